@@ -1,0 +1,90 @@
+"""ctypes binding of libapcost.so (see include/apcost.h for the contract).
+
+There is no CPU fallback: if the library has not been built, or a launch fails,
+a RuntimeError is raised.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+
+from ._build import LIB_PATH
+
+APC_MAX_RANK = 8
+APC_MAX_MESH = 4
+APC_MAX_DTYPES = 8
+APC_TILE_MAX_COLS = 1024
+APC_TILE_MAX_ROWS = 1024
+
+EDGE_GRAD_RESCALE = 1
+EDGE_NO_PRODUCER = 2
+
+
+class ApcParams(ctypes.Structure):
+    _fields_ = [
+        ("mesh_ndim", ctypes.c_int32),
+        ("mesh_size", ctypes.c_int32 * APC_MAX_MESH),
+        ("bw", ctypes.c_double * APC_MAX_MESH),
+        ("lat", ctypes.c_double * APC_MAX_MESH),
+        ("base_latency", ctypes.c_double),
+        ("a2a_scale", ctypes.c_double),
+        ("hbm_bw", ctypes.c_double),
+        ("rw_eff", ctypes.c_double),
+        ("launch_floor", ctypes.c_double),
+        ("compute_eff", ctypes.c_double),
+        ("rescale", ctypes.c_double),
+        ("gpu_flops", ctypes.c_double * APC_MAX_DTYPES),
+        ("transition_scale", ctypes.c_int32),
+    ]
+
+
+EXPORTS = (
+    "apc_version",
+    "apc_last_error",
+    "apc_validate_tables_host",
+    "apc_tensor_tables",
+    "apc_spec_tables",
+    "apc_compute_costs",
+    "apc_redistribute_tables",
+    "apc_segmented_min",
+)
+
+_lib = None
+
+
+def library_path() -> str:
+    return LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    """Loads the built library; raises if it is missing (build it with
+    ``python -m autoparallel_amd._build`` or ``__graft_entry__.build()``)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: the HIP library has not been built "
+                "(run `python -m autoparallel_amd._build`). There is no CPU fallback."
+            )
+        l = ctypes.CDLL(LIB_PATH)
+        for name in EXPORTS:
+            if not hasattr(l, name):
+                raise RuntimeError(f"{LIB_PATH} does not export {name}")
+        l.apc_last_error.restype = ctypes.c_char_p
+        for name in EXPORTS:
+            if name != "apc_last_error":
+                getattr(l, name).restype = ctypes.c_int
+        _lib = l
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = lib().apc_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what} failed ({rc}): {msg}")
+
+
+def vp(ptr) -> ctypes.c_void_p:
+    """int / None -> void*"""
+    return ctypes.c_void_p(ptr if ptr else None)

@@ -1,0 +1,546 @@
+// apcost — sharding-cost evaluation kernels for MI355X (gfx950) and their C ABI.
+//
+// Built with -ffp-contract=off: every fp64 operation below is a single IEEE
+// rounding in the order the reference's Python evaluates it, so results are
+// bit-identical to CPython's floats rather than merely close.
+//
+// Reference functions restated here (batched over the whole graph):
+//   autoparallel/collective_runtime_estimation.py:22-153
+//   autoparallel/compute_estimation.py:211-229, 302-365
+//   autoparallel/optimize_sharding.py:306-379
+//   torch/distributed/tensor/_collective_utils.py:230-313
+//   torch/_prims_common/__init__.py:252-292
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "apcost.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(-3, "%s: %s", what, hipGetErrorString(e));
+  return 0;
+}
+
+constexpr int kBlock = 256;
+
+// ------------------------------------------------------------------------------------------
+// placement codes
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ int kind_of(uint32_t c) { return (int)(c >> 6); }  // 0 R, 1 P, 2 S
+__device__ __forceinline__ int dim_of(uint32_t c) { return (int)(c & 0x0F); }
+
+// compute_estimation.py:302-314
+__device__ __forceinline__ double rw_time(double bytes, const apc_params &p) {
+  double t = bytes / p.hbm_bw * 1e6;
+  t = t / p.rw_eff;
+  return t > p.launch_floor ? t : p.launch_floor;
+}
+
+// torch _collective_utils.py:281-313: latency + bandwidth term of a ring collective
+__device__ __forceinline__ double ring(double gb, const apc_params &p, int d, int hops) {
+  double latency = p.base_latency + (double)hops * p.lat[d];
+  double bw = (gb * (double)hops / (double)p.mesh_size[d]) / p.bw[d];
+  return latency + bw * 1e6;
+}
+
+// collective_runtime_estimation.py:37-153 for one (producer spec, consumer spec) pair.
+// gb = bytes / num_shards / 1024^3 of the producer spec, cont = global contiguity.
+template <int M>
+__device__ __forceinline__ double entry_cost(uint32_t srcp, uint32_t tgtp, double gb, bool cont,
+                                             const apc_params &p) {
+  if (srcp == 0u) {  // fully replicated producer (:56-62)
+    bool tgt_partial = false;
+#pragma unroll
+    for (int i = 0; i < M; ++i) tgt_partial |= kind_of((tgtp >> (8 * i)) & 0xFF) == 1;
+    return tgt_partial ? INFINITY : 0.0;
+  }
+  bool flip = false;
+  if (M == 2) {  // :146-151
+    flip = srcp == 0x4040u && kind_of(tgtp & 0xFF) == 2 && kind_of((tgtp >> 8) & 0xFF) == 2;
+  }
+  double cost = 0.0;
+#pragma unroll
+  for (int k = 0; k < M; ++k) {
+    const int i = (M == 2 && flip) ? 1 - k : k;
+    const uint32_t c = (srcp >> (8 * i)) & 0xFF, t = (tgtp >> (8 * i)) & 0xFF;
+    if (c == t) continue;
+    const double n = (double)p.mesh_size[i];
+    if (!cont) cost += rw_time(gb * 2 * 1073741824.0, p);
+    const int ck = kind_of(c), tk = kind_of(t);
+    if (ck == 2 && tk == 0) {  // all-gather (:83-96)
+      gb *= n;
+      cost += ring(gb, p, i, p.mesh_size[i] - 1);
+      if (dim_of(c) != 0) cost += rw_time(gb * 2 * 1073741824.0, p);
+    } else if (ck == 2 && tk == 2) {  // all-to-all (:97-113)
+      double a2a = ring(gb, p, i, p.mesh_size[i] - 1);
+      a2a *= p.a2a_scale;
+      cost += a2a;
+      const int copies = (dim_of(c) != 0) + (dim_of(t) != 0);
+      cost += (double)copies * rw_time(gb * 2 * 1073741824.0, p);
+    } else if (ck == 1 && tk == 0) {  // all-reduce (:115-117)
+      cost += ring(gb, p, i, 2 * (p.mesh_size[i] - 1));
+    } else if (ck == 1 && tk == 2) {  // reduce-scatter (:118-130)
+      cost += ring(gb, p, i, p.mesh_size[i] - 1);
+      if (dim_of(t) != 0) cost += rw_time(gb * 2 * 1073741824.0, p);
+      gb /= n;
+    } else if (tk == 1 && ck != 1) {  // Shard->Partial, Replicate->Partial banned (:131-138)
+      return INFINITY;
+    }
+    cont = true;  // :141
+  }
+  return cost;
+}
+
+// ------------------------------------------------------------------------------------------
+// a7: bytes + contiguity per tensor
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void tensor_tables_kernel(int64_t n, const int32_t *__restrict__ rank,
+                                                               const int32_t *__restrict__ itemsize,
+                                                               const int64_t *__restrict__ shape,
+                                                               const int64_t *__restrict__ stride,
+                                                               int64_t *__restrict__ bytes,
+                                                               uint8_t *__restrict__ cont) {
+  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (t >= n) return;
+  const int r = rank[t];
+  const int64_t *sh = shape + t * APC_MAX_RANK;
+  const int64_t *st = stride + t * APC_MAX_RANK;
+  int64_t nbytes = itemsize[t];
+  int64_t expected = 1, expected_max = 1;
+  bool ok = true;
+  for (int i = r - 1; i >= 0; --i) {
+    const int64_t x = sh[i], y = st[i];
+    nbytes *= x;
+    if (x == 1) continue;
+    if (y != expected && y != expected_max) ok = false;
+    expected_max *= (x > 1 ? x : 1);
+    expected *= x;
+  }
+  bytes[t] = nbytes;
+  cont[t] = ok ? 1 : 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// a8: local shard shape / stride / counts per spec
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void spec_tables_kernel(
+    apc_params p, int64_t n, const uint32_t *__restrict__ codes, const int32_t *__restrict__ tensor,
+    const int32_t *__restrict__ rank, const int32_t *__restrict__ itemsize,
+    const int64_t *__restrict__ shape, const int64_t *__restrict__ stride, int64_t *__restrict__ shards,
+    int64_t *__restrict__ lshape, int64_t *__restrict__ lstride, int64_t *__restrict__ lnumel,
+    int64_t *__restrict__ lbytes) {
+  const int64_t s = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (s >= n) return;
+  int64_t sh[APC_MAX_RANK], st[APC_MAX_RANK];
+#pragma unroll
+  for (int i = 0; i < APC_MAX_RANK; ++i) sh[i] = st[i] = 0;
+  const int t = tensor[s];
+  int64_t nsh = 0, ne = 0, nb = 0;
+  if (t >= 0) {
+    const int r = rank[t];
+#pragma unroll
+    for (int i = 0; i < APC_MAX_RANK; ++i) {
+      if (i < r) {
+        sh[i] = shape[(int64_t)t * APC_MAX_RANK + i];
+        st[i] = stride[(int64_t)t * APC_MAX_RANK + i];
+      }
+    }
+    nsh = 1;
+    const uint32_t pc = codes[s];
+    for (int i = 0; i < p.mesh_ndim; ++i) {
+      const uint32_t c = (pc >> (8 * i)) & 0xFF;
+      if (kind_of(c) == 2) {
+        const int d = dim_of(c);
+        const int64_t m = p.mesh_size[i];
+        nsh *= m;
+        // compile-time indices keep sh/st in registers
+#pragma unroll
+        for (int j = 0; j < APC_MAX_RANK; ++j) {
+          if (j == d) sh[j] = (sh[j] + m - 1) / m;
+          if (j == d - 1 && d - 1 > 0) st[j] = (st[j] + m - 1) / m;  // compute_estimation.py:225-228
+        }
+      }
+    }
+    ne = 1;
+#pragma unroll
+    for (int i = 0; i < APC_MAX_RANK; ++i)
+      if (i < r) ne *= sh[i];
+    nb = ne * itemsize[t];
+  }
+  shards[s] = nsh;
+  lnumel[s] = ne;
+  lbytes[s] = nb;
+#pragma unroll
+  for (int i = 0; i < APC_MAX_RANK; ++i) {
+    lshape[s * APC_MAX_RANK + i] = sh[i];
+    lstride[s * APC_MAX_RANK + i] = st[i];
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// a9/a10: compute-cost tail per (node, strategy)
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void compute_costs_kernel(
+    apc_params p, int64_t n, const int64_t *__restrict__ flops, const int64_t *__restrict__ rw_bytes,
+    const int8_t *__restrict__ dtype, const uint8_t *__restrict__ zero_cost,
+    const int32_t *__restrict__ num_args, double *__restrict__ compute, double *__restrict__ per_arg,
+    int32_t *__restrict__ error_flag) {
+  const int64_t s = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (s >= n) return;
+  double c = 0.0;
+  if (!zero_cost[s]) {
+    const double rw = rw_time((double)rw_bytes[s], p);
+    const int64_t f = flops[s];
+    if (f == 0) {
+      c = rw;
+    } else {
+      const int dt = dtype[s];
+      const double gf = (dt >= 0 && dt < APC_MAX_DTYPES) ? p.gpu_flops[dt] : 0.0;
+      if (gf == 0.0) {
+        if (error_flag) *error_flag = 1;  // compute_estimation.py:198-201 raises ValueError
+        c = NAN;
+      } else {
+        double t = (double)f / gf * 1e6;
+        t = t / p.compute_eff;
+        c = t > rw ? t : rw;
+      }
+    }
+  }
+  if (compute) compute[s] = c;
+  if (per_arg) per_arg[s] = c / (double)num_args[s];
+}
+
+// ------------------------------------------------------------------------------------------
+// a1-a6: redistribution-cost matrices, one workgroup per tile of one edge's matrix.
+// Producer specs (columns) and consumer specs (rows) of the tile are staged in LDS once;
+// every lane then walks the tile's entries with stride kBlock so that a wavefront
+// writes 64 consecutive fp64 values of a row.
+// ------------------------------------------------------------------------------------------
+struct TableArgs {
+  const int64_t *tensor_bytes;
+  const uint8_t *tensor_contiguous;
+  const uint32_t *spec_codes;
+  const int32_t *spec_tensor;
+  const int32_t *edge_src_begin;
+  const int32_t *edge_n_src;
+  const int32_t *edge_tgt_begin;
+  const int32_t *edge_n_tgt;
+  const int32_t *edge_flags;
+  const int64_t *edge_pt_begin;
+  const int64_t *edge_entry_begin;
+  const int32_t *edge_strat_begin;
+  const double *pt_values;
+  const double *per_arg;
+  const int32_t *tile_edge;
+  const int32_t *tile_row_begin;
+  const int32_t *tile_row_count;
+  const int32_t *tile_col_begin;
+  const int32_t *tile_col_count;
+  double *comm_out;
+  uint8_t *trans_out;
+  double *cost_out;
+};
+
+template <int M>
+__global__ __launch_bounds__(kBlock) void redistribute_tiles_kernel(apc_params p, TableArgs a) {
+  __shared__ double s_gb[APC_TILE_MAX_COLS];
+  __shared__ uint32_t s_src[APC_TILE_MAX_COLS];
+  __shared__ uint8_t s_sflag[APC_TILE_MAX_COLS];  // bit0 valid spec, bit1 contiguous
+  __shared__ uint32_t s_tgt[APC_TILE_MAX_ROWS];
+  __shared__ uint8_t s_tflag[APC_TILE_MAX_ROWS];
+  __shared__ double s_cpa[APC_TILE_MAX_ROWS];
+
+  const int tile = blockIdx.x;
+  const int e = a.tile_edge[tile];
+  const int row0 = a.tile_row_begin[tile], rows = a.tile_row_count[tile];
+  const int col0 = a.tile_col_begin[tile], cols = a.tile_col_count[tile];
+  const int n_src = a.edge_n_src[e];
+  const int src_begin = a.edge_src_begin[e], tgt_begin = a.edge_tgt_begin[e];
+  const int flags = a.edge_flags[e];
+  const int64_t entry_begin = a.edge_entry_begin[e];
+  const int64_t pt_begin = a.edge_pt_begin[e];
+  const int strat_begin = a.edge_strat_begin[e];
+  const int tid = threadIdx.x;
+
+  for (int j = tid; j < cols; j += kBlock) {
+    const int sp = src_begin + col0 + j;
+    const uint32_t codes = a.spec_codes[sp];
+    const int t = a.spec_tensor[sp];
+    uint8_t f = 0;
+    double gb = 0.0;
+    if (t >= 0) {
+      int64_t shards = 1;
+#pragma unroll
+      for (int i = 0; i < M; ++i)
+        if (kind_of((codes >> (8 * i)) & 0xFF) == 2) shards *= p.mesh_size[i];
+      // collective_runtime_estimation.py:66-68
+      gb = (double)a.tensor_bytes[t] / (double)shards / 1024 / 1024 / 1024;
+      f = 1 | (a.tensor_contiguous[t] ? 2 : 0);
+    }
+    s_gb[j] = gb;
+    s_src[j] = codes;
+    s_sflag[j] = f;
+  }
+  for (int j = tid; j < rows; j += kBlock) {
+    const int ts = tgt_begin + row0 + j;
+    s_tgt[j] = a.spec_codes[ts];
+    s_tflag[j] = a.spec_tensor[ts] >= 0 ? 1 : 0;
+    s_cpa[j] = a.per_arg ? a.per_arg[strat_begin + row0 + j] : 0.0;
+  }
+  __syncthreads();
+
+  const int n = rows * cols;
+  int r = tid / cols, c = tid - r * cols;
+  const int dr = kBlock / cols, dc = kBlock - dr * cols;
+  for (int idx = tid; idx < n; idx += kBlock) {
+    const int64_t local = (int64_t)(row0 + r) * n_src + (col0 + c);
+    double comm;
+    int trans = 0;
+    const bool passthrough = (flags & APC_EDGE_NO_PRODUCER) || !(s_sflag[c] & 1) || !s_tflag[r];
+    if (passthrough) {
+      comm = a.pt_values[pt_begin + local];
+    } else {
+      const uint32_t src = s_src[c], tgt = s_tgt[r];
+      comm = entry_cost<M>(src, tgt, s_gb[c], (s_sflag[c] & 2) != 0, p);
+      trans = (src != tgt) ? p.transition_scale : 0;  // optimize_sharding.py:345-351
+    }
+    if (flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;  // :358-359
+    const int64_t o = entry_begin + local;
+    if (a.comm_out) a.comm_out[o] = comm;
+    if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
+    if (a.cost_out) a.cost_out[o] = comm + s_cpa[r] + (double)trans;  // :368-372
+    c += dc;
+    r += dr;
+    if (c >= cols) {
+      c -= cols;
+      r += 1;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// a14: segmented min + first argmin, one wavefront per segment
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void segmented_min_kernel(const double *__restrict__ values,
+                                                               const int64_t *__restrict__ seg_ptr,
+                                                               int64_t n_seg, double *__restrict__ mins,
+                                                               int32_t *__restrict__ args) {
+  const int lane = threadIdx.x & 63;
+  const int64_t seg = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (seg >= n_seg) return;
+  const int64_t lo = seg_ptr[seg], hi = seg_ptr[seg + 1];
+  double best = INFINITY;
+  int64_t arg = INT64_MAX;  // absolute index; INT64_MAX = none seen
+  for (int64_t j = lo + lane; j < hi; j += 64) {
+    const double v = values[j];
+    if (arg == INT64_MAX || v < best) {
+      best = v;
+      arg = j;
+    }
+  }
+  // lexicographic (value, index) min across the wavefront; lanes that saw nothing lose
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const double ob = __shfl_xor(best, off, 64);
+    const int64_t oa = __shfl_xor(arg, off, 64);
+    const bool take = (oa != INT64_MAX) && (arg == INT64_MAX || ob < best || (ob == best && oa < arg));
+    if (take) {
+      best = ob;
+      arg = oa;
+    }
+  }
+  if (lane == 0) {
+    mins[seg] = best;
+    args[seg] = arg == INT64_MAX ? -1 : (int32_t)(arg - lo);
+  }
+}
+
+inline unsigned blocks_for(int64_t n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
+
+int check_params(const apc_params *p) {
+  if (!p) return fail(-1, "params is NULL");
+  if (p->mesh_ndim < 1 || p->mesh_ndim > APC_MAX_MESH)
+    return fail(-1, "mesh_ndim %d outside [1, %d]", p->mesh_ndim, APC_MAX_MESH);
+  for (int i = 0; i < p->mesh_ndim; ++i)
+    if (p->mesh_size[i] < 1) return fail(-1, "mesh_size[%d] = %d must be >= 1", i, p->mesh_size[i]);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int apc_version(void) { return 1; }
+
+const char *apc_last_error(void) { return g_err; }
+
+int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
+                             int64_t n_specs, const uint32_t *spec_codes, const int32_t *spec_tensor,
+                             int64_t n_edges, const int32_t *edge_src_begin, const int32_t *edge_n_src,
+                             const int32_t *edge_tgt_begin, const int32_t *edge_n_tgt,
+                             const int32_t *edge_flags, const int64_t *edge_pt_begin,
+                             const int64_t *edge_entry_begin, const int32_t *edge_strat_begin, int64_t n_pt,
+                             int64_t n_strategies, int64_t n_tiles, const int32_t *tile_edge,
+                             const int32_t *tile_row_begin, const int32_t *tile_row_count,
+                             const int32_t *tile_col_begin, const int32_t *tile_col_count) {
+  if (int rc = check_params(params)) return rc;
+  const int M = params->mesh_ndim;
+  for (int64_t t = 0; t < n_tensors; ++t)
+    if (tensor_rank[t] < 0 || tensor_rank[t] > APC_MAX_RANK)
+      return fail(-2, "tensor %lld: rank %d outside [0, %d]", (long long)t, tensor_rank[t], APC_MAX_RANK);
+  for (int64_t s = 0; s < n_specs; ++s) {
+    const int t = spec_tensor[s];
+    if (t < -1 || t >= n_tensors)
+      return fail(-2, "spec %lld: tensor row %d out of range [-1, %lld)", (long long)s, t, (long long)n_tensors);
+    if (M < 4 && (spec_codes[s] >> (8 * M)) != 0)
+      return fail(-2, "spec %lld: placement bytes beyond mesh ndim %d are set (0x%08x)", (long long)s, M,
+                  spec_codes[s]);
+    for (int i = 0; i < M; ++i) {
+      const uint32_t c = (spec_codes[s] >> (8 * i)) & 0xFF;
+      if ((c >> 6) == 3) return fail(-2, "spec %lld: placement code 0x%02x has no meaning", (long long)s, c);
+      if ((c >> 6) == 0 && c != 0) return fail(-2, "spec %lld: placement code 0x%02x has no meaning", (long long)s, c);
+      if ((c >> 6) == 2 && t >= 0 && (int)(c & 0x0F) >= tensor_rank[t])
+        return fail(-2, "spec %lld: Shard(%d) on a rank-%d tensor", (long long)s, (int)(c & 0x0F), tensor_rank[t]);
+    }
+  }
+  int64_t expect = 0;
+  for (int64_t e = 0; e < n_edges; ++e) {
+    if (edge_entry_begin[e] != expect)
+      return fail(-2, "edge %lld: entry_begin %lld, expected %lld (offsets must be the running sum of n_tgt*n_src)",
+                  (long long)e, (long long)edge_entry_begin[e], (long long)expect);
+    const int64_t ns = edge_n_src[e], nt = edge_n_tgt[e];
+    if (ns < 0 || nt < 0) return fail(-2, "edge %lld: negative strategy count", (long long)e);
+    if (edge_src_begin[e] < 0 || edge_src_begin[e] + ns > n_specs)
+      return fail(-2, "edge %lld: producer spec range [%d, +%lld) outside the spec table", (long long)e,
+                  edge_src_begin[e], (long long)ns);
+    if (edge_tgt_begin[e] < 0 || edge_tgt_begin[e] + nt > n_specs)
+      return fail(-2, "edge %lld: consumer spec range [%d, +%lld) outside the spec table", (long long)e,
+                  edge_tgt_begin[e], (long long)nt);
+    if (edge_strat_begin[e] < 0 || edge_strat_begin[e] + nt > n_strategies)
+      return fail(-2, "edge %lld: strategy rows [%d, +%lld) outside the strategy table", (long long)e,
+                  edge_strat_begin[e], (long long)nt);
+    bool needs_pt = (edge_flags[e] & APC_EDGE_NO_PRODUCER) != 0;
+    if (!needs_pt) {
+      for (int64_t j = 0; j < ns && !needs_pt; ++j) needs_pt = spec_tensor[edge_src_begin[e] + j] < 0;
+      for (int64_t j = 0; j < nt && !needs_pt; ++j) needs_pt = spec_tensor[edge_tgt_begin[e] + j] < 0;
+    }
+    if (needs_pt && (edge_pt_begin[e] < 0 || edge_pt_begin[e] + ns * nt > n_pt))
+      return fail(-2, "edge %lld: pass-through values [%lld, +%lld) outside pt_values", (long long)e,
+                  (long long)edge_pt_begin[e], (long long)(ns * nt));
+    expect += ns * nt;
+  }
+  if (edge_entry_begin[n_edges] != expect)
+    return fail(-2, "entry_begin[n_edges] = %lld, expected %lld", (long long)edge_entry_begin[n_edges],
+                (long long)expect);
+  for (int64_t t = 0; t < n_tiles; ++t) {
+    const int e = tile_edge[t];
+    if (e < 0 || e >= n_edges) return fail(-2, "tile %lld: edge %d out of range", (long long)t, e);
+    if (tile_row_count[t] < 1 || tile_row_count[t] > APC_TILE_MAX_ROWS || tile_row_begin[t] < 0 ||
+        tile_row_begin[t] + tile_row_count[t] > edge_n_tgt[e])
+      return fail(-2, "tile %lld: rows [%d, +%d) outside edge %d (n_tgt %d, max %d per tile)", (long long)t,
+                  tile_row_begin[t], tile_row_count[t], e, edge_n_tgt[e], APC_TILE_MAX_ROWS);
+    if (tile_col_count[t] < 1 || tile_col_count[t] > APC_TILE_MAX_COLS || tile_col_begin[t] < 0 ||
+        tile_col_begin[t] + tile_col_count[t] > edge_n_src[e])
+      return fail(-2, "tile %lld: cols [%d, +%d) outside edge %d (n_src %d, max %d per tile)", (long long)t,
+                  tile_col_begin[t], tile_col_count[t], e, edge_n_src[e], APC_TILE_MAX_COLS);
+  }
+  return 0;
+}
+
+int apc_tensor_tables(int64_t n, const int32_t *rank, const int32_t *itemsize, const int64_t *shape,
+                      const int64_t *stride, int64_t *bytes, uint8_t *cont, void *stream) {
+  if (n < 0) return fail(-1, "n_tensors < 0");
+  if (n == 0) return 0;
+  if (!rank || !itemsize || !shape || !stride || !bytes || !cont) return fail(-1, "apc_tensor_tables: NULL array");
+  hipLaunchKernelGGL(tensor_tables_kernel, dim3(blocks_for(n, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, n,
+                     rank, itemsize, shape, stride, bytes, cont);
+  return check_launch("apc_tensor_tables");
+}
+
+int apc_spec_tables(const apc_params *params, int64_t n, const uint32_t *codes, const int32_t *tensor,
+                    const int32_t *rank, const int32_t *itemsize, const int64_t *shape, const int64_t *stride,
+                    int64_t *shards, int64_t *lshape, int64_t *lstride, int64_t *lnumel, int64_t *lbytes,
+                    void *stream) {
+  if (int rc = check_params(params)) return rc;
+  if (n < 0) return fail(-1, "n_specs < 0");
+  if (n == 0) return 0;
+  if (!codes || !tensor || !rank || !itemsize || !shape || !stride || !shards || !lshape || !lstride || !lnumel ||
+      !lbytes)
+    return fail(-1, "apc_spec_tables: NULL array");
+  hipLaunchKernelGGL(spec_tables_kernel, dim3(blocks_for(n, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, *params,
+                     n, codes, tensor, rank, itemsize, shape, stride, shards, lshape, lstride, lnumel, lbytes);
+  return check_launch("apc_spec_tables");
+}
+
+int apc_compute_costs(const apc_params *params, int64_t n, const int64_t *flops, const int64_t *rw_bytes,
+                      const int8_t *dtype, const uint8_t *zero_cost, const int32_t *num_args, double *compute,
+                      double *per_arg, int32_t *error_flag, void *stream) {
+  if (int rc = check_params(params)) return rc;
+  if (n < 0) return fail(-1, "n_strategies < 0");
+  if (n == 0) return 0;
+  if (!flops || !rw_bytes || !dtype || !zero_cost || !num_args) return fail(-1, "apc_compute_costs: NULL input");
+  hipLaunchKernelGGL(compute_costs_kernel, dim3(blocks_for(n, kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
+                     *params, n, flops, rw_bytes, dtype, zero_cost, num_args, compute, per_arg, error_flag);
+  return check_launch("apc_compute_costs");
+}
+
+int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes, const uint8_t *tensor_contiguous,
+                            const uint32_t *spec_codes, const int32_t *spec_tensor, const int32_t *edge_src_begin,
+                            const int32_t *edge_n_src, const int32_t *edge_tgt_begin, const int32_t *edge_n_tgt,
+                            const int32_t *edge_flags, const int64_t *edge_pt_begin, const int64_t *edge_entry_begin,
+                            const int32_t *edge_strat_begin, const double *pt_values, const double *per_arg,
+                            int64_t n_tiles, const int32_t *tile_edge, const int32_t *tile_row_begin,
+                            const int32_t *tile_row_count, const int32_t *tile_col_begin,
+                            const int32_t *tile_col_count, double *comm_out, uint8_t *trans_out, double *cost_out,
+                            void *stream) {
+  if (int rc = check_params(params)) return rc;
+  if (n_tiles < 0 || n_tiles > INT32_MAX) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
+  if (n_tiles == 0) return 0;
+  if (!tensor_bytes || !tensor_contiguous || !spec_codes || !spec_tensor || !edge_src_begin || !edge_n_src ||
+      !edge_tgt_begin || !edge_n_tgt || !edge_flags || !edge_pt_begin || !edge_entry_begin || !edge_strat_begin ||
+      !tile_edge || !tile_row_begin || !tile_row_count || !tile_col_begin || !tile_col_count)
+    return fail(-1, "apc_redistribute_tables: NULL table");
+  if (cost_out && !per_arg) return fail(-1, "cost_out needs compute_cost_per_arg");
+  TableArgs a{tensor_bytes, tensor_contiguous, spec_codes,      spec_tensor,    edge_src_begin, edge_n_src,
+              edge_tgt_begin, edge_n_tgt,      edge_flags,      edge_pt_begin,  edge_entry_begin, edge_strat_begin,
+              pt_values,    per_arg,           tile_edge,       tile_row_begin, tile_row_count, tile_col_begin,
+              tile_col_count, comm_out,        trans_out,       cost_out};
+  const dim3 grid((unsigned)n_tiles), block(kBlock);
+  hipStream_t s = (hipStream_t)stream;
+  switch (params->mesh_ndim) {
+    case 1: hipLaunchKernelGGL(redistribute_tiles_kernel<1>, grid, block, 0, s, *params, a); break;
+    case 2: hipLaunchKernelGGL(redistribute_tiles_kernel<2>, grid, block, 0, s, *params, a); break;
+    case 3: hipLaunchKernelGGL(redistribute_tiles_kernel<3>, grid, block, 0, s, *params, a); break;
+    default: hipLaunchKernelGGL(redistribute_tiles_kernel<4>, grid, block, 0, s, *params, a); break;
+  }
+  return check_launch("apc_redistribute_tables");
+}
+
+int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_seg, double *mins, int32_t *args,
+                      void *stream) {
+  if (n_seg < 0) return fail(-1, "n_segments < 0");
+  if (n_seg == 0) return 0;
+  if (!seg_ptr || !mins || !args) return fail(-1, "apc_segmented_min: NULL array");
+  hipLaunchKernelGGL(segmented_min_kernel, dim3(blocks_for(n_seg, kBlock / 64)), dim3(kBlock), 0,
+                     (hipStream_t)stream, values, seg_ptr, n_seg, mins, args);
+  return check_launch("apc_segmented_min");
+}
+
+}  // extern "C"

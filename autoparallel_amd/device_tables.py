@@ -1,0 +1,174 @@
+"""Device-resident cost tables: uploads a ``CostTables`` encoding to HBM once and
+runs the HIP kernels of libapcost.so over it through the C ABI.
+
+torch is used for device memory and the current HIP stream only; every
+computation is a kernel of the library.  Without a HIP device (or without the
+built library) construction raises: there is no CPU path.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _native
+from ._native import APC_MAX_RANK, vp
+from .cost_model import CostModelParams
+from .encoding import CostTables
+
+_UPLOAD = (
+    "tensor_rank", "tensor_itemsize", "tensor_shape", "tensor_stride", "spec_codes", "spec_tensor",
+    "strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "strat_num_args",
+    "edge_src_begin", "edge_n_src", "edge_tgt_begin", "edge_n_tgt", "edge_flags", "edge_pt_begin",
+    "edge_entry_begin", "edge_strat_begin", "pt_values", "tile_edge", "tile_row_begin", "tile_row_count",
+    "tile_col_begin", "tile_col_count",
+)
+
+
+def _to_device(a: np.ndarray, device) -> torch.Tensor:
+    if a.dtype == np.uint32:  # same bits; torch's uint32 support is partial
+        a = a.view(np.int32)
+    if a.size == 0:
+        return torch.empty(a.shape, dtype=torch.from_numpy(np.zeros(1, a.dtype)).dtype, device=device)
+    return torch.from_numpy(a).to(device, non_blocking=False)
+
+
+class DeviceCostTables:
+    def __init__(self, tables: CostTables, params: CostModelParams, device="cuda:0", validate=True):
+        if not torch.cuda.is_available():
+            raise RuntimeError("DeviceCostTables needs a HIP device; there is no CPU path")
+        self.lib = _native.lib()
+        self.tables = tables
+        self.params = params
+        self.device = torch.device(device)
+        if validate:
+            tables.validate(params)
+        self.c_params = params.to_c()
+        with torch.cuda.device(self.device):
+            self.d = {k: _to_device(getattr(tables, k), self.device) for k in _UPLOAD}
+        self.tensor_bytes = None
+        self.tensor_contiguous = None
+        self.compute_cost = None
+        self.compute_cost_per_arg = None
+        self.comm = None
+        self.transition = None
+        self.cost = None
+
+    # ---- helpers -------------------------------------------------------------------------
+    def _stream(self):
+        return vp(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _p(self, key):
+        t = self.d[key] if isinstance(key, str) else key
+        return vp(t.data_ptr() if t is not None and t.numel() else 0)
+
+    def _empty(self, shape, dtype):
+        return torch.empty(shape, dtype=dtype, device=self.device)
+
+    # ---- integer tables ------------------------------------------------------------------
+    def run_tensor_tables(self):
+        n = self.tables.n_tensors
+        self.tensor_bytes = self._empty((n,), torch.int64)
+        self.tensor_contiguous = self._empty((n,), torch.uint8)
+        with torch.cuda.device(self.device):
+            rc = self.lib.apc_tensor_tables(
+                ctypes.c_int64(n), self._p("tensor_rank"), self._p("tensor_itemsize"), self._p("tensor_shape"),
+                self._p("tensor_stride"), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
+                self._stream())
+        _native.check(rc, "apc_tensor_tables")
+        return self.tensor_bytes, self.tensor_contiguous
+
+    def run_spec_tables(self):
+        n = self.tables.n_specs
+        out = {
+            "num_shards": self._empty((n,), torch.int64),
+            "local_shape": self._empty((n, APC_MAX_RANK), torch.int64),
+            "local_stride": self._empty((n, APC_MAX_RANK), torch.int64),
+            "local_numel": self._empty((n,), torch.int64),
+            "local_bytes": self._empty((n,), torch.int64),
+        }
+        with torch.cuda.device(self.device):
+            rc = self.lib.apc_spec_tables(
+                ctypes.byref(self.c_params), ctypes.c_int64(n), self._p("spec_codes"), self._p("spec_tensor"),
+                self._p("tensor_rank"), self._p("tensor_itemsize"), self._p("tensor_shape"),
+                self._p("tensor_stride"), self._p(out["num_shards"]), self._p(out["local_shape"]),
+                self._p(out["local_stride"]), self._p(out["local_numel"]), self._p(out["local_bytes"]),
+                self._stream())
+        _native.check(rc, "apc_spec_tables")
+        self.spec_out = out
+        return out
+
+    # ---- per-strategy compute cost ---------------------------------------------------------
+    def run_compute_costs(self):
+        n = self.tables.n_strategies
+        self.compute_cost = self._empty((n,), torch.float64)
+        self.compute_cost_per_arg = self._empty((n,), torch.float64)
+        err = torch.zeros((1,), dtype=torch.int32, device=self.device)
+        with torch.cuda.device(self.device):
+            rc = self.lib.apc_compute_costs(
+                ctypes.byref(self.c_params), ctypes.c_int64(n), self._p("strat_flops"), self._p("strat_rw_bytes"),
+                self._p("strat_dtype"), self._p("strat_zero_cost"), self._p("strat_num_args"),
+                self._p(self.compute_cost), self._p(self.compute_cost_per_arg), self._p(err), self._stream())
+        _native.check(rc, "apc_compute_costs")
+        if int(err.item()) != 0:
+            # compute_estimation.py:198-201
+            raise ValueError(f"a strategy with non-zero flops uses a dtype not supported on {self.params.device_name}")
+        return self.compute_cost, self.compute_cost_per_arg
+
+    # ---- redistribution-cost matrices ------------------------------------------------------
+    def alloc_outputs(self, comm=True, transition=True, cost=True):
+        n = self.tables.n_entries
+        self.comm = self._empty((n,), torch.float64) if comm else None
+        self.transition = self._empty((n,), torch.uint8) if transition else None
+        self.cost = self._empty((n,), torch.float64) if cost else None
+
+    def launch_redistribute_tables(self):
+        """One enqueue of the table kernel over pre-allocated outputs (no allocation,
+        no synchronisation): the timed unit of the benchmark."""
+        with torch.cuda.device(self.device):
+            rc = self.lib.apc_redistribute_tables(
+                ctypes.byref(self.c_params), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
+                self._p("spec_codes"), self._p("spec_tensor"), self._p("edge_src_begin"), self._p("edge_n_src"),
+                self._p("edge_tgt_begin"), self._p("edge_n_tgt"), self._p("edge_flags"), self._p("edge_pt_begin"),
+                self._p("edge_entry_begin"), self._p("edge_strat_begin"), self._p("pt_values"),
+                self._p(self.compute_cost_per_arg), ctypes.c_int64(self.tables.n_tiles), self._p("tile_edge"),
+                self._p("tile_row_begin"), self._p("tile_row_count"), self._p("tile_col_begin"),
+                self._p("tile_col_count"), self._p(self.comm), self._p(self.transition), self._p(self.cost),
+                self._stream())
+        _native.check(rc, "apc_redistribute_tables")
+
+    def run_redistribute_tables(self, comm=True, transition=True, cost=True):
+        if self.tensor_bytes is None:
+            self.run_tensor_tables()
+        if cost and self.compute_cost_per_arg is None:
+            self.run_compute_costs()
+        self.alloc_outputs(comm, transition, cost)
+        self.launch_redistribute_tables()
+        return self.comm, self.transition, self.cost
+
+    def build_all(self):
+        """tensor tables -> compute costs -> cost matrices, all on the current stream."""
+        self.run_tensor_tables()
+        self.run_compute_costs()
+        return self.run_redistribute_tables()
+
+    # ---- segmented min ---------------------------------------------------------------------
+    def segmented_min(self, values: torch.Tensor, seg_ptr):
+        if not isinstance(seg_ptr, torch.Tensor):
+            seg_ptr = torch.from_numpy(np.ascontiguousarray(seg_ptr, dtype=np.int64)).to(self.device)
+        if values.dtype != torch.float64 or seg_ptr.dtype != torch.int64:
+            raise TypeError("segmented_min takes float64 values and an int64 segment pointer")
+        if not (values.is_contiguous() and seg_ptr.is_contiguous()):
+            raise ValueError("segmented_min takes contiguous arrays")
+        n_seg = seg_ptr.numel() - 1
+        if n_seg < 0:
+            raise ValueError("seg_ptr must have at least one element")
+        mins = self._empty((n_seg,), torch.float64)
+        args = self._empty((n_seg,), torch.int32)
+        with torch.cuda.device(self.device):
+            rc = self.lib.apc_segmented_min(self._p(values), self._p(seg_ptr), ctypes.c_int64(n_seg),
+                                            self._p(mins), self._p(args), self._stream())
+        _native.check(rc, "apc_segmented_min")
+        return mins, args

@@ -1,0 +1,279 @@
+"""Flattened strategy / placement encoding: the object graph
+``dict[Node, OpStrategy] -> OpSpec -> DTensorSpec`` that the reference walks in
+``ShardingOptimizer.build_ds`` (autoparallel/optimize_sharding.py:270-380; types at
+torch/distributed/tensor/_op_schema.py:94-141) laid out as CSR arrays over tensors,
+specs, strategies, edges and entries, ready to sit in HBM.
+
+Layout
+------
+tensor table   one row per distinct (shape, stride, dtype): ``tensor_rank``,
+               ``tensor_itemsize``, ``tensor_shape[T, 8]``, ``tensor_stride[T, 8]``.
+spec table     one row per DTensorSpec occurrence: ``spec_codes`` (uint32, byte i =
+               placement code of mesh dim i) and ``spec_tensor`` (row of the tensor
+               table, -1 for "not a DTensorSpec": ``None`` outputs, scalars).
+strategy table one row per (node, strategy): ``strat_flops``, ``strat_rw_bytes``,
+               ``strat_dtype``, ``strat_zero_cost``, ``strat_num_args``;
+               ``node_strat_begin[N + 1]`` is its CSR pointer.
+edge table     one row per (consumer node, argument): producer output specs are spec
+               rows ``[edge_src_begin, +edge_n_src)``, consumer input specs are
+               ``[edge_tgt_begin, +edge_n_tgt)``; the edge's cost matrix occupies
+               entries ``[edge_entry_begin[e], edge_entry_begin[e + 1])``, row-major by
+               consumer strategy (= ``redistribute_cost[argi][ii]`` of strategy ``ss``).
+pt_values      rule-provided costs that survive where either side is not a
+               DTensorSpec (optimize_sharding.py:336-355).
+tiles          rectangles of edge matrices, one per workgroup.
+
+Placement codes: 0x00 Replicate; 0x40|op Partial(op) (op 0 = sum); 0x80|v<<4|d Shard(d)
+with v a variant id (0 = plain ``Shard``).
+"""
+
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass, fields
+
+import numpy as np
+
+from . import _native
+from ._native import APC_MAX_MESH, APC_MAX_RANK, APC_TILE_MAX_COLS, APC_TILE_MAX_ROWS
+
+REPLICATE = 0x00
+PARTIAL_SUM = 0x40
+KIND_REPLICATE, KIND_PARTIAL, KIND_SHARD = 0, 1, 2
+
+# reduce ops of Partial; index = code payload
+PARTIAL_OPS = ("sum", "avg", "min", "max", "product", "band", "bor", "bxor")
+
+EDGE_GRAD_RESCALE = _native.EDGE_GRAD_RESCALE
+EDGE_NO_PRODUCER = _native.EDGE_NO_PRODUCER
+
+DEFAULT_TILE_ENTRIES = 4096
+
+
+def shard_code(dim: int, variant: int = 0) -> int:
+    if not 0 <= dim < 16:
+        raise ValueError(f"Shard dim {dim} outside [0, 16)")
+    if not 0 <= variant < 4:
+        raise ValueError(f"Shard variant {variant} outside [0, 4)")
+    return 0x80 | (variant << 4) | dim
+
+
+def partial_code(op: int | str = 0) -> int:
+    if isinstance(op, str):
+        op = PARTIAL_OPS.index(op)
+    if not 0 <= op < 64:
+        raise ValueError(f"Partial op id {op} outside [0, 64)")
+    return 0x40 | op
+
+
+def code_kind(code: int) -> int:
+    return code >> 6
+
+
+def code_dim(code: int) -> int:
+    return code & 0x0F
+
+
+def pack_codes(codes) -> int:
+    out = 0
+    for i, c in enumerate(codes):
+        out |= (int(c) & 0xFF) << (8 * i)
+    return out
+
+
+def unpack_codes(packed: int, ndim: int) -> tuple:
+    return tuple((int(packed) >> (8 * i)) & 0xFF for i in range(ndim))
+
+
+def _i32(x):
+    return np.ascontiguousarray(x, dtype=np.int32)
+
+
+def _i64(x):
+    return np.ascontiguousarray(x, dtype=np.int64)
+
+
+@dataclass
+class CostTables:
+    mesh_sizes: tuple
+    tensor_rank: np.ndarray
+    tensor_itemsize: np.ndarray
+    tensor_shape: np.ndarray
+    tensor_stride: np.ndarray
+    spec_codes: np.ndarray
+    spec_tensor: np.ndarray
+    strat_flops: np.ndarray
+    strat_rw_bytes: np.ndarray
+    strat_dtype: np.ndarray
+    strat_zero_cost: np.ndarray
+    strat_num_args: np.ndarray
+    node_strat_begin: np.ndarray
+    edge_node: np.ndarray
+    edge_arg: np.ndarray
+    edge_src_begin: np.ndarray
+    edge_n_src: np.ndarray
+    edge_tgt_begin: np.ndarray
+    edge_n_tgt: np.ndarray
+    edge_flags: np.ndarray
+    edge_pt_begin: np.ndarray
+    edge_entry_begin: np.ndarray
+    edge_strat_begin: np.ndarray
+    pt_values: np.ndarray
+    tile_edge: np.ndarray = None
+    tile_row_begin: np.ndarray = None
+    tile_row_count: np.ndarray = None
+    tile_col_begin: np.ndarray = None
+    tile_col_count: np.ndarray = None
+
+    _DTYPES = {
+        "tensor_rank": np.int32, "tensor_itemsize": np.int32, "tensor_shape": np.int64,
+        "tensor_stride": np.int64, "spec_codes": np.uint32, "spec_tensor": np.int32,
+        "strat_flops": np.int64, "strat_rw_bytes": np.int64, "strat_dtype": np.int8,
+        "strat_zero_cost": np.uint8, "strat_num_args": np.int32, "node_strat_begin": np.int64,
+        "edge_node": np.int32, "edge_arg": np.int32, "edge_src_begin": np.int32,
+        "edge_n_src": np.int32, "edge_tgt_begin": np.int32, "edge_n_tgt": np.int32,
+        "edge_flags": np.int32, "edge_pt_begin": np.int64, "edge_entry_begin": np.int64,
+        "edge_strat_begin": np.int32, "pt_values": np.float64, "tile_edge": np.int32,
+        "tile_row_begin": np.int32, "tile_row_count": np.int32, "tile_col_begin": np.int32,
+        "tile_col_count": np.int32,
+    }
+
+    def __post_init__(self):
+        self.mesh_sizes = tuple(int(x) for x in self.mesh_sizes)
+        for name, dt in self._DTYPES.items():
+            v = getattr(self, name)
+            if v is not None:
+                setattr(self, name, np.ascontiguousarray(v, dtype=dt))
+        if self.tensor_shape.ndim != 2 or self.tensor_shape.shape[1] != APC_MAX_RANK:
+            raise ValueError(f"tensor_shape must be [T, {APC_MAX_RANK}]")
+        if self.tensor_stride.shape != self.tensor_shape.shape:
+            raise ValueError("tensor_stride must have the shape of tensor_shape")
+        if self.tile_edge is None:
+            self.build_tiles()
+
+    # ---- sizes -------------------------------------------------------------------------
+    @property
+    def n_tensors(self) -> int:
+        return len(self.tensor_rank)
+
+    @property
+    def n_specs(self) -> int:
+        return len(self.spec_codes)
+
+    @property
+    def n_strategies(self) -> int:
+        return len(self.strat_flops)
+
+    @property
+    def n_nodes(self) -> int:
+        return len(self.node_strat_begin) - 1
+
+    @property
+    def n_edges(self) -> int:
+        return len(self.edge_n_src)
+
+    @property
+    def n_entries(self) -> int:
+        return int(self.edge_entry_begin[-1])
+
+    @property
+    def n_tiles(self) -> int:
+        return len(self.tile_edge)
+
+    def algorithmic_bytes(self, comm=True, transition=True, cost=True) -> int:
+        """Bytes one table build must move at minimum: the outputs written per entry,
+        the placement codes of both spec lists of every edge and a 64-byte edge header."""
+        per_entry = 8 * int(comm) + 1 * int(transition) + 8 * int(cost)
+        m = len(self.mesh_sizes)
+        per_edge = (self.edge_n_src.astype(np.int64) + self.edge_n_tgt.astype(np.int64)) * m + 64
+        return per_entry * self.n_entries + int(per_edge.sum())
+
+    # ---- tiles -------------------------------------------------------------------------
+    def build_tiles(self, tile_entries: int = DEFAULT_TILE_ENTRIES) -> None:
+        """Cuts every edge matrix into rectangles of about ``tile_entries`` entries:
+        whole rows when a row fits the LDS column budget, column chunks otherwise."""
+        ns = self.edge_n_src.astype(np.int64)
+        nt = self.edge_n_tgt.astype(np.int64)
+        live = (ns > 0) & (nt > 0)
+        ns1 = np.maximum(ns, 1)
+        nt1 = np.maximum(nt, 1)
+        ncc = -(-ns1 // APC_TILE_MAX_COLS)  # column chunks per edge
+        cw = -(-ns1 // ncc)  # chunk width
+        rpt = np.clip(tile_entries // cw, 1, APC_TILE_MAX_ROWS)
+        nrt = -(-nt1 // rpt)  # row tiles per edge
+        rpt = -(-nt1 // nrt)  # balanced rows per tile
+        per_edge = np.where(live, ncc * nrt, 0)
+        total = int(per_edge.sum())
+        te = np.repeat(np.arange(self.n_edges, dtype=np.int64), per_edge)
+        first = np.cumsum(per_edge) - per_edge
+        k = np.arange(total, dtype=np.int64) - np.repeat(first, per_edge)
+        ci = k % ncc[te]
+        ri = k // ncc[te]
+        col_begin = ci * cw[te]
+        row_begin = ri * rpt[te]
+        self.tile_edge = _i32(te)
+        self.tile_col_begin = _i32(col_begin)
+        self.tile_col_count = _i32(np.minimum(cw[te], ns[te] - col_begin))
+        self.tile_row_begin = _i32(row_begin)
+        self.tile_row_count = _i32(np.minimum(rpt[te], nt[te] - row_begin))
+
+    # ---- checks ------------------------------------------------------------------------
+    def validate(self, params) -> None:
+        """Structural check through the library's host-side validator; raises
+        RuntimeError naming the first malformed row."""
+        if tuple(params.mesh_sizes) != self.mesh_sizes:
+            raise RuntimeError(f"tables were encoded for mesh {self.mesh_sizes}, params describe {params.mesh_sizes}")
+        if len(self.edge_entry_begin) != self.n_edges + 1:
+            raise RuntimeError("edge_entry_begin must have n_edges + 1 rows")
+        for name in ("edge_src_begin", "edge_tgt_begin", "edge_flags", "edge_pt_begin", "edge_strat_begin",
+                     "edge_n_tgt"):
+            if len(getattr(self, name)) != self.n_edges:
+                raise RuntimeError(f"{name} must have n_edges rows")
+        if len(self.spec_tensor) != self.n_specs:
+            raise RuntimeError("spec_tensor must have n_specs rows")
+        for name in ("strat_rw_bytes", "strat_dtype", "strat_zero_cost", "strat_num_args"):
+            if len(getattr(self, name)) != self.n_strategies:
+                raise RuntimeError(f"{name} must have n_strategies rows")
+        if self.n_strategies and int(self.strat_num_args.min()) < 1:
+            raise RuntimeError("strat_num_args must be >= 1")
+        if (self.strat_flops >= 2**53).any() or (self.strat_rw_bytes >= 2**53).any():
+            raise RuntimeError("flop / byte counts must stay below 2**53 to convert to fp64 exactly")
+        cp = params.to_c()
+
+        def p(a):
+            return a.ctypes.data_as(ctypes.c_void_p)
+
+        rc = _native.lib().apc_validate_tables_host(
+            ctypes.byref(cp), ctypes.c_int64(self.n_tensors), p(self.tensor_rank),
+            ctypes.c_int64(self.n_specs), p(self.spec_codes), p(self.spec_tensor),
+            ctypes.c_int64(self.n_edges), p(self.edge_src_begin), p(self.edge_n_src), p(self.edge_tgt_begin),
+            p(self.edge_n_tgt), p(self.edge_flags), p(self.edge_pt_begin), p(self.edge_entry_begin),
+            p(self.edge_strat_begin), ctypes.c_int64(len(self.pt_values)), ctypes.c_int64(self.n_strategies),
+            ctypes.c_int64(self.n_tiles), p(self.tile_edge), p(self.tile_row_begin), p(self.tile_row_count),
+            p(self.tile_col_begin), p(self.tile_col_count))
+        _native.check(rc, "apc_validate_tables_host")
+        # byte counts must convert to fp64 exactly (the kernels divide them as doubles)
+        if self.n_tensors:
+            r = np.arange(APC_MAX_RANK)[None, :] < self.tensor_rank[:, None]
+            numel = np.where(r, self.tensor_shape, 1).astype(object).prod(axis=1)
+            if (numel * self.tensor_itemsize.astype(object) >= 2**53).any():
+                raise RuntimeError("tensor byte counts must stay below 2**53")
+
+    def as_dict(self) -> dict:
+        """Plain-data view (numpy arrays) of every table."""
+        out = {"mesh_sizes": self.mesh_sizes}
+        for f in fields(self):
+            if f.name != "mesh_sizes":
+                out[f.name] = getattr(self, f.name)
+        return out
+
+    # ---- derived index arrays ------------------------------------------------------------
+    def row_ptr(self) -> np.ndarray:
+        """CSR pointer of matrix rows over the entry array: one segment per
+        (edge, consumer strategy), length = that edge's producer count."""
+        ns = self.edge_n_src.astype(np.int64)
+        nt = self.edge_n_tgt.astype(np.int64)
+        lens = np.repeat(ns, nt)
+        out = np.zeros(len(lens) + 1, np.int64)
+        np.cumsum(lens, out=out[1:])
+        return out

@@ -1,0 +1,154 @@
+/*
+ * apcost — C ABI of the MI355X sharding-cost evaluation library (libapcost.so).
+ *
+ * The reference (pure Python) has no FFI layer; the seam these entry points sit
+ * behind is the pair of per-entry Python calls made by
+ * ShardingOptimizer.build_ds (autoparallel/optimize_sharding.py:270-380):
+ *   estimate_strategy_comms_cost   autoparallel/collective_runtime_estimation.py:146-153
+ *   estimate_strategy_runtime_cost autoparallel/compute_estimation.py:334-365
+ * plus _get_sharded_shape_stride   autoparallel/compute_estimation.py:211-229.
+ * Each entry point below names the reference function(s) it replaces, batched
+ * over the whole graph.
+ *
+ * Conventions
+ *   - Every array pointer is a DEVICE pointer unless the name ends in _host.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Calls
+ *     enqueue work and return; they never synchronise and never allocate.
+ *   - Return value 0 = success; negative = error, text via apc_last_error().
+ *   - The library owns no memory.  Outputs are caller-allocated.
+ *   - No CPU fallback exists: without a HIP device every launch entry fails.
+ *
+ * Flattened graph tables ("encoding")
+ *   placement code, one byte per mesh dim:
+ *       0x00            Replicate
+ *       0x40 | op       Partial(op), op 0 = sum
+ *       0x80 | v<<4 | d Shard(tensor dim d), v = variant (0 plain)
+ *   spec_codes[s]   uint32, byte i = code of mesh dim i (mesh ndim <= 4)
+ *   spec_tensor[s]  int32 row of the tensor table, -1 = "not a DTensorSpec"
+ *   tensor table    rank int32, itemsize int32, shape/stride int64[APC_MAX_RANK]
+ *   edge e = (consumer node, argument):
+ *       producer output specs  spec rows [edge_src_begin, +edge_n_src)
+ *       consumer input specs   spec rows [edge_tgt_begin, +edge_n_tgt)
+ *       matrix entries         [edge_entry_begin[e], +n_tgt*n_src), row = consumer
+ *                              strategy, column = producer strategy
+ *       edge_strat_begin[e]    row of the consumer's first strategy in the
+ *                              per-strategy tables
+ *       edge_pt_begin[e]       offset into pt_values of the rule-provided costs
+ *                              kept where either spec is not a DTensorSpec
+ *       edge_flags             APC_EDGE_*
+ *   tile t = a rectangle of one edge's matrix handled by one workgroup:
+ *       tile_edge, tile_row_begin, tile_row_count, tile_col_begin, tile_col_count
+ */
+#ifndef APCOST_H
+#define APCOST_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define APC_MAX_RANK 8
+#define APC_MAX_MESH 4
+#define APC_MAX_DTYPES 8
+#define APC_TILE_MAX_COLS 1024 /* producer specs staged in LDS per tile */
+#define APC_TILE_MAX_ROWS 1024 /* consumer specs staged in LDS per tile */
+
+#define APC_EDGE_GRAD_RESCALE 1 /* consumer is a parameter-gradient node (optimize_sharding.py:358-359) */
+#define APC_EDGE_NO_PRODUCER 2  /* placeholder / factory pseudo-argument (optimize_sharding.py:312-355) */
+
+/* Cost-model parameters: everything the reference reads from its environment
+ * (torch MeshTopoInfo, DEVICE_LIMITS row, module constants), made explicit. */
+typedef struct apc_params {
+  int32_t mesh_ndim;
+  int32_t mesh_size[APC_MAX_MESH];
+  double bw[APC_MAX_MESH];  /* GB/s per mesh dim   torch _collective_utils.py:256-274 */
+  double lat[APC_MAX_MESH]; /* us per hop          torch _collective_utils.py:258-274 */
+  double base_latency;      /* 6.6 us              torch _collective_utils.py:286 */
+  double a2a_scale;         /* 5                   collective_runtime_estimation.py:30-31 */
+  double hbm_bw;            /* bytes/s             compute_estimation.py:63-166 */
+  double rw_eff;            /* 0.70                compute_estimation.py:307 */
+  double launch_floor;      /* 7 us                compute_estimation.py:309 */
+  double compute_eff;       /* 0.70                compute_estimation.py:361 */
+  double rescale;           /* grad comm rescale   optimize_sharding.py:358-359 */
+  double gpu_flops[APC_MAX_DTYPES]; /* tflops*10^12 per dtype code; 0 = unsupported */
+  int32_t transition_scale; /* 1                   optimize_sharding.py:298 */
+} apc_params;
+
+int apc_version(void);
+const char *apc_last_error(void);
+
+/* Host-side structural check of the tables (HOST pointers).  Replaces the
+ * reference's assertions in ShardingOptimizer.validate
+ * (optimize_sharding.py:908-958) for the flattened form: monotone entry
+ * offsets, spec/tensor/strategy indices in range, rank <= APC_MAX_RANK, shard
+ * dims < rank, tiles inside their edge and within the LDS staging limits. */
+int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank_host,
+                             int64_t n_specs, const uint32_t *spec_codes_host, const int32_t *spec_tensor_host,
+                             int64_t n_edges, const int32_t *edge_src_begin_host, const int32_t *edge_n_src_host,
+                             const int32_t *edge_tgt_begin_host, const int32_t *edge_n_tgt_host,
+                             const int32_t *edge_flags_host, const int64_t *edge_pt_begin_host,
+                             const int64_t *edge_entry_begin_host, const int32_t *edge_strat_begin_host,
+                             int64_t n_pt, int64_t n_strategies, int64_t n_tiles, const int32_t *tile_edge_host,
+                             const int32_t *tile_row_begin_host, const int32_t *tile_row_count_host,
+                             const int32_t *tile_col_begin_host, const int32_t *tile_col_count_host);
+
+/* Bytes and contiguity of every tensor row.
+ * Replaces torch spec_to_bytes (distributed/tensor/_collective_utils.py:230-232) and
+ * check_contiguous_sizes_strides (_prims_common/__init__.py:252-292) as called from
+ * collective_runtime_estimation.py:66-76. */
+int apc_tensor_tables(int64_t n_tensors, const int32_t *tensor_rank, const int32_t *tensor_itemsize,
+                      const int64_t *tensor_shape, const int64_t *tensor_stride, int64_t *tensor_bytes,
+                      uint8_t *tensor_contiguous, void *stream);
+
+/* Local shard shape / stride / element and byte counts and shard count per spec.
+ * Replaces _get_sharded_shape_stride (compute_estimation.py:211-229) and
+ * DTensorSpec.num_shards (torch distributed/tensor/_dtensor_spec.py:555-561).
+ * local_shape / local_stride are [n_specs][APC_MAX_RANK], zero padded. */
+int apc_spec_tables(const apc_params *params, int64_t n_specs, const uint32_t *spec_codes,
+                    const int32_t *spec_tensor, const int32_t *tensor_rank, const int32_t *tensor_itemsize,
+                    const int64_t *tensor_shape, const int64_t *tensor_stride, int64_t *num_shards,
+                    int64_t *local_shape, int64_t *local_stride, int64_t *local_numel, int64_t *local_bytes,
+                    void *stream);
+
+/* Per-(node, strategy) compute cost and compute cost / num_args.
+ * Replaces the arithmetic tail of estimate_strategy_runtime_cost
+ * (compute_estimation.py:334-365) with compute_read_write_time (:302-314), and the
+ * division at optimize_sharding.py:371-373.  A strategy with flops != 0 whose dtype
+ * has no throughput on the device row sets *error_flag (device int32) to 1. */
+int apc_compute_costs(const apc_params *params, int64_t n_strategies, const int64_t *flops,
+                      const int64_t *rw_bytes, const int8_t *dtype_code, const uint8_t *zero_cost,
+                      const int32_t *num_args, double *compute_cost, double *compute_cost_per_arg,
+                      int32_t *error_flag, void *stream);
+
+/* The redistribution-cost matrices of every edge, plus the assembled ILP cost.
+ * Replaces the two inner loops of ShardingOptimizer.build_ds
+ * (optimize_sharding.py:306-379): estimate_strategy_comms_cost /
+ * redistribute_cost / all_to_all_cost (collective_runtime_estimation.py:22-153),
+ * torch allgather_cost / allreduce_cost / reduce_scatter_cost
+ * (distributed/tensor/_collective_utils.py:281-313), the transition tie-break
+ * (:345-351), the grad rescale (:358-359) and cost assembly (:368-372).
+ * comm_out / transition_out / cost_out are [n_entries]; any may be NULL. */
+int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes,
+                            const uint8_t *tensor_contiguous, const uint32_t *spec_codes,
+                            const int32_t *spec_tensor, const int32_t *edge_src_begin,
+                            const int32_t *edge_n_src, const int32_t *edge_tgt_begin,
+                            const int32_t *edge_n_tgt, const int32_t *edge_flags,
+                            const int64_t *edge_pt_begin, const int64_t *edge_entry_begin,
+                            const int32_t *edge_strat_begin, const double *pt_values,
+                            const double *compute_cost_per_arg, int64_t n_tiles, const int32_t *tile_edge,
+                            const int32_t *tile_row_begin, const int32_t *tile_row_count,
+                            const int32_t *tile_col_begin, const int32_t *tile_col_count, double *comm_out,
+                            uint8_t *transition_out, double *cost_out, void *stream);
+
+/* Segmented minimum with first-argmin (relative to the segment start); empty
+ * segments give (+inf, -1).  No counterpart in the reference (which hands the full
+ * table to the ILP solver, optimize_sharding.py:648-659): used for pruning and
+ * warm start. */
+int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_segments, double *seg_min,
+                      int32_t *seg_argmin, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* APCOST_H */
