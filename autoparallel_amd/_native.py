@@ -62,6 +62,11 @@ def lib() -> ctypes.CDLL:
     ``python -m autoparallel_amd._build`` or ``__graft_entry__.build()``)."""
     global _lib
     if _lib is None:
+        # torch ships its own HIP runtime; it must be in the process before this library
+        # is mapped so that both resolve to the same runtime (streams and device pointers
+        # are shared between them).
+        import torch  # noqa: F401
+
         if not os.path.exists(LIB_PATH):
             raise RuntimeError(
                 f"{LIB_PATH} is missing: the HIP library has not been built "

@@ -151,7 +151,7 @@ def mesh_topology(mesh_sizes, devices_per_host=8, base_bw=87.7, inter_factor=0.2
 def make_params(mesh_sizes, device_name="H100", devices_per_host=8, rescale=1.0) -> CostParams:
     n, bw, lat = mesh_topology(mesh_sizes, devices_per_host)
     _, hbm, tflops = device_limit(device_name)
-    gf = [0.0] * NUM_DTYPE_CODES
+    gf = [0.0] * 8
     for name, code in DTYPE_CODES.items():
         if name in tflops:
             # ref: compute_estimation.py:356  gpu_flops = tflops * 10**12

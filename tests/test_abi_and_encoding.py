@@ -1,0 +1,156 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every
+symbol the public header declares; the flattened encoding's tiles cover every
+entry exactly once; the host validator rejects malformed tables; the cost-model
+parameters reproduce the reference's environment lookups."""
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from autoparallel_amd import CostModelParams, _native, get_device_limit, mesh_topology
+from autoparallel_amd.encoding import (EDGE_NO_PRODUCER, CostTables, code_dim, code_kind, pack_codes, partial_code,
+                                       shard_code, unpack_codes)
+from autoparallel_amd.synthetic import stress_dag
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "apcost.h")).read()
+    declared = set(re.findall(r"\b(apc_[a-z_0-9]+)\s*\(", header))
+    assert declared, "no declarations found in include/apcost.h"
+    lib = _native.lib()
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} declared in apcost.h but not exported"
+    assert declared == set(_native.EXPORTS)
+    assert lib.apc_version() == 1
+
+
+def test_params_struct_layout_matches_header():
+    # 4 + 16 (+4 pad) + 32 + 32 + 7*8 + 64 + 4 (+4 pad)
+    assert ctypes.sizeof(_native.ApcParams) == 216
+    assert _native.ApcParams.bw.offset == 24 and _native.ApcParams.gpu_flops.offset == 144
+
+
+def test_placement_codes_round_trip():
+    codes = (0, partial_code("sum"), partial_code("max"), shard_code(3))
+    assert unpack_codes(pack_codes(codes), 4) == codes
+    assert [code_kind(c) for c in codes] == [0, 1, 1, 2]
+    assert code_dim(shard_code(3)) == 3 and shard_code(2, variant=1) != shard_code(2)
+    with pytest.raises(ValueError):
+        shard_code(16)
+
+
+def test_launch_entry_points_fail_loudly_without_a_device():
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a HIP device is present")
+    from autoparallel_amd.device_tables import DeviceCostTables
+
+    tb = stress_dag(seed=0, n_nodes=10, mesh_sizes=(4, 2))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        DeviceCostTables(tb, CostModelParams.from_mesh((4, 2)))
+
+
+@pytest.mark.parametrize("tile_entries", [64, 1000, 4096])
+def test_tiles_cover_every_entry_exactly_once(tile_entries):
+    tb = stress_dag(seed=3, n_nodes=300, mesh_sizes=(4, 4, 2), max_strategies=80, tile_entries=tile_entries)
+    seen = np.zeros(tb.n_entries, np.int32)
+    for t in range(tb.n_tiles):
+        e = tb.tile_edge[t]
+        ns = int(tb.edge_n_src[e])
+        r0, rc, c0, cc = (int(x[t]) for x in (tb.tile_row_begin, tb.tile_row_count, tb.tile_col_begin, tb.tile_col_count))
+        assert 1 <= rc <= _native.APC_TILE_MAX_ROWS and 1 <= cc <= _native.APC_TILE_MAX_COLS
+        rows = np.arange(r0, r0 + rc)[:, None] * ns + np.arange(c0, c0 + cc)[None, :]
+        seen[int(tb.edge_entry_begin[e]) + rows.ravel()] += 1
+    assert (seen == 1).all()
+
+
+def test_wide_edges_are_cut_into_column_chunks():
+    # one consumer with 3 strategies reading a producer with 2500 strategies
+    n_src, n_tgt = 2500, 3
+    tb = CostTables(
+        mesh_sizes=(4,), tensor_rank=[1], tensor_itemsize=[4], tensor_shape=[[64] + [0] * 7],
+        tensor_stride=[[1] + [0] * 7], spec_codes=np.zeros(n_src + n_tgt, np.uint32),
+        spec_tensor=np.zeros(n_src + n_tgt, np.int32), strat_flops=np.zeros(n_tgt), strat_rw_bytes=np.zeros(n_tgt),
+        strat_dtype=np.ones(n_tgt), strat_zero_cost=np.zeros(n_tgt), strat_num_args=np.ones(n_tgt),
+        node_strat_begin=[0, n_tgt], edge_node=[0], edge_arg=[0], edge_src_begin=[0], edge_n_src=[n_src],
+        edge_tgt_begin=[n_src], edge_n_tgt=[n_tgt], edge_flags=[0], edge_pt_begin=[-1],
+        edge_entry_begin=[0, n_src * n_tgt], edge_strat_begin=[0], pt_values=[])
+    assert tb.n_tiles >= 3 and int(tb.tile_col_count.max()) <= _native.APC_TILE_MAX_COLS
+    assert int(tb.tile_col_count.astype(np.int64).dot(tb.tile_row_count)) == n_src * n_tgt
+    tb.validate(CostModelParams.from_mesh((4,)))
+
+
+def _small():
+    return stress_dag(seed=5, n_nodes=40, mesh_sizes=(4, 2), max_strategies=8)
+
+
+def test_validator_accepts_generated_tables():
+    _small().validate(CostModelParams.from_mesh((4, 2)))
+
+
+@pytest.mark.parametrize("mutate, message", [
+    (lambda t: t.tensor_rank.__setitem__(0, 9), "rank"),
+    (lambda t: t.spec_tensor.__setitem__(3, 10**6), "tensor row"),
+    (lambda t: t.spec_codes.__setitem__(0, 0xC0), "no meaning"),
+    (lambda t: t.spec_codes.__setitem__(0, 0x01), "no meaning"),
+    (lambda t: t.spec_codes.__setitem__(0, 0x8F), "Shard"),
+    (lambda t: t.spec_codes.__setitem__(0, 0x800000), "beyond mesh ndim"),
+    (lambda t: t.edge_entry_begin.__setitem__(2, int(t.edge_entry_begin[2]) + 1), "entry_begin"),
+    (lambda t: t.edge_src_begin.__setitem__(1, t.n_specs), "producer spec range"),
+    (lambda t: t.edge_strat_begin.__setitem__(1, t.n_strategies), "strategy rows"),
+    (lambda t: t.tile_row_count.__setitem__(0, 10**4), "rows"),
+    (lambda t: t.tile_col_begin.__setitem__(0, -1), "cols"),
+    (lambda t: t.tile_edge.__setitem__(0, t.n_edges), "edge"),
+])
+def test_validator_rejects_malformed_tables(mutate, message):
+    tb = _small()
+    mutate(tb)
+    with pytest.raises(RuntimeError, match=message):
+        tb.validate(CostModelParams.from_mesh((4, 2)))
+
+
+def test_validator_needs_pass_through_values_for_producerless_edges():
+    tb = _small()
+    e = int(np.nonzero(tb.edge_flags & EDGE_NO_PRODUCER)[0][0])
+    tb.edge_pt_begin[e] = -1
+    with pytest.raises(RuntimeError, match="pass-through"):
+        tb.validate(CostModelParams.from_mesh((4, 2)))
+
+
+def test_validator_rejects_mesh_mismatch():
+    with pytest.raises(RuntimeError, match="mesh"):
+        _small().validate(CostModelParams.from_mesh((2, 4)))
+
+
+def test_cost_model_params_follow_reference_environment():
+    assert mesh_topology((32, 8)) == ((87.7 * 0.22, 87.7), (2.7, 0.6))
+    assert mesh_topology((8, 8, 8)) == ((87.7 * 0.22, 87.7 * 0.22, 87.7), (2.7, 2.7, 0.6))
+    assert mesh_topology((64,))[0] == (87.7 * 0.22,)
+    assert mesh_topology((8,))[0] == (87.7,)  # strict '>' on the device product
+    p = CostModelParams.from_mesh((32, 8), rescale=2.2)
+    assert p.hbm_bw == 3.35 * 1024**4 and p.gpu_flops[3] == 989e12 and p.gpu_flops[1] == 494e12
+    assert p.gpu_flops[5] == 0.0
+    assert get_device_limit("NVIDIA H100 80GB HBM3").name == "H100"
+    with pytest.raises(ValueError, match="Unsupported device"):
+        CostModelParams.from_mesh((8,), device_name="AMD Instinct MI355X")
+    with pytest.raises(ValueError):
+        CostModelParams.from_mesh((2, 2, 2, 2, 2))
+    c = p.to_c()
+    assert c.mesh_ndim == 2 and list(c.mesh_size)[:2] == [32, 8] and c.rescale == 2.2
+
+
+def test_oracle_and_product_agree_on_constants():
+    # the oracle restates the device table and codes independently; both must say the same
+    from oracle import cost_oracle as po
+
+    for mesh in [(64,), (32, 8), (16, 8, 4)]:
+        a, b = po.make_params(mesh), CostModelParams.from_mesh(mesh)
+        assert a.bw == b.bw and a.lat == b.lat and a.hbm_bw == b.hbm_bw and tuple(a.gpu_flops) == tuple(b.gpu_flops)
+    assert po.shard(3) == shard_code(3) and po.partial(2) == partial_code(2)
+    assert po.DTYPE_CODES == __import__("autoparallel_amd.cost_model", fromlist=["x"]).DTYPE_CODES

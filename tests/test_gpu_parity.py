@@ -1,0 +1,246 @@
+"""GPU parity: every kernel, called through the C ABI, against the CPU oracle on the
+same seeded tables.  Bar: bit-exact for integer / byte / index outputs AND for the fp64
+costs (the kernels are built with FMA contraction off and evaluate in the reference's
+operation order); the stated tolerance of the path is 1e-9 relative, asserted as well
+so that a future relaxation of bit-exactness cannot silently exceed it."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from autoparallel_amd import CostModelParams
+from autoparallel_amd.device_tables import DeviceCostTables
+from autoparallel_amd.encoding import CostTables, pack_codes, partial_code, shard_code
+from autoparallel_amd.synthetic import stress_dag
+from oracle import c_oracle
+from oracle import cost_oracle as po
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-9
+
+
+def _assert_costs(got: np.ndarray, want: np.ndarray, what: str):
+    assert got.shape == want.shape, what
+    assert np.array_equal(np.isinf(got), np.isinf(want)), f"{what}: inf pattern differs"
+    fin = np.isfinite(want)
+    denom = np.maximum(np.abs(want[fin]), 1e-300)
+    rel = np.abs(got[fin] - want[fin]) / denom
+    assert rel.size == 0 or rel.max() <= REL_TOL, f"{what}: max rel err {rel.max()}"
+    assert np.array_equal(got, want), f"{what}: not bit-identical ({int((got != want).sum())} entries differ)"
+
+
+def _run_and_compare(tb: CostTables, mesh, rescale, device):
+    p = CostModelParams.from_mesh(mesh, rescale=rescale)
+    op = po.make_params(mesh, rescale=rescale)
+    d = DeviceCostTables(tb, p, device=device)
+    comm, trans, cost = d.build_all()
+    torch.cuda.synchronize()
+    enc = tb.as_dict()
+    want_cc, want_pa = c_oracle.compute_costs(enc, op)
+    want = c_oracle.build_tables(enc, op, per_arg=want_pa)
+    _assert_costs(d.compute_cost.cpu().numpy(), want_cc, "compute_cost")
+    _assert_costs(d.compute_cost_per_arg.cpu().numpy(), want_pa, "compute_cost_per_arg")
+    _assert_costs(comm.cpu().numpy(), want["comm"], "comm")
+    _assert_costs(cost.cpu().numpy(), want["cost"], "cost")
+    assert np.array_equal(trans.cpu().numpy(), want["transition"])
+    return d, want
+
+
+@pytest.mark.parametrize("mesh", [(64,), (32, 8), (8, 8, 8), (64, 4), (16, 8, 4), (6, 3), (5, 3, 2), (2, 3, 2, 2)])
+def test_tables_match_oracle_on_seeded_dags(gpu_device, mesh):
+    tb = stress_dag(seed=11, n_nodes=1500, mesh_sizes=mesh, frac_nonspec_nodes=0.02, frac_noncontiguous=0.2)
+    d, want = _run_and_compare(tb, mesh, 2.2, gpu_device)
+    # integer tables: bit-exact
+    enc = tb.as_dict()
+    wb, wc = c_oracle.tensor_tables(enc)
+    assert np.array_equal(d.tensor_bytes.cpu().numpy(), wb)
+    assert np.array_equal(d.tensor_contiguous.cpu().numpy(), wc)
+    got = d.run_spec_tables()
+    for key, w in zip(("num_shards", "local_shape", "local_stride", "local_numel", "local_bytes"),
+                      c_oracle.spec_tables(enc, mesh)):
+        assert np.array_equal(got[key].cpu().numpy(), w), key
+
+
+def test_python_oracle_agrees_on_a_small_case(gpu_device):
+    # the scalar Python restatement (not only its C twin) against the kernels
+    mesh = (32, 8)
+    tb = stress_dag(seed=2, n_nodes=40, mesh_sizes=mesh, max_strategies=10, frac_nonspec_nodes=0.1)
+    p = CostModelParams.from_mesh(mesh, rescale=2.2)
+    d = DeviceCostTables(tb, p, device=gpu_device)
+    comm, trans, cost = d.build_all()
+    want = po.build_tables(tb.as_dict(), po.make_params(mesh, rescale=2.2))
+    assert np.array_equal(comm.cpu().numpy(), np.asarray(want["comm"]))
+    assert np.array_equal(cost.cpu().numpy(), np.asarray(want["cost"]))
+    assert np.array_equal(trans.cpu().numpy(), np.asarray(want["transition"], dtype=np.uint8))
+
+
+def _two_node_tables(mesh, shape, stride, itemsize, src_codes, tgt_codes, flags=0, num_args=1, flops=0, rw=0):
+    """producer node (strategies = src_codes) -> consumer node (input specs = tgt_codes)."""
+    ns, nt = len(src_codes), len(tgt_codes)
+    rank = len(shape)
+    pad = [0] * (8 - rank)
+    specs = [pack_codes(c) for c in src_codes] + [pack_codes(c) for c in tgt_codes]
+    return CostTables(
+        mesh_sizes=mesh, tensor_rank=[rank], tensor_itemsize=[itemsize], tensor_shape=[list(shape) + pad],
+        tensor_stride=[list(stride) + pad], spec_codes=specs, spec_tensor=[0] * (ns + nt),
+        strat_flops=[0] * ns + [flops] * nt, strat_rw_bytes=[0] * ns + [rw] * nt, strat_dtype=[3] * (ns + nt),
+        strat_zero_cost=[1] * ns + [0 if (flops or rw) else 1] * nt, strat_num_args=[1] * ns + [num_args] * nt,
+        node_strat_begin=[0, ns, ns + nt], edge_node=[1], edge_arg=[0], edge_src_begin=[0], edge_n_src=[ns],
+        edge_tgt_begin=[ns], edge_n_tgt=[nt], edge_flags=[flags], edge_pt_begin=[-1],
+        edge_entry_begin=[0, ns * nt], edge_strat_begin=[ns], pt_values=[])
+
+
+def test_known_answer_values_on_device(gpu_device):
+    """The hand-derived values (mesh (32, 8), [4096, 4096] bf16) straight from the kernel."""
+    R, P, S0, S1 = 0, partial_code(), shard_code(0), shard_code(1)
+    src = [(S0, S0), (P, P), (S0, S1), (R, R), (S0, R)]
+    tgt = [(R, S0), (R, R), (S0, S0), (S0, R), (S0, S1), (P, R)]
+    tb = _two_node_tables((32, 8), [4096, 4096], [4096, 1], 2, src, tgt)
+    d = DeviceCostTables(tb, CostModelParams.from_mesh((32, 8)), device=gpu_device)
+    comm, trans, _ = d.build_all()
+    m = comm.cpu().numpy().reshape(len(tgt), len(src))
+    assert m[0, 0] == 286.43246022079404  # (S0,S0) -> (R,S0)
+    assert m[1, 0] == 609.0198034363015  # (S0,S0) -> (R,R)
+    assert m[2, 1] == 609.0198034363015  # (P,P) -> (S0,S0): flipped order
+    assert m[3, 2] == 27.543354475484605  # (S0,S1) -> (S0,R)
+    assert m[4, 0] == 67.08959654717788  # (S0,S0) -> (S0,S1)
+    assert m[2, 0] == 0.0 and m[0, 3] == 0.0  # identity, replicated source
+    assert math.isinf(m[5, 3]) and math.isinf(m[5, 0])  # -> Partial banned
+    t = trans.cpu().numpy().reshape(len(tgt), len(src))
+    assert t[2, 0] == 0 and t[0, 0] == 1 and t[3, 4] == 0
+    # fp32 [8192, 4096] all-reduce on the inter-host dim
+    tb = _two_node_tables((32, 8), [8192, 4096], [4096, 1], 4, [(P, R)], [(R, R)])
+    d = DeviceCostTables(tb, CostModelParams.from_mesh((32, 8)), device=gpu_device)
+    assert d.build_all()[0].cpu().numpy()[0] == 12726.477454130818
+
+
+def test_compute_cost_known_answer_and_assembly(gpu_device):
+    S0 = shard_code(0)
+    flops, rw = 68719476736, 67108864
+    tb = _two_node_tables((32, 8), [4096, 4096], [4096, 1], 2, [(S0, S0)], [(0, S0)], flags=1, num_args=2,
+                          flops=flops, rw=rw)
+    d = DeviceCostTables(tb, CostModelParams.from_mesh((32, 8), rescale=2.2), device=gpu_device)
+    comm, trans, cost = d.build_all()
+    cc = d.compute_cost.cpu().numpy()
+    assert cc[1] == 99.26256931388127 and cc[0] == 0.0
+    assert comm.cpu().numpy()[0] == 286.43246022079404 / 2.2  # grad rescale is a division
+    assert cost.cpu().numpy()[0] == 286.43246022079404 / 2.2 + 99.26256931388127 / 2 + 1
+
+
+def test_unsupported_dtype_raises(gpu_device):
+    tb = _two_node_tables((4,), [64, 64], [64, 1], 2, [(0,)], [(0,)], flops=10, rw=10)
+    tb.strat_dtype[:] = 6
+    d = DeviceCostTables(tb, CostModelParams.from_mesh((4,)), device=gpu_device)
+    d.run_tensor_tables()
+    with pytest.raises(ValueError, match="dtype"):
+        d.run_compute_costs()
+
+
+def test_wide_and_degenerate_edges(gpu_device):
+    """Column-chunked tiles (producer with > 1024 strategies), single-entry edges and a
+    graph with zero edges."""
+    rng = np.random.default_rng(0)
+    n_src, n_tgt = 2600, 7
+    opts = [0, partial_code(), shard_code(0), shard_code(1), shard_code(2)]
+    src = [tuple(rng.choice(opts, 3)) for _ in range(n_src)]
+    tgt = [tuple(rng.choice(opts, 3)) for _ in range(n_tgt)]
+    tb = _two_node_tables((4, 2, 2), [64, 32, 16], [512, 16, 1], 4, src, tgt)
+    assert int(tb.tile_col_count.max()) <= 1024 and tb.n_tiles > 1
+    _run_and_compare(tb, (4, 2, 2), 1.0, gpu_device)
+    tb = _two_node_tables((4,), [64], [1], 4, [(shard_code(0),)], [(0,)])
+    _run_and_compare(tb, (4,), 1.0, gpu_device)
+    empty = CostTables(
+        mesh_sizes=(4,), tensor_rank=[], tensor_itemsize=[], tensor_shape=np.zeros((0, 8)),
+        tensor_stride=np.zeros((0, 8)), spec_codes=[], spec_tensor=[], strat_flops=[], strat_rw_bytes=[],
+        strat_dtype=[], strat_zero_cost=[], strat_num_args=[], node_strat_begin=[0], edge_node=[], edge_arg=[],
+        edge_src_begin=[], edge_n_src=[], edge_tgt_begin=[], edge_n_tgt=[], edge_flags=[], edge_pt_begin=[],
+        edge_entry_begin=[0], edge_strat_begin=[], pt_values=[])
+    d = DeviceCostTables(empty, CostModelParams.from_mesh((4,)), device=gpu_device)
+    comm, trans, cost = d.build_all()
+    assert comm.numel() == 0 and trans.numel() == 0 and cost.numel() == 0
+
+
+def test_tile_size_does_not_change_results(gpu_device):
+    mesh = (16, 8, 4)
+    base = None
+    for te in (64, 777, 4096, 16384):
+        tb = stress_dag(seed=4, n_nodes=400, mesh_sizes=mesh, tile_entries=te)
+        d = DeviceCostTables(tb, CostModelParams.from_mesh(mesh), device=gpu_device)
+        out = [x.cpu().numpy() for x in d.build_all()]
+        if base is None:
+            base = out
+        else:
+            for a, b in zip(base, out):
+                assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("max_len", [3, 40, 700])
+def test_segmented_min_matches_oracle(gpu_device, max_len):
+    rng = np.random.default_rng(max_len)
+    lens = rng.integers(0, max_len + 1, size=5000)
+    ptr = np.zeros(len(lens) + 1, np.int64)
+    np.cumsum(lens, out=ptr[1:])
+    vals = rng.choice([0.0, 1.0, 2.5, 7.0, 1e4, np.inf], size=int(ptr[-1]))
+    tb = stress_dag(seed=0, n_nodes=5, mesh_sizes=(2,))
+    d = DeviceCostTables(tb, CostModelParams.from_mesh((2,)), device=gpu_device)
+    mins, args = d.segmented_min(torch.from_numpy(vals).to(gpu_device), ptr)
+    wm, wa = c_oracle.segmented_min(vals, ptr)
+    assert np.array_equal(mins.cpu().numpy(), wm)
+    assert np.array_equal(args.cpu().numpy(), wa)
+    nz = lens > 0
+    assert np.array_equal(wm[nz], np.minimum.reduceat(vals, ptr[:-1][nz]))
+
+
+def test_row_min_of_cost_tables(gpu_device):
+    mesh = (32, 8)
+    tb = stress_dag(seed=9, n_nodes=800, mesh_sizes=mesh)
+    d, want = _run_and_compare(tb, mesh, 2.2, gpu_device)
+    rp = tb.row_ptr()
+    mins, args = d.segmented_min(d.cost, rp)
+    wm, wa = c_oracle.segmented_min(want["cost"], rp)
+    assert np.array_equal(mins.cpu().numpy(), wm) and np.array_equal(args.cpu().numpy(), wa)
+
+
+def test_full_size_stress_properties(gpu_device):
+    """The raw-throughput workload at a size the CPU cannot check entry by entry in test
+    time: size-independent properties instead.  (a) the diagonal property: wherever the
+    producer and consumer placements are identical the comm cost is exactly 0 and the
+    transition flag 0; (b) a sampled 2000-edge slice is bit-identical to the oracle;
+    (c) row minima are <= every sampled entry of their row."""
+    mesh = (16, 8, 4)
+    tb = stress_dag(seed=0, n_nodes=40_000, mesh_sizes=mesh)
+    p = CostModelParams.from_mesh(mesh, rescale=2.2)
+    d = DeviceCostTables(tb, p, device=gpu_device)
+    comm, trans, cost = d.build_all()
+    torch.cuda.synchronize()
+    assert comm.numel() == tb.n_entries > 50_000_000
+    # (b)
+    lo, hi = 17_000, 19_000
+    want = c_oracle.build_tables(tb.as_dict(), po.make_params(mesh, rescale=2.2), edge_range=(lo, hi))
+    a, b = int(tb.edge_entry_begin[lo]), int(tb.edge_entry_begin[hi])
+    assert np.array_equal(comm[a:b].cpu().numpy(), want["comm"])
+    assert np.array_equal(cost[a:b].cpu().numpy(), want["cost"])
+    assert np.array_equal(trans[a:b].cpu().numpy(), want["transition"])
+    # (a) on the same slice, from the tables
+    got_c, got_t = comm[a:b].cpu().numpy(), trans[a:b].cpu().numpy()
+    off = 0
+    for e in range(lo, hi):
+        ns, nt = int(tb.edge_n_src[e]), int(tb.edge_n_tgt[e])
+        if not (tb.edge_flags[e] & 2):
+            s = tb.spec_codes[tb.edge_src_begin[e]:tb.edge_src_begin[e] + ns]
+            t = tb.spec_codes[tb.edge_tgt_begin[e]:tb.edge_tgt_begin[e] + nt]
+            valid = (tb.spec_tensor[tb.edge_src_begin[e]] >= 0)
+            if valid:
+                same = (t[:, None] == s[None, :]).ravel()
+                assert (got_c[off:off + ns * nt][same] == 0.0).all()
+                assert (got_t[off:off + ns * nt] == (~same).astype(np.uint8)).all()
+        off += ns * nt
+    # (c)
+    mins, _ = d.segmented_min(cost, tb.row_ptr())
+    rp = torch.from_numpy(tb.row_ptr()).to(gpu_device)
+    seg_of_entry = torch.repeat_interleave(torch.arange(rp.numel() - 1, device=gpu_device)[:200_000],
+                                           (rp[1:] - rp[:-1])[:200_000])
+    assert bool((cost[: seg_of_entry.numel()] >= mins[seg_of_entry]).all())
