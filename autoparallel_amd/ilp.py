@@ -1,0 +1,121 @@
+"""A small sparse 0/1 linear program container and its solve through HiGHS
+(``scipy.optimize.milp``).
+
+It plays the role PuLP + CBC play for the reference planner
+(autoparallel/optimize_sharding.py:86, 648-659): named linear constraints over binary
+variables and a linear objective.  Constraints are appended as whole index/coefficient
+arrays so a planner can emit thousands of rows per numpy call.
+"""
+
+from __future__ import annotations
+
+import time
+
+import numpy as np
+
+_NAME_COUNTERS: dict = {}
+
+
+def next_name(prefix: str) -> str:
+    idx = _NAME_COUNTERS.setdefault(prefix, 0)
+    _NAME_COUNTERS[prefix] += 1
+    return f"{prefix}_{idx:03}"
+
+
+class BinaryProgram:
+    def __init__(self, n_vars: int, name: str = "AutoParallel"):
+        self.name = name
+        self.n_vars = int(n_vars)
+        self._cols: list = []
+        self._vals: list = []
+        self._row_len: list = []
+        self._lb: list = []
+        self._ub: list = []
+        self._names: list = []
+        self.upper = np.ones(self.n_vars, np.float64)  # variable upper bounds (0 = forced off)
+        self.objective = np.zeros(self.n_vars, np.float64)
+        self.status = None
+        self.x = None
+        self.objective_value = None
+        self.solve_seconds = None
+
+    @property
+    def n_constraints(self) -> int:
+        return len(self._names)
+
+    # ---- building ------------------------------------------------------------------------
+    def add_row(self, cols, vals, lb, ub, name: str) -> None:
+        cols = np.asarray(cols, np.int64)
+        vals = np.broadcast_to(np.asarray(vals, np.float64), cols.shape)
+        self._cols.append(cols)
+        self._vals.append(vals)
+        self._row_len.append(len(cols))
+        self._lb.append(float(lb))
+        self._ub.append(float(ub))
+        self._names.append(name)
+
+    def add_rows(self, cols, vals, row_lengths, lb, ub, prefix: str) -> None:
+        """Many rows at once: ``cols`` / ``vals`` are the concatenated rows,
+        ``row_lengths`` their lengths; every row gets bounds [lb, ub]."""
+        cols = np.asarray(cols, np.int64)
+        vals = np.broadcast_to(np.asarray(vals, np.float64), cols.shape)
+        row_lengths = np.asarray(row_lengths, np.int64)
+        assert int(row_lengths.sum()) == len(cols)
+        self._cols.append(cols)
+        self._vals.append(vals)
+        self._row_len.extend(int(x) for x in row_lengths)
+        self._lb.extend([float(lb)] * len(row_lengths))
+        self._ub.extend([float(ub)] * len(row_lengths))
+        self._names.extend(next_name(prefix) for _ in range(len(row_lengths)))
+
+    def force_zero(self, var_ids) -> None:
+        self.upper[np.asarray(var_ids, np.int64)] = 0.0
+
+    def matrix(self):
+        from scipy.sparse import csr_matrix
+
+        if not self._names:
+            return csr_matrix((0, self.n_vars))
+        indptr = np.zeros(len(self._row_len) + 1, np.int64)
+        np.cumsum(self._row_len, out=indptr[1:])
+        cols = np.concatenate(self._cols) if self._cols else np.zeros(0, np.int64)
+        vals = np.concatenate(self._vals) if self._vals else np.zeros(0, np.float64)
+        m = csr_matrix((vals, cols, indptr), shape=(len(self._row_len), self.n_vars))
+        m.sum_duplicates()
+        return m
+
+    # ---- solving -------------------------------------------------------------------------
+    def solve(self, verbose: bool = False, time_limit: float | None = None, mip_rel_gap: float | None = None):
+        from scipy.optimize import Bounds, LinearConstraint, milp
+
+        a = self.matrix()
+        t0 = time.time()
+        options = {"disp": bool(verbose)}
+        if time_limit is not None:
+            options["time_limit"] = float(time_limit)
+        if mip_rel_gap is not None:
+            options["mip_rel_gap"] = float(mip_rel_gap)
+        constraints = [LinearConstraint(a, np.asarray(self._lb), np.asarray(self._ub))] if self._names else []
+        res = milp(self.objective, integrality=np.ones(self.n_vars), bounds=Bounds(np.zeros(self.n_vars), self.upper),
+                   constraints=constraints, options=options)
+        self.solve_seconds = time.time() - t0
+        self.raw = res
+        # scipy: 0 optimal, 1 iteration/time limit, 2 infeasible, 3 unbounded, 4 other
+        if res.status == 0 or (res.status == 1 and res.x is not None):
+            self.status = 1
+            self.x = np.rint(res.x).astype(np.int8)
+            self.objective_value = float(res.fun)
+        else:
+            self.status = -1
+            self.x = None
+            self.objective_value = None
+        return self.status
+
+    # ---- inspection ------------------------------------------------------------------------
+    def violated_constraints(self, x=None, tol: float = 1e-6) -> list:
+        x = self.x if x is None else x
+        if x is None or not self._names:
+            return []
+        act = self.matrix() @ np.asarray(x, np.float64)
+        bad = np.nonzero((act < np.asarray(self._lb) - tol) | (act > np.asarray(self._ub) + tol))[0]
+        return [self._names[i] for i in bad]

@@ -1,0 +1,550 @@
+"""``ShardingOptimizer``: the planner class of the reference
+(autoparallel/optimize_sharding.py:129-958) with its cost-table build replaced by one
+batched pass over HIP kernels.
+
+Same constructor, attributes and methods as the reference class, so its callers
+(autoparallel/api.py:273-282, 398-445) can use it unchanged:
+
+    opt = ShardingOptimizer(gm, mesh, rescale_grad_comm_cost_for_mp=1.0, repeated_subgraphs=False)
+    opt.strats, opt.ds, opt.num_inp_out, opt.num_args, opt.prob, opt.res, opt.cluster_links
+    opt.add_grad_param_constraints(), add_parameter_memory_constraint(), add_node_constraint(),
+    add_sharded_input_constraint(), add_sharded_output_constraint(), get_solution(), get_log(),
+    print_costs_for_node()
+
+What differs underneath:
+  * ``build_ds`` flattens ``strats`` once (graphs/encode.py), sends the tables to the GPU,
+    runs the integer shard-shape kernel, the compute-cost kernel and the redistribution-cost
+    kernel, and copies the three result arrays back.  ``ds`` is a read-only mapping view over
+    those arrays: a record dict is materialised only when a key is looked up.
+  * every ILP variable is an entry index of the flattened tables; constraints are emitted
+    as sparse index arrays and solved by HiGHS through scipy (PuLP / CBC are not required).
+  * the environment inputs the reference reads implicitly (devices per host, device row)
+    are explicit: class attributes ``devices_per_host`` / ``device_name``, defaulting to the
+    values the reference's own tests patch in (8, "H100").
+There is no CPU path for the tables: without a HIP device construction raises.
+"""
+
+from __future__ import annotations
+
+import math
+import operator
+import time
+from collections.abc import Mapping
+from typing import Optional
+
+import numpy as np
+import torch
+from torch.distributed.tensor._dtensor_spec import DTensorSpec
+from torch.distributed.tensor.placement_types import Placement, Replicate, Shard
+
+from .cost_model import CostModelParams
+from .graphs.cost_inputs import fill_flops_and_bytes
+from .graphs.encode import EncodedGraph, all_input_nodes, encode_graph
+from .graphs.strategies import StrategyEnumerator
+from .ilp import BinaryProgram, next_name
+
+
+class DeviceBackend:
+    """Runs the table kernels on the GPU (the only backend of the product)."""
+
+    def __init__(self, tables, params: CostModelParams, device="cuda:0"):
+        from .device_tables import DeviceCostTables
+
+        self.dev = DeviceCostTables(tables, params, device=device)
+        self.timings = {}
+
+    def local_shapes(self):
+        out = self.dev.run_spec_tables()
+        return out["local_shape"].cpu().numpy(), out["local_stride"].cpu().numpy()
+
+    def upload_strategy_inputs(self, tables):
+        d = self.dev
+        for k in ("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost"):
+            d.d[k].copy_(torch.from_numpy(getattr(tables, k)))
+
+    def build(self):
+        d = self.dev
+        t0 = time.perf_counter()
+        d.build_all()
+        torch.cuda.synchronize(d.device)
+        self.timings["kernels_s"] = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        out = {
+            "comm": d.comm.cpu().numpy(),
+            "transition": d.transition.cpu().numpy(),
+            "cost": d.cost.cpu().numpy(),
+            "compute_per_arg": d.compute_cost_per_arg.cpu().numpy(),
+        }
+        self.timings["copy_back_s"] = time.perf_counter() - t0
+        return out
+
+    def row_min(self, row_ptr):
+        mins, args = self.dev.segmented_min(self.dev.cost, row_ptr)
+        return mins.cpu().numpy(), args.cpu().numpy()
+
+
+class CostRecords(Mapping):
+    """``ds``: (s_i, argi, ss, ii) -> record, backed by the flat result arrays."""
+
+    def __init__(self, optimizer: "ShardingOptimizer"):
+        self._o = optimizer
+
+    def _index(self, key) -> int:
+        s_i, argi, ss, ii = key
+        enc = self._o.encoded
+        e = enc.edge_of.get((s_i, argi))
+        if e is None:
+            raise KeyError(key)
+        tb = enc.tables
+        ns, nt = int(tb.edge_n_src[e]), int(tb.edge_n_tgt[e])
+        if not (0 <= ss < nt and 0 <= ii < ns):
+            raise KeyError(key)
+        return int(tb.edge_entry_begin[e]) + ss * ns + ii
+
+    def __getitem__(self, key):
+        o = self._o
+        idx = self._index(key)
+        s_i, argi, ss, _ = key
+        full = o.strats[o.nodes[s_i]].strategies[ss]
+        return {
+            "va": int(o.var_of_entry[idx]),
+            "cost": float(o.cost[idx]),
+            "compute_cost": float(o.compute_cost_per_arg[o.encoded.strat_begin[s_i] + ss]),
+            "comm_cost": float(o.comm_cost[idx]),
+            "sharding_transition_cost": int(o.transition_cost[idx]),
+            "full_strat": full,
+            "out_strat": full.output_specs,
+            "inp_strat": full.input_specs[argi],
+        }
+
+    def __contains__(self, key):
+        try:
+            self._index(key)
+            return True
+        except (KeyError, TypeError, ValueError):
+            return False
+
+    def __len__(self):
+        return self._o.encoded.tables.n_entries
+
+    def __iter__(self):
+        enc = self._o.encoded
+        tb = enc.tables
+        for e, (s_i, argi) in enumerate(enc.edge_keys):
+            ns, nt = int(tb.edge_n_src[e]), int(tb.edge_n_tgt[e])
+            for ss in range(nt):
+                for ii in range(ns):
+                    yield (s_i, argi, ss, ii)
+
+    def key_of_entry(self, idx: int):
+        tb = self._o.encoded.tables
+        e = int(np.searchsorted(tb.edge_entry_begin, idx, side="right")) - 1
+        s_i, argi = self._o.encoded.edge_keys[e]
+        ns = int(tb.edge_n_src[e])
+        local = idx - int(tb.edge_entry_begin[e])
+        return (s_i, argi, local // ns, local % ns)
+
+
+class ShardingOptimizer:
+    # environment of the cost model, explicit (the reference reads torch.cuda.device_count()
+    # and torch.cuda.get_device_name(); its tests patch them to 8 and "H100")
+    devices_per_host = 8
+    device_name = "H100"
+    device = "cuda:0"
+    backend_cls = DeviceBackend
+    solver_time_limit: Optional[float] = None
+
+    def __init__(self, gm, mesh, rescale_grad_comm_cost_for_mp=1.0, repeated_subgraphs=False):
+        self.gm = gm
+        self.graph = gm.graph
+        self.nodes = list(self.graph.nodes)
+        self.mesh = mesh
+        self.rescale_grad_comm_cost_for_mp = rescale_grad_comm_cost_for_mp
+        self.node_map = {node: i for i, node in enumerate(self.graph.nodes)}
+        self.timings = {}
+        t0 = time.perf_counter()
+        self.strats = self.build_sharding_metadata()
+        self.timings["enumerate_s"] = time.perf_counter() - t0
+
+        self.cluster_links = {}
+        if repeated_subgraphs:
+            raise NotImplementedError("repeated_subgraphs=True (ILP variable sharing across identical layers) "
+                                      "is not implemented yet")
+        self.ds, self.num_inp_out, self.num_args = self.build_ds()
+        self.validate()
+        self.prob = BinaryProgram(self.encoded.tables.n_entries, "AutoParallel")
+        self.res = None
+        self.add_default_constraints()
+
+    # ------------------------------------------------------------------------------------
+    def build_sharding_metadata(self):
+        self.enumerator = StrategyEnumerator(self.mesh)
+        return self.enumerator.enumerate(self.graph)
+
+    def _grad_param_nodes(self):
+        from torch._functorch._aot_autograd.fx_utils import get_param_and_grad_nodes
+
+        try:
+            return set(x[1] for x in get_param_and_grad_nodes(self.graph).values())
+        except (KeyError, AttributeError):
+            return set()  # a graph without AOT descriptors has no parameter gradients to rescale
+
+    def cost_model_params(self) -> CostModelParams:
+        return CostModelParams.from_mesh(tuple(self.mesh.shape), device_name=self.device_name,
+                                         devices_per_host=self.devices_per_host,
+                                         rescale=self.rescale_grad_comm_cost_for_mp)
+
+    def build_ds(self):
+        """Batched table build: encode -> shard-shape kernel -> flop / byte inference ->
+        compute-cost kernel -> redistribution-cost kernel -> copy back."""
+        t0 = time.perf_counter()
+        self.encoded: EncodedGraph = encode_graph(self.graph, self.strats, tuple(self.mesh.shape),
+                                                  self._grad_param_nodes())
+        self.timings["encode_s"] = time.perf_counter() - t0
+        self.params = self.cost_model_params()
+        tb = self.encoded.tables
+        t0 = time.perf_counter()
+        self.backend = self.backend_cls(tb, self.params, self.device)
+        local_shape, local_stride = self.backend.local_shapes()
+        self.timings["upload_and_shapes_s"] = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        self.cost_input_stats = {}
+        fill_flops_and_bytes(self.encoded, self.strats, local_shape, local_stride, self.cost_input_stats)
+        self.backend.upload_strategy_inputs(tb)
+        self.timings["flops_bytes_s"] = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        out = self.backend.build()
+        self.timings["tables_s"] = time.perf_counter() - t0
+        self.timings.update({f"backend_{k}": v for k, v in getattr(self.backend, "timings", {}).items()})
+        self.comm_cost = out["comm"]
+        self.transition_cost = out["transition"]
+        self.cost = out["cost"].copy()
+        self.compute_cost_per_arg = out["compute_per_arg"]
+        self.var_of_entry = np.arange(tb.n_entries, dtype=np.int64)
+        # the recomputed costs are written back into OpSpec.redistribute_cost, which
+        # print_costs_for_node reads (optimize_sharding.py:361-363)
+        t0 = time.perf_counter()
+        self._write_back_redistribute_cost()
+        self.timings["write_back_s"] = time.perf_counter() - t0
+        return CostRecords(self), self.encoded.num_inp_out, self.encoded.num_args
+
+    def _write_back_redistribute_cost(self):
+        tb = self.encoded.tables
+        comm = self.comm_cost
+        for e, (s_i, argi) in enumerate(self.encoded.edge_keys):
+            ns, nt = int(tb.edge_n_src[e]), int(tb.edge_n_tgt[e])
+            b = int(tb.edge_entry_begin[e])
+            rows = comm[b:b + ns * nt].reshape(nt, ns).tolist()
+            for s, row in zip(self.strats[self.nodes[s_i]].strategies, rows):
+                s.redistribute_cost[argi] = row
+
+    # ------------------------------------------------------------------------------------
+    def _all_input_nodes(self, node):
+        return all_input_nodes(node)
+
+    def walk_over_options(self, node, constrain_arg=None):
+        tgt = self.strats[node]
+        for argi in range(len(tgt.strategies[0].input_specs)):
+            if constrain_arg is not None and argi != constrain_arg:
+                continue
+            for oi, s in enumerate(tgt.strategies):
+                for ii in range(len(s.redistribute_cost[argi])):
+                    yield argi, oi, ii
+
+    def _edge(self, s_i, argi):
+        e = self.encoded.edge_of[(s_i, argi)]
+        tb = self.encoded.tables
+        return int(tb.edge_entry_begin[e]), int(tb.edge_n_tgt[e]), int(tb.edge_n_src[e])
+
+    # ---- default constraints (optimize_sharding.py:402-542) --------------------------------
+    def add_unique_decision_constraint(self):
+        """For every (node, argument): exactly one (output, input) strategy pair."""
+        tb = self.encoded.tables
+        lens = tb.edge_entry_begin[1:] - tb.edge_entry_begin[:-1]
+        self.prob.add_rows(self.var_of_entry, 1.0, lens, 1.0, 1.0, "unique_decision")
+
+    def add_same_output_across_args_constraint(self):
+        """All arguments of a node agree on the node's output strategy."""
+        cols, vals, lens = [], [], []
+        for s_i, node in enumerate(self.nodes):
+            if node.op != "call_function" or len(self._all_input_nodes(node)) <= 1:
+                continue
+            b0, nt, ns0 = self._edge(s_i, 0)
+            for argi in range(1, len(self._all_input_nodes(node))):
+                ba, nta, nsa = self._edge(s_i, argi)
+                assert nta == nt
+                first = b0 + np.arange(nt)[:, None] * ns0 + np.arange(ns0)[None, :]
+                other = ba + np.arange(nt)[:, None] * nsa + np.arange(nsa)[None, :]
+                cols.append(np.concatenate([first, other], axis=1).ravel())
+                vals.append(np.tile(np.concatenate([np.ones(ns0), -np.ones(nsa)]), nt))
+                lens.append(np.full(nt, ns0 + nsa))
+        if cols:
+            self.prob.add_rows(self.var_of_entry[np.concatenate(cols)], np.concatenate(vals), np.concatenate(lens),
+                               0.0, 0.0, "same_across_args")
+
+    def add_output_input_consistent_constraint(self):
+        """The producer's chosen output strategy is the column its consumers read."""
+        cols, vals, lens = [], [], []
+        for s_i, node in enumerate(self.nodes):
+            if node.op == "output":
+                continue
+            bp, ntp, nsp = self._edge(s_i, 0)
+            for user in node.users:
+                if user.op == "output":
+                    continue
+                s_j = self.node_map[user]
+                argj = [i for i, n in enumerate(user.all_input_nodes) if n == node]
+                assert len(argj) == 1
+                bc, ntc, nsc = self._edge(s_j, argj[0])
+                assert nsc == ntp, f"{node} has {ntp} strategies, {user} arg {argj[0]} reads {nsc}"
+                prod = bp + np.arange(ntp)[:, None] * nsp + np.arange(nsp)[None, :]  # row o of producer
+                cons = bc + np.arange(ntc)[None, :] * nsc + np.arange(nsc)[:, None]  # column o of consumer
+                cols.append(np.concatenate([prod, cons], axis=1).ravel())
+                vals.append(np.tile(np.concatenate([np.ones(nsp), -np.ones(ntc)]), ntp))
+                lens.append(np.full(ntp, nsp + ntc))
+        if cols:
+            self.prob.add_rows(self.var_of_entry[np.concatenate(cols)], np.concatenate(vals), np.concatenate(lens),
+                               0.0, 0.0, "output_input_consistent")
+
+    def add_inf_cost_constraint(self):
+        """Non-finite costs become 10000 and their variable is forced to 0."""
+        bad = np.nonzero(~np.isfinite(self.cost))[0]
+        self.cost[bad] = self.params.inf_replacement_cost
+        self.prob.force_zero(self.var_of_entry[bad])
+        self.inf_entries = bad
+
+    def add_default_constraints(self):
+        self.add_unique_decision_constraint()
+        self.add_same_output_across_args_constraint()
+        self.add_output_input_consistent_constraint()
+        self.add_inf_cost_constraint()
+
+    # ---- solve (optimize_sharding.py:648-701) ------------------------------------------------
+    def get_solution(self, verbose=False):
+        obj = np.zeros(self.prob.n_vars)
+        np.add.at(obj, self.var_of_entry, self.cost)  # duplicate variables: costs add up
+        self.prob.objective = obj
+        status = self.prob.solve(verbose=verbose, time_limit=self.solver_time_limit)
+        if status == -1:
+            print(self.get_violated_constraints_log())
+            raise RuntimeError("Unsolvable problem")
+        chosen = np.nonzero(self.prob.x[self.var_of_entry] == 1)[0]
+        self.res = [self.ds.key_of_entry(int(i)) for i in chosen]
+        self.res_entries = chosen
+
+        opt = {}
+        nodes = self.nodes
+        for key in self.res:
+            opt.setdefault(nodes[key[0]], []).append(self.ds[key])
+        seen = set()
+        for r in self.res:
+            key = (r[0], r[1])
+            if key in seen:
+                raise RuntimeError(
+                    f"Multiple solutions for {nodes[key[0]]}, key={key}, "
+                    f"solutions: {[str(x['full_strat']) for x in opt[nodes[key[0]]]]}")
+            seen.add(key)
+        for k in opt.values():
+            assert all(k[0]["full_strat"] == kk["full_strat"] for kk in k), \
+                f"{[kk['va'] for kk in k]}: {[str(kk['full_strat']) for kk in k]}"
+        return {k: v[0]["full_strat"] for k, v in opt.items()}
+
+    def objective_value(self) -> float:
+        return float(self.cost[self.res_entries].sum())
+
+    def get_violated_constraints_log(self):
+        names = self.prob.violated_constraints()
+        return f"Violated constraints: {names}"
+
+    # ---- user constraints (optimize_sharding.py:703-906) ---------------------------------------
+    def _add_node_constraint(self, node, output_constraint_indices, constraint_name=None):
+        if constraint_name is None:
+            constraint_name = "user_constraint"
+        s_i = self.node_map[node]
+        rows = np.asarray(sorted(output_constraint_indices), np.int64)
+        for argi in range(self.num_args[s_i]):
+            b, nt, ns = self._edge(s_i, argi)
+            idx = (b + rows[:, None] * ns + np.arange(ns)[None, :]).ravel()
+            self.prob.add_row(self.var_of_entry[idx], 1.0, 1.0, 1.0, next_name(constraint_name))
+
+    def add_grad_param_constraints(self):
+        """A parameter and its gradient choose the same placement."""
+        from torch._functorch._aot_autograd.fx_utils import get_param_and_grad_nodes
+
+        for param, grad in get_param_and_grad_nodes(self.graph).values():
+            if grad is None:
+                continue
+            s_i, s_j = self.node_map[param], self.node_map[grad]
+            num_out = self.num_inp_out[(s_i, 0)]["num_output_strat"]
+            num_inp_g = self.num_inp_out[(s_j, 0)]["num_input_strat"]
+            strat_p = [str(s.output_specs) for s in self.strats[param].strategies]
+            assert num_out == len(strat_p)
+            strat_gp = [str(s.output_specs) for s in self.strats[grad].strategies]
+            bp, _, nsp = self._edge(s_i, 0)
+            bg, _, nsg = self._edge(s_j, 0)
+            for oi in range(num_out):
+                sp = strat_p[oi]
+                if sp not in strat_gp:
+                    continue
+                ooi = strat_gp.index(sp)
+                g = bg + ooi * nsg + np.arange(num_inp_g)
+                cols = np.concatenate([g, [bp + oi * nsp]])
+                vals = np.concatenate([np.ones(num_inp_g), [-1.0]])
+                self.prob.add_row(self.var_of_entry[cols], vals, 0.0, 0.0, next_name("grad_param_constraint"))
+
+    def add_parameter_memory_constraint(self, memory_factor_low: float, memory_factor_high: float):
+        """Sum over parameters of (local size / global size) stays within [low, high] x #params."""
+        from torch._functorch._aot_autograd.fx_utils import get_param_nodes
+
+        world_size = math.prod(self.mesh.shape)
+        cols, vals = [], []
+        considered = 0
+        for node in get_param_nodes(self.graph):
+            s_i = self.node_map[node]
+            if node.meta["val"].numel() < world_size:
+                continue
+            considered += 1
+            b, nt, ns = self._edge(s_i, 0)
+            for oi in range(self.num_inp_out[(s_i, 0)]["num_output_strat"]):
+                spec: DTensorSpec = self.strats[node].strategies[oi].input_specs[0]
+                shape = list(spec.tensor_meta.shape)
+                old = math.prod(shape)
+                for n, p in zip(self.mesh.shape, spec.placements):
+                    if p.is_shard():
+                        shape[p.dim] = (shape[p.dim] + n - 1) // n
+                cols.append(b + oi * ns)
+                vals.append(math.prod(shape) / old)
+        cols = self.var_of_entry[np.asarray(cols, np.int64)]
+        self.prob.add_row(cols, vals, -np.inf, memory_factor_high * considered, "memory_constraint_high")
+        self.prob.add_row(cols, vals, memory_factor_low * considered, np.inf, "memory_constraint_low")
+
+    def add_node_constraint(self, node, placement=None, constraint_name=None):
+        assert node in self.strats, (node, self.strats.keys())
+        if placement is None:
+            placement = (Shard(0),) + (Replicate(),) * (self.mesh.ndim - 1)
+        wanted = [i for i, s in enumerate(self.strats[node].strategies) if s.output_specs.placements == placement]
+        if not wanted:
+            raise RuntimeError(f"Couldn't find appropriate constraint {node} {constraint_name} {placement}")
+        self._add_node_constraint(node, output_constraint_indices=wanted, constraint_name=constraint_name)
+
+    def add_sharded_input_constraint(self, input_placements: Optional[list[Optional[tuple[Placement, ...]]]] = None):
+        from torch._functorch._aot_autograd.descriptors import PlainAOTInput
+        from torch._functorch._aot_autograd.fx_utils import get_plain_input_and_grad_nodes
+
+        pending = None if input_placements is None else dict(enumerate(input_placements))
+        for desc, (node, grad_node) in get_plain_input_and_grad_nodes(self.graph).items():
+            if pending is None:
+                placement = None
+            else:
+                assert isinstance(desc, PlainAOTInput)
+                placement = pending.pop(desc.idx)
+            self.add_node_constraint(node, placement, constraint_name="input_constraint")
+            if grad_node is not None:
+                self.add_node_constraint(grad_node, placement, constraint_name="grad_input_constraint")
+        ignored = [i for i, p in (pending or {}).items() if p is not None]
+        if ignored:
+            raise RuntimeError(
+                f"We were unable to respect placements for inputs at indices {ignored}.  The traced joint graph has "
+                "no dedicated placeholder node for these inputs (typically because inputs alias each other); "
+                "remove the explicit placement (use None) or clone the inputs before tracing.")
+
+    def add_sharded_output_constraint(self, output_placements=None):
+        from torch._functorch._aot_autograd.descriptors import PlainAOTOutput
+        from torch._functorch._aot_autograd.fx_utils import get_plain_output_and_tangent_nodes
+
+        pending = None if output_placements is None else dict(enumerate(output_placements))
+        for desc, (node, tangent_node) in get_plain_output_and_tangent_nodes(self.graph).items():
+            if pending is None:
+                placement = None
+            else:
+                assert isinstance(desc, PlainAOTOutput)
+                placement = pending.pop(desc.idx)
+            self.add_node_constraint(node, placement, constraint_name="output_constraint")
+            if tangent_node is not None:
+                self.add_node_constraint(tangent_node, placement, constraint_name="grad_output_constraint")
+        ignored = [i for i, p in (pending or {}).items() if p is not None]
+        if ignored:
+            raise RuntimeError(
+                f"We were unable to respect placements for outputs at indices {ignored}.  The traced joint graph has "
+                "no dedicated output node for these outputs (typically because outputs alias each other); "
+                "remove the explicit placement (use None) or clone the outputs before returning them.")
+
+    # ---- reporting (optimize_sharding.py:569-646) ------------------------------------------------
+    def get_log(self, colored=False):
+        from torch.fx.graph import _color_fns, _identity
+
+        opt = {}
+        nodes = self.nodes
+        for key in self.res:
+            opt.setdefault(nodes[key[0]], []).append(self.ds[key])
+        code = self.graph.python_code("self", colored=colored).src.strip().split("\n")
+        txt_color = _color_fns["blue"] if colored else _identity
+        attr_color = _color_fns["red"] if colored else _identity
+        l_id = 1
+        plc_txt, cost_txt = txt_color("# placement="), txt_color(", cost=")
+        for node in nodes:
+            if node.op == "output":
+                continue
+            d = opt[node]
+            strat = str(d[0]["full_strat"])
+            costs = [(x["comm_cost"], x["compute_cost"], x["sharding_transition_cost"]) for x in d]
+            line = f"  {plc_txt}{attr_color(strat)} {cost_txt}{attr_color(str(costs))}"
+            if node.op == "placeholder":
+                code.insert(l_id, f"    # {node.name}: {line}")
+                l_id += 1
+                continue
+            while not code[l_id].lstrip().startswith(repr(node)):
+                l_id += 1
+            code[l_id] += line
+            l_id += 1
+        code = "\n".join(code)
+        idx = self.res_entries
+        strat_rows = np.asarray([self.encoded.strat_begin[k[0]] + k[2] for k in self.res], np.int64)
+        code += f"\ntotal_cost: {self.cost[idx].sum():.2f}"
+        code += f"\n  comm_cost: {self.comm_cost[idx].sum():.2f}"
+        code += f"\n  compute_cost: {self.compute_cost_per_arg[strat_rows].sum():.2f}"
+        code += f"\n  transition_cost: {self.transition_cost[idx].astype(np.float64).sum():.2f}"
+        code += "\n" + self.get_violated_constraints_log()
+        return code
+
+    def print_costs_for_node(self, node, arg=0, **kwargs):
+        from tabulate import tabulate
+        from torch.distributed.tensor._op_schema import _pretty_print_spec
+
+        tgt = self.strats[node]
+        src = self.strats[self._all_input_nodes(node)[arg]]
+        headers = [""] + [_pretty_print_spec(x.output_specs) for x in src.strategies]
+        costs = [[str(x)] + x.redistribute_cost[arg] for x in tgt.strategies]
+        print(tabulate(costs, headers=headers, **kwargs))
+
+    # ---- warm-start helpers built on the segmented min kernel -------------------------------------
+    def row_minima(self):
+        """min / first-argmin over producer strategies for every (edge, consumer strategy)."""
+        return self.backend.row_min(self.encoded.tables.row_ptr())
+
+    # ---- structural checks (optimize_sharding.py:908-958) -------------------------------------------
+    def validate(self):
+        for node in self.graph.nodes:
+            if node.op != "call_function":
+                continue
+            strat0 = self.strats[node].strategies[0]
+            inputs = self._all_input_nodes(node)
+            n_in = len(inputs)
+            assert (len(strat0.redistribute_cost) == n_in) or (n_in == 0 and len(strat0.redistribute_cost) == 1), \
+                f"{node}, {len(strat0.redistribute_cost)}, {n_in}"
+            ospec = strat0.output_specs
+            if isinstance(ospec, (list, tuple)):
+                for spec in ospec:
+                    if spec:
+                        assert spec.tensor_meta is not None, f"{node} doesn't have a tensor_meta"
+            elif ospec is not None:
+                assert ospec.tensor_meta is not None, f"{node} doesn't have a tensor_meta"
+            for ispec in strat0.input_specs:
+                if isinstance(ispec, (list, tuple)):
+                    for spec in ispec:
+                        assert spec.tensor_meta is not None, f"{node} input_spec doesn't have a tensor_meta"
+                elif ispec is not None:
+                    assert ispec.tensor_meta is not None, f"{node} input_spec doesn't have a tensor_meta"
+            for i, arg in enumerate(inputs):
+                n_arg = len(self.strats[arg].strategies)
+                assert len(strat0.redistribute_cost[i]) == n_arg, f"{node}, {len(strat0.redistribute_cost[i])}, {n_arg}"

@@ -1,0 +1,34 @@
+"""Test-only table backend: the CPU oracle behind the planner's backend interface, so the
+host logic (encoding, ILP) can be exercised without a GPU and so GPU-built tables can be
+compared with oracle-built ones through the same solver.  Never used by the product."""
+
+import numpy as np
+
+from oracle import c_oracle
+from oracle import cost_oracle as po
+
+
+class OracleBackend:
+    def __init__(self, tables, params, device=None):
+        self.tables = tables
+        self.params = po.make_params(params.mesh_sizes, device_name=params.device_name, rescale=params.rescale)
+        assert self.params.bw == params.bw and self.params.lat == params.lat
+        self.timings = {}
+
+    def local_shapes(self):
+        _, lshape, lstride, _, _ = c_oracle.spec_tables(self.tables.as_dict(), self.tables.mesh_sizes)
+        return lshape, lstride
+
+    def upload_strategy_inputs(self, tables):
+        pass
+
+    def build(self):
+        enc = self.tables.as_dict()
+        compute, per_arg = c_oracle.compute_costs(enc, self.params)
+        out = c_oracle.build_tables(enc, self.params, per_arg=per_arg)
+        out["compute_per_arg"] = per_arg
+        self.cost = out["cost"]
+        return out
+
+    def row_min(self, row_ptr):
+        return c_oracle.segmented_min(self.cost, row_ptr)
