@@ -27,6 +27,25 @@ _UPLOAD = (
 )
 
 
+def _real_tensors():
+    """The planner is usually called while a graph-capture context keeps a FakeTensorMode
+    (or another dispatch mode) active; device buffers must be real allocations."""
+    from torch.utils._python_dispatch import _disable_current_modes
+
+    return _disable_current_modes()
+
+
+def _guarded(fn):
+    import functools
+
+    @functools.wraps(fn)
+    def wrapper(*args, **kwargs):
+        with _real_tensors():
+            return fn(*args, **kwargs)
+
+    return wrapper
+
+
 def _to_device(a: np.ndarray, device) -> torch.Tensor:
     if a.dtype == np.uint32:  # same bits; torch's uint32 support is partial
         a = a.view(np.int32)
@@ -36,6 +55,7 @@ def _to_device(a: np.ndarray, device) -> torch.Tensor:
 
 
 class DeviceCostTables:
+    @_guarded
     def __init__(self, tables: CostTables, params: CostModelParams, device="cuda:0", validate=True):
         if not torch.cuda.is_available():
             raise RuntimeError("DeviceCostTables needs a HIP device; there is no CPU path")
@@ -68,6 +88,7 @@ class DeviceCostTables:
         return torch.empty(shape, dtype=dtype, device=self.device)
 
     # ---- integer tables ------------------------------------------------------------------
+    @_guarded
     def run_tensor_tables(self):
         n = self.tables.n_tensors
         self.tensor_bytes = self._empty((n,), torch.int64)
@@ -80,6 +101,7 @@ class DeviceCostTables:
         _native.check(rc, "apc_tensor_tables")
         return self.tensor_bytes, self.tensor_contiguous
 
+    @_guarded
     def run_spec_tables(self):
         n = self.tables.n_specs
         out = {
@@ -101,6 +123,7 @@ class DeviceCostTables:
         return out
 
     # ---- per-strategy compute cost ---------------------------------------------------------
+    @_guarded
     def run_compute_costs(self):
         n = self.tables.n_strategies
         self.compute_cost = self._empty((n,), torch.float64)
@@ -118,12 +141,14 @@ class DeviceCostTables:
         return self.compute_cost, self.compute_cost_per_arg
 
     # ---- redistribution-cost matrices ------------------------------------------------------
+    @_guarded
     def alloc_outputs(self, comm=True, transition=True, cost=True):
         n = self.tables.n_entries
         self.comm = self._empty((n,), torch.float64) if comm else None
         self.transition = self._empty((n,), torch.uint8) if transition else None
         self.cost = self._empty((n,), torch.float64) if cost else None
 
+    @_guarded
     def launch_redistribute_tables(self):
         """One enqueue of the table kernel over pre-allocated outputs (no allocation,
         no synchronisation): the timed unit of the benchmark."""
@@ -139,6 +164,7 @@ class DeviceCostTables:
                 self._stream())
         _native.check(rc, "apc_redistribute_tables")
 
+    @_guarded
     def run_redistribute_tables(self, comm=True, transition=True, cost=True):
         if self.tensor_bytes is None:
             self.run_tensor_tables()
@@ -148,6 +174,7 @@ class DeviceCostTables:
         self.launch_redistribute_tables()
         return self.comm, self.transition, self.cost
 
+    @_guarded
     def build_all(self):
         """tensor tables -> compute costs -> cost matrices, all on the current stream."""
         self.run_tensor_tables()
@@ -155,6 +182,7 @@ class DeviceCostTables:
         return self.run_redistribute_tables()
 
     # ---- segmented min ---------------------------------------------------------------------
+    @_guarded
     def segmented_min(self, values: torch.Tensor, seg_ptr):
         if not isinstance(seg_ptr, torch.Tensor):
             seg_ptr = torch.from_numpy(np.ascontiguousarray(seg_ptr, dtype=np.int64)).to(self.device)

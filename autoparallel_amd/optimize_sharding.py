@@ -54,15 +54,27 @@ class DeviceBackend:
         self.timings = {}
 
     def local_shapes(self):
-        out = self.dev.run_spec_tables()
-        return out["local_shape"].cpu().numpy(), out["local_stride"].cpu().numpy()
+        from .device_tables import _real_tensors
+
+        with _real_tensors():
+            out = self.dev.run_spec_tables()
+            return out["local_shape"].cpu().numpy(), out["local_stride"].cpu().numpy()
 
     def upload_strategy_inputs(self, tables):
+        from .device_tables import _real_tensors
+
         d = self.dev
-        for k in ("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost"):
-            d.d[k].copy_(torch.from_numpy(getattr(tables, k)))
+        with _real_tensors():
+            for k in ("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost"):
+                d.d[k].copy_(torch.from_numpy(getattr(tables, k)))
 
     def build(self):
+        from .device_tables import _real_tensors
+
+        with _real_tensors():
+            return self._build()
+
+    def _build(self):
         d = self.dev
         t0 = time.perf_counter()
         d.build_all()
@@ -79,8 +91,11 @@ class DeviceBackend:
         return out
 
     def row_min(self, row_ptr):
-        mins, args = self.dev.segmented_min(self.dev.cost, row_ptr)
-        return mins.cpu().numpy(), args.cpu().numpy()
+        from .device_tables import _real_tensors
+
+        with _real_tensors():
+            mins, args = self.dev.segmented_min(self.dev.cost, row_ptr)
+            return mins.cpu().numpy(), args.cpu().numpy()
 
 
 class CostRecords(Mapping):
