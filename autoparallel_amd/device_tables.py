@@ -181,6 +181,60 @@ class DeviceCostTables:
         self.run_compute_costs()
         return self.run_redistribute_tables()
 
+    # ---- one full device-side pass with pre-bound arguments -------------------------------------
+    @_guarded
+    def prepare_step(self, row_min=True):
+        """Allocates every output once and returns ``{kernel name: zero-argument launcher}``
+        in launch order.  A launcher only enqueues (no allocation, no synchronisation), so a
+        timed loop measures the kernels and not Python argument marshalling."""
+        self.run_tensor_tables()
+        spec = self.run_spec_tables()
+        self.run_compute_costs()
+        self.alloc_outputs(True, True, True)
+        lib, P, cp = self.lib, self._p, ctypes.byref(self.c_params)
+        stream = self._stream()
+        tb = self.tables
+        err = torch.zeros((1,), dtype=torch.int32, device=self.device)
+        self._step_keepalive = [err, spec]
+        a_tensor = (ctypes.c_int64(tb.n_tensors), P("tensor_rank"), P("tensor_itemsize"), P("tensor_shape"),
+                    P("tensor_stride"), P(self.tensor_bytes), P(self.tensor_contiguous), stream)
+        a_spec = (cp, ctypes.c_int64(tb.n_specs), P("spec_codes"), P("spec_tensor"), P("tensor_rank"),
+                  P("tensor_itemsize"), P("tensor_shape"), P("tensor_stride"), P(spec["num_shards"]),
+                  P(spec["local_shape"]), P(spec["local_stride"]), P(spec["local_numel"]), P(spec["local_bytes"]),
+                  stream)
+        a_compute = (cp, ctypes.c_int64(tb.n_strategies), P("strat_flops"), P("strat_rw_bytes"), P("strat_dtype"),
+                     P("strat_zero_cost"), P("strat_num_args"), P(self.compute_cost), P(self.compute_cost_per_arg),
+                     P(err), stream)
+        a_tables = (cp, P(self.tensor_bytes), P(self.tensor_contiguous), P("spec_codes"), P("spec_tensor"),
+                    P("edge_src_begin"), P("edge_n_src"), P("edge_tgt_begin"), P("edge_n_tgt"), P("edge_flags"),
+                    P("edge_pt_begin"), P("edge_entry_begin"), P("edge_strat_begin"), P("pt_values"),
+                    P(self.compute_cost_per_arg), ctypes.c_int64(tb.n_tiles), P("tile_edge"), P("tile_row_begin"),
+                    P("tile_row_count"), P("tile_col_begin"), P("tile_col_count"), P(self.comm), P(self.transition),
+                    P(self.cost), stream)
+
+        def bind(fn, args, what):
+            def launch():
+                rc = fn(*args)
+                if rc != 0:
+                    _native.check(rc, what)
+            return launch
+
+        step = {
+            "tensor_tables": bind(lib.apc_tensor_tables, a_tensor, "apc_tensor_tables"),
+            "spec_tables": bind(lib.apc_spec_tables, a_spec, "apc_spec_tables"),
+            "compute_costs": bind(lib.apc_compute_costs, a_compute, "apc_compute_costs"),
+            "redistribute_tables": bind(lib.apc_redistribute_tables, a_tables, "apc_redistribute_tables"),
+        }
+        if row_min:
+            row_ptr = torch.from_numpy(tb.row_ptr()).to(self.device)
+            n_seg = row_ptr.numel() - 1
+            self.row_min = self._empty((n_seg,), torch.float64)
+            self.row_argmin = self._empty((n_seg,), torch.int32)
+            self._step_keepalive.append(row_ptr)
+            a_min = (P(self.cost), P(row_ptr), ctypes.c_int64(n_seg), P(self.row_min), P(self.row_argmin), stream)
+            step["segmented_min"] = bind(lib.apc_segmented_min, a_min, "apc_segmented_min")
+        return step
+
     # ---- segmented min ---------------------------------------------------------------------
     @_guarded
     def segmented_min(self, values: torch.Tensor, seg_ptr):
