@@ -14,8 +14,8 @@ from ._build import LIB_PATH
 APC_MAX_RANK = 8
 APC_MAX_MESH = 4
 APC_MAX_DTYPES = 8
-APC_TILE_MAX_COLS = 1024
-APC_TILE_MAX_ROWS = 1024
+APC_TILE_MAX_COLS = 256
+APC_TILE_MAX_ROWS = 256
 
 EDGE_GRAD_RESCALE = 1
 EDGE_NO_PRODUCER = 2
@@ -36,6 +36,18 @@ class ApcParams(ctypes.Structure):
         ("rescale", ctypes.c_double),
         ("gpu_flops", ctypes.c_double * APC_MAX_DTYPES),
         ("transition_scale", ctypes.c_int32),
+    ]
+
+
+class ApcTile(ctypes.Structure):
+    _fields_ = [
+        ("edge", ctypes.c_int32),
+        ("row_begin", ctypes.c_int32), ("row_count", ctypes.c_int32),
+        ("col_begin", ctypes.c_int32), ("col_count", ctypes.c_int32),
+        ("src_begin", ctypes.c_int32), ("n_src", ctypes.c_int32), ("tgt_begin", ctypes.c_int32),
+        ("flags", ctypes.c_int32), ("strat_begin", ctypes.c_int32),
+        ("entry_begin", ctypes.c_int64), ("pt_begin", ctypes.c_int64),
+        ("reserved", ctypes.c_int32 * 2),
     ]
 
 

@@ -228,101 +228,200 @@ __global__ __launch_bounds__(kBlock) void compute_costs_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// a1-a6: redistribution-cost matrices, one workgroup per tile of one edge's matrix.
-// Producer specs (columns) and consumer specs (rows) of the tile are staged in LDS once;
-// every lane then walks the tile's entries with stride kBlock so that a wavefront
-// writes 64 consecutive fp64 values of a row.
+// a1-a6: redistribution-cost matrices.  One wavefront (a 64-thread workgroup) per tile of
+// one edge's matrix.
+//
+// The cost of an entry is a sum of per-mesh-dim terms; each term is an expensive
+// expression (fp64 divisions) of ONE quantity only: the running comm_bytes_gb at that
+// dim.  That quantity takes few distinct values inside a tile: it starts from
+// bytes / num_shards (decided by WHICH mesh dims the producer shards: a mask of M bits) and
+// every earlier dim either left it alone or applied its single possible update (x n after
+// an all-gather when the producer shards that dim, / n after a reduce-scatter when it does
+// not).  State (level L, mask, history) therefore indexes all values that can occur; the
+// prologue evaluates every collective / read-write term once per state into LDS, in
+// exactly the reference's operation order, and the per-entry loop only looks terms up and
+// adds them in the reference's order.  Results are bit-identical to evaluating every entry
+// directly (entry_cost), which remains the path for the rare cases the states do not
+// cover: producer specs of one edge that point at different tensors, and the 2-D
+// (Partial, Partial) -> all-Shard order flip.
 // ------------------------------------------------------------------------------------------
+constexpr int kTileThreads = 64;
+
 struct TableArgs {
   const int64_t *tensor_bytes;
   const uint8_t *tensor_contiguous;
   const uint32_t *spec_codes;
   const int32_t *spec_tensor;
-  const int32_t *edge_src_begin;
-  const int32_t *edge_n_src;
-  const int32_t *edge_tgt_begin;
-  const int32_t *edge_n_tgt;
-  const int32_t *edge_flags;
-  const int64_t *edge_pt_begin;
-  const int64_t *edge_entry_begin;
-  const int32_t *edge_strat_begin;
   const double *pt_values;
   const double *per_arg;
-  const int32_t *tile_edge;
-  const int32_t *tile_row_begin;
-  const int32_t *tile_row_count;
-  const int32_t *tile_col_begin;
-  const int32_t *tile_col_count;
+  const apc_tile *tiles;
   double *comm_out;
   uint8_t *trans_out;
   double *cost_out;
 };
 
 template <int M>
-__global__ __launch_bounds__(kBlock) void redistribute_tiles_kernel(apc_params p, TableArgs a) {
-  __shared__ double s_gb[APC_TILE_MAX_COLS];
+struct States {
+  // level L in [0, M]: 2^M masks x 2^L histories
+  static constexpr int kCount = (1 << M) * ((1 << (M + 1)) - 1);
+  __device__ static __forceinline__ int index(int level, int mask, int hist) {
+    return (((1 << level) - 1) << M) + (mask << level) + hist;
+  }
+};
+
+template <int M>
+__global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_params p, TableArgs a) {
+  constexpr int NS = States<M>::kCount;
   __shared__ uint32_t s_src[APC_TILE_MAX_COLS];
-  __shared__ uint8_t s_sflag[APC_TILE_MAX_COLS];  // bit0 valid spec, bit1 contiguous
+  __shared__ int32_t s_stensor[APC_TILE_MAX_COLS];
   __shared__ uint32_t s_tgt[APC_TILE_MAX_ROWS];
-  __shared__ uint8_t s_tflag[APC_TILE_MAX_ROWS];
+  __shared__ uint8_t s_tflag[APC_TILE_MAX_ROWS];  // bit0 valid spec, bit1 any Partial, bit2 all Shard
   __shared__ double s_cpa[APC_TILE_MAX_ROWS];
+  __shared__ double s_rw[NS];   // read+write time of the running bytes
+  __shared__ double s_ag[NS];   // all-gather of the previous dim (bytes already multiplied)
+  __shared__ double s_rs[NS];   // reduce-scatter of this level's dim
+  __shared__ double s_a2a[NS];  // all-to-all of this level's dim
+  __shared__ double s_ar[NS];   // all-reduce of this level's dim
+  __shared__ int s_uniform;
 
-  const int tile = blockIdx.x;
-  const int e = a.tile_edge[tile];
-  const int row0 = a.tile_row_begin[tile], rows = a.tile_row_count[tile];
-  const int col0 = a.tile_col_begin[tile], cols = a.tile_col_count[tile];
-  const int n_src = a.edge_n_src[e];
-  const int src_begin = a.edge_src_begin[e], tgt_begin = a.edge_tgt_begin[e];
-  const int flags = a.edge_flags[e];
-  const int64_t entry_begin = a.edge_entry_begin[e];
-  const int64_t pt_begin = a.edge_pt_begin[e];
-  const int strat_begin = a.edge_strat_begin[e];
+  const apc_tile tile = a.tiles[blockIdx.x];
+  const int rows = tile.row_count, cols = tile.col_count;
+  const int row0 = tile.row_begin, col0 = tile.col_begin;
+  const int n_src = tile.n_src;
+  const int flags = tile.flags;
   const int tid = threadIdx.x;
+  const bool no_producer = (flags & APC_EDGE_NO_PRODUCER) != 0;
 
-  for (int j = tid; j < cols; j += kBlock) {
-    const int sp = src_begin + col0 + j;
-    const uint32_t codes = a.spec_codes[sp];
+  // ---- stage the tile's producer / consumer specs -------------------------------------------
+  if (tid == 0) s_uniform = 1;
+  __syncthreads();
+  const int t0 = a.spec_tensor[tile.src_begin + col0];
+  for (int j = tid; j < cols; j += kTileThreads) {
+    const int sp = tile.src_begin + col0 + j;
     const int t = a.spec_tensor[sp];
-    uint8_t f = 0;
-    double gb = 0.0;
-    if (t >= 0) {
+    s_src[j] = a.spec_codes[sp];
+    s_stensor[j] = t;
+    if (t != t0) s_uniform = 0;
+  }
+  for (int j = tid; j < rows; j += kTileThreads) {
+    const int ts = tile.tgt_begin + row0 + j;
+    const uint32_t tg = a.spec_codes[ts];
+    bool any_partial = false, all_shard = true;
+#pragma unroll
+    for (int i = 0; i < M; ++i) {
+      const int k = kind_of((tg >> (8 * i)) & 0xFF);
+      any_partial |= k == 1;
+      all_shard &= k == 2;
+    }
+    s_tgt[j] = tg;
+    s_tflag[j] = (a.spec_tensor[ts] >= 0 ? 1 : 0) | (any_partial ? 2 : 0) | (all_shard ? 4 : 0);
+    s_cpa[j] = a.per_arg ? a.per_arg[tile.strat_begin + row0 + j] : 0.0;
+  }
+  __syncthreads();
+  const bool uniform = s_uniform != 0 && t0 >= 0 && !no_producer;
+
+  // ---- evaluate every reachable state once ---------------------------------------------------
+  bool tile_cont = true;
+  if (uniform) {
+    const double bytes = (double)a.tensor_bytes[t0];
+    tile_cont = a.tensor_contiguous[t0] != 0;
+    for (int k = tid; k < NS; k += kTileThreads) {
+      const int level = 31 - __clz((k >> M) + 1);
+      const int rem = k - ((((1 << level) - 1)) << M);
+      const int mask = rem >> level, hist = rem & ((1 << level) - 1);
       int64_t shards = 1;
 #pragma unroll
       for (int i = 0; i < M; ++i)
-        if (kind_of((codes >> (8 * i)) & 0xFF) == 2) shards *= p.mesh_size[i];
-      // collective_runtime_estimation.py:66-68
-      gb = (double)a.tensor_bytes[t] / (double)shards / 1024 / 1024 / 1024;
-      f = 1 | (a.tensor_contiguous[t] ? 2 : 0);
+        if ((mask >> i) & 1) shards *= p.mesh_size[i];
+      double gb = bytes / (double)shards / 1024 / 1024 / 1024;  // collective_runtime_estimation.py:66-68
+#pragma unroll
+      for (int i = 0; i < M; ++i) {
+        if (i < level && ((hist >> i) & 1)) {
+          const double n = (double)p.mesh_size[i];
+          if ((mask >> i) & 1) gb *= n; else gb /= n;
+        }
+      }
+      s_rw[k] = rw_time(gb * 2 * 1073741824.0, p);
+      double ag = 0.0, rs = 0.0, a2a = 0.0, ar = 0.0;
+      if (level >= 1) ag = ring(gb, p, level - 1, p.mesh_size[level - 1] - 1);
+      if (level < M) {
+        rs = ring(gb, p, level, p.mesh_size[level] - 1);
+        a2a = rs;
+        a2a *= p.a2a_scale;
+        ar = ring(gb, p, level, 2 * (p.mesh_size[level] - 1));
+      }
+      s_ag[k] = ag;
+      s_rs[k] = rs;
+      s_a2a[k] = a2a;
+      s_ar[k] = ar;
     }
-    s_gb[j] = gb;
-    s_src[j] = codes;
-    s_sflag[j] = f;
-  }
-  for (int j = tid; j < rows; j += kBlock) {
-    const int ts = tgt_begin + row0 + j;
-    s_tgt[j] = a.spec_codes[ts];
-    s_tflag[j] = a.spec_tensor[ts] >= 0 ? 1 : 0;
-    s_cpa[j] = a.per_arg ? a.per_arg[strat_begin + row0 + j] : 0.0;
   }
   __syncthreads();
 
+  // ---- entries ---------------------------------------------------------------------------------
   const int n = rows * cols;
   int r = tid / cols, c = tid - r * cols;
-  const int dr = kBlock / cols, dc = kBlock - dr * cols;
-  for (int idx = tid; idx < n; idx += kBlock) {
+  const int dr = kTileThreads / cols, dc = kTileThreads - dr * cols;
+  for (int idx = tid; idx < n; idx += kTileThreads) {
     const int64_t local = (int64_t)(row0 + r) * n_src + (col0 + c);
     double comm;
     int trans = 0;
-    const bool passthrough = (flags & APC_EDGE_NO_PRODUCER) || !(s_sflag[c] & 1) || !s_tflag[r];
-    if (passthrough) {
-      comm = a.pt_values[pt_begin + local];
+    const int tf = s_tflag[r];
+    const int st = s_stensor[c];
+    if (no_producer || st < 0 || !(tf & 1)) {
+      comm = a.pt_values[tile.pt_begin + local];
     } else {
       const uint32_t src = s_src[c], tgt = s_tgt[r];
-      comm = entry_cost<M>(src, tgt, s_gb[c], (s_sflag[c] & 2) != 0, p);
       trans = (src != tgt) ? p.transition_scale : 0;  // optimize_sharding.py:345-351
+      const bool flipped = M == 2 && src == 0x4040u && (tf & 4);
+      if (src == 0u) {  // fully replicated producer
+        comm = (tf & 2) ? INFINITY : 0.0;
+      } else if (!uniform || flipped) {
+        int64_t shards = 1;
+#pragma unroll
+        for (int i = 0; i < M; ++i)
+          if (kind_of((src >> (8 * i)) & 0xFF) == 2) shards *= p.mesh_size[i];
+        const double gb = (double)a.tensor_bytes[st] / (double)shards / 1024 / 1024 / 1024;
+        comm = entry_cost<M>(src, tgt, gb, a.tensor_contiguous[st] != 0, p);
+      } else {
+        int mask = 0;
+#pragma unroll
+        for (int i = 0; i < M; ++i) mask |= (kind_of((src >> (8 * i)) & 0xFF) == 2 ? 1 : 0) << i;
+        int hist = 0;
+        bool cont = tile_cont;
+        double cost = 0.0;
+#pragma unroll
+        for (int i = 0; i < M; ++i) {
+          const uint32_t cc = (src >> (8 * i)) & 0xFF, tt = (tgt >> (8 * i)) & 0xFF;
+          if (cc == tt) continue;
+          const int k = States<M>::index(i, mask, hist);
+          if (!cont) cost += s_rw[k];
+          const int ck = kind_of(cc), tk = kind_of(tt);
+          if (ck == 2 && tk == 0) {  // all-gather
+            hist |= 1 << i;
+            const int k2 = States<M>::index(i + 1, mask, hist);
+            cost += s_ag[k2];
+            if (dim_of(cc) != 0) cost += s_rw[k2];
+          } else if (ck == 2 && tk == 2) {  // all-to-all
+            cost += s_a2a[k];
+            const int copies = (dim_of(cc) != 0) + (dim_of(tt) != 0);
+            cost += (double)copies * s_rw[k];
+          } else if (ck == 1 && tk == 0) {  // all-reduce
+            cost += s_ar[k];
+          } else if (ck == 1 && tk == 2) {  // reduce-scatter
+            cost += s_rs[k];
+            if (dim_of(tt) != 0) cost += s_rw[k];
+            hist |= 1 << i;
+          } else if (tk == 1 && ck != 1) {  // -> Partial from Shard / Replicate: banned
+            cost = INFINITY;
+          }
+          cont = true;
+        }
+        comm = cost;
+      }
     }
     if (flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;  // :358-359
-    const int64_t o = entry_begin + local;
+    const int64_t o = tile.entry_begin + local;
     if (a.comm_out) a.comm_out[o] = comm;
     if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
     if (a.cost_out) a.cost_out[o] = comm + s_cpa[r] + (double)trans;  // :368-372
@@ -397,9 +496,7 @@ int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const 
                              const int32_t *edge_tgt_begin, const int32_t *edge_n_tgt,
                              const int32_t *edge_flags, const int64_t *edge_pt_begin,
                              const int64_t *edge_entry_begin, const int32_t *edge_strat_begin, int64_t n_pt,
-                             int64_t n_strategies, int64_t n_tiles, const int32_t *tile_edge,
-                             const int32_t *tile_row_begin, const int32_t *tile_row_count,
-                             const int32_t *tile_col_begin, const int32_t *tile_col_count) {
+                             int64_t n_strategies, int64_t n_tiles, const apc_tile *tiles) {
   if (int rc = check_params(params)) return rc;
   const int M = params->mesh_ndim;
   for (int64_t t = 0; t < n_tensors; ++t)
@@ -450,16 +547,21 @@ int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const 
     return fail(-2, "entry_begin[n_edges] = %lld, expected %lld", (long long)edge_entry_begin[n_edges],
                 (long long)expect);
   for (int64_t t = 0; t < n_tiles; ++t) {
-    const int e = tile_edge[t];
+    const apc_tile &tl = tiles[t];
+    const int e = tl.edge;
     if (e < 0 || e >= n_edges) return fail(-2, "tile %lld: edge %d out of range", (long long)t, e);
-    if (tile_row_count[t] < 1 || tile_row_count[t] > APC_TILE_MAX_ROWS || tile_row_begin[t] < 0 ||
-        tile_row_begin[t] + tile_row_count[t] > edge_n_tgt[e])
+    if (tl.row_count < 1 || tl.row_count > APC_TILE_MAX_ROWS || tl.row_begin < 0 ||
+        tl.row_begin + tl.row_count > edge_n_tgt[e])
       return fail(-2, "tile %lld: rows [%d, +%d) outside edge %d (n_tgt %d, max %d per tile)", (long long)t,
-                  tile_row_begin[t], tile_row_count[t], e, edge_n_tgt[e], APC_TILE_MAX_ROWS);
-    if (tile_col_count[t] < 1 || tile_col_count[t] > APC_TILE_MAX_COLS || tile_col_begin[t] < 0 ||
-        tile_col_begin[t] + tile_col_count[t] > edge_n_src[e])
+                  tl.row_begin, tl.row_count, e, edge_n_tgt[e], APC_TILE_MAX_ROWS);
+    if (tl.col_count < 1 || tl.col_count > APC_TILE_MAX_COLS || tl.col_begin < 0 ||
+        tl.col_begin + tl.col_count > edge_n_src[e])
       return fail(-2, "tile %lld: cols [%d, +%d) outside edge %d (n_src %d, max %d per tile)", (long long)t,
-                  tile_col_begin[t], tile_col_count[t], e, edge_n_src[e], APC_TILE_MAX_COLS);
+                  tl.col_begin, tl.col_count, e, edge_n_src[e], APC_TILE_MAX_COLS);
+    if (tl.src_begin != edge_src_begin[e] || tl.n_src != edge_n_src[e] || tl.tgt_begin != edge_tgt_begin[e] ||
+        tl.flags != edge_flags[e] || tl.strat_begin != edge_strat_begin[e] ||
+        tl.entry_begin != edge_entry_begin[e] || tl.pt_begin != edge_pt_begin[e])
+      return fail(-2, "tile %lld: record does not repeat the fields of edge %d", (long long)t, e);
   }
   return 0;
 }
@@ -502,27 +604,18 @@ int apc_compute_costs(const apc_params *params, int64_t n, const int64_t *flops,
 }
 
 int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes, const uint8_t *tensor_contiguous,
-                            const uint32_t *spec_codes, const int32_t *spec_tensor, const int32_t *edge_src_begin,
-                            const int32_t *edge_n_src, const int32_t *edge_tgt_begin, const int32_t *edge_n_tgt,
-                            const int32_t *edge_flags, const int64_t *edge_pt_begin, const int64_t *edge_entry_begin,
-                            const int32_t *edge_strat_begin, const double *pt_values, const double *per_arg,
-                            int64_t n_tiles, const int32_t *tile_edge, const int32_t *tile_row_begin,
-                            const int32_t *tile_row_count, const int32_t *tile_col_begin,
-                            const int32_t *tile_col_count, double *comm_out, uint8_t *trans_out, double *cost_out,
-                            void *stream) {
+                            const uint32_t *spec_codes, const int32_t *spec_tensor, const double *pt_values,
+                            const double *per_arg, int64_t n_tiles, const apc_tile *tiles, double *comm_out,
+                            uint8_t *trans_out, double *cost_out, void *stream) {
   if (int rc = check_params(params)) return rc;
   if (n_tiles < 0 || n_tiles > INT32_MAX) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tiles == 0) return 0;
-  if (!tensor_bytes || !tensor_contiguous || !spec_codes || !spec_tensor || !edge_src_begin || !edge_n_src ||
-      !edge_tgt_begin || !edge_n_tgt || !edge_flags || !edge_pt_begin || !edge_entry_begin || !edge_strat_begin ||
-      !tile_edge || !tile_row_begin || !tile_row_count || !tile_col_begin || !tile_col_count)
+  if (!tensor_bytes || !tensor_contiguous || !spec_codes || !spec_tensor || !tiles)
     return fail(-1, "apc_redistribute_tables: NULL table");
   if (cost_out && !per_arg) return fail(-1, "cost_out needs compute_cost_per_arg");
-  TableArgs a{tensor_bytes, tensor_contiguous, spec_codes,      spec_tensor,    edge_src_begin, edge_n_src,
-              edge_tgt_begin, edge_n_tgt,      edge_flags,      edge_pt_begin,  edge_entry_begin, edge_strat_begin,
-              pt_values,    per_arg,           tile_edge,       tile_row_begin, tile_row_count, tile_col_begin,
-              tile_col_count, comm_out,        trans_out,       cost_out};
-  const dim3 grid((unsigned)n_tiles), block(kBlock);
+  TableArgs a{tensor_bytes, tensor_contiguous, spec_codes, spec_tensor, pt_values, per_arg, tiles,
+              comm_out,     trans_out,         cost_out};
+  const dim3 grid((unsigned)n_tiles), block(kTileThreads);
   hipStream_t s = (hipStream_t)stream;
   switch (params->mesh_ndim) {
     case 1: hipLaunchKernelGGL(redistribute_tiles_kernel<1>, grid, block, 0, s, *params, a); break;

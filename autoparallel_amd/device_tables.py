@@ -22,8 +22,7 @@ _UPLOAD = (
     "tensor_rank", "tensor_itemsize", "tensor_shape", "tensor_stride", "spec_codes", "spec_tensor",
     "strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "strat_num_args",
     "edge_src_begin", "edge_n_src", "edge_tgt_begin", "edge_n_tgt", "edge_flags", "edge_pt_begin",
-    "edge_entry_begin", "edge_strat_begin", "pt_values", "tile_edge", "tile_row_begin", "tile_row_count",
-    "tile_col_begin", "tile_col_count",
+    "edge_entry_begin", "edge_strat_begin", "pt_values", "tile_records",
 )
 
 
@@ -49,6 +48,8 @@ def _guarded(fn):
 def _to_device(a: np.ndarray, device) -> torch.Tensor:
     if a.dtype == np.uint32:  # same bits; torch's uint32 support is partial
         a = a.view(np.int32)
+    if a.dtype.names is not None:  # packed records travel as raw int32 words
+        a = np.ascontiguousarray(a).view(np.int32).reshape(len(a), a.dtype.itemsize // 4)
     if a.size == 0:
         return torch.empty(a.shape, dtype=torch.from_numpy(np.zeros(1, a.dtype)).dtype, device=device)
     return torch.from_numpy(a).to(device, non_blocking=False)
@@ -155,13 +156,9 @@ class DeviceCostTables:
         with torch.cuda.device(self.device):
             rc = self.lib.apc_redistribute_tables(
                 ctypes.byref(self.c_params), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
-                self._p("spec_codes"), self._p("spec_tensor"), self._p("edge_src_begin"), self._p("edge_n_src"),
-                self._p("edge_tgt_begin"), self._p("edge_n_tgt"), self._p("edge_flags"), self._p("edge_pt_begin"),
-                self._p("edge_entry_begin"), self._p("edge_strat_begin"), self._p("pt_values"),
-                self._p(self.compute_cost_per_arg), ctypes.c_int64(self.tables.n_tiles), self._p("tile_edge"),
-                self._p("tile_row_begin"), self._p("tile_row_count"), self._p("tile_col_begin"),
-                self._p("tile_col_count"), self._p(self.comm), self._p(self.transition), self._p(self.cost),
-                self._stream())
+                self._p("spec_codes"), self._p("spec_tensor"), self._p("pt_values"),
+                self._p(self.compute_cost_per_arg), ctypes.c_int64(self.tables.n_tiles), self._p("tile_records"),
+                self._p(self.comm), self._p(self.transition), self._p(self.cost), self._stream())
         _native.check(rc, "apc_redistribute_tables")
 
     @_guarded
@@ -206,11 +203,8 @@ class DeviceCostTables:
                      P("strat_zero_cost"), P("strat_num_args"), P(self.compute_cost), P(self.compute_cost_per_arg),
                      P(err), stream)
         a_tables = (cp, P(self.tensor_bytes), P(self.tensor_contiguous), P("spec_codes"), P("spec_tensor"),
-                    P("edge_src_begin"), P("edge_n_src"), P("edge_tgt_begin"), P("edge_n_tgt"), P("edge_flags"),
-                    P("edge_pt_begin"), P("edge_entry_begin"), P("edge_strat_begin"), P("pt_values"),
-                    P(self.compute_cost_per_arg), ctypes.c_int64(tb.n_tiles), P("tile_edge"), P("tile_row_begin"),
-                    P("tile_row_count"), P("tile_col_begin"), P("tile_col_count"), P(self.comm), P(self.transition),
-                    P(self.cost), stream)
+                    P("pt_values"), P(self.compute_cost_per_arg), ctypes.c_int64(tb.n_tiles), P("tile_records"),
+                    P(self.comm), P(self.transition), P(self.cost), stream)
 
         def bind(fn, args, what):
             def launch():

@@ -47,7 +47,15 @@ PARTIAL_OPS = ("sum", "avg", "min", "max", "product", "band", "bor", "bxor")
 EDGE_GRAD_RESCALE = _native.EDGE_GRAD_RESCALE
 EDGE_NO_PRODUCER = _native.EDGE_NO_PRODUCER
 
-DEFAULT_TILE_ENTRIES = 4096
+DEFAULT_TILE_ENTRIES = 2048
+
+# numpy mirror of the C struct apc_tile (64 bytes)
+TILE_DTYPE = np.dtype([
+    ("edge", "<i4"), ("row_begin", "<i4"), ("row_count", "<i4"), ("col_begin", "<i4"), ("col_count", "<i4"),
+    ("src_begin", "<i4"), ("n_src", "<i4"), ("tgt_begin", "<i4"), ("flags", "<i4"), ("strat_begin", "<i4"),
+    ("entry_begin", "<i8"), ("pt_begin", "<i8"), ("reserved", "<i4", (2,)),
+])
+assert TILE_DTYPE.itemsize == 64
 
 
 def shard_code(dim: int, variant: int = 0) -> int:
@@ -124,6 +132,7 @@ class CostTables:
     tile_row_count: np.ndarray = None
     tile_col_begin: np.ndarray = None
     tile_col_count: np.ndarray = None
+    tile_records: np.ndarray = None
 
     _DTYPES = {
         "tensor_rank": np.int32, "tensor_itemsize": np.int32, "tensor_shape": np.int64,
@@ -150,6 +159,8 @@ class CostTables:
             raise ValueError("tensor_stride must have the shape of tensor_shape")
         if self.tile_edge is None:
             self.build_tiles()
+        elif self.tile_records is None:
+            self.pack_tile_records()
 
     # ---- sizes -------------------------------------------------------------------------
     @property
@@ -216,6 +227,24 @@ class CostTables:
         self.tile_col_count = _i32(np.minimum(cw[te], ns[te] - col_begin))
         self.tile_row_begin = _i32(row_begin)
         self.tile_row_count = _i32(np.minimum(rpt[te], nt[te] - row_begin))
+        self.pack_tile_records()
+
+    def pack_tile_records(self) -> None:
+        """The tile rectangles plus the fields of their edge, as the packed records the
+        table kernel reads (C struct ``apc_tile``)."""
+        te = self.tile_edge.astype(np.int64)
+        rec = np.zeros(len(te), TILE_DTYPE)
+        rec["edge"] = self.tile_edge
+        rec["row_begin"], rec["row_count"] = self.tile_row_begin, self.tile_row_count
+        rec["col_begin"], rec["col_count"] = self.tile_col_begin, self.tile_col_count
+        rec["src_begin"] = self.edge_src_begin[te]
+        rec["n_src"] = self.edge_n_src[te]
+        rec["tgt_begin"] = self.edge_tgt_begin[te]
+        rec["flags"] = self.edge_flags[te]
+        rec["strat_begin"] = self.edge_strat_begin[te]
+        rec["entry_begin"] = self.edge_entry_begin[:-1][te] if len(te) else 0
+        rec["pt_begin"] = self.edge_pt_begin[te]
+        self.tile_records = rec
 
     # ---- checks ------------------------------------------------------------------------
     def validate(self, params) -> None:
@@ -239,6 +268,8 @@ class CostTables:
         if (self.strat_flops >= 2**53).any() or (self.strat_rw_bytes >= 2**53).any():
             raise RuntimeError("flop / byte counts must stay below 2**53 to convert to fp64 exactly")
         cp = params.to_c()
+        if self.tile_records is None or len(self.tile_records) != self.n_tiles:
+            raise RuntimeError("tile_records must have one record per tile (call pack_tile_records())")
 
         def p(a):
             return a.ctypes.data_as(ctypes.c_void_p)
@@ -249,8 +280,7 @@ class CostTables:
             ctypes.c_int64(self.n_edges), p(self.edge_src_begin), p(self.edge_n_src), p(self.edge_tgt_begin),
             p(self.edge_n_tgt), p(self.edge_flags), p(self.edge_pt_begin), p(self.edge_entry_begin),
             p(self.edge_strat_begin), ctypes.c_int64(len(self.pt_values)), ctypes.c_int64(self.n_strategies),
-            ctypes.c_int64(self.n_tiles), p(self.tile_edge), p(self.tile_row_begin), p(self.tile_row_count),
-            p(self.tile_col_begin), p(self.tile_col_count))
+            ctypes.c_int64(self.n_tiles), p(self.tile_records))
         _native.check(rc, "apc_validate_tables_host")
         # byte counts must convert to fp64 exactly (the kernels divide them as doubles)
         if self.n_tensors:

@@ -36,8 +36,7 @@
  *       edge_pt_begin[e]       offset into pt_values of the rule-provided costs
  *                              kept where either spec is not a DTensorSpec
  *       edge_flags             APC_EDGE_*
- *   tile t = a rectangle of one edge's matrix handled by one workgroup:
- *       tile_edge, tile_row_begin, tile_row_count, tile_col_begin, tile_col_count
+ *   tile t = a rectangle of one edge's matrix handled by one workgroup (apc_tile)
  */
 #ifndef APCOST_H
 #define APCOST_H
@@ -51,11 +50,28 @@ extern "C" {
 #define APC_MAX_RANK 8
 #define APC_MAX_MESH 4
 #define APC_MAX_DTYPES 8
-#define APC_TILE_MAX_COLS 1024 /* producer specs staged in LDS per tile */
-#define APC_TILE_MAX_ROWS 1024 /* consumer specs staged in LDS per tile */
+#define APC_TILE_MAX_COLS 256 /* producer specs staged in LDS per tile */
+#define APC_TILE_MAX_ROWS 256 /* consumer specs staged in LDS per tile */
 
 #define APC_EDGE_GRAD_RESCALE 1 /* consumer is a parameter-gradient node (optimize_sharding.py:358-359) */
 #define APC_EDGE_NO_PRODUCER 2  /* placeholder / factory pseudo-argument (optimize_sharding.py:312-355) */
+
+/* One tile: a rows x cols rectangle of one edge's matrix, handled by one workgroup.
+ * The record repeats the fields of its edge so that the kernel reaches everything it
+ * needs with one load; apc_validate_tables_host checks it against the edge arrays. */
+typedef struct apc_tile {
+  int32_t edge;
+  int32_t row_begin, row_count; /* consumer strategies */
+  int32_t col_begin, col_count; /* producer strategies */
+  int32_t src_begin;            /* = edge_src_begin[edge] */
+  int32_t n_src;                /* = edge_n_src[edge] */
+  int32_t tgt_begin;            /* = edge_tgt_begin[edge] */
+  int32_t flags;                /* = edge_flags[edge] */
+  int32_t strat_begin;          /* = edge_strat_begin[edge] */
+  int64_t entry_begin;          /* = edge_entry_begin[edge] */
+  int64_t pt_begin;             /* = edge_pt_begin[edge] */
+  int32_t reserved[2];
+} apc_tile;
 
 /* Cost-model parameters: everything the reference reads from its environment
  * (torch MeshTopoInfo, DEVICE_LIMITS row, module constants), made explicit. */
@@ -89,9 +105,7 @@ int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const 
                              const int32_t *edge_tgt_begin_host, const int32_t *edge_n_tgt_host,
                              const int32_t *edge_flags_host, const int64_t *edge_pt_begin_host,
                              const int64_t *edge_entry_begin_host, const int32_t *edge_strat_begin_host,
-                             int64_t n_pt, int64_t n_strategies, int64_t n_tiles, const int32_t *tile_edge_host,
-                             const int32_t *tile_row_begin_host, const int32_t *tile_row_count_host,
-                             const int32_t *tile_col_begin_host, const int32_t *tile_col_count_host);
+                             int64_t n_pt, int64_t n_strategies, int64_t n_tiles, const apc_tile *tiles_host);
 
 /* Bytes and contiguity of every tensor row.
  * Replaces torch spec_to_bytes (distributed/tensor/_collective_utils.py:230-232) and
@@ -131,15 +145,9 @@ int apc_compute_costs(const apc_params *params, int64_t n_strategies, const int6
  * comm_out / transition_out / cost_out are [n_entries]; any may be NULL. */
 int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes,
                             const uint8_t *tensor_contiguous, const uint32_t *spec_codes,
-                            const int32_t *spec_tensor, const int32_t *edge_src_begin,
-                            const int32_t *edge_n_src, const int32_t *edge_tgt_begin,
-                            const int32_t *edge_n_tgt, const int32_t *edge_flags,
-                            const int64_t *edge_pt_begin, const int64_t *edge_entry_begin,
-                            const int32_t *edge_strat_begin, const double *pt_values,
-                            const double *compute_cost_per_arg, int64_t n_tiles, const int32_t *tile_edge,
-                            const int32_t *tile_row_begin, const int32_t *tile_row_count,
-                            const int32_t *tile_col_begin, const int32_t *tile_col_count, double *comm_out,
-                            uint8_t *transition_out, double *cost_out, void *stream);
+                            const int32_t *spec_tensor, const double *pt_values,
+                            const double *compute_cost_per_arg, int64_t n_tiles, const apc_tile *tiles,
+                            double *comm_out, uint8_t *transition_out, double *cost_out, void *stream);
 
 /* Segmented minimum with first-argmin (relative to the segment start); empty
  * segments give (+inf, -1).  No counterpart in the reference (which hands the full

@@ -31,6 +31,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_params_struct_layout_matches_header():
     # 4 + 16 (+4 pad) + 32 + 32 + 7*8 + 64 + 4 (+4 pad)
+    assert ctypes.sizeof(_native.ApcTile) == 64 and _native.ApcTile.entry_begin.offset == 40
     assert ctypes.sizeof(_native.ApcParams) == 216
     assert _native.ApcParams.bw.offset == 24 and _native.ApcParams.gpu_flops.offset == 144
 
@@ -106,12 +107,23 @@ def test_validator_accepts_generated_tables():
     (lambda t: t.edge_strat_begin.__setitem__(1, t.n_strategies), "strategy rows"),
     (lambda t: t.tile_row_count.__setitem__(0, 10**4), "rows"),
     (lambda t: t.tile_col_begin.__setitem__(0, -1), "cols"),
-    (lambda t: t.tile_edge.__setitem__(0, t.n_edges), "edge"),
 ])
 def test_validator_rejects_malformed_tables(mutate, message):
     tb = _small()
     mutate(tb)
+    tb.pack_tile_records()
     with pytest.raises(RuntimeError, match=message):
+        tb.validate(CostModelParams.from_mesh((4, 2)))
+
+
+def test_validator_rejects_tile_record_that_disagrees_with_its_edge():
+    tb = _small()
+    tb.tile_records["src_begin"][0] += 1
+    with pytest.raises(RuntimeError, match="does not repeat"):
+        tb.validate(CostModelParams.from_mesh((4, 2)))
+    tb = _small()
+    tb.tile_records["edge"][0] = tb.n_edges
+    with pytest.raises(RuntimeError, match="out of range"):
         tb.validate(CostModelParams.from_mesh((4, 2)))
 
 
@@ -119,6 +131,7 @@ def test_validator_needs_pass_through_values_for_producerless_edges():
     tb = _small()
     e = int(np.nonzero(tb.edge_flags & EDGE_NO_PRODUCER)[0][0])
     tb.edge_pt_begin[e] = -1
+    tb.pack_tile_records()
     with pytest.raises(RuntimeError, match="pass-through"):
         tb.validate(CostModelParams.from_mesh((4, 2)))
 
