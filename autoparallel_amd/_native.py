@@ -14,8 +14,8 @@ from ._build import LIB_PATH
 APC_MAX_RANK = 8
 APC_MAX_MESH = 4
 APC_MAX_DTYPES = 8
-APC_TILE_MAX_COLS = 256
-APC_TILE_MAX_ROWS = 256
+APC_TILE_MAX_COLS = 128
+APC_TILE_MAX_ROWS = 128
 
 EDGE_GRAD_RESCALE = 1
 EDGE_NO_PRODUCER = 2
@@ -55,6 +55,7 @@ EXPORTS = (
     "apc_version",
     "apc_last_error",
     "apc_validate_tables_host",
+    "apc_tensor_terms_count",
     "apc_tensor_tables",
     "apc_spec_tables",
     "apc_compute_costs",
@@ -92,6 +93,7 @@ def lib() -> ctypes.CDLL:
         for name in EXPORTS:
             if name != "apc_last_error":
                 getattr(l, name).restype = ctypes.c_int
+        l.apc_tensor_terms_count.restype = ctypes.c_int64
         _lib = l
     return _lib
 

@@ -109,15 +109,41 @@ __device__ __forceinline__ double entry_cost(uint32_t srcp, uint32_t tgtp, doubl
 }
 
 // ------------------------------------------------------------------------------------------
-// a7: bytes + contiguity per tensor
+// Running-bytes states.  The redistribution cost of an entry is a sum of per-mesh-dim terms,
+// and every term is an expensive expression (fp64 divisions) of ONE quantity only: the
+// running comm_bytes_gb at that dim.  For a given tensor that quantity takes few distinct
+// values: it starts from bytes / num_shards (decided by WHICH mesh dims the producer
+// shards: a mask of M bits) and every earlier dim either left it alone or applied its
+// single possible update (x n after an all-gather when the producer shards that dim, / n
+// after a reduce-scatter when it does not).  State (level L, mask, history) indexes every
+// value that can occur; level L in [0, M] has 2^M masks x 2^L histories.
 // ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void tensor_tables_kernel(int64_t n, const int32_t *__restrict__ rank,
-                                                               const int32_t *__restrict__ itemsize,
-                                                               const int64_t *__restrict__ shape,
-                                                               const int64_t *__restrict__ stride,
-                                                               int64_t *__restrict__ bytes,
-                                                               uint8_t *__restrict__ cont) {
-  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+template <int M>
+struct States {
+  static constexpr int kCount = (1 << M) * ((1 << (M + 1)) - 1);
+  __device__ static __forceinline__ int index(int level, int mask, int hist) {
+    return (((1 << level) - 1) << M) + (mask << level) + hist;
+  }
+};
+constexpr int kTermArrays = 4;  // rw, ag, rs, ar
+
+__host__ __device__ constexpr int states_count(int m) { return (1 << m) * ((1 << (m + 1)) - 1); }
+
+// ------------------------------------------------------------------------------------------
+// a7: bytes + contiguity per tensor, and (optionally) the per-state cost terms of the tensor:
+//   terms[t][0][k] read+write time of the running bytes          (compute_estimation.py:302-314)
+//   terms[t][1][k] all-gather on dim level-1, bytes already x n   (torch _collective_utils.py:281-288)
+//   terms[t][2][k] reduce-scatter on dim level (x a2a_scale = all-to-all)      (:302-313)
+//   terms[t][3][k] all-reduce on dim level                                      (:291-299)
+// each evaluated once, in the reference's operation order.  One 64-thread workgroup per tensor.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void tensor_tables_kernel(apc_params p, int64_t n, const int32_t *__restrict__ rank,
+                                                           const int32_t *__restrict__ itemsize,
+                                                           const int64_t *__restrict__ shape,
+                                                           const int64_t *__restrict__ stride,
+                                                           int64_t *__restrict__ bytes, uint8_t *__restrict__ cont,
+                                                           double *__restrict__ terms) {
+  const int64_t t = blockIdx.x;
   if (t >= n) return;
   const int r = rank[t];
   const int64_t *sh = shape + t * APC_MAX_RANK;
@@ -125,7 +151,7 @@ __global__ __launch_bounds__(kBlock) void tensor_tables_kernel(int64_t n, const 
   int64_t nbytes = itemsize[t];
   int64_t expected = 1, expected_max = 1;
   bool ok = true;
-  for (int i = r - 1; i >= 0; --i) {
+  for (int i = r - 1; i >= 0; --i) {  // every lane computes the same few integers
     const int64_t x = sh[i], y = st[i];
     nbytes *= x;
     if (x == 1) continue;
@@ -133,8 +159,40 @@ __global__ __launch_bounds__(kBlock) void tensor_tables_kernel(int64_t n, const 
     expected_max *= (x > 1 ? x : 1);
     expected *= x;
   }
-  bytes[t] = nbytes;
-  cont[t] = ok ? 1 : 0;
+  if (threadIdx.x == 0) {
+    bytes[t] = nbytes;
+    cont[t] = ok ? 1 : 0;
+  }
+  if (!terms) return;
+  const int M = p.mesh_ndim;
+  const int ns = states_count(M);
+  double *out = terms + t * (int64_t)(kTermArrays * ns);
+  const double fbytes = (double)nbytes;
+  for (int k = threadIdx.x; k < ns; k += 64) {
+    const int level = 31 - __clz((k >> M) + 1);
+    const int rem = k - (((1 << level) - 1) << M);
+    const int mask = rem >> level, hist = rem & ((1 << level) - 1);
+    int64_t shards = 1;
+    for (int i = 0; i < M; ++i)
+      if ((mask >> i) & 1) shards *= p.mesh_size[i];
+    double gb = fbytes / (double)shards / 1024 / 1024 / 1024;  // collective_runtime_estimation.py:66-68
+    for (int i = 0; i < level; ++i) {
+      if ((hist >> i) & 1) {
+        const double m = (double)p.mesh_size[i];
+        if ((mask >> i) & 1) gb *= m; else gb /= m;  // :86 / :128
+      }
+    }
+    double ag = 0.0, rs = 0.0, ar = 0.0;
+    if (level >= 1) ag = ring(gb, p, level - 1, p.mesh_size[level - 1] - 1);
+    if (level < M) {
+      rs = ring(gb, p, level, p.mesh_size[level] - 1);
+      ar = ring(gb, p, level, 2 * (p.mesh_size[level] - 1));
+    }
+    out[k] = rw_time(gb * 2 * 1073741824.0, p);
+    out[ns + k] = ag;
+    out[2 * ns + k] = rs;
+    out[3 * ns + k] = ar;
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -229,27 +287,19 @@ __global__ __launch_bounds__(kBlock) void compute_costs_kernel(
 
 // ------------------------------------------------------------------------------------------
 // a1-a6: redistribution-cost matrices.  One wavefront (a 64-thread workgroup) per tile of
-// one edge's matrix.
-//
-// The cost of an entry is a sum of per-mesh-dim terms; each term is an expensive
-// expression (fp64 divisions) of ONE quantity only: the running comm_bytes_gb at that
-// dim.  That quantity takes few distinct values inside a tile: it starts from
-// bytes / num_shards (decided by WHICH mesh dims the producer shards: a mask of M bits) and
-// every earlier dim either left it alone or applied its single possible update (x n after
-// an all-gather when the producer shards that dim, / n after a reduce-scatter when it does
-// not).  State (level L, mask, history) therefore indexes all values that can occur; the
-// prologue evaluates every collective / read-write term once per state into LDS, in
-// exactly the reference's operation order, and the per-entry loop only looks terms up and
-// adds them in the reference's order.  Results are bit-identical to evaluating every entry
-// directly (entry_cost), which remains the path for the rare cases the states do not
-// cover: producer specs of one edge that point at different tensors, and the 2-D
-// (Partial, Partial) -> all-Shard order flip.
+// one edge's matrix.  The tile's producer and consumer specs and the per-state terms of the
+// edge's tensor are staged in LDS; the per-entry loop walks the mesh dims, looks the terms
+// of the current state up and adds them in the reference's order, so results are
+// bit-identical to evaluating every entry directly (entry_cost).  The direct evaluation
+// remains the path for the rare cases the states do not cover: producer specs of one edge
+// that point at different tensors, and the 2-D (Partial, Partial) -> all-Shard order flip.
 // ------------------------------------------------------------------------------------------
 constexpr int kTileThreads = 64;
 
 struct TableArgs {
   const int64_t *tensor_bytes;
   const uint8_t *tensor_contiguous;
+  const double *tensor_terms;
   const uint32_t *spec_codes;
   const int32_t *spec_tensor;
   const double *pt_values;
@@ -260,28 +310,41 @@ struct TableArgs {
   double *cost_out;
 };
 
-template <int M>
-struct States {
-  // level L in [0, M]: 2^M masks x 2^L histories
-  static constexpr int kCount = (1 << M) * ((1 << (M + 1)) - 1);
-  __device__ static __forceinline__ int index(int level, int mask, int hist) {
-    return (((1 << level) - 1) << M) + (mask << level) + hist;
-  }
-};
+// What one mesh dim contributes, by (producer class, consumer class) with classes
+// 0 Replicate, 1 Partial, 2 Shard(0), 3 Shard(d != 0); only consulted when the two placement
+// codes differ.  One byte per pair:
+//   bits 0-1  term array: 0 none, 1 all-gather, 2 reduce-scatter, 3 all-reduce
+//   bits 2-3  number of read+write reshuffles added after the collective
+//   bit  4    all-to-all: the reduce-scatter shaped term times a2a_scale
+//   bit  5    banned transition (-> Partial from Replicate / Shard): cost is inf
+//   bit  6    the running bytes change after this dim (x n after all-gather, / n after
+//             reduce-scatter)
+// collective_runtime_estimation.py:83-138.
+__host__ __device__ constexpr uint32_t pair_action(int c, int t) {
+  constexpr uint32_t AG = 1, RS = 2, AR = 3, A2A = 2u | (1u << 4), BAN = 1u << 5, UPD = 1u << 6;
+  const uint32_t cn = c == 3, tn = t == 3;
+  if (t == 1) return c == 1 ? 0u : BAN;            // -> Partial
+  if (c == 0) return 0u;                           // Replicate -> Replicate / Shard: local
+  if (c == 1) return t == 0 ? AR : (RS | (tn << 2) | UPD);
+  return t == 0 ? (AG | (cn << 2) | UPD) : (A2A | ((cn + tn) << 2));
+}
+__host__ __device__ constexpr uint32_t pair_row(int c) {
+  return pair_action(c, 0) | (pair_action(c, 1) << 8) | (pair_action(c, 2) << 16) | (pair_action(c, 3) << 24);
+}
+__device__ __forceinline__ int placement_class(uint32_t code) {
+  const int k = kind_of(code);
+  return k == 2 ? 2 + (dim_of(code) != 0 ? 1 : 0) : k;
+}
 
 template <int M>
 __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_params p, TableArgs a) {
   constexpr int NS = States<M>::kCount;
-  __shared__ uint32_t s_src[APC_TILE_MAX_COLS];
-  __shared__ int32_t s_stensor[APC_TILE_MAX_COLS];
-  __shared__ uint32_t s_tgt[APC_TILE_MAX_ROWS];
-  __shared__ uint8_t s_tflag[APC_TILE_MAX_ROWS];  // bit0 valid spec, bit1 any Partial, bit2 all Shard
+  constexpr int CW = 2 + M;  // words per staged producer spec: codes, info, one action row per mesh dim
+  // term arrays in LDS: [0] zeros, [1] all-gather, [2] reduce-scatter, [3] all-reduce, [4] read+write
+  __shared__ double s_terms[5 * NS];
+  __shared__ uint32_t s_col[APC_TILE_MAX_COLS * CW];
+  __shared__ uint2 s_row[APC_TILE_MAX_ROWS];  // x = codes, y = info
   __shared__ double s_cpa[APC_TILE_MAX_ROWS];
-  __shared__ double s_rw[NS];   // read+write time of the running bytes
-  __shared__ double s_ag[NS];   // all-gather of the previous dim (bytes already multiplied)
-  __shared__ double s_rs[NS];   // reduce-scatter of this level's dim
-  __shared__ double s_a2a[NS];  // all-to-all of this level's dim
-  __shared__ double s_ar[NS];   // all-reduce of this level's dim
   __shared__ int s_uniform;
 
   const apc_tile tile = a.tiles[blockIdx.x];
@@ -299,132 +362,141 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
   for (int j = tid; j < cols; j += kTileThreads) {
     const int sp = tile.src_begin + col0 + j;
     const int t = a.spec_tensor[sp];
-    s_src[j] = a.spec_codes[sp];
-    s_stensor[j] = t;
+    const uint32_t codes = a.spec_codes[sp];
+    // info: bit0 valid spec, bit1 fully replicated, bits 4.. mask of sharded mesh dims
+    uint32_t info = (t >= 0 ? 1u : 0u) | (codes == 0u ? 2u : 0u);
+#pragma unroll
+    for (int i = 0; i < M; ++i) {
+      const uint32_t c = (codes >> (8 * i)) & 0xFF;
+      const int cls = placement_class(c);
+      info |= (cls >= 2 ? 1u : 0u) << (4 + i);
+      s_col[j * CW + 2 + i] = cls == 0 ? pair_row(0) : cls == 1 ? pair_row(1) : cls == 2 ? pair_row(2) : pair_row(3);
+    }
+    s_col[j * CW] = codes;
+    s_col[j * CW + 1] = info;
     if (t != t0) s_uniform = 0;
   }
   for (int j = tid; j < rows; j += kTileThreads) {
     const int ts = tile.tgt_begin + row0 + j;
     const uint32_t tg = a.spec_codes[ts];
-    bool any_partial = false, all_shard = true;
+    // info: bit0 valid spec, bits 1 + 5i .. : 8 x class of mesh dim i, bit 30 every dim is a Shard
+    uint32_t info = a.spec_tensor[ts] >= 0 ? 1u : 0u;
+    bool all_shard = true;
 #pragma unroll
     for (int i = 0; i < M; ++i) {
-      const int k = kind_of((tg >> (8 * i)) & 0xFF);
-      any_partial |= k == 1;
-      all_shard &= k == 2;
+      const uint32_t t = (tg >> (8 * i)) & 0xFF;
+      info |= (uint32_t)(placement_class(t) * 8) << (1 + 5 * i);
+      all_shard &= kind_of(t) == 2;
     }
-    s_tgt[j] = tg;
-    s_tflag[j] = (a.spec_tensor[ts] >= 0 ? 1 : 0) | (any_partial ? 2 : 0) | (all_shard ? 4 : 0);
+    if (all_shard) info |= 1u << 30;
+    s_row[j] = make_uint2(tg, info);
     s_cpa[j] = a.per_arg ? a.per_arg[tile.strat_begin + row0 + j] : 0.0;
+  }
+  if (t0 >= 0 && !no_producer) {
+    // global layout per tensor: [rw][ag][rs][ar]
+    const double *terms = a.tensor_terms + (int64_t)t0 * (kTermArrays * NS);
+    for (int k = tid; k < NS; k += kTileThreads) {
+      s_terms[k] = 0.0;
+      s_terms[4 * NS + k] = terms[k];
+      s_terms[NS + k] = terms[NS + k];
+      s_terms[2 * NS + k] = terms[2 * NS + k];
+      s_terms[3 * NS + k] = terms[3 * NS + k];
+    }
   }
   __syncthreads();
   const bool uniform = s_uniform != 0 && t0 >= 0 && !no_producer;
 
-  // ---- evaluate every reachable state once ---------------------------------------------------
-  bool tile_cont = true;
-  if (uniform) {
-    const double bytes = (double)a.tensor_bytes[t0];
-    tile_cont = a.tensor_contiguous[t0] != 0;
-    for (int k = tid; k < NS; k += kTileThreads) {
-      const int level = 31 - __clz((k >> M) + 1);
-      const int rem = k - ((((1 << level) - 1)) << M);
-      const int mask = rem >> level, hist = rem & ((1 << level) - 1);
-      int64_t shards = 1;
-#pragma unroll
-      for (int i = 0; i < M; ++i)
-        if ((mask >> i) & 1) shards *= p.mesh_size[i];
-      double gb = bytes / (double)shards / 1024 / 1024 / 1024;  // collective_runtime_estimation.py:66-68
-#pragma unroll
-      for (int i = 0; i < M; ++i) {
-        if (i < level && ((hist >> i) & 1)) {
-          const double n = (double)p.mesh_size[i];
-          if ((mask >> i) & 1) gb *= n; else gb /= n;
-        }
-      }
-      s_rw[k] = rw_time(gb * 2 * 1073741824.0, p);
-      double ag = 0.0, rs = 0.0, a2a = 0.0, ar = 0.0;
-      if (level >= 1) ag = ring(gb, p, level - 1, p.mesh_size[level - 1] - 1);
-      if (level < M) {
-        rs = ring(gb, p, level, p.mesh_size[level] - 1);
-        a2a = rs;
-        a2a *= p.a2a_scale;
-        ar = ring(gb, p, level, 2 * (p.mesh_size[level] - 1));
-      }
-      s_ag[k] = ag;
-      s_rs[k] = rs;
-      s_a2a[k] = a2a;
-      s_ar[k] = ar;
-    }
-  }
-  __syncthreads();
-
-  // ---- entries ---------------------------------------------------------------------------------
   const int n = rows * cols;
   int r = tid / cols, c = tid - r * cols;
   const int dr = kTileThreads / cols, dc = kTileThreads - dr * cols;
+
+  if (uniform) {
+    // ---- fast loop: straight-line code per mesh dim, terms looked up by running-bytes state ----
+    const bool tile_cont = a.tensor_contiguous[t0] != 0;
+    const double a2a_scale = p.a2a_scale;
+    for (int idx = tid; idx < n; idx += kTileThreads) {
+      const uint32_t src = s_col[c * CW], cinfo = s_col[c * CW + 1];
+      const uint2 rowv = s_row[r];
+      const uint32_t tgt = rowv.x, tinfo = rowv.y;
+      const uint32_t x = src ^ tgt;
+      const uint32_t mask = (cinfo >> 4) & 0xF;
+      uint32_t hist = 0, seen = 0;
+      // a fully replicated producer returns before the non-contiguity term (:56-62)
+      bool cont = tile_cont || (cinfo & 2u);
+      double cost = 0.0;
+#pragma unroll
+      for (int i = 0; i < M; ++i) {
+        const bool neq = ((x >> (8 * i)) & 0xFF) != 0;
+        const uint32_t tsh = (tinfo >> (1 + 5 * i)) & 0x1F;
+        uint32_t e = (s_col[c * CW + 2 + i] >> tsh) & 0x7F;
+        e = neq ? e : 0u;
+        const uint32_t sel = e & 3u;
+        const uint32_t k = (uint32_t)States<M>::index(i, 0, 0) + (mask << i) + hist;
+        const uint32_t upd = (e >> 6) & 1u;
+        hist |= upd << i;
+        const uint32_t k2 = (uint32_t)States<M>::index(i + 1, 0, 0) + (mask << (i + 1)) + hist;
+        const uint32_t kk = sel == 1u ? k2 : k;  // the all-gather is charged on the gathered bytes
+        if (!tile_cont) {  // (uniform over the tile)
+          cost += (neq && !cont) ? s_terms[4 * NS + k] : 0.0;
+          cont = cont || neq;
+        }
+        double term = s_terms[sel * NS + kk];
+        const double rw = s_terms[4 * NS + kk];
+        term *= (e & 16u) ? a2a_scale : 1.0;
+        cost += term;
+        cost += (double)((e >> 2) & 3u) * rw;
+        seen |= e;
+      }
+      double comm = (seen & 32u) ? INFINITY : cost;
+      const int64_t local = (int64_t)(row0 + r) * n_src + (col0 + c);
+      int trans = x != 0u ? p.transition_scale : 0;  // optimize_sharding.py:345-351
+      if (M == 2 && src == 0x4040u && (tinfo >> 30)) {  // (Partial, Partial) -> all Shard walks dim 1 first
+        const double gb = (double)a.tensor_bytes[t0] / 1024 / 1024 / 1024;
+        comm = entry_cost<M>(src, tgt, gb, tile_cont, p);
+      }
+      if (!(cinfo & tinfo & 1u)) {  // either side is not a DTensorSpec: keep the rule's value
+        comm = a.pt_values[tile.pt_begin + local];
+        trans = 0;
+      }
+      if (flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;  // :358-359
+      const int64_t o = tile.entry_begin + local;
+      if (a.comm_out) a.comm_out[o] = comm;
+      if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
+      if (a.cost_out) a.cost_out[o] = comm + s_cpa[r] + (double)trans;  // :368-372
+      c += dc;
+      r += dr;
+      if (c >= cols) {
+        c -= cols;
+        r += 1;
+      }
+    }
+    return;
+  }
+
+  // ---- generic loop: pass-through edges and edges whose producer specs name different tensors ----
   for (int idx = tid; idx < n; idx += kTileThreads) {
     const int64_t local = (int64_t)(row0 + r) * n_src + (col0 + c);
     double comm;
     int trans = 0;
-    const int tf = s_tflag[r];
-    const int st = s_stensor[c];
-    if (no_producer || st < 0 || !(tf & 1)) {
+    const uint32_t src = s_col[c * CW], cinfo = s_col[c * CW + 1];
+    const uint32_t tgt = s_row[r].x, tinfo = s_row[r].y;
+    if (no_producer || !(cinfo & tinfo & 1u)) {
       comm = a.pt_values[tile.pt_begin + local];
     } else {
-      const uint32_t src = s_src[c], tgt = s_tgt[r];
-      trans = (src != tgt) ? p.transition_scale : 0;  // optimize_sharding.py:345-351
-      const bool flipped = M == 2 && src == 0x4040u && (tf & 4);
-      if (src == 0u) {  // fully replicated producer
-        comm = (tf & 2) ? INFINITY : 0.0;
-      } else if (!uniform || flipped) {
-        int64_t shards = 1;
+      trans = (src != tgt) ? p.transition_scale : 0;
+      const int st = a.spec_tensor[tile.src_begin + col0 + c];
+      int64_t shards = 1;
 #pragma unroll
-        for (int i = 0; i < M; ++i)
-          if (kind_of((src >> (8 * i)) & 0xFF) == 2) shards *= p.mesh_size[i];
-        const double gb = (double)a.tensor_bytes[st] / (double)shards / 1024 / 1024 / 1024;
-        comm = entry_cost<M>(src, tgt, gb, a.tensor_contiguous[st] != 0, p);
-      } else {
-        int mask = 0;
-#pragma unroll
-        for (int i = 0; i < M; ++i) mask |= (kind_of((src >> (8 * i)) & 0xFF) == 2 ? 1 : 0) << i;
-        int hist = 0;
-        bool cont = tile_cont;
-        double cost = 0.0;
-#pragma unroll
-        for (int i = 0; i < M; ++i) {
-          const uint32_t cc = (src >> (8 * i)) & 0xFF, tt = (tgt >> (8 * i)) & 0xFF;
-          if (cc == tt) continue;
-          const int k = States<M>::index(i, mask, hist);
-          if (!cont) cost += s_rw[k];
-          const int ck = kind_of(cc), tk = kind_of(tt);
-          if (ck == 2 && tk == 0) {  // all-gather
-            hist |= 1 << i;
-            const int k2 = States<M>::index(i + 1, mask, hist);
-            cost += s_ag[k2];
-            if (dim_of(cc) != 0) cost += s_rw[k2];
-          } else if (ck == 2 && tk == 2) {  // all-to-all
-            cost += s_a2a[k];
-            const int copies = (dim_of(cc) != 0) + (dim_of(tt) != 0);
-            cost += (double)copies * s_rw[k];
-          } else if (ck == 1 && tk == 0) {  // all-reduce
-            cost += s_ar[k];
-          } else if (ck == 1 && tk == 2) {  // reduce-scatter
-            cost += s_rs[k];
-            if (dim_of(tt) != 0) cost += s_rw[k];
-            hist |= 1 << i;
-          } else if (tk == 1 && ck != 1) {  // -> Partial from Shard / Replicate: banned
-            cost = INFINITY;
-          }
-          cont = true;
-        }
-        comm = cost;
-      }
+      for (int i = 0; i < M; ++i)
+        if (kind_of((src >> (8 * i)) & 0xFF) == 2) shards *= p.mesh_size[i];
+      const double gb = (double)a.tensor_bytes[st] / (double)shards / 1024 / 1024 / 1024;
+      comm = entry_cost<M>(src, tgt, gb, a.tensor_contiguous[st] != 0, p);
     }
-    if (flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;  // :358-359
+    if (flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;
     const int64_t o = tile.entry_begin + local;
     if (a.comm_out) a.comm_out[o] = comm;
     if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
-    if (a.cost_out) a.cost_out[o] = comm + s_cpa[r] + (double)trans;  // :368-372
+    if (a.cost_out) a.cost_out[o] = comm + s_cpa[r] + (double)trans;
     c += dc;
     r += dr;
     if (c >= cols) {
@@ -435,28 +507,31 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
 }
 
 // ------------------------------------------------------------------------------------------
-// a14: segmented min + first argmin, one wavefront per segment
+// a14: segmented min + first argmin.  G consecutive lanes share one segment (G = 4 .. 64,
+// chosen by the host from the mean segment length), so short segments do not leave most of
+// a wavefront idle.
 // ------------------------------------------------------------------------------------------
+template <int G>
 __global__ __launch_bounds__(kBlock) void segmented_min_kernel(const double *__restrict__ values,
                                                                const int64_t *__restrict__ seg_ptr,
                                                                int64_t n_seg, double *__restrict__ mins,
                                                                int32_t *__restrict__ args) {
-  const int lane = threadIdx.x & 63;
-  const int64_t seg = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
-  if (seg >= n_seg) return;
-  const int64_t lo = seg_ptr[seg], hi = seg_ptr[seg + 1];
+  const int sub = threadIdx.x & (G - 1);
+  const int64_t seg = (int64_t)blockIdx.x * (kBlock / G) + (threadIdx.x / G);
+  const bool live = seg < n_seg;
+  const int64_t lo = live ? seg_ptr[seg] : 0, hi = live ? seg_ptr[seg + 1] : 0;
   double best = INFINITY;
   int64_t arg = INT64_MAX;  // absolute index; INT64_MAX = none seen
-  for (int64_t j = lo + lane; j < hi; j += 64) {
+  for (int64_t j = lo + sub; j < hi; j += G) {
     const double v = values[j];
     if (arg == INT64_MAX || v < best) {
       best = v;
       arg = j;
     }
   }
-  // lexicographic (value, index) min across the wavefront; lanes that saw nothing lose
+  // lexicographic (value, index) min inside the group; lanes that saw nothing lose
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
+  for (int off = G / 2; off > 0; off >>= 1) {
     const double ob = __shfl_xor(best, off, 64);
     const int64_t oa = __shfl_xor(arg, off, 64);
     const bool take = (oa != INT64_MAX) && (arg == INT64_MAX || ob < best || (ob == best && oa < arg));
@@ -465,10 +540,17 @@ __global__ __launch_bounds__(kBlock) void segmented_min_kernel(const double *__r
       arg = oa;
     }
   }
-  if (lane == 0) {
+  if (live && sub == 0) {
     mins[seg] = best;
     args[seg] = arg == INT64_MAX ? -1 : (int32_t)(arg - lo);
   }
+}
+
+template <int G>
+void launch_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_seg, double *mins, int32_t *args,
+                          hipStream_t stream) {
+  hipLaunchKernelGGL(segmented_min_kernel<G>, dim3((unsigned)((n_seg + kBlock / G - 1) / (kBlock / G))), dim3(kBlock),
+                     0, stream, values, seg_ptr, n_seg, mins, args);
 }
 
 inline unsigned blocks_for(int64_t n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
@@ -566,13 +648,20 @@ int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const 
   return 0;
 }
 
-int apc_tensor_tables(int64_t n, const int32_t *rank, const int32_t *itemsize, const int64_t *shape,
-                      const int64_t *stride, int64_t *bytes, uint8_t *cont, void *stream) {
-  if (n < 0) return fail(-1, "n_tensors < 0");
+int64_t apc_tensor_terms_count(int mesh_ndim) {
+  if (mesh_ndim < 1 || mesh_ndim > APC_MAX_MESH) return 0;
+  return (int64_t)kTermArrays * states_count(mesh_ndim);
+}
+
+int apc_tensor_tables(const apc_params *params, int64_t n, const int32_t *rank, const int32_t *itemsize,
+                      const int64_t *shape, const int64_t *stride, int64_t *bytes, uint8_t *cont, double *terms,
+                      void *stream) {
+  if (int rc = check_params(params)) return rc;
+  if (n < 0 || n > INT32_MAX) return fail(-1, "n_tensors %lld out of range", (long long)n);
   if (n == 0) return 0;
   if (!rank || !itemsize || !shape || !stride || !bytes || !cont) return fail(-1, "apc_tensor_tables: NULL array");
-  hipLaunchKernelGGL(tensor_tables_kernel, dim3(blocks_for(n, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, n,
-                     rank, itemsize, shape, stride, bytes, cont);
+  hipLaunchKernelGGL(tensor_tables_kernel, dim3((unsigned)n), dim3(64), 0, (hipStream_t)stream, *params, n, rank,
+                     itemsize, shape, stride, bytes, cont, terms);
   return check_launch("apc_tensor_tables");
 }
 
@@ -604,17 +693,18 @@ int apc_compute_costs(const apc_params *params, int64_t n, const int64_t *flops,
 }
 
 int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes, const uint8_t *tensor_contiguous,
-                            const uint32_t *spec_codes, const int32_t *spec_tensor, const double *pt_values,
+                            const double *tensor_terms, const uint32_t *spec_codes, const int32_t *spec_tensor,
+                            const double *pt_values,
                             const double *per_arg, int64_t n_tiles, const apc_tile *tiles, double *comm_out,
                             uint8_t *trans_out, double *cost_out, void *stream) {
   if (int rc = check_params(params)) return rc;
   if (n_tiles < 0 || n_tiles > INT32_MAX) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tiles == 0) return 0;
-  if (!tensor_bytes || !tensor_contiguous || !spec_codes || !spec_tensor || !tiles)
+  if (!tensor_bytes || !tensor_contiguous || !tensor_terms || !spec_codes || !spec_tensor || !tiles)
     return fail(-1, "apc_redistribute_tables: NULL table");
   if (cost_out && !per_arg) return fail(-1, "cost_out needs compute_cost_per_arg");
-  TableArgs a{tensor_bytes, tensor_contiguous, spec_codes, spec_tensor, pt_values, per_arg, tiles,
-              comm_out,     trans_out,         cost_out};
+  TableArgs a{tensor_bytes, tensor_contiguous, tensor_terms, spec_codes, spec_tensor, pt_values,
+              per_arg,      tiles,             comm_out,     trans_out,  cost_out};
   const dim3 grid((unsigned)n_tiles), block(kTileThreads);
   hipStream_t s = (hipStream_t)stream;
   switch (params->mesh_ndim) {
@@ -626,13 +716,19 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
   return check_launch("apc_redistribute_tables");
 }
 
-int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_seg, double *mins, int32_t *args,
-                      void *stream) {
-  if (n_seg < 0) return fail(-1, "n_segments < 0");
+int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_seg, int64_t n_values, double *mins,
+                      int32_t *args, void *stream) {
+  if (n_seg < 0 || n_values < 0) return fail(-1, "negative count");
   if (n_seg == 0) return 0;
-  if (!seg_ptr || !mins || !args) return fail(-1, "apc_segmented_min: NULL array");
-  hipLaunchKernelGGL(segmented_min_kernel, dim3(blocks_for(n_seg, kBlock / 64)), dim3(kBlock), 0,
-                     (hipStream_t)stream, values, seg_ptr, n_seg, mins, args);
+  if (!seg_ptr || !mins || !args || (!values && n_values > 0)) return fail(-1, "apc_segmented_min: NULL array");
+  if (n_seg > (int64_t)INT32_MAX * 4) return fail(-1, "n_segments %lld too large", (long long)n_seg);
+  hipStream_t s = (hipStream_t)stream;
+  const double mean = (double)n_values / (double)n_seg;
+  if (mean <= 4) launch_segmented_min<4>(values, seg_ptr, n_seg, mins, args, s);
+  else if (mean <= 8) launch_segmented_min<8>(values, seg_ptr, n_seg, mins, args, s);
+  else if (mean <= 16) launch_segmented_min<16>(values, seg_ptr, n_seg, mins, args, s);
+  else if (mean <= 32) launch_segmented_min<32>(values, seg_ptr, n_seg, mins, args, s);
+  else launch_segmented_min<64>(values, seg_ptr, n_seg, mins, args, s);
   return check_launch("apc_segmented_min");
 }
 

@@ -50,8 +50,8 @@ extern "C" {
 #define APC_MAX_RANK 8
 #define APC_MAX_MESH 4
 #define APC_MAX_DTYPES 8
-#define APC_TILE_MAX_COLS 256 /* producer specs staged in LDS per tile */
-#define APC_TILE_MAX_ROWS 256 /* consumer specs staged in LDS per tile */
+#define APC_TILE_MAX_COLS 128 /* producer specs staged in LDS per tile */
+#define APC_TILE_MAX_ROWS 128 /* consumer specs staged in LDS per tile */
 
 #define APC_EDGE_GRAD_RESCALE 1 /* consumer is a parameter-gradient node (optimize_sharding.py:358-359) */
 #define APC_EDGE_NO_PRODUCER 2  /* placeholder / factory pseudo-argument (optimize_sharding.py:312-355) */
@@ -107,13 +107,22 @@ int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const 
                              const int64_t *edge_entry_begin_host, const int32_t *edge_strat_begin_host,
                              int64_t n_pt, int64_t n_strategies, int64_t n_tiles, const apc_tile *tiles_host);
 
-/* Bytes and contiguity of every tensor row.
+/* Number of doubles per tensor in the tensor_terms table for a mesh of this ndim
+ * (4 term arrays x the number of running-bytes states); 0 for an unsupported ndim. */
+int64_t apc_tensor_terms_count(int mesh_ndim);
+
+/* Bytes and contiguity of every tensor row, and the tensor's collective / read-write cost
+ * terms for every running-bytes state (tensor_terms: [n_tensors][apc_tensor_terms_count]).
  * Replaces torch spec_to_bytes (distributed/tensor/_collective_utils.py:230-232) and
  * check_contiguous_sizes_strides (_prims_common/__init__.py:252-292) as called from
- * collective_runtime_estimation.py:66-76. */
-int apc_tensor_tables(int64_t n_tensors, const int32_t *tensor_rank, const int32_t *tensor_itemsize,
-                      const int64_t *tensor_shape, const int64_t *tensor_stride, int64_t *tensor_bytes,
-                      uint8_t *tensor_contiguous, void *stream);
+ * collective_runtime_estimation.py:66-76, and evaluates allgather_cost / reduce_scatter_cost /
+ * allreduce_cost (torch _collective_utils.py:281-313) and compute_read_write_time
+ * (compute_estimation.py:302-314) once per value comm_bytes_gb can take for the tensor
+ * (collective_runtime_estimation.py:66-68, :86, :128).  tensor_terms may be NULL (then
+ * apc_redistribute_tables cannot be used with the outputs). */
+int apc_tensor_tables(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
+                      const int32_t *tensor_itemsize, const int64_t *tensor_shape, const int64_t *tensor_stride,
+                      int64_t *tensor_bytes, uint8_t *tensor_contiguous, double *tensor_terms, void *stream);
 
 /* Local shard shape / stride / element and byte counts and shard count per spec.
  * Replaces _get_sharded_shape_stride (compute_estimation.py:211-229) and
@@ -144,17 +153,18 @@ int apc_compute_costs(const apc_params *params, int64_t n_strategies, const int6
  * (:345-351), the grad rescale (:358-359) and cost assembly (:368-372).
  * comm_out / transition_out / cost_out are [n_entries]; any may be NULL. */
 int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes,
-                            const uint8_t *tensor_contiguous, const uint32_t *spec_codes,
-                            const int32_t *spec_tensor, const double *pt_values,
+                            const uint8_t *tensor_contiguous, const double *tensor_terms,
+                            const uint32_t *spec_codes, const int32_t *spec_tensor, const double *pt_values,
                             const double *compute_cost_per_arg, int64_t n_tiles, const apc_tile *tiles,
                             double *comm_out, uint8_t *transition_out, double *cost_out, void *stream);
 
 /* Segmented minimum with first-argmin (relative to the segment start); empty
  * segments give (+inf, -1).  No counterpart in the reference (which hands the full
  * table to the ILP solver, optimize_sharding.py:648-659): used for pruning and
- * warm start. */
-int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_segments, double *seg_min,
-                      int32_t *seg_argmin, void *stream);
+ * warm start.  n_values = seg_ptr[n_segments] (the host knows it; it selects how many lanes
+ * share a segment). */
+int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_segments, int64_t n_values,
+                      double *seg_min, int32_t *seg_argmin, void *stream);
 
 #ifdef __cplusplus
 }
