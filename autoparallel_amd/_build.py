@@ -7,7 +7,8 @@ import subprocess
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 _ROOT = os.path.dirname(_PKG)
-LIB_PATH = os.path.join(_PKG, "libapcost.so")
+# APCOST_LIBRARY names another build of the same sources (a debug or instrumented one)
+LIB_PATH = os.environ.get("APCOST_LIBRARY") or os.path.join(_PKG, "libapcost.so")
 SOURCES = [os.path.join(_PKG, "csrc", "apcost.hip")]
 INCLUDE = os.path.join(_ROOT, "include")
 

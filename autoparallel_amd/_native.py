@@ -47,7 +47,7 @@ class ApcTile(ctypes.Structure):
         ("src_begin", ctypes.c_int32), ("n_src", ctypes.c_int32), ("tgt_begin", ctypes.c_int32),
         ("flags", ctypes.c_int32), ("strat_begin", ctypes.c_int32),
         ("entry_begin", ctypes.c_int64), ("pt_begin", ctypes.c_int64),
-        ("reserved", ctypes.c_int32 * 2),
+        ("tensor", ctypes.c_int32), ("reserved", ctypes.c_int32),
     ]
 
 

@@ -294,7 +294,6 @@ __global__ __launch_bounds__(kBlock) void compute_costs_kernel(
 // remains the path for the rare cases the states do not cover: producer specs of one edge
 // that point at different tensors, and the 2-D (Partial, Partial) -> all-Shard order flip.
 // ------------------------------------------------------------------------------------------
-constexpr int kTileThreads = 64;
 
 struct TableArgs {
   const int64_t *tensor_bytes;
@@ -313,20 +312,19 @@ struct TableArgs {
 // What one mesh dim contributes, by (producer class, consumer class) with classes
 // 0 Replicate, 1 Partial, 2 Shard(0), 3 Shard(d != 0); only consulted when the two placement
 // codes differ.  One byte per pair:
-//   bits 0-1  term array: 0 none, 1 all-gather, 2 reduce-scatter, 3 all-reduce
-//   bits 2-3  number of read+write reshuffles added after the collective
-//   bit  4    all-to-all: the reduce-scatter shaped term times a2a_scale
+//   bits 0-2  term array: 0 none, 1 all-gather, 2 reduce-scatter, 3 all-reduce, 4 all-to-all
+//   bits 3-4  number of read+write reshuffles added after the collective
 //   bit  5    banned transition (-> Partial from Replicate / Shard): cost is inf
 //   bit  6    the running bytes change after this dim (x n after all-gather, / n after
 //             reduce-scatter)
 // collective_runtime_estimation.py:83-138.
 __host__ __device__ constexpr uint32_t pair_action(int c, int t) {
-  constexpr uint32_t AG = 1, RS = 2, AR = 3, A2A = 2u | (1u << 4), BAN = 1u << 5, UPD = 1u << 6;
+  constexpr uint32_t AG = 1, RS = 2, AR = 3, A2A = 4, BAN = 1u << 5, UPD = 1u << 6;
   const uint32_t cn = c == 3, tn = t == 3;
   if (t == 1) return c == 1 ? 0u : BAN;            // -> Partial
   if (c == 0) return 0u;                           // Replicate -> Replicate / Shard: local
-  if (c == 1) return t == 0 ? AR : (RS | (tn << 2) | UPD);
-  return t == 0 ? (AG | (cn << 2) | UPD) : (A2A | ((cn + tn) << 2));
+  if (c == 1) return t == 0 ? AR : (RS | (tn << 3) | UPD);
+  return t == 0 ? (AG | (cn << 3) | UPD) : (A2A | ((cn + tn) << 3));
 }
 __host__ __device__ constexpr uint32_t pair_row(int c) {
   return pair_action(c, 0) | (pair_action(c, 1) << 8) | (pair_action(c, 2) << 16) | (pair_action(c, 3) << 24);
@@ -336,12 +334,110 @@ __device__ __forceinline__ int placement_class(uint32_t code) {
   return k == 2 ? 2 + (dim_of(code) != 0 ? 1 : 0) : k;
 }
 
-template <int M>
+constexpr int kLdsTermArrays = 6;  // zeros, all-gather, reduce-scatter, all-reduce, all-to-all, read+write
+
+// The per-entry loop of a tile whose producer specs all name one tensor.  Straight-line code:
+// all lookups of an entry are independent of its fp additions, so they are issued together.
+template <int M, int kTileThreads, bool CONT, bool RESCALE>
+__device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const TableArgs &a, const apc_tile &tile,
+                                                     const double *s_terms, const uint32_t *s_col,
+                                                     const uint2 *s_row, const double *s_cpa, int t0) {
+  constexpr int NS = States<M>::kCount;
+  constexpr int CW = 2 + M;
+  const int rows = tile.row_count, cols = tile.col_count;
+  const int tid = threadIdx.x;
+  const int n = rows * cols;
+  int r = tid / cols, c = tid - r * cols;
+  const int dr = kTileThreads / cols, dc = kTileThreads - dr * cols;
+  const int64_t tile_base = tile.entry_begin + (int64_t)tile.row_begin * tile.n_src + tile.col_begin;
+  // only the 2-D order flip evaluates an entry directly; (Partial, Partial) shards nothing
+  const double gb_unsharded = M == 2 ? (double)a.tensor_bytes[t0] / 1024 / 1024 / 1024 : 0.0;
+  // Every spec of the tile is a DTensorSpec on one tensor (the caller checked): the loop
+  // below issues no vector memory loads, so its stores are never waited for.
+  for (int idx = tid; idx < n; idx += kTileThreads) {
+    const uint32_t src = s_col[c * CW], cinfo = s_col[c * CW + 1];
+    const uint2 rowv = s_row[r];
+    const uint32_t tgt = rowv.x, tinfo = rowv.y;
+    const double cpa = s_cpa[r];
+    const uint32_t x = src ^ tgt;
+    const uint32_t mask = (cinfo >> 4) & 0xF;
+    // ---- integer part: which term of which state each mesh dim adds ------------------------
+    uint32_t hist = 0, seen = 0;
+    uint32_t term_at[M], rw_at[M], nc_at[M], copies[M];
+    bool neq[M];
+#pragma unroll
+    for (int i = 0; i < M; ++i) {
+      neq[i] = ((x >> (8 * i)) & 0xFF) != 0;
+      const uint32_t tsh = (tinfo >> (1 + 5 * i)) & 0x1F;
+      uint32_t e = (s_col[c * CW + 2 + i] >> tsh) & 0x7F;
+      e = neq[i] ? e : 0u;
+      const uint32_t sel = e & 7u;
+      const uint32_t k = (uint32_t)States<M>::index(i, 0, 0) + (mask << i) + hist;
+      hist |= ((e >> 6) & 1u) << i;
+      const uint32_t k2 = (uint32_t)States<M>::index(i + 1, 0, 0) + (mask << (i + 1)) + hist;
+      const uint32_t kk = sel == 1u ? k2 : k;  // the all-gather is charged on the gathered bytes
+      term_at[i] = sel * NS + kk;
+      rw_at[i] = 5 * NS + kk;
+      nc_at[i] = 5 * NS + k;
+      copies[i] = (e >> 3) & 3u;
+      seen |= e;
+    }
+    // ---- lookups ------------------------------------------------------------------------------
+    double term[M], rw[M], nc[M];
+#pragma unroll
+    for (int i = 0; i < M; ++i) {
+      term[i] = s_terms[term_at[i]];
+      rw[i] = s_terms[rw_at[i]];
+      if (!CONT) nc[i] = s_terms[nc_at[i]];
+    }
+    // ---- additions in the reference's order ------------------------------------------------------
+    double cost = 0.0;
+    // a fully replicated producer returns before the non-contiguity term (:56-62)
+    bool cont = CONT || (cinfo & 2u);
+#pragma unroll
+    for (int i = 0; i < M; ++i) {
+      if (!CONT) {
+        cost += (neq[i] && !cont) ? nc[i] : 0.0;
+        cont = cont || neq[i];
+      }
+      cost += term[i];
+      cost += (double)copies[i] * rw[i];
+    }
+    double comm = (seen & 32u) ? INFINITY : cost;
+    const int64_t local = (int64_t)r * tile.n_src + c;
+    int trans = x != 0u ? p.transition_scale : 0;  // optimize_sharding.py:345-351
+    if (M == 2 && src == 0x4040u && (tinfo >> 30)) {  // (Partial, Partial) -> all Shard walks dim 1 first
+      comm = entry_cost<M>(src, tgt, gb_unsharded, CONT, p);
+    }
+    if (RESCALE) comm = comm / p.rescale;  // :358-359
+    const int64_t o = tile_base + local;
+#if defined(APC_EXP_NO_STORE)
+    if (comm == -1.0) a.comm_out[o] = comm;
+#elif defined(APC_EXP_NO_COMPUTE)
+    a.comm_out[o] = cpa;
+    if (APC_EXP_NO_COMPUTE <= 2) a.cost_out[o] = cpa;
+    if (APC_EXP_NO_COMPUTE <= 1) a.trans_out[o] = (uint8_t)idx;
+#else
+    if (a.comm_out) a.comm_out[o] = comm;
+    if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
+    if (a.cost_out) a.cost_out[o] = comm + cpa + (double)trans;  // :368-372
+#endif
+    c += dc;
+    r += dr;
+    if (c >= cols) {
+      c -= cols;
+      r += 1;
+    }
+  }
+}
+
+template <int M, int kTileThreads>
 __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_params p, TableArgs a) {
   constexpr int NS = States<M>::kCount;
   constexpr int CW = 2 + M;  // words per staged producer spec: codes, info, one action row per mesh dim
-  // term arrays in LDS: [0] zeros, [1] all-gather, [2] reduce-scatter, [3] all-reduce, [4] read+write
-  __shared__ double s_terms[5 * NS];
+  // term arrays in LDS: [0] zeros, [1] all-gather, [2] reduce-scatter, [3] all-reduce,
+  // [4] all-to-all (= reduce-scatter shaped term x a2a_scale, :22-32), [5] read+write
+  __shared__ double s_terms[kLdsTermArrays * NS];
   __shared__ uint32_t s_col[APC_TILE_MAX_COLS * CW];
   __shared__ uint2 s_row[APC_TILE_MAX_ROWS];  // x = codes, y = info
   __shared__ double s_cpa[APC_TILE_MAX_ROWS];
@@ -358,7 +454,24 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
   // ---- stage the tile's producer / consumer specs -------------------------------------------
   if (tid == 0) s_uniform = 1;
   __syncthreads();
-  const int t0 = a.spec_tensor[tile.src_begin + col0];
+  const int t0 = tile.tensor;  // spec_tensor of the tile's first producer spec (checked by the host)
+  const bool terms_wanted = t0 >= 0 && !no_producer;
+  if (terms_wanted) {
+    // global layout per tensor: [rw][ag][rs][ar]
+    const double *terms = a.tensor_terms + (int64_t)t0 * (kTermArrays * NS);
+    for (int k = tid; k < NS; k += kTileThreads) {
+      const double rs = terms[2 * NS + k];
+      double a2a = rs;
+      a2a *= p.a2a_scale;
+      s_terms[k] = 0.0;
+      s_terms[NS + k] = terms[NS + k];
+      s_terms[2 * NS + k] = rs;
+      s_terms[3 * NS + k] = terms[3 * NS + k];
+      s_terms[4 * NS + k] = a2a;
+      s_terms[5 * NS + k] = terms[k];
+    }
+  }
+  const bool tile_cont = terms_wanted ? a.tensor_contiguous[t0] != 0 : true;
   for (int j = tid; j < cols; j += kTileThreads) {
     const int sp = tile.src_begin + col0 + j;
     const int t = a.spec_tensor[sp];
@@ -374,7 +487,7 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
     }
     s_col[j * CW] = codes;
     s_col[j * CW + 1] = info;
-    if (t != t0) s_uniform = 0;
+    if (t != t0 || t < 0) s_uniform = 0;
   }
   for (int j = tid; j < rows; j += kTileThreads) {
     const int ts = tile.tgt_begin + row0 + j;
@@ -389,19 +502,9 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
       all_shard &= kind_of(t) == 2;
     }
     if (all_shard) info |= 1u << 30;
+    if (!(info & 1u)) s_uniform = 0;  // a consumer spec that is not a DTensorSpec: generic loop
     s_row[j] = make_uint2(tg, info);
     s_cpa[j] = a.per_arg ? a.per_arg[tile.strat_begin + row0 + j] : 0.0;
-  }
-  if (t0 >= 0 && !no_producer) {
-    // global layout per tensor: [rw][ag][rs][ar]
-    const double *terms = a.tensor_terms + (int64_t)t0 * (kTermArrays * NS);
-    for (int k = tid; k < NS; k += kTileThreads) {
-      s_terms[k] = 0.0;
-      s_terms[4 * NS + k] = terms[k];
-      s_terms[NS + k] = terms[NS + k];
-      s_terms[2 * NS + k] = terms[2 * NS + k];
-      s_terms[3 * NS + k] = terms[3 * NS + k];
-    }
   }
   __syncthreads();
   const bool uniform = s_uniform != 0 && t0 >= 0 && !no_producer;
@@ -411,64 +514,13 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
   const int dr = kTileThreads / cols, dc = kTileThreads - dr * cols;
 
   if (uniform) {
-    // ---- fast loop: straight-line code per mesh dim, terms looked up by running-bytes state ----
-    const bool tile_cont = a.tensor_contiguous[t0] != 0;
-    const double a2a_scale = p.a2a_scale;
-    for (int idx = tid; idx < n; idx += kTileThreads) {
-      const uint32_t src = s_col[c * CW], cinfo = s_col[c * CW + 1];
-      const uint2 rowv = s_row[r];
-      const uint32_t tgt = rowv.x, tinfo = rowv.y;
-      const uint32_t x = src ^ tgt;
-      const uint32_t mask = (cinfo >> 4) & 0xF;
-      uint32_t hist = 0, seen = 0;
-      // a fully replicated producer returns before the non-contiguity term (:56-62)
-      bool cont = tile_cont || (cinfo & 2u);
-      double cost = 0.0;
-#pragma unroll
-      for (int i = 0; i < M; ++i) {
-        const bool neq = ((x >> (8 * i)) & 0xFF) != 0;
-        const uint32_t tsh = (tinfo >> (1 + 5 * i)) & 0x1F;
-        uint32_t e = (s_col[c * CW + 2 + i] >> tsh) & 0x7F;
-        e = neq ? e : 0u;
-        const uint32_t sel = e & 3u;
-        const uint32_t k = (uint32_t)States<M>::index(i, 0, 0) + (mask << i) + hist;
-        const uint32_t upd = (e >> 6) & 1u;
-        hist |= upd << i;
-        const uint32_t k2 = (uint32_t)States<M>::index(i + 1, 0, 0) + (mask << (i + 1)) + hist;
-        const uint32_t kk = sel == 1u ? k2 : k;  // the all-gather is charged on the gathered bytes
-        if (!tile_cont) {  // (uniform over the tile)
-          cost += (neq && !cont) ? s_terms[4 * NS + k] : 0.0;
-          cont = cont || neq;
-        }
-        double term = s_terms[sel * NS + kk];
-        const double rw = s_terms[4 * NS + kk];
-        term *= (e & 16u) ? a2a_scale : 1.0;
-        cost += term;
-        cost += (double)((e >> 2) & 3u) * rw;
-        seen |= e;
-      }
-      double comm = (seen & 32u) ? INFINITY : cost;
-      const int64_t local = (int64_t)(row0 + r) * n_src + (col0 + c);
-      int trans = x != 0u ? p.transition_scale : 0;  // optimize_sharding.py:345-351
-      if (M == 2 && src == 0x4040u && (tinfo >> 30)) {  // (Partial, Partial) -> all Shard walks dim 1 first
-        const double gb = (double)a.tensor_bytes[t0] / 1024 / 1024 / 1024;
-        comm = entry_cost<M>(src, tgt, gb, tile_cont, p);
-      }
-      if (!(cinfo & tinfo & 1u)) {  // either side is not a DTensorSpec: keep the rule's value
-        comm = a.pt_values[tile.pt_begin + local];
-        trans = 0;
-      }
-      if (flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;  // :358-359
-      const int64_t o = tile.entry_begin + local;
-      if (a.comm_out) a.comm_out[o] = comm;
-      if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
-      if (a.cost_out) a.cost_out[o] = comm + s_cpa[r] + (double)trans;  // :368-372
-      c += dc;
-      r += dr;
-      if (c >= cols) {
-        c -= cols;
-        r += 1;
-      }
+    const bool rescale = (flags & APC_EDGE_GRAD_RESCALE) != 0;
+    if (tile_cont) {
+      if (rescale) uniform_tile_entries<M, kTileThreads, true, true>(p, a, tile, s_terms, s_col, s_row, s_cpa, t0);
+      else uniform_tile_entries<M, kTileThreads, true, false>(p, a, tile, s_terms, s_col, s_row, s_cpa, t0);
+    } else {
+      if (rescale) uniform_tile_entries<M, kTileThreads, false, true>(p, a, tile, s_terms, s_col, s_row, s_cpa, t0);
+      else uniform_tile_entries<M, kTileThreads, false, false>(p, a, tile, s_terms, s_col, s_row, s_cpa, t0);
     }
     return;
   }
@@ -644,6 +696,8 @@ int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const 
         tl.flags != edge_flags[e] || tl.strat_begin != edge_strat_begin[e] ||
         tl.entry_begin != edge_entry_begin[e] || tl.pt_begin != edge_pt_begin[e])
       return fail(-2, "tile %lld: record does not repeat the fields of edge %d", (long long)t, e);
+    if (tl.tensor != spec_tensor[edge_src_begin[e] + tl.col_begin])
+      return fail(-2, "tile %lld: tensor %d is not the tensor of its first producer spec", (long long)t, tl.tensor);
   }
   return 0;
 }
@@ -695,24 +749,32 @@ int apc_compute_costs(const apc_params *params, int64_t n, const int64_t *flops,
 int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes, const uint8_t *tensor_contiguous,
                             const double *tensor_terms, const uint32_t *spec_codes, const int32_t *spec_tensor,
                             const double *pt_values,
-                            const double *per_arg, int64_t n_tiles, const apc_tile *tiles, double *comm_out,
-                            uint8_t *trans_out, double *cost_out, void *stream) {
+                            const double *per_arg, int64_t n_tiles, const apc_tile *tiles, int64_t n_entries,
+                            double *comm_out, uint8_t *trans_out, double *cost_out, void *stream) {
   if (int rc = check_params(params)) return rc;
   if (n_tiles < 0 || n_tiles > INT32_MAX) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tiles == 0) return 0;
+  if (n_entries < 0) return fail(-1, "n_entries < 0");
   if (!tensor_bytes || !tensor_contiguous || !tensor_terms || !spec_codes || !spec_tensor || !tiles)
     return fail(-1, "apc_redistribute_tables: NULL table");
   if (cost_out && !per_arg) return fail(-1, "cost_out needs compute_cost_per_arg");
   TableArgs a{tensor_bytes, tensor_contiguous, tensor_terms, spec_codes, spec_tensor, pt_values,
               per_arg,      tiles,             comm_out,     trans_out,  cost_out};
-  const dim3 grid((unsigned)n_tiles), block(kTileThreads);
+  const dim3 grid((unsigned)n_tiles);
   hipStream_t s = (hipStream_t)stream;
+  // small matrices (traced graphs): one wavefront per tile; large ones: two wavefronts share
+  // the staged specs and terms of a tile
+  const bool wide = n_entries / n_tiles >= 512;
+#define APC_LAUNCH(M_)                                                                                  \
+  if (wide) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 128>), grid, dim3(128), 0, s, *params, a); \
+  else hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 64>), grid, dim3(64), 0, s, *params, a)
   switch (params->mesh_ndim) {
-    case 1: hipLaunchKernelGGL(redistribute_tiles_kernel<1>, grid, block, 0, s, *params, a); break;
-    case 2: hipLaunchKernelGGL(redistribute_tiles_kernel<2>, grid, block, 0, s, *params, a); break;
-    case 3: hipLaunchKernelGGL(redistribute_tiles_kernel<3>, grid, block, 0, s, *params, a); break;
-    default: hipLaunchKernelGGL(redistribute_tiles_kernel<4>, grid, block, 0, s, *params, a); break;
+    case 1: APC_LAUNCH(1); break;
+    case 2: APC_LAUNCH(2); break;
+    case 3: APC_LAUNCH(3); break;
+    default: APC_LAUNCH(4); break;
   }
+#undef APC_LAUNCH
   return check_launch("apc_redistribute_tables");
 }
 

@@ -161,7 +161,8 @@ class DeviceCostTables:
                 ctypes.byref(self.c_params), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
                 self._p(self.tensor_terms), self._p("spec_codes"), self._p("spec_tensor"), self._p("pt_values"),
                 self._p(self.compute_cost_per_arg), ctypes.c_int64(self.tables.n_tiles), self._p("tile_records"),
-                self._p(self.comm), self._p(self.transition), self._p(self.cost), self._stream())
+                ctypes.c_int64(self.tables.n_entries), self._p(self.comm), self._p(self.transition),
+                self._p(self.cost), self._stream())
         _native.check(rc, "apc_redistribute_tables")
 
     @_guarded
@@ -208,7 +209,7 @@ class DeviceCostTables:
         a_tables = (cp, P(self.tensor_bytes), P(self.tensor_contiguous), P(self.tensor_terms), P("spec_codes"),
                     P("spec_tensor"),
                     P("pt_values"), P(self.compute_cost_per_arg), ctypes.c_int64(tb.n_tiles), P("tile_records"),
-                    P(self.comm), P(self.transition), P(self.cost), stream)
+                    ctypes.c_int64(tb.n_entries), P(self.comm), P(self.transition), P(self.cost), stream)
 
         def bind(fn, args, what):
             def launch():

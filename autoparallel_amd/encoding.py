@@ -53,7 +53,7 @@ DEFAULT_TILE_ENTRIES = 2048
 TILE_DTYPE = np.dtype([
     ("edge", "<i4"), ("row_begin", "<i4"), ("row_count", "<i4"), ("col_begin", "<i4"), ("col_count", "<i4"),
     ("src_begin", "<i4"), ("n_src", "<i4"), ("tgt_begin", "<i4"), ("flags", "<i4"), ("strat_begin", "<i4"),
-    ("entry_begin", "<i8"), ("pt_begin", "<i8"), ("reserved", "<i4", (2,)),
+    ("entry_begin", "<i8"), ("pt_begin", "<i8"), ("tensor", "<i4"), ("reserved", "<i4"),
 ])
 assert TILE_DTYPE.itemsize == 64
 
@@ -244,6 +244,10 @@ class CostTables:
         rec["strat_begin"] = self.edge_strat_begin[te]
         rec["entry_begin"] = self.edge_entry_begin[:-1][te] if len(te) else 0
         rec["pt_begin"] = self.edge_pt_begin[te]
+        if len(te) and self.n_specs:
+            # (indices are clipped here; validate() reports ranges that fall outside the table)
+            first = np.clip(self.edge_src_begin[te].astype(np.int64) + self.tile_col_begin, 0, self.n_specs - 1)
+            rec["tensor"] = self.spec_tensor[first]
         self.tile_records = rec
 
     # ---- checks ------------------------------------------------------------------------

@@ -70,7 +70,8 @@ typedef struct apc_tile {
   int32_t strat_begin;          /* = edge_strat_begin[edge] */
   int64_t entry_begin;          /* = edge_entry_begin[edge] */
   int64_t pt_begin;             /* = edge_pt_begin[edge] */
-  int32_t reserved[2];
+  int32_t tensor;               /* = spec_tensor[src_begin + col_begin] */
+  int32_t reserved;
 } apc_tile;
 
 /* Cost-model parameters: everything the reference reads from its environment
@@ -156,7 +157,8 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
                             const uint8_t *tensor_contiguous, const double *tensor_terms,
                             const uint32_t *spec_codes, const int32_t *spec_tensor, const double *pt_values,
                             const double *compute_cost_per_arg, int64_t n_tiles, const apc_tile *tiles,
-                            double *comm_out, uint8_t *transition_out, double *cost_out, void *stream);
+                            int64_t n_entries, double *comm_out, uint8_t *transition_out, double *cost_out,
+                            void *stream);
 
 /* Segmented minimum with first-argmin (relative to the segment start); empty
  * segments give (+inf, -1).  No counterpart in the reference (which hands the full
