@@ -40,6 +40,9 @@ def parse_args():
     ap.add_argument("--tile-entries", type=int, default=None)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU-baseline sample duration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 1 GiB device-to-device copy three times (reference reading for the "
+                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
     return ap.parse_args()
 
 
@@ -124,6 +127,15 @@ def main():
         print("bench.py needs a HIP device (there is no CPU path for the product)", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if args.calibrate_copy:
+        src = torch.ones(1 << 27, dtype=torch.float64, device="cuda:0")  # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 8, "calibrate_copy_bytes_written": src.numel() * 8,
+                          "copies": 3}))
+        return
     from autoparallel_amd.device_tables import DeviceCostTables
 
     t_setup = time.perf_counter()
