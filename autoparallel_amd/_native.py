@@ -14,8 +14,8 @@ from ._build import LIB_PATH
 APC_MAX_RANK = 8
 APC_MAX_MESH = 4
 APC_MAX_DTYPES = 8
-APC_TILE_MAX_COLS = 128
-APC_TILE_MAX_ROWS = 128
+APC_TILE_MAX_COLS = 64
+APC_TILE_MAX_ROWS = 64
 
 EDGE_GRAD_RESCALE = 1
 EDGE_NO_PRODUCER = 2

@@ -354,6 +354,9 @@ __device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const 
   const double gb_unsharded = M == 2 ? (double)a.tensor_bytes[t0] / 1024 / 1024 / 1024 : 0.0;
   // Every spec of the tile is a DTensorSpec on one tensor (the caller checked): the loop
   // below issues no vector memory loads, so its stores are never waited for.
+#if defined(APC_EXP_PROLOGUE_ONLY)
+  if (n > 0) return;
+#endif
   for (int idx = tid; idx < n; idx += kTileThreads) {
     const uint32_t src = s_col[c * CW], cinfo = s_col[c * CW + 1];
     const uint2 rowv = s_row[r];

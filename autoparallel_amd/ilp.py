@@ -84,18 +84,47 @@ class BinaryProgram:
         m.sum_duplicates()
         return m
 
+    def deduplicated(self):
+        """(matrix, lb, ub) with repeated rows removed.  Variable sharing makes many
+        constraints of linked nodes literally identical; rows are compared through two
+        independent 64-bit hashes of their (column, coefficient) pairs."""
+        a = self.matrix()
+        lb, ub = np.asarray(self._lb), np.asarray(self._ub)
+        if a.shape[0] == 0:
+            return a, lb, ub
+        a.sort_indices()
+        a.eliminate_zeros()
+        indptr = a.indptr.astype(np.int64)
+        nnz_rows = np.nonzero(np.diff(indptr) > 0)[0]
+        cols = a.indices.astype(np.uint64)
+        vals = a.data.view(np.uint64)
+        with np.errstate(over="ignore"):
+            h1 = (cols * np.uint64(0x9E3779B97F4A7C15) + np.uint64(0x632BE59BD9B4E019)) ^ (vals * np.uint64(0xD6E8FEB86659FD93))
+            h2 = (cols * np.uint64(0xC2B2AE3D27D4EB4F) + np.uint64(0x165667B19E3779F9)) ^ (vals * np.uint64(0xFF51AFD7ED558CCD))
+            h1 = h1 * (h1 >> np.uint64(29) | np.uint64(1))
+            h2 = h2 * (h2 >> np.uint64(31) | np.uint64(1))
+            r1 = np.zeros(a.shape[0], np.uint64)
+            r2 = np.zeros(a.shape[0], np.uint64)
+            r1[nnz_rows] = np.add.reduceat(h1, indptr[nnz_rows])
+            r2[nnz_rows] = np.add.reduceat(h2, indptr[nnz_rows])
+        sig = np.stack([r1, r2, np.diff(indptr).astype(np.uint64), lb.view(np.uint64), ub.view(np.uint64)], axis=1)
+        _, keep = np.unique(sig, axis=0, return_index=True)
+        keep.sort()
+        self.rows_before_dedupe, self.rows_after_dedupe = a.shape[0], len(keep)
+        return a[keep], lb[keep], ub[keep]
+
     # ---- solving -------------------------------------------------------------------------
     def solve(self, verbose: bool = False, time_limit: float | None = None, mip_rel_gap: float | None = None):
         from scipy.optimize import Bounds, LinearConstraint, milp
 
-        a = self.matrix()
+        a, lb, ub = self.deduplicated()
         t0 = time.time()
         options = {"disp": bool(verbose)}
         if time_limit is not None:
             options["time_limit"] = float(time_limit)
         if mip_rel_gap is not None:
             options["mip_rel_gap"] = float(mip_rel_gap)
-        constraints = [LinearConstraint(a, np.asarray(self._lb), np.asarray(self._ub))] if self._names else []
+        constraints = [LinearConstraint(a, lb, ub)] if self._names else []
         res = milp(self.objective, integrality=np.ones(self.n_vars), bounds=Bounds(np.zeros(self.n_vars), self.upper),
                    constraints=constraints, options=options)
         self.solve_seconds = time.time() - t0

@@ -160,6 +160,43 @@ class CostRecords(Mapping):
         return (s_i, argi, local // ns, local % ns)
 
 
+class ClusterLinks(Mapping):
+    """``cluster_links``: key of a linked entry -> key of the entry whose ILP variable it
+    shares (optimize_sharding.py:211-231), derived from the node representatives."""
+
+    def __init__(self, optimizer: "ShardingOptimizer"):
+        self._o = optimizer
+
+    def _rep(self, key):
+        s_i, argi, ss, ii = key
+        o = self._o
+        if key not in o.ds:
+            raise KeyError(key)
+        rep = o.node_representative.get(o.nodes[s_i])
+        if rep is None:
+            raise KeyError(key)
+        return (o.node_map[rep], argi, ss, ii)
+
+    def __getitem__(self, key):
+        return self._rep(key)
+
+    def __contains__(self, key):
+        try:
+            self._rep(key)
+            return True
+        except (KeyError, TypeError, ValueError):
+            return False
+
+    def __iter__(self):
+        o = self._o
+        for key in o.ds:
+            if o.nodes[key[0]] in o.node_representative:
+                yield key
+
+    def __len__(self):
+        return int(self._o._linked_entry.sum())
+
+
 class ShardingOptimizer:
     # environment of the cost model, explicit (the reference reads torch.cuda.device_count()
     # and torch.cuda.get_device_name(); its tests patch them to 8 and "H100")
@@ -181,13 +218,18 @@ class ShardingOptimizer:
         self.strats = self.build_sharding_metadata()
         self.timings["enumerate_s"] = time.perf_counter() - t0
 
-        self.cluster_links = {}
+        self.node_representative = {}
         if repeated_subgraphs:
-            raise NotImplementedError("repeated_subgraphs=True (ILP variable sharing across identical layers) "
-                                      "is not implemented yet")
+            from .graphs.clustering import cluster_nodes
+
+            t0 = time.perf_counter()
+            self.node_representative = cluster_nodes(self.graph, self.strats)
+            self.timings["cluster_s"] = time.perf_counter() - t0
         self.ds, self.num_inp_out, self.num_args = self.build_ds()
         self.validate()
-        self.prob = BinaryProgram(self.encoded.tables.n_entries, "AutoParallel")
+        self.cluster_links = ClusterLinks(self)
+        self.create_cluster_links()
+        self.prob = BinaryProgram(self.n_variables, "AutoParallel")
         self.res = None
         self.add_default_constraints()
 
@@ -242,6 +284,29 @@ class ShardingOptimizer:
         self._write_back_redistribute_cost()
         self.timings["write_back_s"] = time.perf_counter() - t0
         return CostRecords(self), self.encoded.num_inp_out, self.encoded.num_args
+
+    def create_cluster_links(self):
+        """Entries of a linked node share the ILP variables of its representative's entries
+        (same argument, same strategy pair)."""
+        tb = self.encoded.tables
+        ident = np.arange(tb.n_entries, dtype=np.int64)
+        self._identity_vars = ident
+        var = ident.copy()
+        for node, rep in self.node_representative.items():
+            s1, s0 = self.node_map[node], self.node_map[rep]
+            assert self.num_args[s1] == self.num_args[s0], f"clustering linked {node} and {rep} with different arity"
+            for argi in range(self.num_args[s1]):
+                b1, nt1, ns1 = self._edge(s1, argi)
+                b0, nt0, ns0 = self._edge(s0, argi)
+                assert (nt1, ns1) == (nt0, ns0), (
+                    f"Problem with graph clustering: {rep} and {node} don't have the same number of input/output "
+                    "placements. Please report a bug")
+                var[b1:b1 + nt1 * ns1] = np.arange(b0, b0 + nt0 * ns0)
+        # compact variable ids: one per distinct representative entry
+        uniq, inverse = np.unique(var, return_inverse=True)
+        self.var_of_entry = inverse.astype(np.int64)
+        self.n_variables = len(uniq)
+        self._linked_entry = var != ident
 
     def _write_back_redistribute_cost(self):
         tb = self.encoded.tables

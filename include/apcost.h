@@ -50,8 +50,8 @@ extern "C" {
 #define APC_MAX_RANK 8
 #define APC_MAX_MESH 4
 #define APC_MAX_DTYPES 8
-#define APC_TILE_MAX_COLS 128 /* producer specs staged in LDS per tile */
-#define APC_TILE_MAX_ROWS 128 /* consumer specs staged in LDS per tile */
+#define APC_TILE_MAX_COLS 64 /* producer specs staged in LDS per tile */
+#define APC_TILE_MAX_ROWS 64 /* consumer specs staged in LDS per tile */
 
 #define APC_EDGE_GRAD_RESCALE 1 /* consumer is a parameter-gradient node (optimize_sharding.py:358-359) */
 #define APC_EDGE_NO_PRODUCER 2  /* placeholder / factory pseudo-argument (optimize_sharding.py:312-355) */
