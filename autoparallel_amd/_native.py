@@ -16,6 +16,7 @@ APC_MAX_MESH = 4
 APC_MAX_DTYPES = 8
 APC_TILE_MAX_COLS = 64
 APC_TILE_MAX_ROWS = 64
+APC_TILE_MAX_DUPS = 127
 
 EDGE_GRAD_RESCALE = 1
 EDGE_NO_PRODUCER = 2
@@ -41,13 +42,12 @@ class ApcParams(ctypes.Structure):
 
 class ApcTile(ctypes.Structure):
     _fields_ = [
-        ("edge", ctypes.c_int32),
-        ("row_begin", ctypes.c_int32), ("row_count", ctypes.c_int32),
-        ("col_begin", ctypes.c_int32), ("col_count", ctypes.c_int32),
+        ("edge", ctypes.c_int32), ("row_begin", ctypes.c_int32), ("col_begin", ctypes.c_int32),
+        ("counts", ctypes.c_int32),
         ("src_begin", ctypes.c_int32), ("n_src", ctypes.c_int32), ("tgt_begin", ctypes.c_int32),
-        ("flags", ctypes.c_int32), ("strat_begin", ctypes.c_int32),
+        ("flags", ctypes.c_int32), ("strat_begin", ctypes.c_int32), ("tensor", ctypes.c_int32),
         ("entry_begin", ctypes.c_int64), ("pt_begin", ctypes.c_int64),
-        ("tensor", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("dup_begin", ctypes.c_int32), ("dup_count", ctypes.c_int32),
     ]
 
 

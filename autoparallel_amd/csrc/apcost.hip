@@ -304,6 +304,7 @@ struct TableArgs {
   const double *pt_values;
   const double *per_arg;
   const apc_tile *tiles;
+  const int64_t *dup_entry_begin;
   double *comm_out;
   uint8_t *trans_out;
   double *cost_out;
@@ -341,10 +342,11 @@ constexpr int kLdsTermArrays = 6;  // zeros, all-gather, reduce-scatter, all-red
 template <int M, int kTileThreads, bool CONT, bool RESCALE>
 __device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const TableArgs &a, const apc_tile &tile,
                                                      const double *s_terms, const uint32_t *s_col,
-                                                     const uint2 *s_row, const double *s_cpa, int t0) {
+                                                     const uint2 *s_row, const double *s_cpa, const int64_t *s_dup,
+                                                     int t0) {
   constexpr int NS = States<M>::kCount;
   constexpr int CW = 2 + M;
-  const int rows = tile.row_count, cols = tile.col_count;
+  const int rows = tile.counts & 0xFFFF, cols = tile.counts >> 16;
   const int tid = threadIdx.x;
   const int n = rows * cols;
   int r = tid / cols, c = tid - r * cols;
@@ -421,9 +423,16 @@ __device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const 
     if (APC_EXP_NO_COMPUTE <= 2) a.cost_out[o] = cpa;
     if (APC_EXP_NO_COMPUTE <= 1) a.trans_out[o] = (uint8_t)idx;
 #else
+    const double total = comm + cpa + (double)trans;  // :368-372
     if (a.comm_out) a.comm_out[o] = comm;
     if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
-    if (a.cost_out) a.cost_out[o] = comm + cpa + (double)trans;  // :368-372
+    if (a.cost_out) a.cost_out[o] = total;
+    for (int d = 0; d < tile.dup_count; ++d) {  // identical edges receive the same values
+      const int64_t od = o + s_dup[d];
+      if (a.comm_out) a.comm_out[od] = comm;
+      if (a.trans_out) a.trans_out[od] = (uint8_t)trans;
+      if (a.cost_out) a.cost_out[od] = total;
+    }
 #endif
     c += dc;
     r += dr;
@@ -444,10 +453,11 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
   __shared__ uint32_t s_col[APC_TILE_MAX_COLS * CW];
   __shared__ uint2 s_row[APC_TILE_MAX_ROWS];  // x = codes, y = info
   __shared__ double s_cpa[APC_TILE_MAX_ROWS];
+  __shared__ int64_t s_dup[APC_TILE_MAX_DUPS];  // entry offsets of identical edges, relative to this edge
   __shared__ int s_uniform;
 
   const apc_tile tile = a.tiles[blockIdx.x];
-  const int rows = tile.row_count, cols = tile.col_count;
+  const int rows = tile.counts & 0xFFFF, cols = tile.counts >> 16;
   const int row0 = tile.row_begin, col0 = tile.col_begin;
   const int n_src = tile.n_src;
   const int flags = tile.flags;
@@ -475,6 +485,8 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
     }
   }
   const bool tile_cont = terms_wanted ? a.tensor_contiguous[t0] != 0 : true;
+  for (int j = tid; j < tile.dup_count; j += kTileThreads)
+    s_dup[j] = a.dup_entry_begin[tile.dup_begin + j] - tile.entry_begin;
   for (int j = tid; j < cols; j += kTileThreads) {
     const int sp = tile.src_begin + col0 + j;
     const int t = a.spec_tensor[sp];
@@ -519,11 +531,11 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
   if (uniform) {
     const bool rescale = (flags & APC_EDGE_GRAD_RESCALE) != 0;
     if (tile_cont) {
-      if (rescale) uniform_tile_entries<M, kTileThreads, true, true>(p, a, tile, s_terms, s_col, s_row, s_cpa, t0);
-      else uniform_tile_entries<M, kTileThreads, true, false>(p, a, tile, s_terms, s_col, s_row, s_cpa, t0);
+      if (rescale) uniform_tile_entries<M, kTileThreads, true, true>(p, a, tile, s_terms, s_col, s_row, s_cpa, s_dup, t0);
+      else uniform_tile_entries<M, kTileThreads, true, false>(p, a, tile, s_terms, s_col, s_row, s_cpa, s_dup, t0);
     } else {
-      if (rescale) uniform_tile_entries<M, kTileThreads, false, true>(p, a, tile, s_terms, s_col, s_row, s_cpa, t0);
-      else uniform_tile_entries<M, kTileThreads, false, false>(p, a, tile, s_terms, s_col, s_row, s_cpa, t0);
+      if (rescale) uniform_tile_entries<M, kTileThreads, false, true>(p, a, tile, s_terms, s_col, s_row, s_cpa, s_dup, t0);
+      else uniform_tile_entries<M, kTileThreads, false, false>(p, a, tile, s_terms, s_col, s_row, s_cpa, s_dup, t0);
     }
     return;
   }
@@ -549,9 +561,16 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
     }
     if (flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;
     const int64_t o = tile.entry_begin + local;
+    const double total = comm + s_cpa[r] + (double)trans;
     if (a.comm_out) a.comm_out[o] = comm;
     if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
-    if (a.cost_out) a.cost_out[o] = comm + s_cpa[r] + (double)trans;
+    if (a.cost_out) a.cost_out[o] = total;
+    for (int d = 0; d < tile.dup_count; ++d) {
+      const int64_t od = o + s_dup[d];
+      if (a.comm_out) a.comm_out[od] = comm;
+      if (a.trans_out) a.trans_out[od] = (uint8_t)trans;
+      if (a.cost_out) a.cost_out[od] = total;
+    }
     c += dc;
     r += dr;
     if (c >= cols) {
@@ -633,7 +652,8 @@ int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const 
                              const int32_t *edge_tgt_begin, const int32_t *edge_n_tgt,
                              const int32_t *edge_flags, const int64_t *edge_pt_begin,
                              const int64_t *edge_entry_begin, const int32_t *edge_strat_begin, int64_t n_pt,
-                             int64_t n_strategies, int64_t n_tiles, const apc_tile *tiles) {
+                             int64_t n_strategies, int64_t n_tiles, const apc_tile *tiles, int64_t n_dups,
+                             const int64_t *dup_entry_begin) {
   if (int rc = check_params(params)) return rc;
   const int M = params->mesh_ndim;
   for (int64_t t = 0; t < n_tensors; ++t)
@@ -686,21 +706,40 @@ int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const 
   for (int64_t t = 0; t < n_tiles; ++t) {
     const apc_tile &tl = tiles[t];
     const int e = tl.edge;
+    const int row_count = tl.counts & 0xFFFF, col_count = tl.counts >> 16;
     if (e < 0 || e >= n_edges) return fail(-2, "tile %lld: edge %d out of range", (long long)t, e);
-    if (tl.row_count < 1 || tl.row_count > APC_TILE_MAX_ROWS || tl.row_begin < 0 ||
-        tl.row_begin + tl.row_count > edge_n_tgt[e])
+    if (row_count < 1 || row_count > APC_TILE_MAX_ROWS || tl.row_begin < 0 ||
+        tl.row_begin + row_count > edge_n_tgt[e])
       return fail(-2, "tile %lld: rows [%d, +%d) outside edge %d (n_tgt %d, max %d per tile)", (long long)t,
-                  tl.row_begin, tl.row_count, e, edge_n_tgt[e], APC_TILE_MAX_ROWS);
-    if (tl.col_count < 1 || tl.col_count > APC_TILE_MAX_COLS || tl.col_begin < 0 ||
-        tl.col_begin + tl.col_count > edge_n_src[e])
+                  tl.row_begin, row_count, e, edge_n_tgt[e], APC_TILE_MAX_ROWS);
+    if (col_count < 1 || col_count > APC_TILE_MAX_COLS || tl.col_begin < 0 ||
+        tl.col_begin + col_count > edge_n_src[e])
       return fail(-2, "tile %lld: cols [%d, +%d) outside edge %d (n_src %d, max %d per tile)", (long long)t,
-                  tl.col_begin, tl.col_count, e, edge_n_src[e], APC_TILE_MAX_COLS);
+                  tl.col_begin, col_count, e, edge_n_src[e], APC_TILE_MAX_COLS);
     if (tl.src_begin != edge_src_begin[e] || tl.n_src != edge_n_src[e] || tl.tgt_begin != edge_tgt_begin[e] ||
         tl.flags != edge_flags[e] || tl.strat_begin != edge_strat_begin[e] ||
         tl.entry_begin != edge_entry_begin[e] || tl.pt_begin != edge_pt_begin[e])
       return fail(-2, "tile %lld: record does not repeat the fields of edge %d", (long long)t, e);
     if (tl.tensor != spec_tensor[edge_src_begin[e] + tl.col_begin])
       return fail(-2, "tile %lld: tensor %d is not the tensor of its first producer spec", (long long)t, tl.tensor);
+    if (tl.dup_count < 0 || tl.dup_count > APC_TILE_MAX_DUPS || tl.dup_begin < 0 ||
+        (int64_t)tl.dup_begin + tl.dup_count > n_dups)
+      return fail(-2, "tile %lld: duplicate list [%d, +%d) outside dup_entry_begin", (long long)t, tl.dup_begin,
+                  tl.dup_count);
+    for (int d = 0; d < tl.dup_count; ++d) {
+      // the offset must be the start of another edge with the same matrix shape
+      const int64_t off = dup_entry_begin[tl.dup_begin + d];
+      int64_t lo = 0, hi = n_edges;  // first edge whose entry_begin >= off, then skip empty edges
+      while (lo < hi) {
+        const int64_t mid = (lo + hi) / 2;
+        if (edge_entry_begin[mid] < off) lo = mid + 1; else hi = mid;
+      }
+      while (lo < n_edges && (int64_t)edge_n_src[lo] * edge_n_tgt[lo] == 0) ++lo;
+      if (lo >= n_edges || edge_entry_begin[lo] != off || lo == e || edge_n_src[lo] != edge_n_src[e] ||
+          edge_n_tgt[lo] != edge_n_tgt[e])
+        return fail(-2, "tile %lld: duplicate offset %lld is not the start of an edge shaped like edge %d",
+                    (long long)t, (long long)off, e);
+    }
   }
   return 0;
 }
@@ -752,8 +791,9 @@ int apc_compute_costs(const apc_params *params, int64_t n, const int64_t *flops,
 int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes, const uint8_t *tensor_contiguous,
                             const double *tensor_terms, const uint32_t *spec_codes, const int32_t *spec_tensor,
                             const double *pt_values,
-                            const double *per_arg, int64_t n_tiles, const apc_tile *tiles, int64_t n_entries,
-                            double *comm_out, uint8_t *trans_out, double *cost_out, void *stream) {
+                            const double *per_arg, int64_t n_tiles, const apc_tile *tiles,
+                            const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *trans_out,
+                            double *cost_out, void *stream) {
   if (int rc = check_params(params)) return rc;
   if (n_tiles < 0 || n_tiles > INT32_MAX) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tiles == 0) return 0;
@@ -761,13 +801,14 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
   if (!tensor_bytes || !tensor_contiguous || !tensor_terms || !spec_codes || !spec_tensor || !tiles)
     return fail(-1, "apc_redistribute_tables: NULL table");
   if (cost_out && !per_arg) return fail(-1, "cost_out needs compute_cost_per_arg");
-  TableArgs a{tensor_bytes, tensor_contiguous, tensor_terms, spec_codes, spec_tensor, pt_values,
-              per_arg,      tiles,             comm_out,     trans_out,  cost_out};
+  TableArgs a{tensor_bytes, tensor_contiguous, tensor_terms,    spec_codes, spec_tensor, pt_values,
+              per_arg,      tiles,             dup_entry_begin, comm_out,   trans_out,   cost_out};
   const dim3 grid((unsigned)n_tiles);
   hipStream_t s = (hipStream_t)stream;
   // small matrices (traced graphs): one wavefront per tile; large ones: two wavefronts share
   // the staged specs and terms of a tile
-  const bool wide = n_entries / n_tiles >= 512;
+  // (n_entries counts de-duplicated edges too: per computed tile the estimate is an upper bound)
+  const bool wide = n_entries / n_tiles >= 512 && n_tiles >= 4096;
 #define APC_LAUNCH(M_)                                                                                  \
   if (wide) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 128>), grid, dim3(128), 0, s, *params, a); \
   else hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 64>), grid, dim3(64), 0, s, *params, a)

@@ -9,6 +9,7 @@ built library) construction raises: there is no CPU path.
 from __future__ import annotations
 
 import ctypes
+import os
 
 import numpy as np
 import torch
@@ -22,7 +23,7 @@ _UPLOAD = (
     "tensor_rank", "tensor_itemsize", "tensor_shape", "tensor_stride", "spec_codes", "spec_tensor",
     "strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "strat_num_args",
     "edge_src_begin", "edge_n_src", "edge_tgt_begin", "edge_n_tgt", "edge_flags", "edge_pt_begin",
-    "edge_entry_begin", "edge_strat_begin", "pt_values", "tile_records",
+    "edge_entry_begin", "edge_strat_begin", "pt_values", "tile_records", "dup_entry_begin",
 )
 
 
@@ -78,6 +79,14 @@ class DeviceCostTables:
         self.comm = None
         self.transition = None
         self.cost = None
+
+    @_guarded
+    def refresh(self, *names):
+        """Re-uploads host tables that changed after construction (strategy inputs filled in
+        from the shard-shape table, tiles rebuilt with de-duplication)."""
+        with torch.cuda.device(self.device):
+            for k in names:
+                self.d[k] = _to_device(getattr(self.tables, k), self.device)
 
     # ---- helpers -------------------------------------------------------------------------
     def _stream(self):
@@ -161,7 +170,7 @@ class DeviceCostTables:
                 ctypes.byref(self.c_params), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
                 self._p(self.tensor_terms), self._p("spec_codes"), self._p("spec_tensor"), self._p("pt_values"),
                 self._p(self.compute_cost_per_arg), ctypes.c_int64(self.tables.n_tiles), self._p("tile_records"),
-                ctypes.c_int64(self.tables.n_entries), self._p(self.comm), self._p(self.transition),
+                self._p("dup_entry_begin"), ctypes.c_int64(self.tables.n_entries), self._p(self.comm), self._p(self.transition),
                 self._p(self.cost), self._stream())
         _native.check(rc, "apc_redistribute_tables")
 
@@ -191,7 +200,7 @@ class DeviceCostTables:
         self.run_tensor_tables()
         spec = self.run_spec_tables()
         self.run_compute_costs()
-        self.alloc_outputs(True, True, True)
+        self.alloc_outputs(True, os.environ.get('APC_EXP_NO_TRANS') is None, True)
         lib, P, cp = self.lib, self._p, ctypes.byref(self.c_params)
         stream = self._stream()
         tb = self.tables
@@ -209,7 +218,7 @@ class DeviceCostTables:
         a_tables = (cp, P(self.tensor_bytes), P(self.tensor_contiguous), P(self.tensor_terms), P("spec_codes"),
                     P("spec_tensor"),
                     P("pt_values"), P(self.compute_cost_per_arg), ctypes.c_int64(tb.n_tiles), P("tile_records"),
-                    ctypes.c_int64(tb.n_entries), P(self.comm), P(self.transition), P(self.cost), stream)
+                    P("dup_entry_begin"), ctypes.c_int64(tb.n_entries), P(self.comm), P(self.transition), P(self.cost), stream)
 
         def bind(fn, args, what):
             def launch():

@@ -35,7 +35,7 @@ from dataclasses import dataclass, fields
 import numpy as np
 
 from . import _native
-from ._native import APC_MAX_MESH, APC_MAX_RANK, APC_TILE_MAX_COLS, APC_TILE_MAX_ROWS
+from ._native import APC_MAX_MESH, APC_MAX_RANK, APC_TILE_MAX_COLS, APC_TILE_MAX_DUPS, APC_TILE_MAX_ROWS
 
 REPLICATE = 0x00
 PARTIAL_SUM = 0x40
@@ -51,9 +51,9 @@ DEFAULT_TILE_ENTRIES = 2048
 
 # numpy mirror of the C struct apc_tile (64 bytes)
 TILE_DTYPE = np.dtype([
-    ("edge", "<i4"), ("row_begin", "<i4"), ("row_count", "<i4"), ("col_begin", "<i4"), ("col_count", "<i4"),
+    ("edge", "<i4"), ("row_begin", "<i4"), ("col_begin", "<i4"), ("counts", "<i4"),
     ("src_begin", "<i4"), ("n_src", "<i4"), ("tgt_begin", "<i4"), ("flags", "<i4"), ("strat_begin", "<i4"),
-    ("entry_begin", "<i8"), ("pt_begin", "<i8"), ("tensor", "<i4"), ("reserved", "<i4"),
+    ("tensor", "<i4"), ("entry_begin", "<i8"), ("pt_begin", "<i8"), ("dup_begin", "<i4"), ("dup_count", "<i4"),
 ])
 assert TILE_DTYPE.itemsize == 64
 
@@ -133,6 +133,10 @@ class CostTables:
     tile_col_begin: np.ndarray = None
     tile_col_count: np.ndarray = None
     tile_records: np.ndarray = None
+    edge_canonical: np.ndarray = None  # edge -> the identical edge that is tiled (itself unless de-duplicated)
+    dup_entry_begin: np.ndarray = None  # entry offsets of the duplicates, grouped by canonical edge
+    edge_dup_begin: np.ndarray = None
+    edge_dup_count: np.ndarray = None
 
     _DTYPES = {
         "tensor_rank": np.int32, "tensor_itemsize": np.int32, "tensor_shape": np.int64,
@@ -200,12 +204,64 @@ class CostTables:
         return per_entry * self.n_entries + int(per_edge.sum())
 
     # ---- tiles -------------------------------------------------------------------------
-    def build_tiles(self, tile_entries: int = DEFAULT_TILE_ENTRIES) -> None:
+    def edge_signatures(self) -> list:
+        """One digest per edge over everything its matrix depends on: both spec lists
+        (codes and tensor rows), flags, the consumer strategies' compute-cost inputs and
+        the pass-through values.  Equal digests = bit-identical comm / transition / cost."""
+        import hashlib
+
+        sb, ns = self.edge_src_begin.astype(np.int64), self.edge_n_src.astype(np.int64)
+        tb, nt = self.edge_tgt_begin.astype(np.int64), self.edge_n_tgt.astype(np.int64)
+        st = self.edge_strat_begin.astype(np.int64)
+        codes, tensor = self.spec_codes, self.spec_tensor
+        strat = np.rec.fromarrays([self.strat_flops, self.strat_rw_bytes, self.strat_dtype, self.strat_zero_cost,
+                                   self.strat_num_args])
+        out = []
+        for e in range(self.n_edges):
+            h = hashlib.blake2b(digest_size=16)
+            h.update(np.array([ns[e], nt[e], self.edge_flags[e]], np.int64).tobytes())
+            h.update(codes[sb[e]:sb[e] + ns[e]].tobytes())
+            h.update(tensor[sb[e]:sb[e] + ns[e]].tobytes())
+            h.update(codes[tb[e]:tb[e] + nt[e]].tobytes())
+            h.update(tensor[tb[e]:tb[e] + nt[e]].tobytes())
+            h.update(strat[st[e]:st[e] + nt[e]].tobytes())
+            if self.edge_pt_begin[e] >= 0:
+                b = int(self.edge_pt_begin[e])
+                h.update(self.pt_values[b:b + int(ns[e] * nt[e])].tobytes())
+            out.append(h.digest())
+        return out
+
+    def build_tiles(self, tile_entries: int = DEFAULT_TILE_ENTRIES, dedupe: bool = False,
+                    max_copies: int = 8) -> None:
         """Cuts every edge matrix into rectangles of about ``tile_entries`` entries:
-        whole rows when a row fits the LDS column budget, column chunks otherwise."""
+        whole rows when a row fits the LDS column budget, column chunks otherwise.  With
+        ``dedupe`` only the first of every group of identical edges is tiled; its tiles
+        store their values to all copies.  (Call it after the strategy table is final:
+        the compute-cost inputs are part of an edge's identity.)  One tiled edge serves at
+        most ``max_copies - 1`` duplicates, so a long run of identical edges still spreads
+        over many workgroups."""
         ns = self.edge_n_src.astype(np.int64)
         nt = self.edge_n_tgt.astype(np.int64)
-        live = (ns > 0) & (nt > 0)
+        canonical = np.arange(self.n_edges, dtype=np.int64)
+        if dedupe and self.n_edges:
+            first: dict = {}  # signature -> [canonical edge, copies it already serves]
+            for e, sig in enumerate(self.edge_signatures()):
+                slot = first.get(sig)
+                if slot is None or slot[1] >= min(APC_TILE_MAX_DUPS, max(int(max_copies) - 1, 0)):
+                    first[sig] = [e, 0]  # a new canonical edge (also when the previous one is full)
+                else:
+                    canonical[e] = slot[0]
+                    slot[1] += 1
+        self.edge_canonical = canonical
+        is_dup = canonical != np.arange(self.n_edges)
+        # duplicates grouped by canonical edge (stable: in edge order)
+        dup_edges = np.nonzero(is_dup)[0]
+        order = np.argsort(canonical[dup_edges], kind="stable")
+        dup_edges = dup_edges[order]
+        self.dup_entry_begin = _i64(self.edge_entry_begin[:-1][dup_edges]) if self.n_edges else _i64([])
+        self.edge_dup_count = np.bincount(canonical[dup_edges], minlength=self.n_edges).astype(np.int64)
+        self.edge_dup_begin = np.cumsum(self.edge_dup_count) - self.edge_dup_count
+        live = (ns > 0) & (nt > 0) & ~is_dup
         ns1 = np.maximum(ns, 1)
         nt1 = np.maximum(nt, 1)
         ncc = -(-ns1 // APC_TILE_MAX_COLS)  # column chunks per edge
@@ -216,8 +272,8 @@ class CostTables:
         per_edge = np.where(live, ncc * nrt, 0)
         total = int(per_edge.sum())
         te = np.repeat(np.arange(self.n_edges, dtype=np.int64), per_edge)
-        first = np.cumsum(per_edge) - per_edge
-        k = np.arange(total, dtype=np.int64) - np.repeat(first, per_edge)
+        first_tile = np.cumsum(per_edge) - per_edge
+        k = np.arange(total, dtype=np.int64) - np.repeat(first_tile, per_edge)
         ci = k % ncc[te]
         ri = k // ncc[te]
         col_begin = ci * cw[te]
@@ -233,20 +289,30 @@ class CostTables:
         """The tile rectangles plus the fields of their edge, as the packed records the
         table kernel reads (C struct ``apc_tile``)."""
         te = self.tile_edge.astype(np.int64)
+        if self.edge_canonical is None or len(self.edge_canonical) != self.n_edges:
+            self.edge_canonical = np.arange(self.n_edges, dtype=np.int64)
+            self.dup_entry_begin = _i64([])
+            self.edge_dup_count = np.zeros(self.n_edges, np.int64)
+            self.edge_dup_begin = np.zeros(self.n_edges, np.int64)
         rec = np.zeros(len(te), TILE_DTYPE)
+        inside = (te >= 0) & (te < self.n_edges)
+        tc = np.where(inside, te, 0)  # (out-of-range tiles are reported by validate())
         rec["edge"] = self.tile_edge
-        rec["row_begin"], rec["row_count"] = self.tile_row_begin, self.tile_row_count
-        rec["col_begin"], rec["col_count"] = self.tile_col_begin, self.tile_col_count
-        rec["src_begin"] = self.edge_src_begin[te]
-        rec["n_src"] = self.edge_n_src[te]
-        rec["tgt_begin"] = self.edge_tgt_begin[te]
-        rec["flags"] = self.edge_flags[te]
-        rec["strat_begin"] = self.edge_strat_begin[te]
-        rec["entry_begin"] = self.edge_entry_begin[:-1][te] if len(te) else 0
-        rec["pt_begin"] = self.edge_pt_begin[te]
-        if len(te) and self.n_specs:
+        rec["row_begin"], rec["col_begin"] = self.tile_row_begin, self.tile_col_begin
+        rec["counts"] = (self.tile_row_count.astype(np.int64) & 0xFFFF) | ((self.tile_col_count.astype(np.int64) & 0x7FFF) << 16)
+        if len(te) and self.n_edges:
+            rec["src_begin"] = self.edge_src_begin[tc]
+            rec["n_src"] = self.edge_n_src[tc]
+            rec["tgt_begin"] = self.edge_tgt_begin[tc]
+            rec["flags"] = self.edge_flags[tc]
+            rec["strat_begin"] = self.edge_strat_begin[tc]
+            rec["entry_begin"] = self.edge_entry_begin[:-1][tc]
+            rec["pt_begin"] = self.edge_pt_begin[tc]
+            rec["dup_begin"] = self.edge_dup_begin[tc]
+            rec["dup_count"] = self.edge_dup_count[tc]
+        if len(te) and self.n_specs and self.n_edges:
             # (indices are clipped here; validate() reports ranges that fall outside the table)
-            first = np.clip(self.edge_src_begin[te].astype(np.int64) + self.tile_col_begin, 0, self.n_specs - 1)
+            first = np.clip(self.edge_src_begin[tc].astype(np.int64) + self.tile_col_begin, 0, self.n_specs - 1)
             rec["tensor"] = self.spec_tensor[first]
         self.tile_records = rec
 
@@ -284,8 +350,19 @@ class CostTables:
             ctypes.c_int64(self.n_edges), p(self.edge_src_begin), p(self.edge_n_src), p(self.edge_tgt_begin),
             p(self.edge_n_tgt), p(self.edge_flags), p(self.edge_pt_begin), p(self.edge_entry_begin),
             p(self.edge_strat_begin), ctypes.c_int64(len(self.pt_values)), ctypes.c_int64(self.n_strategies),
-            ctypes.c_int64(self.n_tiles), p(self.tile_records))
+            ctypes.c_int64(self.n_tiles), p(self.tile_records), ctypes.c_int64(len(self.dup_entry_begin)),
+            p(self.dup_entry_begin))
         _native.check(rc, "apc_validate_tables_host")
+        # every edge is either tiled completely or a duplicate of an edge that is
+        area = np.zeros(self.n_edges, np.int64)
+        np.add.at(area, self.tile_edge.astype(np.int64),
+                  self.tile_row_count.astype(np.int64) * self.tile_col_count.astype(np.int64))
+        want = self.edge_n_src.astype(np.int64) * self.edge_n_tgt.astype(np.int64)
+        tiled = self.edge_canonical == np.arange(self.n_edges)
+        if not np.array_equal(area[tiled], want[tiled]) or area[~tiled].any():
+            raise RuntimeError("tiles do not cover every (non-duplicate) edge matrix exactly once")
+        if int(self.edge_dup_count.sum()) != int((~tiled).sum()) or len(self.dup_entry_begin) != int((~tiled).sum()):
+            raise RuntimeError("duplicate-edge lists do not account for every de-duplicated edge")
         # byte counts must convert to fp64 exactly (the kernels divide them as doubles)
         if self.n_tensors:
             r = np.arange(APC_MAX_RANK)[None, :] < self.tensor_rank[:, None]

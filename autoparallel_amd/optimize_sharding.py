@@ -61,12 +61,11 @@ class DeviceBackend:
             return out["local_shape"].cpu().numpy(), out["local_stride"].cpu().numpy()
 
     def upload_strategy_inputs(self, tables):
-        from .device_tables import _real_tensors
-
-        d = self.dev
-        with _real_tensors():
-            for k in ("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost"):
-                d.d[k].copy_(torch.from_numpy(getattr(tables, k)))
+        """The strategy table is final: tile the edges (identical edges once) and send both."""
+        tables.build_tiles(dedupe=True)
+        tables.validate(self.dev.params)
+        self.dev.refresh("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "tile_records",
+                         "dup_entry_begin")
 
     def build(self):
         from .device_tables import _real_tensors

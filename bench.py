@@ -40,6 +40,8 @@ def parse_args():
     ap.add_argument("--tile-entries", type=int, default=None)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU-baseline sample duration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-dedupe", action="store_true", help="tile every edge even if an identical one exists")
+    ap.add_argument("--max-copies", type=int, default=4, help="identical edges served by one tiled edge")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy three times (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -153,8 +155,14 @@ def main():
             torch.cuda.synchronize()
             local_shape, local_stride = spec["local_shape"].cpu().numpy(), spec["local_stride"].cpu().numpy()
         finish(local_shape, local_stride)
-        for k in ("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost"):
-            dev.d[k].copy_(torch.from_numpy(getattr(tables, k)))
+        t1 = time.perf_counter()
+        if not args.no_dedupe:
+            # identical edges (repeated layers) are tiled once per group of --max-copies
+            tables.build_tiles(args.tile_entries or 2048, dedupe=True, max_copies=args.max_copies)
+            tables.validate(params)
+        host_timings["dedupe_tiles_s"] = time.perf_counter() - t1
+        dev.refresh("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "tile_records",
+                    "dup_entry_begin")
     step = dev.prepare_step(row_min=True)
     torch.cuda.synchronize()
     host_timings["upload_and_prepare_s"] = time.perf_counter() - t0
@@ -195,7 +203,7 @@ def main():
 
     # copy-back of the results, for the PCIe-inclusive figure
     t0 = time.perf_counter()
-    host_out = [dev.comm.cpu(), dev.transition.cpu(), dev.cost.cpu()]
+    host_out = [x.cpu() for x in (dev.comm, dev.transition, dev.cost) if x is not None]
     copy_back_s = time.perf_counter() - t0
     del host_out
 
@@ -218,7 +226,8 @@ def main():
         "dtype": "f64",
         "data": "synthetic",
         "config": {**desc, "edges": tables.n_edges, "strategies": tables.n_strategies, "specs": tables.n_specs,
-                   "entries": E, "tiles": tables.n_tiles, "device_row": params.device_name,
+                   "entries": E, "tiles": tables.n_tiles,
+                   "edges_deduplicated": int((tables.edge_canonical != np.arange(tables.n_edges)).sum()), "device_row": params.device_name,
                    "devices_per_host": 8, "step": "tensor_tables + spec_tables + compute_costs + "
                                                    "redistribute_tables(comm, transition, cost) + segmented_min(rows)"},
         "roofline": {"bound": "hbm", "kernel": "redistribute_tiles_kernel", "achieved": achieved,

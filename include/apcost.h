@@ -52,26 +52,33 @@ extern "C" {
 #define APC_MAX_DTYPES 8
 #define APC_TILE_MAX_COLS 64 /* producer specs staged in LDS per tile */
 #define APC_TILE_MAX_ROWS 64 /* consumer specs staged in LDS per tile */
+#define APC_TILE_MAX_DUPS 127 /* identical edges served by one tile (offsets staged in LDS) */
 
 #define APC_EDGE_GRAD_RESCALE 1 /* consumer is a parameter-gradient node (optimize_sharding.py:358-359) */
 #define APC_EDGE_NO_PRODUCER 2  /* placeholder / factory pseudo-argument (optimize_sharding.py:312-355) */
 
 /* One tile: a rows x cols rectangle of one edge's matrix, handled by one workgroup.
  * The record repeats the fields of its edge so that the kernel reaches everything it
- * needs with one load; apc_validate_tables_host checks it against the edge arrays. */
+ * needs with one load; apc_validate_tables_host checks it against the edge arrays.
+ * Edges whose matrices are provably identical (same spec lists, tensor, flags, consumer
+ * compute costs: the layers of a transformer) may be tiled once: the tile then lists the
+ * entry offsets of the other copies (dup_entry_begin[dup_begin .. dup_begin + dup_count))
+ * and every value is stored to all of them. */
 typedef struct apc_tile {
   int32_t edge;
-  int32_t row_begin, row_count; /* consumer strategies */
-  int32_t col_begin, col_count; /* producer strategies */
-  int32_t src_begin;            /* = edge_src_begin[edge] */
-  int32_t n_src;                /* = edge_n_src[edge] */
-  int32_t tgt_begin;            /* = edge_tgt_begin[edge] */
-  int32_t flags;                /* = edge_flags[edge] */
-  int32_t strat_begin;          /* = edge_strat_begin[edge] */
-  int64_t entry_begin;          /* = edge_entry_begin[edge] */
-  int64_t pt_begin;             /* = edge_pt_begin[edge] */
-  int32_t tensor;               /* = spec_tensor[src_begin + col_begin] */
-  int32_t reserved;
+  int32_t row_begin;   /* first consumer strategy */
+  int32_t col_begin;   /* first producer strategy */
+  int32_t counts;      /* row_count | col_count << 16 */
+  int32_t src_begin;   /* = edge_src_begin[edge] */
+  int32_t n_src;       /* = edge_n_src[edge] */
+  int32_t tgt_begin;   /* = edge_tgt_begin[edge] */
+  int32_t flags;       /* = edge_flags[edge] */
+  int32_t strat_begin; /* = edge_strat_begin[edge] */
+  int32_t tensor;      /* = spec_tensor[src_begin + col_begin] */
+  int64_t entry_begin; /* = edge_entry_begin[edge] */
+  int64_t pt_begin;    /* = edge_pt_begin[edge] */
+  int32_t dup_begin;   /* first row of dup_entry_begin for this tile's edge */
+  int32_t dup_count;   /* number of identical edges that receive the same values */
 } apc_tile;
 
 /* Cost-model parameters: everything the reference reads from its environment
@@ -99,14 +106,16 @@ const char *apc_last_error(void);
  * reference's assertions in ShardingOptimizer.validate
  * (optimize_sharding.py:908-958) for the flattened form: monotone entry
  * offsets, spec/tensor/strategy indices in range, rank <= APC_MAX_RANK, shard
- * dims < rank, tiles inside their edge and within the LDS staging limits. */
+ * dims < rank, tiles inside their edge and within the LDS staging limits, duplicate
+ * offsets naming edges of the same shape. */
 int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank_host,
                              int64_t n_specs, const uint32_t *spec_codes_host, const int32_t *spec_tensor_host,
                              int64_t n_edges, const int32_t *edge_src_begin_host, const int32_t *edge_n_src_host,
                              const int32_t *edge_tgt_begin_host, const int32_t *edge_n_tgt_host,
                              const int32_t *edge_flags_host, const int64_t *edge_pt_begin_host,
                              const int64_t *edge_entry_begin_host, const int32_t *edge_strat_begin_host,
-                             int64_t n_pt, int64_t n_strategies, int64_t n_tiles, const apc_tile *tiles_host);
+                             int64_t n_pt, int64_t n_strategies, int64_t n_tiles, const apc_tile *tiles_host,
+                             int64_t n_dups, const int64_t *dup_entry_begin_host);
 
 /* Number of doubles per tensor in the tensor_terms table for a mesh of this ndim
  * (4 term arrays x the number of running-bytes states); 0 for an unsupported ndim. */
@@ -157,8 +166,8 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
                             const uint8_t *tensor_contiguous, const double *tensor_terms,
                             const uint32_t *spec_codes, const int32_t *spec_tensor, const double *pt_values,
                             const double *compute_cost_per_arg, int64_t n_tiles, const apc_tile *tiles,
-                            int64_t n_entries, double *comm_out, uint8_t *transition_out, double *cost_out,
-                            void *stream);
+                            const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out,
+                            uint8_t *transition_out, double *cost_out, void *stream);
 
 /* Segmented minimum with first-argmin (relative to the segment start); empty
  * segments give (+inf, -1).  No counterpart in the reference (which hands the full

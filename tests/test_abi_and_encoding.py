@@ -71,6 +71,63 @@ def test_tiles_cover_every_entry_exactly_once(tile_entries):
     assert (seen == 1).all()
 
 
+def twin_graph(tb: CostTables) -> CostTables:
+    """A copy of every node, spec and edge appended to the tables (tensors shared): every
+    edge then has an identical twin, like the layers of a transformer."""
+    S, NS, NP = tb.n_strategies, tb.n_specs, len(tb.pt_values)
+    cat = np.concatenate
+    eb = tb.edge_entry_begin
+    return CostTables(
+        mesh_sizes=tb.mesh_sizes, tensor_rank=tb.tensor_rank, tensor_itemsize=tb.tensor_itemsize,
+        tensor_shape=tb.tensor_shape, tensor_stride=tb.tensor_stride,
+        spec_codes=cat([tb.spec_codes, tb.spec_codes]), spec_tensor=cat([tb.spec_tensor, tb.spec_tensor]),
+        strat_flops=cat([tb.strat_flops] * 2), strat_rw_bytes=cat([tb.strat_rw_bytes] * 2),
+        strat_dtype=cat([tb.strat_dtype] * 2), strat_zero_cost=cat([tb.strat_zero_cost] * 2),
+        strat_num_args=cat([tb.strat_num_args] * 2),
+        node_strat_begin=cat([tb.node_strat_begin, tb.node_strat_begin[1:] + S]),
+        edge_node=cat([tb.edge_node, tb.edge_node + tb.n_nodes]), edge_arg=cat([tb.edge_arg] * 2),
+        edge_src_begin=cat([tb.edge_src_begin, tb.edge_src_begin + NS]), edge_n_src=cat([tb.edge_n_src] * 2),
+        edge_tgt_begin=cat([tb.edge_tgt_begin, tb.edge_tgt_begin + NS]), edge_n_tgt=cat([tb.edge_n_tgt] * 2),
+        edge_flags=cat([tb.edge_flags] * 2),
+        edge_pt_begin=cat([tb.edge_pt_begin, np.where(tb.edge_pt_begin >= 0, tb.edge_pt_begin + NP, -1)]),
+        edge_entry_begin=cat([eb, eb[1:] + eb[-1]]), edge_strat_begin=cat([tb.edge_strat_begin, tb.edge_strat_begin + S]),
+        pt_values=cat([tb.pt_values] * 2))
+
+
+def test_deduplicated_tiles_write_every_entry_exactly_once():
+    base = stress_dag(seed=8, n_nodes=120, mesh_sizes=(4, 2), max_strategies=20)
+    tb = twin_graph(base)
+    tb.build_tiles(256, dedupe=True)
+    tb.validate(CostModelParams.from_mesh((4, 2)))
+    n_dup = int((tb.edge_canonical != np.arange(tb.n_edges)).sum())
+    assert n_dup >= base.n_edges  # every appended edge has its original as twin
+    seen = np.zeros(tb.n_entries, np.int32)
+    rec = tb.tile_records
+    for t in range(tb.n_tiles):
+        e = int(rec["edge"][t])
+        ns = int(tb.edge_n_src[e])
+        rc, cc = int(rec["counts"][t]) & 0xFFFF, int(rec["counts"][t]) >> 16
+        local = (np.arange(rec["row_begin"][t], rec["row_begin"][t] + rc)[:, None] * ns
+                 + np.arange(rec["col_begin"][t], rec["col_begin"][t] + cc)[None, :]).ravel()
+        seen[int(tb.edge_entry_begin[e]) + local] += 1
+        for d in range(int(rec["dup_count"][t])):
+            seen[int(tb.dup_entry_begin[int(rec["dup_begin"][t]) + d]) + local] += 1
+    assert (seen == 1).all()
+    # edges that differ in anything their matrix depends on are not merged
+    other = twin_graph(base)
+    other.strat_flops[other.n_strategies // 2:] += 1
+    other.build_tiles(256, dedupe=True)
+    assert int((other.edge_canonical != np.arange(other.n_edges)).sum()) < n_dup
+
+
+def test_validator_rejects_bad_duplicate_offsets():
+    tb = twin_graph(stress_dag(seed=8, n_nodes=60, mesh_sizes=(4, 2), max_strategies=10))
+    tb.build_tiles(256, dedupe=True)
+    tb.dup_entry_begin[0] += 1
+    with pytest.raises(RuntimeError, match="duplicate offset"):
+        tb.validate(CostModelParams.from_mesh((4, 2)))
+
+
 def test_wide_edges_are_cut_into_column_chunks():
     # one consumer with 3 strategies reading a producer with 2500 strategies
     n_src, n_tgt = 2500, 3

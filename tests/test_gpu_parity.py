@@ -163,6 +163,18 @@ def test_wide_and_degenerate_edges(gpu_device):
     assert comm.numel() == 0 and trans.numel() == 0 and cost.numel() == 0
 
 
+def test_deduplicated_edges_receive_identical_values(gpu_device):
+    """Identical edges tiled once and stored to every copy: still bit-identical to the oracle,
+    which evaluates every edge on its own."""
+    from test_abi_and_encoding import twin_graph
+
+    for mesh in [(32, 8), (4, 4, 2)]:
+        tb = twin_graph(stress_dag(seed=21, n_nodes=600, mesh_sizes=mesh, frac_nonspec_nodes=0.02))
+        tb.build_tiles(512, dedupe=True)
+        assert int((tb.edge_canonical != np.arange(tb.n_edges)).sum()) >= tb.n_edges // 2
+        _run_and_compare(tb, mesh, 2.2, gpu_device)
+
+
 def test_tile_size_does_not_change_results(gpu_device):
     mesh = (16, 8, 4)
     base = None
