@@ -60,9 +60,9 @@ class DeviceBackend:
             out = self.dev.run_spec_tables()
             return out["local_shape"].cpu().numpy(), out["local_stride"].cpu().numpy()
 
-    def upload_strategy_inputs(self, tables):
+    def upload_strategy_inputs(self, tables, tile_entries=2048, dedupe=True, max_copies=4):
         """The strategy table is final: tile the edges (identical edges once) and send both."""
-        tables.build_tiles(dedupe=True)
+        tables.build_tiles(tile_entries, dedupe=dedupe, max_copies=max_copies)
         tables.validate(self.dev.params)
         self.dev.refresh("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "tile_records",
                          "dup_entry_begin")
@@ -204,6 +204,11 @@ class ShardingOptimizer:
     device = "cuda:0"
     backend_cls = DeviceBackend
     solver_time_limit: Optional[float] = None
+    # tiling of the edge matrices: entries per tile, whether identical edges (repeated layers)
+    # are evaluated once, and how many copies one evaluated edge may serve
+    tile_entries = 2048
+    dedupe = True
+    max_copies = 4
 
     def __init__(self, gm, mesh, rescale_grad_comm_cost_for_mp=1.0, repeated_subgraphs=False):
         self.gm = gm
@@ -266,7 +271,7 @@ class ShardingOptimizer:
         t0 = time.perf_counter()
         self.cost_input_stats = {}
         fill_flops_and_bytes(self.encoded, self.strats, local_shape, local_stride, self.cost_input_stats)
-        self.backend.upload_strategy_inputs(tb)
+        self.backend.upload_strategy_inputs(tb, self.tile_entries, self.dedupe, self.max_copies)
         self.timings["flops_bytes_s"] = time.perf_counter() - t0
         t0 = time.perf_counter()
         out = self.backend.build()

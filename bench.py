@@ -40,6 +40,8 @@ def parse_args():
     ap.add_argument("--tile-entries", type=int, default=None)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU-baseline sample duration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-solve", action="store_true", help="skip the ILP leg of the plan wall-time")
+    ap.add_argument("--no-clustering", action="store_true", help="one ILP variable per entry (no variable sharing)")
     ap.add_argument("--no-dedupe", action="store_true", help="tile every edge even if an identical one exists")
     ap.add_argument("--max-copies", type=int, default=4, help="identical edges served by one tiled edge")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -49,7 +51,7 @@ def parse_args():
 
 
 def build_workload(args):
-    """-> (tables, params, description dict, finish callback or None, host timings)"""
+    """-> (tables, params, description, device tables or None, planner or None, host timings)"""
     from autoparallel_amd import CostModelParams
 
     if args.workload == "stress":
@@ -61,22 +63,69 @@ def build_workload(args):
         timings = {"generate_s": time.perf_counter() - t0}
         desc = {"workload": f"synthetic stress DAG, seed 0, {args.stress_nodes} nodes, mesh {mesh}",
                 "mesh": list(mesh)}
-        return tables, CostModelParams.from_mesh(mesh, rescale=2.2), desc, None, timings
+        return tables, CostModelParams.from_mesh(mesh, rescale=2.2), desc, None, None, timings
+
+    # traced workloads go through the product path: capture -> ShardingOptimizer (which
+    # enumerates, clusters, encodes, builds the device tables and copies them back)
+    import dataclasses
+
+    import torch
+
+    from autoparallel_amd.api import AutoParallelPlanner
     from autoparallel_amd.graphs import workloads
+    from autoparallel_amd.graphs.llama3 import Llama, SingleBlock
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
 
-    encoded, strats, info = workloads.traced_tables(args.workload, n_layers=args.layers)
-    mesh = info["mesh_sizes"]
-    cfg = info["config"]
+    cfg, mesh_sizes, batch, seq = workloads.WORKLOADS[args.workload]
+    if args.layers is not None:
+        cfg = dataclasses.replace(cfg, n_layers=args.layers)
+    mesh = workloads.logical_mesh(mesh_sizes)
+    with torch.device("meta"):
+        model = SingleBlock(cfg) if args.workload == "block_1k" else Llama(cfg)
+    if args.workload == "block_1k":
+        def input_fn():
+            return torch.randn(batch, seq, cfg.dim, dtype=torch.bfloat16, requires_grad=True)
+    else:
+        def input_fn():
+            return torch.randint(0, cfg.vocab_size, (batch, seq))
+
+    class Optimizer(ShardingOptimizer):
+        tile_entries = args.tile_entries or 2048
+        dedupe = not args.no_dedupe
+        max_copies = args.max_copies
+
+    class Planner(AutoParallelPlanner):
+        optimizer_cls = Optimizer
+
+    planner = Planner(model, input_fn, mesh, param_dtype=torch.bfloat16, reduce_dtype=torch.float32,
+                      repeated_subgraphs=not args.no_clustering)
+    planner.__enter__()
+    opt = planner.sharding_optimizer
     desc = {"workload": f"{args.workload} joint fwd+bwd graph ({cfg.n_layers} layers, dim {cfg.dim}, "
-                        f"batch {info['batch']}, seq {info['seq']}, bf16 params / fp32 reduce), logical mesh {mesh}",
-            "mesh": list(mesh), "graph_nodes": len(encoded.nodes)}
+                        f"batch {batch}, seq {seq}, bf16 params / fp32 reduce), logical mesh {tuple(mesh_sizes)}",
+            "mesh": list(mesh_sizes), "graph_nodes": len(opt.nodes), "ilp_variables": opt.n_variables,
+            "clustered_nodes": len(opt.node_representative)}
+    return opt.encoded.tables, opt.params, desc, opt.backend.dev, planner, dict(planner.timings)
 
-    def finish(local_shape, local_stride):
-        workloads.finish_strategy_inputs(encoded, strats, local_shape, local_stride, info)
-        info["ctx"].__exit__(None, None, None)
 
-    # bf16 parameters reduced in fp32: rescale = 4 / 2 * 1.1
-    return encoded.tables, CostModelParams.from_mesh(mesh, rescale=2.2), desc, finish, info["timings"]
+def solve_plan(planner, args):
+    """The ILP leg of the plan (input / output constraints of the reference's Llama example:
+    examples/example_llama3.py:205-218)."""
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    t0 = time.perf_counter()
+    planner.add_parameter_memory_constraint(low=None, high=None)
+    nd = planner.mesh.ndim
+    x_sharding = (Shard(0),) + (Replicate(),) * (nd - 1)
+    out_sharding = (Shard(0), Shard(2)) if (nd == 2 and args.workload != "block_1k") else x_sharding
+    planner.add_input_constraints([x_sharding])
+    planner.add_output_constraints([out_sharding])
+    constraints_s = time.perf_counter() - t0
+    planner.optimize_placement()
+    opt = planner.sharding_optimizer
+    return {"constraints_s": constraints_s, "solve_s": planner.timings["solve_s"],
+            "objective": opt.objective_value(), "ilp_rows": getattr(opt.prob, "rows_after_dedupe", None),
+            "ilp_variables": opt.n_variables}
 
 
 def cpu_baseline(tables, params, target_seconds):
@@ -141,28 +190,18 @@ def main():
     from autoparallel_amd.device_tables import DeviceCostTables
 
     t_setup = time.perf_counter()
-    tables, params, desc, finish, host_timings = build_workload(args)
-    if args.tile_entries:
-        tables.build_tiles(args.tile_entries)
-    t0 = time.perf_counter()
-    dev = DeviceCostTables(tables, params, device="cuda:0")
-    if finish is not None:
-        from autoparallel_amd.device_tables import _real_tensors
+    tables, params, desc, dev, planner, host_timings = build_workload(args)
+    # a traced workload keeps its capture context (a fake-tensor mode) open until the plan is
+    # solved; the measurements below work on real device buffers
+    from autoparallel_amd.device_tables import _real_tensors
 
-        # the capture context keeps a fake-tensor mode active until finish() closes it
-        with _real_tensors():
-            spec = dev.run_spec_tables()
-            torch.cuda.synchronize()
-            local_shape, local_stride = spec["local_shape"].cpu().numpy(), spec["local_stride"].cpu().numpy()
-        finish(local_shape, local_stride)
-        t1 = time.perf_counter()
-        if not args.no_dedupe:
-            # identical edges (repeated layers) are tiled once per group of --max-copies
-            tables.build_tiles(args.tile_entries or 2048, dedupe=True, max_copies=args.max_copies)
-            tables.validate(params)
-        host_timings["dedupe_tiles_s"] = time.perf_counter() - t1
-        dev.refresh("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "tile_records",
-                    "dup_entry_begin")
+    guard = _real_tensors()
+    guard.__enter__()
+    t0 = time.perf_counter()
+    if dev is None:
+        if args.tile_entries:
+            tables.build_tiles(args.tile_entries)
+        dev = DeviceCostTables(tables, params, device="cuda:0")
     step = dev.prepare_step(row_min=True)
     torch.cuda.synchronize()
     host_timings["upload_and_prepare_s"] = time.perf_counter() - t0
@@ -243,6 +282,22 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(tables, params, args.cpu_seconds)
+    guard.__exit__(None, None, None)
+    if planner is not None:
+        plan = {"stages_s": {k: round(v, 4) for k, v in host_timings.items()}}
+        if not args.no_solve:
+            plan.update(solve_plan(planner, args))
+        table_stage = host_timings.get("optimizer_tables_s", 0.0)
+        other = host_timings.get("capture_s", 0.0) + host_timings.get("optimizer_s", 0.0) - table_stage \
+            + plan.get("constraints_s", 0.0) + plan.get("solve_s", 0.0)
+        plan["total_with_gpu_tables_s"] = other + table_stage
+        if "cpu_baseline" in result:
+            # the same plan with the tables built by the CPU port: only the table stage differs
+            cpu_tables = E / result["cpu_baseline"]["value"]
+            plan["cpu_table_stage_s"] = cpu_tables
+            plan["total_with_cpu_tables_s"] = other + cpu_tables
+        result["plan_wall_time"] = plan
+        planner.__exit__(None, None, None)
     print(json.dumps(result))
 
 

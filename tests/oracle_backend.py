@@ -19,7 +19,7 @@ class OracleBackend:
         _, lshape, lstride, _, _ = c_oracle.spec_tables(self.tables.as_dict(), self.tables.mesh_sizes)
         return lshape, lstride
 
-    def upload_strategy_inputs(self, tables):
+    def upload_strategy_inputs(self, tables, *args, **kwargs):
         pass
 
     def build(self):
