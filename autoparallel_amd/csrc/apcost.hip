@@ -16,6 +16,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "apcost.h"
@@ -204,51 +205,64 @@ __global__ __launch_bounds__(kBlock) void spec_tables_kernel(
     const int64_t *__restrict__ shape, const int64_t *__restrict__ stride, int64_t *__restrict__ shards,
     int64_t *__restrict__ lshape, int64_t *__restrict__ lstride, int64_t *__restrict__ lnumel,
     int64_t *__restrict__ lbytes) {
-  const int64_t s = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (s >= n) return;
+  // each thread derives one spec; the two [kBlock][8] result blocks are transposed through LDS
+  // so that the workgroup writes them as two contiguous 16 KB runs
+  __shared__ int64_t s_shape[kBlock * (APC_MAX_RANK + 1)];
+  __shared__ int64_t s_stride[kBlock * (APC_MAX_RANK + 1)];
+  const int64_t base = (int64_t)blockIdx.x * kBlock;
+  const int64_t s = base + threadIdx.x;
   int64_t sh[APC_MAX_RANK], st[APC_MAX_RANK];
 #pragma unroll
   for (int i = 0; i < APC_MAX_RANK; ++i) sh[i] = st[i] = 0;
-  const int t = tensor[s];
   int64_t nsh = 0, ne = 0, nb = 0;
-  if (t >= 0) {
-    const int r = rank[t];
+  if (s < n) {
+    const int t = tensor[s];
+    if (t >= 0) {
+      const int r = rank[t];
 #pragma unroll
-    for (int i = 0; i < APC_MAX_RANK; ++i) {
-      if (i < r) {
-        sh[i] = shape[(int64_t)t * APC_MAX_RANK + i];
-        st[i] = stride[(int64_t)t * APC_MAX_RANK + i];
-      }
-    }
-    nsh = 1;
-    const uint32_t pc = codes[s];
-    for (int i = 0; i < p.mesh_ndim; ++i) {
-      const uint32_t c = (pc >> (8 * i)) & 0xFF;
-      if (kind_of(c) == 2) {
-        const int d = dim_of(c);
-        const int64_t m = p.mesh_size[i];
-        nsh *= m;
-        // compile-time indices keep sh/st in registers
-#pragma unroll
-        for (int j = 0; j < APC_MAX_RANK; ++j) {
-          if (j == d) sh[j] = (sh[j] + m - 1) / m;
-          if (j == d - 1 && d - 1 > 0) st[j] = (st[j] + m - 1) / m;  // compute_estimation.py:225-228
+      for (int i = 0; i < APC_MAX_RANK; ++i) {
+        if (i < r) {
+          sh[i] = shape[(int64_t)t * APC_MAX_RANK + i];
+          st[i] = stride[(int64_t)t * APC_MAX_RANK + i];
         }
       }
-    }
-    ne = 1;
+      nsh = 1;
+      const uint32_t pc = codes[s];
+      for (int i = 0; i < p.mesh_ndim; ++i) {
+        const uint32_t c = (pc >> (8 * i)) & 0xFF;
+        if (kind_of(c) == 2) {
+          const int d = dim_of(c);
+          const int64_t m = p.mesh_size[i];
+          nsh *= m;
+          // compile-time indices keep sh/st in registers
 #pragma unroll
-    for (int i = 0; i < APC_MAX_RANK; ++i)
-      if (i < r) ne *= sh[i];
-    nb = ne * itemsize[t];
+          for (int j = 0; j < APC_MAX_RANK; ++j) {
+            if (j == d) sh[j] = (sh[j] + m - 1) / m;
+            if (j == d - 1 && d - 1 > 0) st[j] = (st[j] + m - 1) / m;  // compute_estimation.py:225-228
+          }
+        }
+      }
+      ne = 1;
+#pragma unroll
+      for (int i = 0; i < APC_MAX_RANK; ++i)
+        if (i < r) ne *= sh[i];
+      nb = ne * itemsize[t];
+    }
+    shards[s] = nsh;
+    lnumel[s] = ne;
+    lbytes[s] = nb;
   }
-  shards[s] = nsh;
-  lnumel[s] = ne;
-  lbytes[s] = nb;
 #pragma unroll
   for (int i = 0; i < APC_MAX_RANK; ++i) {
-    lshape[s * APC_MAX_RANK + i] = sh[i];
-    lstride[s * APC_MAX_RANK + i] = st[i];
+    s_shape[threadIdx.x * (APC_MAX_RANK + 1) + i] = sh[i];
+    s_stride[threadIdx.x * (APC_MAX_RANK + 1) + i] = st[i];
+  }
+  __syncthreads();
+  const int64_t live = (n - base < kBlock ? n - base : kBlock) * APC_MAX_RANK;
+  for (int k = threadIdx.x; k < live; k += kBlock) {
+    const int row = k / APC_MAX_RANK, col = k % APC_MAX_RANK;
+    lshape[base * APC_MAX_RANK + k] = s_shape[row * (APC_MAX_RANK + 1) + col];
+    lstride[base * APC_MAX_RANK + k] = s_stride[row * (APC_MAX_RANK + 1) + col];
   }
 }
 
@@ -829,12 +843,21 @@ int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_se
   if (!seg_ptr || !mins || !args || (!values && n_values > 0)) return fail(-1, "apc_segmented_min: NULL array");
   if (n_seg > (int64_t)INT32_MAX * 4) return fail(-1, "n_segments %lld too large", (long long)n_seg);
   hipStream_t s = (hipStream_t)stream;
+  // lanes per segment: about a quarter of the mean length, so most lanes of a group have work in every
+  // pass over their segment (APC_SEGMIN_GROUP overrides, for tuning)
   const double mean = (double)n_values / (double)n_seg;
-  if (mean <= 4) launch_segmented_min<4>(values, seg_ptr, n_seg, mins, args, s);
-  else if (mean <= 8) launch_segmented_min<8>(values, seg_ptr, n_seg, mins, args, s);
-  else if (mean <= 16) launch_segmented_min<16>(values, seg_ptr, n_seg, mins, args, s);
-  else if (mean <= 32) launch_segmented_min<32>(values, seg_ptr, n_seg, mins, args, s);
-  else launch_segmented_min<64>(values, seg_ptr, n_seg, mins, args, s);
+  int g = mean <= 16 ? 4 : mean <= 64 ? 8 : mean <= 256 ? 16 : mean <= 1024 ? 32 : 64;
+  if (const char *env = getenv("APC_SEGMIN_GROUP")) g = atoi(env);
+  switch (g) {
+    case 1: launch_segmented_min<1>(values, seg_ptr, n_seg, mins, args, s); break;
+    case 2: launch_segmented_min<2>(values, seg_ptr, n_seg, mins, args, s); break;
+    case 4: launch_segmented_min<4>(values, seg_ptr, n_seg, mins, args, s); break;
+    case 8: launch_segmented_min<8>(values, seg_ptr, n_seg, mins, args, s); break;
+    case 16: launch_segmented_min<16>(values, seg_ptr, n_seg, mins, args, s); break;
+    case 32: launch_segmented_min<32>(values, seg_ptr, n_seg, mins, args, s); break;
+    case 64: launch_segmented_min<64>(values, seg_ptr, n_seg, mins, args, s); break;
+    default: return fail(-1, "segment group width %d is not a power of two up to 64", g);
+  }
   return check_launch("apc_segmented_min");
 }
 
