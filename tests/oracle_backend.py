@@ -11,6 +11,7 @@ from oracle import cost_oracle as po
 class OracleBackend:
     def __init__(self, tables, params, device=None):
         self.tables = tables
+        self.product_params = params
         self.params = po.make_params(params.mesh_sizes, device_name=params.device_name, rescale=params.rescale)
         assert self.params.bw == params.bw and self.params.lat == params.lat
         self.timings = {}
@@ -19,8 +20,10 @@ class OracleBackend:
         _, lshape, lstride, _, _ = c_oracle.spec_tables(self.tables.as_dict(), self.tables.mesh_sizes)
         return lshape, lstride
 
-    def upload_strategy_inputs(self, tables, *args, **kwargs):
-        pass
+    def upload_strategy_inputs(self, tables, tile_entries=2048, dedupe=True, max_copies=4):
+        # host-side tiling / de-duplication runs as in the product (the oracle ignores the tiles)
+        tables.build_tiles(tile_entries, dedupe=dedupe, max_copies=max_copies)
+        tables.validate(self.product_params)
 
     def build(self):
         enc = self.tables.as_dict()
