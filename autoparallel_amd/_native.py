@@ -37,6 +37,12 @@ class ApcParams(ctypes.Structure):
         ("rescale", ctypes.c_double),
         ("gpu_flops", ctypes.c_double * APC_MAX_DTYPES),
         ("transition_scale", ctypes.c_int32),
+        ("inv_bw", ctypes.c_double * APC_MAX_MESH),
+        ("inv_mesh", ctypes.c_double * APC_MAX_MESH),
+        ("inv_hbm_bw", ctypes.c_double),
+        ("inv_rw_eff", ctypes.c_double),
+        ("shards", ctypes.c_double * (1 << APC_MAX_MESH)),
+        ("inv_shards", ctypes.c_double * (1 << APC_MAX_MESH)),
     ]
 
 
@@ -55,7 +61,6 @@ EXPORTS = (
     "apc_version",
     "apc_last_error",
     "apc_validate_tables_host",
-    "apc_tensor_terms_count",
     "apc_tensor_tables",
     "apc_spec_tables",
     "apc_compute_costs",
@@ -93,7 +98,6 @@ def lib() -> ctypes.CDLL:
         for name in EXPORTS:
             if name != "apc_last_error":
                 getattr(l, name).restype = ctypes.c_int
-        l.apc_tensor_terms_count.restype = ctypes.c_int64
         _lib = l
     return _lib
 

@@ -61,6 +61,31 @@ __device__ __forceinline__ double ring(double gb, const apc_params &p, int d, in
   return latency + bw * 1e6;
 }
 
+// a / b for a divisor whose correctly rounded reciprocal y = RN(1 / b) is known: one
+// multiply and two Newton corrections, each residual computed exactly by an FMA.  With y
+// correctly rounded the second correction returns the correctly rounded quotient (Markstein),
+// i.e. the same bits as the division instruction sequence, at a sixth of its cost.  The
+// reciprocals travel in apc_params and are checked against 1.0 / b on the host.
+__device__ __forceinline__ double div_by(double a, double b, double y) {
+  double q = a * y;
+  double r = __builtin_fma(-b, q, a);
+  q = __builtin_fma(r, y, q);
+  r = __builtin_fma(-b, q, a);
+  return __builtin_fma(r, y, q);
+}
+
+__device__ __forceinline__ double rw_time_r(double bytes, const apc_params &p) {
+  double t = div_by(bytes, p.hbm_bw, p.inv_hbm_bw) * 1e6;
+  t = div_by(t, p.rw_eff, p.inv_rw_eff);
+  return t > p.launch_floor ? t : p.launch_floor;
+}
+
+__device__ __forceinline__ double ring_r(double gb, const apc_params &p, int d, int hops) {
+  const double latency = p.base_latency + (double)hops * p.lat[d];
+  const double bw = div_by(div_by(gb * (double)hops, (double)p.mesh_size[d], p.inv_mesh[d]), p.bw[d], p.inv_bw[d]);
+  return latency + bw * 1e6;
+}
+
 // collective_runtime_estimation.py:37-153 for one (producer spec, consumer spec) pair.
 // gb = bytes / num_shards / 1024^3 of the producer spec, cont = global contiguity.
 template <int M>
@@ -126,25 +151,16 @@ struct States {
     return (((1 << level) - 1) << M) + (mask << level) + hist;
   }
 };
-constexpr int kTermArrays = 4;  // rw, ag, rs, ar
-
-__host__ __device__ constexpr int states_count(int m) { return (1 << m) * ((1 << (m + 1)) - 1); }
-
 // ------------------------------------------------------------------------------------------
-// a7: bytes + contiguity per tensor, and (optionally) the per-state cost terms of the tensor:
-//   terms[t][0][k] read+write time of the running bytes          (compute_estimation.py:302-314)
-//   terms[t][1][k] all-gather on dim level-1, bytes already x n   (torch _collective_utils.py:281-288)
-//   terms[t][2][k] reduce-scatter on dim level (x a2a_scale = all-to-all)      (:302-313)
-//   terms[t][3][k] all-reduce on dim level                                      (:291-299)
-// each evaluated once, in the reference's operation order.  One 64-thread workgroup per tensor.
+// a7: bytes + contiguity per tensor
 // ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void tensor_tables_kernel(apc_params p, int64_t n, const int32_t *__restrict__ rank,
-                                                           const int32_t *__restrict__ itemsize,
-                                                           const int64_t *__restrict__ shape,
-                                                           const int64_t *__restrict__ stride,
-                                                           int64_t *__restrict__ bytes, uint8_t *__restrict__ cont,
-                                                           double *__restrict__ terms) {
-  const int64_t t = blockIdx.x;
+__global__ __launch_bounds__(kBlock) void tensor_tables_kernel(int64_t n, const int32_t *__restrict__ rank,
+                                                               const int32_t *__restrict__ itemsize,
+                                                               const int64_t *__restrict__ shape,
+                                                               const int64_t *__restrict__ stride,
+                                                               int64_t *__restrict__ bytes,
+                                                               uint8_t *__restrict__ cont) {
+  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (t >= n) return;
   const int r = rank[t];
   const int64_t *sh = shape + t * APC_MAX_RANK;
@@ -152,7 +168,7 @@ __global__ __launch_bounds__(64) void tensor_tables_kernel(apc_params p, int64_t
   int64_t nbytes = itemsize[t];
   int64_t expected = 1, expected_max = 1;
   bool ok = true;
-  for (int i = r - 1; i >= 0; --i) {  // every lane computes the same few integers
+  for (int i = r - 1; i >= 0; --i) {
     const int64_t x = sh[i], y = st[i];
     nbytes *= x;
     if (x == 1) continue;
@@ -160,40 +176,8 @@ __global__ __launch_bounds__(64) void tensor_tables_kernel(apc_params p, int64_t
     expected_max *= (x > 1 ? x : 1);
     expected *= x;
   }
-  if (threadIdx.x == 0) {
-    bytes[t] = nbytes;
-    cont[t] = ok ? 1 : 0;
-  }
-  if (!terms) return;
-  const int M = p.mesh_ndim;
-  const int ns = states_count(M);
-  double *out = terms + t * (int64_t)(kTermArrays * ns);
-  const double fbytes = (double)nbytes;
-  for (int k = threadIdx.x; k < ns; k += 64) {
-    const int level = 31 - __clz((k >> M) + 1);
-    const int rem = k - (((1 << level) - 1) << M);
-    const int mask = rem >> level, hist = rem & ((1 << level) - 1);
-    int64_t shards = 1;
-    for (int i = 0; i < M; ++i)
-      if ((mask >> i) & 1) shards *= p.mesh_size[i];
-    double gb = fbytes / (double)shards / 1024 / 1024 / 1024;  // collective_runtime_estimation.py:66-68
-    for (int i = 0; i < level; ++i) {
-      if ((hist >> i) & 1) {
-        const double m = (double)p.mesh_size[i];
-        if ((mask >> i) & 1) gb *= m; else gb /= m;  // :86 / :128
-      }
-    }
-    double ag = 0.0, rs = 0.0, ar = 0.0;
-    if (level >= 1) ag = ring(gb, p, level - 1, p.mesh_size[level - 1] - 1);
-    if (level < M) {
-      rs = ring(gb, p, level, p.mesh_size[level] - 1);
-      ar = ring(gb, p, level, 2 * (p.mesh_size[level] - 1));
-    }
-    out[k] = rw_time(gb * 2 * 1073741824.0, p);
-    out[ns + k] = ag;
-    out[2 * ns + k] = rs;
-    out[3 * ns + k] = ar;
-  }
+  bytes[t] = nbytes;
+  cont[t] = ok ? 1 : 0;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -312,7 +296,6 @@ __global__ __launch_bounds__(kBlock) void compute_costs_kernel(
 struct TableArgs {
   const int64_t *tensor_bytes;
   const uint8_t *tensor_contiguous;
-  const double *tensor_terms;
   const uint32_t *spec_codes;
   const int32_t *spec_tensor;
   const double *pt_values;
@@ -484,18 +467,36 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
   const int t0 = tile.tensor;  // spec_tensor of the tile's first producer spec (checked by the host)
   const bool terms_wanted = t0 >= 0 && !no_producer;
   if (terms_wanted) {
-    // global layout per tensor: [rw][ag][rs][ar]
-    const double *terms = a.tensor_terms + (int64_t)t0 * (kTermArrays * NS);
+    // every collective / read-write term the tile can need, once per running-bytes state, in
+    // the reference's operation order (collective_runtime_estimation.py:66-68, :86, :128;
+    // torch _collective_utils.py:281-313; compute_estimation.py:302-314)
+    const double fbytes = (double)a.tensor_bytes[t0];
     for (int k = tid; k < NS; k += kTileThreads) {
-      const double rs = terms[2 * NS + k];
+      const int level = 31 - __clz((k >> M) + 1);
+      const int rem = k - (((1 << level) - 1) << M);
+      const int mask = rem >> level, hist = rem & ((1 << level) - 1);
+      double gb = div_by(fbytes, p.shards[mask], p.inv_shards[mask]) * 0x1p-30;  // / 1024 / 1024 / 1024
+#pragma unroll
+      for (int i = 0; i < M; ++i) {
+        if (i < level && ((hist >> i) & 1)) {
+          const double m = (double)p.mesh_size[i];
+          gb = ((mask >> i) & 1) ? gb * m : div_by(gb, m, p.inv_mesh[i]);
+        }
+      }
+      double ag = 0.0, rs = 0.0, ar = 0.0;
+      if (level >= 1) ag = ring_r(gb, p, level - 1, p.mesh_size[level - 1] - 1);
+      if (level < M) {
+        rs = ring_r(gb, p, level, p.mesh_size[level] - 1);
+        ar = ring_r(gb, p, level, 2 * (p.mesh_size[level] - 1));
+      }
       double a2a = rs;
       a2a *= p.a2a_scale;
       s_terms[k] = 0.0;
-      s_terms[NS + k] = terms[NS + k];
+      s_terms[NS + k] = ag;
       s_terms[2 * NS + k] = rs;
-      s_terms[3 * NS + k] = terms[3 * NS + k];
+      s_terms[3 * NS + k] = ar;
       s_terms[4 * NS + k] = a2a;
-      s_terms[5 * NS + k] = terms[k];
+      s_terms[5 * NS + k] = rw_time_r(gb * 2 * 1073741824.0, p);
     }
   }
   const bool tile_cont = terms_wanted ? a.tensor_contiguous[t0] != 0 : true;
@@ -647,8 +648,21 @@ int check_params(const apc_params *p) {
   if (!p) return fail(-1, "params is NULL");
   if (p->mesh_ndim < 1 || p->mesh_ndim > APC_MAX_MESH)
     return fail(-1, "mesh_ndim %d outside [1, %d]", p->mesh_ndim, APC_MAX_MESH);
-  for (int i = 0; i < p->mesh_ndim; ++i)
+  for (int i = 0; i < p->mesh_ndim; ++i) {
     if (p->mesh_size[i] < 1) return fail(-1, "mesh_size[%d] = %d must be >= 1", i, p->mesh_size[i]);
+    // the kernels divide through these reciprocals: they must be the correctly rounded ones
+    if (p->inv_mesh[i] != 1.0 / (double)p->mesh_size[i] || p->inv_bw[i] != 1.0 / p->bw[i])
+      return fail(-1, "inv_mesh[%d] / inv_bw[%d] are not 1.0 / mesh_size, 1.0 / bw", i, i);
+  }
+  if (p->inv_hbm_bw != 1.0 / p->hbm_bw || p->inv_rw_eff != 1.0 / p->rw_eff)
+    return fail(-1, "inv_hbm_bw / inv_rw_eff are not 1.0 / hbm_bw, 1.0 / rw_eff");
+  for (int mask = 0; mask < (1 << p->mesh_ndim); ++mask) {
+    double shards = 1.0;
+    for (int i = 0; i < p->mesh_ndim; ++i)
+      if ((mask >> i) & 1) shards *= (double)p->mesh_size[i];
+    if (p->shards[mask] != shards || p->inv_shards[mask] != 1.0 / shards)
+      return fail(-1, "shards[%d] / inv_shards[%d] do not match the mesh", mask, mask);
+  }
   return 0;
 }
 
@@ -758,20 +772,13 @@ int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const 
   return 0;
 }
 
-int64_t apc_tensor_terms_count(int mesh_ndim) {
-  if (mesh_ndim < 1 || mesh_ndim > APC_MAX_MESH) return 0;
-  return (int64_t)kTermArrays * states_count(mesh_ndim);
-}
-
-int apc_tensor_tables(const apc_params *params, int64_t n, const int32_t *rank, const int32_t *itemsize,
-                      const int64_t *shape, const int64_t *stride, int64_t *bytes, uint8_t *cont, double *terms,
-                      void *stream) {
-  if (int rc = check_params(params)) return rc;
-  if (n < 0 || n > INT32_MAX) return fail(-1, "n_tensors %lld out of range", (long long)n);
+int apc_tensor_tables(int64_t n, const int32_t *rank, const int32_t *itemsize, const int64_t *shape,
+                      const int64_t *stride, int64_t *bytes, uint8_t *cont, void *stream) {
+  if (n < 0) return fail(-1, "n_tensors < 0");
   if (n == 0) return 0;
   if (!rank || !itemsize || !shape || !stride || !bytes || !cont) return fail(-1, "apc_tensor_tables: NULL array");
-  hipLaunchKernelGGL(tensor_tables_kernel, dim3((unsigned)n), dim3(64), 0, (hipStream_t)stream, *params, n, rank,
-                     itemsize, shape, stride, bytes, cont, terms);
+  hipLaunchKernelGGL(tensor_tables_kernel, dim3(blocks_for(n, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, n,
+                     rank, itemsize, shape, stride, bytes, cont);
   return check_launch("apc_tensor_tables");
 }
 
@@ -803,8 +810,7 @@ int apc_compute_costs(const apc_params *params, int64_t n, const int64_t *flops,
 }
 
 int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes, const uint8_t *tensor_contiguous,
-                            const double *tensor_terms, const uint32_t *spec_codes, const int32_t *spec_tensor,
-                            const double *pt_values,
+                            const uint32_t *spec_codes, const int32_t *spec_tensor, const double *pt_values,
                             const double *per_arg, int64_t n_tiles, const apc_tile *tiles,
                             const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *trans_out,
                             double *cost_out, void *stream) {
@@ -812,17 +818,18 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
   if (n_tiles < 0 || n_tiles > INT32_MAX) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tiles == 0) return 0;
   if (n_entries < 0) return fail(-1, "n_entries < 0");
-  if (!tensor_bytes || !tensor_contiguous || !tensor_terms || !spec_codes || !spec_tensor || !tiles)
+  if (!tensor_bytes || !tensor_contiguous || !spec_codes || !spec_tensor || !tiles)
     return fail(-1, "apc_redistribute_tables: NULL table");
   if (cost_out && !per_arg) return fail(-1, "cost_out needs compute_cost_per_arg");
-  TableArgs a{tensor_bytes, tensor_contiguous, tensor_terms,    spec_codes, spec_tensor, pt_values,
-              per_arg,      tiles,             dup_entry_begin, comm_out,   trans_out,   cost_out};
+  TableArgs a{tensor_bytes, tensor_contiguous, spec_codes, spec_tensor, pt_values, per_arg,
+              tiles,        dup_entry_begin,   comm_out,   trans_out,   cost_out};
   const dim3 grid((unsigned)n_tiles);
   hipStream_t s = (hipStream_t)stream;
   // small matrices (traced graphs): one wavefront per tile; large ones: two wavefronts share
   // the staged specs and terms of a tile
-  // (n_entries counts de-duplicated edges too: per computed tile the estimate is an upper bound)
-  const bool wide = n_entries / n_tiles >= 512 && n_tiles >= 4096;
+  // (n_entries counts the copies written for de-duplicated edges too: work per tile either way)
+  bool wide = n_entries / n_tiles >= 512;
+  if (const char *env = getenv("APC_TILE_THREADS")) wide = atoi(env) >= 128;  // tuning override
 #define APC_LAUNCH(M_)                                                                                  \
   if (wide) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 128>), grid, dim3(128), 0, s, *params, a); \
   else hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 64>), grid, dim3(64), 0, s, *params, a)

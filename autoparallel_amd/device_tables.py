@@ -68,12 +68,10 @@ class DeviceCostTables:
         if validate:
             tables.validate(params)
         self.c_params = params.to_c()
-        self.terms_per_tensor = int(self.lib.apc_tensor_terms_count(ctypes.c_int(params.ndim)))
         with torch.cuda.device(self.device):
             self.d = {k: _to_device(getattr(tables, k), self.device) for k in _UPLOAD}
         self.tensor_bytes = None
         self.tensor_contiguous = None
-        self.tensor_terms = None
         self.compute_cost = None
         self.compute_cost_per_arg = None
         self.comm = None
@@ -105,12 +103,11 @@ class DeviceCostTables:
         n = self.tables.n_tensors
         self.tensor_bytes = self._empty((n,), torch.int64)
         self.tensor_contiguous = self._empty((n,), torch.uint8)
-        self.tensor_terms = self._empty((n, self.terms_per_tensor), torch.float64)
         with torch.cuda.device(self.device):
             rc = self.lib.apc_tensor_tables(
-                ctypes.byref(self.c_params), ctypes.c_int64(n), self._p("tensor_rank"), self._p("tensor_itemsize"),
-                self._p("tensor_shape"), self._p("tensor_stride"), self._p(self.tensor_bytes),
-                self._p(self.tensor_contiguous), self._p(self.tensor_terms), self._stream())
+                ctypes.c_int64(n), self._p("tensor_rank"), self._p("tensor_itemsize"), self._p("tensor_shape"),
+                self._p("tensor_stride"), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
+                self._stream())
         _native.check(rc, "apc_tensor_tables")
         return self.tensor_bytes, self.tensor_contiguous
 
@@ -168,7 +165,7 @@ class DeviceCostTables:
         with torch.cuda.device(self.device):
             rc = self.lib.apc_redistribute_tables(
                 ctypes.byref(self.c_params), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
-                self._p(self.tensor_terms), self._p("spec_codes"), self._p("spec_tensor"), self._p("pt_values"),
+                self._p("spec_codes"), self._p("spec_tensor"), self._p("pt_values"),
                 self._p(self.compute_cost_per_arg), ctypes.c_int64(self.tables.n_tiles), self._p("tile_records"),
                 self._p("dup_entry_begin"), ctypes.c_int64(self.tables.n_entries), self._p(self.comm), self._p(self.transition),
                 self._p(self.cost), self._stream())
@@ -206,8 +203,8 @@ class DeviceCostTables:
         tb = self.tables
         err = torch.zeros((1,), dtype=torch.int32, device=self.device)
         self._step_keepalive = [err, spec]
-        a_tensor = (cp, ctypes.c_int64(tb.n_tensors), P("tensor_rank"), P("tensor_itemsize"), P("tensor_shape"),
-                    P("tensor_stride"), P(self.tensor_bytes), P(self.tensor_contiguous), P(self.tensor_terms), stream)
+        a_tensor = (ctypes.c_int64(tb.n_tensors), P("tensor_rank"), P("tensor_itemsize"), P("tensor_shape"),
+                    P("tensor_stride"), P(self.tensor_bytes), P(self.tensor_contiguous), stream)
         a_spec = (cp, ctypes.c_int64(tb.n_specs), P("spec_codes"), P("spec_tensor"), P("tensor_rank"),
                   P("tensor_itemsize"), P("tensor_shape"), P("tensor_stride"), P(spec["num_shards"]),
                   P(spec["local_shape"]), P(spec["local_stride"]), P(spec["local_numel"]), P(spec["local_bytes"]),
@@ -215,8 +212,7 @@ class DeviceCostTables:
         a_compute = (cp, ctypes.c_int64(tb.n_strategies), P("strat_flops"), P("strat_rw_bytes"), P("strat_dtype"),
                      P("strat_zero_cost"), P("strat_num_args"), P(self.compute_cost), P(self.compute_cost_per_arg),
                      P(err), stream)
-        a_tables = (cp, P(self.tensor_bytes), P(self.tensor_contiguous), P(self.tensor_terms), P("spec_codes"),
-                    P("spec_tensor"),
+        a_tables = (cp, P(self.tensor_bytes), P(self.tensor_contiguous), P("spec_codes"), P("spec_tensor"),
                     P("pt_values"), P(self.compute_cost_per_arg), ctypes.c_int64(tb.n_tiles), P("tile_records"),
                     P("dup_entry_begin"), ctypes.c_int64(tb.n_entries), P(self.comm), P(self.transition), P(self.cost), stream)
 

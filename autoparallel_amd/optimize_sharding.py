@@ -60,7 +60,7 @@ class DeviceBackend:
             out = self.dev.run_spec_tables()
             return out["local_shape"].cpu().numpy(), out["local_stride"].cpu().numpy()
 
-    def upload_strategy_inputs(self, tables, tile_entries=2048, dedupe=True, max_copies=4):
+    def upload_strategy_inputs(self, tables, tile_entries=2048, dedupe=True, max_copies=8):
         """The strategy table is final: tile the edges (identical edges once) and send both."""
         tables.build_tiles(tile_entries, dedupe=dedupe, max_copies=max_copies)
         tables.validate(self.dev.params)
@@ -208,7 +208,7 @@ class ShardingOptimizer:
     # are evaluated once, and how many copies one evaluated edge may serve
     tile_entries = 2048
     dedupe = True
-    max_copies = 4
+    max_copies = 8
 
     def __init__(self, gm, mesh, rescale_grad_comm_cost_for_mp=1.0, repeated_subgraphs=False):
         self.gm = gm

@@ -43,7 +43,7 @@ def parse_args():
     ap.add_argument("--no-solve", action="store_true", help="skip the ILP leg of the plan wall-time")
     ap.add_argument("--no-clustering", action="store_true", help="one ILP variable per entry (no variable sharing)")
     ap.add_argument("--no-dedupe", action="store_true", help="tile every edge even if an identical one exists")
-    ap.add_argument("--max-copies", type=int, default=4, help="identical edges served by one tiled edge")
+    ap.add_argument("--max-copies", type=int, default=8, help="identical edges served by one tiled edge")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy three times (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")

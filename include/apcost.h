@@ -97,6 +97,14 @@ typedef struct apc_params {
   double rescale;           /* grad comm rescale   optimize_sharding.py:358-359 */
   double gpu_flops[APC_MAX_DTYPES]; /* tflops*10^12 per dtype code; 0 = unsupported */
   int32_t transition_scale; /* 1                   optimize_sharding.py:298 */
+  /* Derived values, checked by the library: the kernels divide by constants through their
+   * correctly rounded reciprocals (same bits as a division, a sixth of the instructions). */
+  double inv_bw[APC_MAX_MESH];   /* 1.0 / bw[i] */
+  double inv_mesh[APC_MAX_MESH]; /* 1.0 / mesh_size[i] */
+  double inv_hbm_bw;             /* 1.0 / hbm_bw */
+  double inv_rw_eff;             /* 1.0 / rw_eff */
+  double shards[1 << APC_MAX_MESH];     /* product of mesh_size[i] over the bits of the index */
+  double inv_shards[1 << APC_MAX_MESH]; /* 1.0 / shards[mask] */
 } apc_params;
 
 int apc_version(void);
@@ -117,22 +125,13 @@ int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const 
                              int64_t n_pt, int64_t n_strategies, int64_t n_tiles, const apc_tile *tiles_host,
                              int64_t n_dups, const int64_t *dup_entry_begin_host);
 
-/* Number of doubles per tensor in the tensor_terms table for a mesh of this ndim
- * (4 term arrays x the number of running-bytes states); 0 for an unsupported ndim. */
-int64_t apc_tensor_terms_count(int mesh_ndim);
-
-/* Bytes and contiguity of every tensor row, and the tensor's collective / read-write cost
- * terms for every running-bytes state (tensor_terms: [n_tensors][apc_tensor_terms_count]).
+/* Bytes and contiguity of every tensor row.
  * Replaces torch spec_to_bytes (distributed/tensor/_collective_utils.py:230-232) and
  * check_contiguous_sizes_strides (_prims_common/__init__.py:252-292) as called from
- * collective_runtime_estimation.py:66-76, and evaluates allgather_cost / reduce_scatter_cost /
- * allreduce_cost (torch _collective_utils.py:281-313) and compute_read_write_time
- * (compute_estimation.py:302-314) once per value comm_bytes_gb can take for the tensor
- * (collective_runtime_estimation.py:66-68, :86, :128).  tensor_terms may be NULL (then
- * apc_redistribute_tables cannot be used with the outputs). */
-int apc_tensor_tables(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
-                      const int32_t *tensor_itemsize, const int64_t *tensor_shape, const int64_t *tensor_stride,
-                      int64_t *tensor_bytes, uint8_t *tensor_contiguous, double *tensor_terms, void *stream);
+ * collective_runtime_estimation.py:66-76. */
+int apc_tensor_tables(int64_t n_tensors, const int32_t *tensor_rank, const int32_t *tensor_itemsize,
+                      const int64_t *tensor_shape, const int64_t *tensor_stride, int64_t *tensor_bytes,
+                      uint8_t *tensor_contiguous, void *stream);
 
 /* Local shard shape / stride / element and byte counts and shard count per spec.
  * Replaces _get_sharded_shape_stride (compute_estimation.py:211-229) and
@@ -163,8 +162,8 @@ int apc_compute_costs(const apc_params *params, int64_t n_strategies, const int6
  * (:345-351), the grad rescale (:358-359) and cost assembly (:368-372).
  * comm_out / transition_out / cost_out are [n_entries]; any may be NULL. */
 int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes,
-                            const uint8_t *tensor_contiguous, const double *tensor_terms,
-                            const uint32_t *spec_codes, const int32_t *spec_tensor, const double *pt_values,
+                            const uint8_t *tensor_contiguous, const uint32_t *spec_codes,
+                            const int32_t *spec_tensor, const double *pt_values,
                             const double *compute_cost_per_arg, int64_t n_tiles, const apc_tile *tiles,
                             const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out,
                             uint8_t *transition_out, double *cost_out, void *stream);

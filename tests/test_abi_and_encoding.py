@@ -32,8 +32,10 @@ def test_library_exports_every_declared_symbol():
 def test_params_struct_layout_matches_header():
     # 4 + 16 (+4 pad) + 32 + 32 + 7*8 + 64 + 4 (+4 pad)
     assert ctypes.sizeof(_native.ApcTile) == 64 and _native.ApcTile.entry_begin.offset == 40
-    assert ctypes.sizeof(_native.ApcParams) == 216
+    # 216 bytes of model parameters + 4 + 4 + 1 + 1 + 16 + 16 derived doubles
+    assert ctypes.sizeof(_native.ApcParams) == 216 + 42 * 8
     assert _native.ApcParams.bw.offset == 24 and _native.ApcParams.gpu_flops.offset == 144
+    assert _native.ApcParams.inv_bw.offset == 216
 
 
 def test_placement_codes_round_trip():
