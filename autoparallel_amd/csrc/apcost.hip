@@ -152,6 +152,21 @@ struct States {
   }
 };
 // ------------------------------------------------------------------------------------------
+// XCD-aware work order.  The dispatcher deals workgroups to the chip's 8 XCDs round-robin by
+// workgroup id, and every XCD has its own L2.  With the plain order, neighbouring units of
+// work (which write neighbouring memory and share the cache lines at their boundaries) sit
+// in eight different L2s and those lines are written back in parts.  The launchers round the
+// grid up to a multiple of 2^shift and the kernel takes unit (id mod 2^shift) * per + id /
+// 2^shift, so each XCD walks one contiguous share of the units.  (Measured: helps the tile
+// kernel, whose units end at arbitrary byte offsets; the kernels whose workgroups write
+// whole aligned blocks are faster in the plain order.)
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ int64_t xcd_chunked_unit(int shift) {
+  const int64_t per = gridDim.x >> shift;
+  return (int64_t)(blockIdx.x & ((1u << shift) - 1)) * per + (blockIdx.x >> shift);
+}
+
+// ------------------------------------------------------------------------------------------
 // a7: bytes + contiguity per tensor
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void tensor_tables_kernel(int64_t n, const int32_t *__restrict__ rank,
@@ -284,13 +299,18 @@ __global__ __launch_bounds__(kBlock) void compute_costs_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// a1-a6: redistribution-cost matrices.  One wavefront (a 64-thread workgroup) per tile of
-// one edge's matrix.  The tile's producer and consumer specs and the per-state terms of the
-// edge's tensor are staged in LDS; the per-entry loop walks the mesh dims, looks the terms
-// of the current state up and adds them in the reference's order, so results are
-// bit-identical to evaluating every entry directly (entry_cost).  The direct evaluation
-// remains the path for the rare cases the states do not cover: producer specs of one edge
-// that point at different tensors, and the 2-D (Partial, Partial) -> all-Shard order flip.
+// a1-a6: redistribution-cost matrices.  The unit of work is a tile: a rectangle of one edge's
+// matrix.  A tile's producer and consumer specs and the per-state terms of the edge's tensor
+// are staged in LDS (TileStage); the per-entry loop walks the mesh dims, looks the terms of
+// the current state up and adds them in the reference's order, so results are bit-identical
+// to evaluating every entry directly (entry_cost).  The direct evaluation remains the path
+// for the rare cases the states do not cover: producer specs of one edge that point at
+// different tensors, and the 2-D (Partial, Partial) -> all-Shard order flip.
+//
+// One workgroup per tile.  (A variant in which a workgroup walked a run of tiles, one
+// wavefront staging tile t+1 while the others computed tile t, was measured slower: the
+// staging of a tile is a chain of two dependent loads, and many short workgroups overlap
+// those chains better than one staging wavefront per workgroup does.)
 // ------------------------------------------------------------------------------------------
 
 struct TableArgs {
@@ -334,144 +354,80 @@ __device__ __forceinline__ int placement_class(uint32_t code) {
 
 constexpr int kLdsTermArrays = 6;  // zeros, all-gather, reduce-scatter, all-reduce, all-to-all, read+write
 
-// The per-entry loop of a tile whose producer specs all name one tensor.  Straight-line code:
-// all lookups of an entry are independent of its fp additions, so they are issued together.
-template <int M, int kTileThreads, bool CONT, bool RESCALE>
-__device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const TableArgs &a, const apc_tile &tile,
-                                                     const double *s_terms, const uint32_t *s_col,
-                                                     const uint2 *s_row, const double *s_cpa, const int64_t *s_dup,
-                                                     int t0) {
-  constexpr int NS = States<M>::kCount;
-  constexpr int CW = 2 + M;
-  const int rows = tile.counts & 0xFFFF, cols = tile.counts >> 16;
-  const int tid = threadIdx.x;
-  const int n = rows * cols;
-  int r = tid / cols, c = tid - r * cols;
-  const int dr = kTileThreads / cols, dc = kTileThreads - dr * cols;
-  const int64_t tile_base = tile.entry_begin + (int64_t)tile.row_begin * tile.n_src + tile.col_begin;
-  // only the 2-D order flip evaluates an entry directly; (Partial, Partial) shards nothing
-  const double gb_unsharded = M == 2 ? (double)a.tensor_bytes[t0] / 1024 / 1024 / 1024 : 0.0;
-  // Every spec of the tile is a DTensorSpec on one tensor (the caller checked): the loop
-  // below issues no vector memory loads, so its stores are never waited for.
-#if defined(APC_EXP_PROLOGUE_ONLY)
-  if (n > 0) return;
-#endif
-  for (int idx = tid; idx < n; idx += kTileThreads) {
-    const uint32_t src = s_col[c * CW], cinfo = s_col[c * CW + 1];
-    const uint2 rowv = s_row[r];
-    const uint32_t tgt = rowv.x, tinfo = rowv.y;
-    const double cpa = s_cpa[r];
-    const uint32_t x = src ^ tgt;
-    const uint32_t mask = (cinfo >> 4) & 0xF;
-    // ---- integer part: which term of which state each mesh dim adds ------------------------
-    uint32_t hist = 0, seen = 0;
-    uint32_t term_at[M], rw_at[M], nc_at[M], copies[M];
-    bool neq[M];
-#pragma unroll
-    for (int i = 0; i < M; ++i) {
-      neq[i] = ((x >> (8 * i)) & 0xFF) != 0;
-      const uint32_t tsh = (tinfo >> (1 + 5 * i)) & 0x1F;
-      uint32_t e = (s_col[c * CW + 2 + i] >> tsh) & 0x7F;
-      e = neq[i] ? e : 0u;
-      const uint32_t sel = e & 7u;
-      const uint32_t k = (uint32_t)States<M>::index(i, 0, 0) + (mask << i) + hist;
-      hist |= ((e >> 6) & 1u) << i;
-      const uint32_t k2 = (uint32_t)States<M>::index(i + 1, 0, 0) + (mask << (i + 1)) + hist;
-      const uint32_t kk = sel == 1u ? k2 : k;  // the all-gather is charged on the gathered bytes
-      term_at[i] = sel * NS + kk;
-      rw_at[i] = 5 * NS + kk;
-      nc_at[i] = 5 * NS + k;
-      copies[i] = (e >> 3) & 3u;
-      seen |= e;
-    }
-    // ---- lookups ------------------------------------------------------------------------------
-    double term[M], rw[M], nc[M];
-#pragma unroll
-    for (int i = 0; i < M; ++i) {
-      term[i] = s_terms[term_at[i]];
-      rw[i] = s_terms[rw_at[i]];
-      if (!CONT) nc[i] = s_terms[nc_at[i]];
-    }
-    // ---- additions in the reference's order ------------------------------------------------------
-    double cost = 0.0;
-    // a fully replicated producer returns before the non-contiguity term (:56-62)
-    bool cont = CONT || (cinfo & 2u);
-#pragma unroll
-    for (int i = 0; i < M; ++i) {
-      if (!CONT) {
-        cost += (neq[i] && !cont) ? nc[i] : 0.0;
-        cont = cont || neq[i];
-      }
-      cost += term[i];
-      cost += (double)copies[i] * rw[i];
-    }
-    double comm = (seen & 32u) ? INFINITY : cost;
-    const int64_t local = (int64_t)r * tile.n_src + c;
-    int trans = x != 0u ? p.transition_scale : 0;  // optimize_sharding.py:345-351
-    if (M == 2 && src == 0x4040u && (tinfo >> 30)) {  // (Partial, Partial) -> all Shard walks dim 1 first
-      comm = entry_cost<M>(src, tgt, gb_unsharded, CONT, p);
-    }
-    if (RESCALE) comm = comm / p.rescale;  // :358-359
-    const int64_t o = tile_base + local;
-#if defined(APC_EXP_NO_STORE)
-    if (comm == -1.0) a.comm_out[o] = comm;
-#elif defined(APC_EXP_NO_COMPUTE)
-    a.comm_out[o] = cpa;
-    if (APC_EXP_NO_COMPUTE <= 2) a.cost_out[o] = cpa;
-    if (APC_EXP_NO_COMPUTE <= 1) a.trans_out[o] = (uint8_t)idx;
-#else
-    const double total = comm + cpa + (double)trans;  // :368-372
-    if (a.comm_out) a.comm_out[o] = comm;
-    if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
-    if (a.cost_out) a.cost_out[o] = total;
-    for (int d = 0; d < tile.dup_count; ++d) {  // identical edges receive the same values
-      const int64_t od = o + s_dup[d];
-      if (a.comm_out) a.comm_out[od] = comm;
-      if (a.trans_out) a.trans_out[od] = (uint8_t)trans;
-      if (a.cost_out) a.cost_out[od] = total;
-    }
-#endif
-    c += dc;
-    r += dr;
-    if (c >= cols) {
-      c -= cols;
-      r += 1;
+// Words of the staged action rows per producer spec: one row per mesh dim, padded to a power
+// of two so that a spec's rows are one aligned LDS read.
+template <int M>
+struct ActionRows {
+  static constexpr int kWords = M == 1 ? 1 : M == 2 ? 2 : 4;
+  __device__ static __forceinline__ void load(const uint32_t *s_act, int c, uint32_t (&act)[M]) {
+    if constexpr (M == 1) {
+      act[0] = s_act[c];
+    } else if constexpr (M == 2) {
+      const uint2 v = reinterpret_cast<const uint2 *>(s_act)[c];
+      act[0] = v.x;
+      act[1] = v.y;
+    } else {
+      const uint4 v = reinterpret_cast<const uint4 *>(s_act)[c];
+      act[0] = v.x;
+      act[1] = v.y;
+      act[2] = v.z;
+      if constexpr (M == 4) act[3] = v.w;
     }
   }
+};
+
+// Everything the entry loops need about one tile, in LDS.
+template <int M>
+struct TileStage {
+  // term arrays: [0] zeros, [1] all-gather, [2] reduce-scatter, [3] all-reduce,
+  // [4] all-to-all (= reduce-scatter shaped term x a2a_scale, :22-32), [5] read+write
+  double terms[kLdsTermArrays * States<M>::kCount];
+  uint2 colh[APC_TILE_MAX_COLS];  // producer specs: x = codes, y = info
+  alignas(16) uint32_t act[APC_TILE_MAX_COLS * ActionRows<M>::kWords];  // one action row per mesh dim
+  uint2 row[APC_TILE_MAX_ROWS];   // consumer specs: x = codes, y = info
+  double cpa[APC_TILE_MAX_ROWS];  // compute cost / num_args of the consumer strategies
+  int64_t dup[APC_TILE_MAX_DUPS];  // entry offsets of identical edges, relative to this edge
+  double gb_unsharded;  // bytes / 1024^3 of the tile's tensor
+  int mixed;            // some spec is not a DTensorSpec on the tile's tensor: generic loop
+  int cont;             // the tile's tensor is contiguous
+};
+
+// The fields of a tile record the entry loops use.
+struct TileView {
+  int rows, cols, row_begin, col_begin, n_src, flags, dup_count, src_begin;
+  int64_t entry_begin, pt_begin;
+};
+
+__device__ __forceinline__ int uniform_i32(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ int64_t uniform_i64(int64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
 }
 
-template <int M, int kTileThreads>
-__global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_params p, TableArgs a) {
+__device__ __forceinline__ TileView view_of(const apc_tile &tile) {
+  return TileView{tile.counts & 0xFFFF, tile.counts >> 16, tile.row_begin, tile.col_begin, tile.n_src,
+                  tile.flags,           tile.dup_count,    tile.src_begin, tile.entry_begin, tile.pt_begin};
+}
+
+// Stages tile `tile` with `nthreads` cooperating threads (this thread is `tid`).  The caller
+// synchronises before the stage is read.  Only global loads and LDS writes: no stores.
+template <int M>
+__device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs &a, const apc_tile &tile,
+                                           TileStage<M> &st, int tid, int nthreads) {
   constexpr int NS = States<M>::kCount;
-  constexpr int CW = 2 + M;  // words per staged producer spec: codes, info, one action row per mesh dim
-  // term arrays in LDS: [0] zeros, [1] all-gather, [2] reduce-scatter, [3] all-reduce,
-  // [4] all-to-all (= reduce-scatter shaped term x a2a_scale, :22-32), [5] read+write
-  __shared__ double s_terms[kLdsTermArrays * NS];
-  __shared__ uint32_t s_col[APC_TILE_MAX_COLS * CW];
-  __shared__ uint2 s_row[APC_TILE_MAX_ROWS];  // x = codes, y = info
-  __shared__ double s_cpa[APC_TILE_MAX_ROWS];
-  __shared__ int64_t s_dup[APC_TILE_MAX_DUPS];  // entry offsets of identical edges, relative to this edge
-  __shared__ int s_uniform;
-
-  const apc_tile tile = a.tiles[blockIdx.x];
+  constexpr int AW = ActionRows<M>::kWords;
   const int rows = tile.counts & 0xFFFF, cols = tile.counts >> 16;
-  const int row0 = tile.row_begin, col0 = tile.col_begin;
-  const int n_src = tile.n_src;
-  const int flags = tile.flags;
-  const int tid = threadIdx.x;
-  const bool no_producer = (flags & APC_EDGE_NO_PRODUCER) != 0;
-
-  // ---- stage the tile's producer / consumer specs -------------------------------------------
-  if (tid == 0) s_uniform = 1;
-  __syncthreads();
   const int t0 = tile.tensor;  // spec_tensor of the tile's first producer spec (checked by the host)
+  const bool no_producer = (tile.flags & APC_EDGE_NO_PRODUCER) != 0;
   const bool terms_wanted = t0 >= 0 && !no_producer;
+  bool mixed = !terms_wanted;
   if (terms_wanted) {
     // every collective / read-write term the tile can need, once per running-bytes state, in
     // the reference's operation order (collective_runtime_estimation.py:66-68, :86, :128;
     // torch _collective_utils.py:281-313; compute_estimation.py:302-314)
     const double fbytes = (double)a.tensor_bytes[t0];
-    for (int k = tid; k < NS; k += kTileThreads) {
+    for (int k = tid; k < NS; k += nthreads) {
       const int level = 31 - __clz((k >> M) + 1);
       const int rem = k - (((1 << level) - 1) << M);
       const int mask = rem >> level, hist = rem & ((1 << level) - 1);
@@ -491,19 +447,25 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
       }
       double a2a = rs;
       a2a *= p.a2a_scale;
-      s_terms[k] = 0.0;
-      s_terms[NS + k] = ag;
-      s_terms[2 * NS + k] = rs;
-      s_terms[3 * NS + k] = ar;
-      s_terms[4 * NS + k] = a2a;
-      s_terms[5 * NS + k] = rw_time_r(gb * 2 * 1073741824.0, p);
+      st.terms[k] = 0.0;
+      st.terms[NS + k] = ag;
+      st.terms[2 * NS + k] = rs;
+      st.terms[3 * NS + k] = ar;
+      st.terms[4 * NS + k] = a2a;
+      st.terms[5 * NS + k] = rw_time_r(gb * 2 * 1073741824.0, p);
     }
+    if (tid == 0) {
+      st.gb_unsharded = fbytes / 1024 / 1024 / 1024;
+      st.cont = a.tensor_contiguous[t0] != 0;
+    }
+  } else if (tid == 0) {
+    st.gb_unsharded = 0.0;
+    st.cont = 1;
   }
-  const bool tile_cont = terms_wanted ? a.tensor_contiguous[t0] != 0 : true;
-  for (int j = tid; j < tile.dup_count; j += kTileThreads)
-    s_dup[j] = a.dup_entry_begin[tile.dup_begin + j] - tile.entry_begin;
-  for (int j = tid; j < cols; j += kTileThreads) {
-    const int sp = tile.src_begin + col0 + j;
+  for (int j = tid; j < tile.dup_count; j += nthreads)
+    st.dup[j] = a.dup_entry_begin[tile.dup_begin + j] - tile.entry_begin;
+  for (int j = tid; j < cols; j += nthreads) {
+    const int sp = tile.src_begin + tile.col_begin + j;
     const int t = a.spec_tensor[sp];
     const uint32_t codes = a.spec_codes[sp];
     // info: bit0 valid spec, bit1 fully replicated, bits 4.. mask of sharded mesh dims
@@ -513,14 +475,13 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
       const uint32_t c = (codes >> (8 * i)) & 0xFF;
       const int cls = placement_class(c);
       info |= (cls >= 2 ? 1u : 0u) << (4 + i);
-      s_col[j * CW + 2 + i] = cls == 0 ? pair_row(0) : cls == 1 ? pair_row(1) : cls == 2 ? pair_row(2) : pair_row(3);
+      st.act[j * AW + i] = cls == 0 ? pair_row(0) : cls == 1 ? pair_row(1) : cls == 2 ? pair_row(2) : pair_row(3);
     }
-    s_col[j * CW] = codes;
-    s_col[j * CW + 1] = info;
-    if (t != t0 || t < 0) s_uniform = 0;
+    st.colh[j] = make_uint2(codes, info);
+    if (t != t0 || t < 0) mixed = true;
   }
-  for (int j = tid; j < rows; j += kTileThreads) {
-    const int ts = tile.tgt_begin + row0 + j;
+  for (int j = tid; j < rows; j += nthreads) {
+    const int ts = tile.tgt_begin + tile.row_begin + j;
     const uint32_t tg = a.spec_codes[ts];
     // info: bit0 valid spec, bits 1 + 5i .. : 8 x class of mesh dim i, bit 30 every dim is a Shard
     uint32_t info = a.spec_tensor[ts] >= 0 ? 1u : 0u;
@@ -532,67 +493,219 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
       all_shard &= kind_of(t) == 2;
     }
     if (all_shard) info |= 1u << 30;
-    if (!(info & 1u)) s_uniform = 0;  // a consumer spec that is not a DTensorSpec: generic loop
-    s_row[j] = make_uint2(tg, info);
-    s_cpa[j] = a.per_arg ? a.per_arg[tile.strat_begin + row0 + j] : 0.0;
+    if (!(info & 1u)) mixed = true;  // a consumer spec that is not a DTensorSpec
+    st.row[j] = make_uint2(tg, info);
+    st.cpa[j] = a.per_arg ? a.per_arg[tile.strat_begin + tile.row_begin + j] : 0.0;
   }
-  __syncthreads();
-  const bool uniform = s_uniform != 0 && t0 >= 0 && !no_producer;
+  if (mixed) st.mixed = 1;  // cleared by the caller before staging
+}
 
-  const int n = rows * cols;
-  int r = tid / cols, c = tid - r * cols;
-  const int dr = kTileThreads / cols, dc = kTileThreads - dr * cols;
-
-  if (uniform) {
-    const bool rescale = (flags & APC_EDGE_GRAD_RESCALE) != 0;
-    if (tile_cont) {
-      if (rescale) uniform_tile_entries<M, kTileThreads, true, true>(p, a, tile, s_terms, s_col, s_row, s_cpa, s_dup, t0);
-      else uniform_tile_entries<M, kTileThreads, true, false>(p, a, tile, s_terms, s_col, s_row, s_cpa, s_dup, t0);
-    } else {
-      if (rescale) uniform_tile_entries<M, kTileThreads, false, true>(p, a, tile, s_terms, s_col, s_row, s_cpa, s_dup, t0);
-      else uniform_tile_entries<M, kTileThreads, false, false>(p, a, tile, s_terms, s_col, s_row, s_cpa, s_dup, t0);
+// One entry of a tile whose producer specs all name one tensor (column c, row r of the tile).
+// Straight-line code: all lookups of an entry are independent of its fp additions, so they
+// are issued together; no vector memory loads.
+template <int M, bool CONT, bool RESCALE>
+__device__ __forceinline__ void uniform_entry(const apc_params &p, const TileStage<M> &st, int r, int c,
+                                              double &comm_o, double &total_o, int &trans_o) {
+  constexpr int NS = States<M>::kCount;
+  const uint2 colv = st.colh[c];
+  const uint32_t src = colv.x, cinfo = colv.y;
+  uint32_t act[M];
+  ActionRows<M>::load(st.act, c, act);
+  const uint2 rowv = st.row[r];
+  const uint32_t tgt = rowv.x, tinfo = rowv.y;
+  const double cpa = st.cpa[r];
+  const uint32_t x = src ^ tgt;
+  const uint32_t mask = (cinfo >> 4) & 0xF;
+  // ---- integer part: which term of which state each mesh dim adds ------------------------
+  uint32_t hist = 0, seen = 0;
+  uint32_t term_at[M], rw_at[M], nc_at[M], copies[M];
+  bool neq[M];
+#pragma unroll
+  for (int i = 0; i < M; ++i) {
+    neq[i] = ((x >> (8 * i)) & 0xFF) != 0;
+    const uint32_t tsh = (tinfo >> (1 + 5 * i)) & 0x1F;
+    uint32_t e = (act[i] >> tsh) & 0x7F;
+    e = neq[i] ? e : 0u;
+    const uint32_t sel = e & 7u;
+    const uint32_t k = (uint32_t)States<M>::index(i, 0, 0) + (mask << i) + hist;
+    hist |= ((e >> 6) & 1u) << i;
+    const uint32_t k2 = (uint32_t)States<M>::index(i + 1, 0, 0) + (mask << (i + 1)) + hist;
+    const uint32_t kk = sel == 1u ? k2 : k;  // the all-gather is charged on the gathered bytes
+    term_at[i] = sel * NS + kk;
+    rw_at[i] = 5 * NS + kk;
+    nc_at[i] = 5 * NS + k;
+    copies[i] = (e >> 3) & 3u;
+    seen |= e;
+  }
+  // ---- lookups ------------------------------------------------------------------------------
+  double term[M], rw[M], nc[M];
+#pragma unroll
+  for (int i = 0; i < M; ++i) {
+    term[i] = st.terms[term_at[i]];
+    rw[i] = st.terms[rw_at[i]];
+    if (!CONT) nc[i] = st.terms[nc_at[i]];
+  }
+  // ---- additions in the reference's order (0.0 + t == t for these non-negative terms) ------------
+  double cost = 0.0;
+  // a fully replicated producer returns before the non-contiguity term (:56-62)
+  bool cont = CONT || (cinfo & 2u);
+#pragma unroll
+  for (int i = 0; i < M; ++i) {
+    if (!CONT) {
+      cost += (neq[i] && !cont) ? nc[i] : 0.0;
+      cont = cont || neq[i];
     }
-    return;
+    if (CONT && i == 0) cost = term[0];
+    else cost += term[i];
+    cost += (double)copies[i] * rw[i];
   }
+  double comm = (seen & 32u) ? INFINITY : cost;
+  const int trans = x != 0u ? p.transition_scale : 0;  // optimize_sharding.py:345-351
+  if (M == 2 && src == 0x4040u && (tinfo >> 30)) {  // (Partial, Partial) -> all Shard walks dim 1 first
+    comm = entry_cost<M>(src, tgt, st.gb_unsharded, CONT, p);
+  }
+  if (RESCALE) comm = comm / p.rescale;  // :358-359
+  comm_o = comm;
+  total_o = comm + cpa + (double)trans;  // :368-372
+  trans_o = trans;
+}
 
-  // ---- generic loop: pass-through edges and edges whose producer specs name different tensors ----
-  for (int idx = tid; idx < n; idx += kTileThreads) {
-    const int64_t local = (int64_t)(row0 + r) * n_src + (col0 + c);
+// The three output streams of one tile: wave-uniform bases, so an entry's addresses are a
+// scalar base plus a 32-bit lane offset (the host checks that a tile spans < 4 GiB).
+struct TileOut {
+  double *comm;
+  uint8_t *trans;
+  double *cost;
+};
+
+// Stores one entry's values to its edge and to every identical edge.  ALL: every output
+// array is present (no per-store checks).
+template <bool ALL>
+__device__ __forceinline__ void store_entry(const TileOut &o, int dup_count, const int64_t *s_dup, uint32_t local,
+                                            double comm, double total, int trans) {
+  const uint32_t off8 = local * 8u;
+  if (ALL || o.comm) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.comm) + off8) = comm;
+  if (ALL || o.trans) o.trans[local] = (uint8_t)trans;
+  if (ALL || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost) + off8) = total;
+  for (int d = 0; d < dup_count; ++d) {
+    const int64_t delta = uniform_i64(s_dup[d]);
+    if (ALL || o.comm) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.comm + delta) + off8) = comm;
+    if (ALL || o.trans) (o.trans + delta)[local] = (uint8_t)trans;
+    if (ALL || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost + delta) + off8) = total;
+  }
+}
+
+// The per-entry loop of such a tile for `nthreads` threads (this one is `tid`): a flattened
+// (row, column) walk, so a wavefront writes 64 consecutive entries.
+template <int M, bool CONT, bool RESCALE, bool ALL>
+__device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M> &st,
+                                                     const TileView &v, int tid, int nthreads) {
+  const int n = v.rows * v.cols;
+  const int dr = nthreads / v.cols, dc = nthreads - dr * v.cols;
+  const int64_t tile_base = v.entry_begin + (int64_t)v.row_begin * v.n_src + v.col_begin;
+  // A full-width tile is one contiguous run of entries: lanes are shifted so that every
+  // wavefront store starts on a 64-entry boundary of the output arrays (whole 128-byte lines
+  // of the fp64 streams) instead of straddling one more line than it fills.
+  int first = tid - (v.cols == v.n_src ? (int)(tile_base & 63) : 0);
+  if (first < 0) first += nthreads;
+  int r = first / v.cols, c = first - r * v.cols;
+  const TileOut out{a.comm_out ? a.comm_out + tile_base : nullptr, a.trans_out ? a.trans_out + tile_base : nullptr,
+                    a.cost_out ? a.cost_out + tile_base : nullptr};
+  for (int idx = first; idx < n; idx += nthreads) {
+    double comm, total;
+    int trans;
+    uniform_entry<M, CONT, RESCALE>(p, st, r, c, comm, total, trans);
+    store_entry<ALL>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
+                     trans);
+    c += dc;
+    r += dr;
+    if (c >= v.cols) {
+      c -= v.cols;
+      r += 1;
+    }
+  }
+}
+
+// Generic loop: pass-through edges and edges whose producer specs name different tensors.
+template <int M>
+__device__ __forceinline__ void generic_tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M> &st,
+                                                     const TileView &v, int tid, int nthreads) {
+  const int n = v.rows * v.cols;
+  int r = tid / v.cols, c = tid - r * v.cols;
+  const int dr = nthreads / v.cols, dc = nthreads - dr * v.cols;
+  const bool no_producer = (v.flags & APC_EDGE_NO_PRODUCER) != 0;
+  for (int idx = tid; idx < n; idx += nthreads) {
+    const int64_t local = (int64_t)(v.row_begin + r) * v.n_src + (v.col_begin + c);
     double comm;
     int trans = 0;
-    const uint32_t src = s_col[c * CW], cinfo = s_col[c * CW + 1];
-    const uint32_t tgt = s_row[r].x, tinfo = s_row[r].y;
+    const uint32_t src = st.colh[c].x, cinfo = st.colh[c].y;
+    const uint32_t tgt = st.row[r].x, tinfo = st.row[r].y;
     if (no_producer || !(cinfo & tinfo & 1u)) {
-      comm = a.pt_values[tile.pt_begin + local];
+      comm = a.pt_values[v.pt_begin + local];
     } else {
       trans = (src != tgt) ? p.transition_scale : 0;
-      const int st = a.spec_tensor[tile.src_begin + col0 + c];
+      const int sten = a.spec_tensor[v.src_begin + v.col_begin + c];
       int64_t shards = 1;
 #pragma unroll
       for (int i = 0; i < M; ++i)
         if (kind_of((src >> (8 * i)) & 0xFF) == 2) shards *= p.mesh_size[i];
-      const double gb = (double)a.tensor_bytes[st] / (double)shards / 1024 / 1024 / 1024;
-      comm = entry_cost<M>(src, tgt, gb, a.tensor_contiguous[st] != 0, p);
+      const double gb = (double)a.tensor_bytes[sten] / (double)shards / 1024 / 1024 / 1024;
+      comm = entry_cost<M>(src, tgt, gb, a.tensor_contiguous[sten] != 0, p);
     }
-    if (flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;
-    const int64_t o = tile.entry_begin + local;
-    const double total = comm + s_cpa[r] + (double)trans;
+    if (v.flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;
+    const int64_t o = v.entry_begin + local;
+    const double total = comm + st.cpa[r] + (double)trans;
     if (a.comm_out) a.comm_out[o] = comm;
     if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
     if (a.cost_out) a.cost_out[o] = total;
-    for (int d = 0; d < tile.dup_count; ++d) {
-      const int64_t od = o + s_dup[d];
+    for (int d = 0; d < v.dup_count; ++d) {
+      const int64_t od = o + st.dup[d];
       if (a.comm_out) a.comm_out[od] = comm;
       if (a.trans_out) a.trans_out[od] = (uint8_t)trans;
       if (a.cost_out) a.cost_out[od] = total;
     }
     c += dc;
     r += dr;
-    if (c >= cols) {
-      c -= cols;
+    if (c >= v.cols) {
+      c -= v.cols;
       r += 1;
     }
   }
+}
+
+// All entries of a staged tile.
+template <int M>
+__device__ __forceinline__ void tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M> &st,
+                                             const TileView &v, int tid, int nthreads) {
+  if (uniform_i32(st.mixed)) {
+    generic_tile_entries<M>(p, a, st, v, tid, nthreads);
+    return;
+  }
+  const bool rescale = (v.flags & APC_EDGE_GRAD_RESCALE) != 0;
+  const bool all = a.comm_out && a.trans_out && a.cost_out;
+#define APC_TILE_LOOP(CONT_, RESCALE_)                                               \
+  if (all) uniform_tile_entries<M, CONT_, RESCALE_, true>(p, a, st, v, tid, nthreads); \
+  else uniform_tile_entries<M, CONT_, RESCALE_, false>(p, a, st, v, tid, nthreads)
+  if (uniform_i32(st.cont)) {
+    if (rescale) { APC_TILE_LOOP(true, true); } else { APC_TILE_LOOP(true, false); }
+  } else {
+    if (rescale) { APC_TILE_LOOP(false, true); } else { APC_TILE_LOOP(false, false); }
+  }
+#undef APC_TILE_LOOP
+}
+
+template <int M, int kTileThreads>
+__global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_params p, TableArgs a, int n_tiles,
+                                                                          int xcd_shift) {
+  __shared__ TileStage<M> s_stage;
+  const int64_t tile_id = xcd_chunked_unit(xcd_shift);
+  if (tile_id >= n_tiles) return;
+  const apc_tile tile = a.tiles[tile_id];
+  if (threadIdx.x == 0) s_stage.mixed = 0;
+  __syncthreads();
+  stage_tile<M>(p, a, tile, s_stage, threadIdx.x, kTileThreads);
+  __syncthreads();
+  tile_entries<M>(p, a, s_stage, view_of(tile), threadIdx.x, kTileThreads);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -635,14 +748,24 @@ __global__ __launch_bounds__(kBlock) void segmented_min_kernel(const double *__r
   }
 }
 
-template <int G>
-void launch_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_seg, double *mins, int32_t *args,
-                          hipStream_t stream) {
-  hipLaunchKernelGGL(segmented_min_kernel<G>, dim3((unsigned)((n_seg + kBlock / G - 1) / (kBlock / G))), dim3(kBlock),
-                     0, stream, values, seg_ptr, n_seg, mins, args);
+// 8 XCDs; APC_XCD_SHIFT=0 restores the plain work order (tuning)
+int xcd_shift() {
+  static const int shift = [] {
+    const char *env = getenv("APC_XCD_SHIFT");
+    const int v = env ? atoi(env) : 3;
+    return v < 0 ? 0 : v > 5 ? 5 : v;
+  }();
+  return shift;
 }
 
 inline unsigned blocks_for(int64_t n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
+
+template <int G>
+void launch_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_seg, double *mins, int32_t *args,
+                          hipStream_t stream) {
+  hipLaunchKernelGGL(segmented_min_kernel<G>, dim3(blocks_for(n_seg, kBlock / G)), dim3(kBlock), 0, stream, values,
+                     seg_ptr, n_seg, mins, args);
+}
 
 int check_params(const apc_params *p) {
   if (!p) return fail(-1, "params is NULL");
@@ -709,6 +832,9 @@ int apc_validate_tables_host(const apc_params *params, int64_t n_tensors, const 
                   (long long)e, (long long)edge_entry_begin[e], (long long)expect);
     const int64_t ns = edge_n_src[e], nt = edge_n_tgt[e];
     if (ns < 0 || nt < 0) return fail(-2, "edge %lld: negative strategy count", (long long)e);
+    if (ns > APC_MAX_STRATEGIES || nt > APC_MAX_STRATEGIES)
+      return fail(-2, "edge %lld: %lld x %lld strategies, at most %d a side", (long long)e, (long long)nt,
+                  (long long)ns, APC_MAX_STRATEGIES);
     if (edge_src_begin[e] < 0 || edge_src_begin[e] + ns > n_specs)
       return fail(-2, "edge %lld: producer spec range [%d, +%lld) outside the spec table", (long long)e,
                   edge_src_begin[e], (long long)ns);
@@ -815,7 +941,7 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
                             const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *trans_out,
                             double *cost_out, void *stream) {
   if (int rc = check_params(params)) return rc;
-  if (n_tiles < 0 || n_tiles > INT32_MAX) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
+  if (n_tiles < 0 || n_tiles > (1 << 30)) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tiles == 0) return 0;
   if (n_entries < 0) return fail(-1, "n_entries < 0");
   if (!tensor_bytes || !tensor_contiguous || !spec_codes || !spec_tensor || !tiles)
@@ -823,16 +949,17 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
   if (cost_out && !per_arg) return fail(-1, "cost_out needs compute_cost_per_arg");
   TableArgs a{tensor_bytes, tensor_contiguous, spec_codes, spec_tensor, pt_values, per_arg,
               tiles,        dup_entry_begin,   comm_out,   trans_out,   cost_out};
-  const dim3 grid((unsigned)n_tiles);
+  const int nt = (int)n_tiles, xs = xcd_shift();
   hipStream_t s = (hipStream_t)stream;
-  // small matrices (traced graphs): one wavefront per tile; large ones: two wavefronts share
-  // the staged specs and terms of a tile
-  // (n_entries counts the copies written for de-duplicated edges too: work per tile either way)
-  bool wide = n_entries / n_tiles >= 512;
-  if (const char *env = getenv("APC_TILE_THREADS")) wide = atoi(env) >= 128;  // tuning override
-#define APC_LAUNCH(M_)                                                                                  \
-  if (wide) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 128>), grid, dim3(128), 0, s, *params, a); \
-  else hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 64>), grid, dim3(64), 0, s, *params, a)
+  // small matrices (traced graphs): one wavefront per tile; larger ones: two wavefronts share a
+  // tile's staged inputs.  (n_entries counts the copies written for de-duplicated edges too:
+  // work per tile either way.)
+  const dim3 grid((unsigned)(((n_tiles + (1 << xs) - 1) >> xs) << xs));  // rounded up for xcd_chunked_unit
+  int threads = n_entries / n_tiles >= 512 ? 128 : 64;
+  if (const char *env = getenv("APC_TILE_THREADS")) threads = atoi(env);  // tuning override
+#define APC_LAUNCH(M_)                                                                                         \
+  if (threads >= 128) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 128>), grid, dim3(128), 0, s, *params, a, nt, xs); \
+  else hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 64>), grid, dim3(64), 0, s, *params, a, nt, xs)
   switch (params->mesh_ndim) {
     case 1: APC_LAUNCH(1); break;
     case 2: APC_LAUNCH(2); break;
