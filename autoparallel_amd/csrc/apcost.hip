@@ -724,13 +724,22 @@ __global__ __launch_bounds__(kBlock) void segmented_min_kernel(const double *__r
   const int64_t lo = live ? seg_ptr[seg] : 0, hi = live ? seg_ptr[seg + 1] : 0;
   double best = INFINITY;
   int64_t arg = INT64_MAX;  // absolute index; INT64_MAX = none seen
-  for (int64_t j = lo + sub; j < hi; j += G) {
-    const double v = values[j];
+  auto take = [&](double v, int64_t j) {
     if (arg == INT64_MAX || v < best) {
       best = v;
       arg = j;
     }
+  };
+  // four independent loads in flight per lane, taken in index order (first minimum wins)
+  int64_t j = lo + sub;
+  for (; j + 3 * G < hi; j += 4 * G) {
+    const double v0 = values[j], v1 = values[j + G], v2 = values[j + 2 * G], v3 = values[j + 3 * G];
+    take(v0, j);
+    take(v1, j + G);
+    take(v2, j + 2 * G);
+    take(v3, j + 3 * G);
   }
+  for (; j < hi; j += G) take(values[j], j);
   // lexicographic (value, index) min inside the group; lanes that saw nothing lose
 #pragma unroll
   for (int off = G / 2; off > 0; off >>= 1) {
@@ -977,10 +986,12 @@ int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_se
   if (!seg_ptr || !mins || !args || (!values && n_values > 0)) return fail(-1, "apc_segmented_min: NULL array");
   if (n_seg > (int64_t)INT32_MAX * 4) return fail(-1, "n_segments %lld too large", (long long)n_seg);
   hipStream_t s = (hipStream_t)stream;
-  // lanes per segment: about a quarter of the mean length, so most lanes of a group have work in every
-  // pass over their segment (APC_SEGMIN_GROUP overrides, for tuning)
+  // lanes per segment: about a tenth of the mean length, so that a lane has several
+  // independent loads in flight (measured best on both benchmark tables; APC_SEGMIN_GROUP
+  // overrides, for tuning)
   const double mean = (double)n_values / (double)n_seg;
-  int g = mean <= 16 ? 4 : mean <= 64 ? 8 : mean <= 256 ? 16 : mean <= 1024 ? 32 : 64;
+  int g = 2;
+  while (g < 64 && g * 12 <= mean) g *= 2;
   if (const char *env = getenv("APC_SEGMIN_GROUP")) g = atoi(env);
   switch (g) {
     case 1: launch_segmented_min<1>(values, seg_ptr, n_seg, mins, args, s); break;

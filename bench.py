@@ -28,6 +28,16 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 
+# HBM bytes per launch of the redistribution kernel, measured with rocprofv3 --pmc
+# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, KiB per dispatch; the factors come from the same
+# counters read on a plain 1 GiB copy, --calibrate-copy).  A hardware counter cannot be read
+# from inside this process, so the figure is the one of the profiled run of the same command
+# and only reported for exactly that table: (entries, tiles, algorithmic bytes) must match.
+MEASURED_TRAFFIC_BYTES = {
+    (1_821_368, 1_616, 32_348_914): (670.7 * 2.000 + 31_430.3) * 1024,             # llama3_8b, mesh (32, 8)
+    (464_235_576, 498_134, 8_003_825_874): (164_953.0 * 2.000 + 7_724_841.2) * 1024,  # stress, mesh (16, 8, 4)
+}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -270,7 +280,8 @@ def main():
                    "devices_per_host": 8, "step": "tensor_tables + spec_tables + compute_costs + "
                                                    "redistribute_tables(comm, transition, cost) + segmented_min(rows)"},
         "roofline": {"bound": "hbm", "kernel": "redistribute_tiles_kernel", "achieved": achieved,
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((E, tables.n_tiles, alg_bytes)),
                      "algorithmic_bytes_per_launch": alg_bytes,
                      "avg_launch_us": t_kernel * 1e6, "min_launch_us": kernel_ms_min["redistribute_tables"] * 1e3,
                      "timing": "HIP events around every launch of the kernel inside the timed region"},
