@@ -11,12 +11,15 @@ Applying the plan (re-tracing with collectives, compilation) is outside this pac
 
 from __future__ import annotations
 
+import logging
 import time
 
 import torch
 
 from .graphs.capture import capture_joint_graph
 from .optimize_sharding import ShardingOptimizer
+
+logger = logging.getLogger(__name__)
 
 
 class AutoParallelPlanner:
@@ -42,6 +45,7 @@ class AutoParallelPlanner:
                                         device=self.trace_device)
         self.gm, self.joint_with_descriptors = self._ctx.__enter__()
         self.timings["capture_s"] = time.perf_counter() - t0
+        logger.info("%s %.3f s", "capture_s", self.timings["capture_s"])
         # api.py:264-272: gradients reduced in a wider dtype than the parameters cost more to
         # communicate; x1.1 breaks the tie towards reducing in the wider dtype
         rescale = 1.0
@@ -54,6 +58,7 @@ class AutoParallelPlanner:
                                                      repeated_subgraphs=self.repeated_subgraphs)
         self.sharding_optimizer.add_grad_param_constraints()
         self.timings["optimizer_s"] = time.perf_counter() - t0
+        logger.info("%s %.3f s", "optimizer_s", self.timings["optimizer_s"])
         self.timings.update({f"optimizer_{k}": v for k, v in self.sharding_optimizer.timings.items()})
         return self
 
@@ -86,6 +91,7 @@ class AutoParallelPlanner:
         t0 = time.perf_counter()
         self.sharding_placement = self.sharding_optimizer.get_solution(verbose=False)
         self.timings["solve_s"] = time.perf_counter() - t0
+        logger.info("%s %.3f s", "solve_s", self.timings["solve_s"])
         if verbose:
             print(self.sharding_optimizer.get_log())
         if self.sharding_optimizer.prob.status == -1:

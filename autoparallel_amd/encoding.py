@@ -31,6 +31,7 @@ from __future__ import annotations
 
 import ctypes
 from dataclasses import dataclass, fields
+from typing import Optional
 
 import numpy as np
 
@@ -47,7 +48,14 @@ PARTIAL_OPS = ("sum", "avg", "min", "max", "product", "band", "bor", "bxor")
 EDGE_GRAD_RESCALE = _native.EDGE_GRAD_RESCALE
 EDGE_NO_PRODUCER = _native.EDGE_NO_PRODUCER
 
-DEFAULT_TILE_ENTRIES = 2048
+# Tiling chosen when the caller names no tile size (measured on one MI355X): an edge matrix of
+# up to 64 x 64 entries is best served by one tile (its producer specs and cost terms are
+# staged once); a table that would then have too few tiles to fill the chip several times
+# over is cut finer (fewer copies per tiled edge first, then smaller tiles), as long as a
+# tile still stores a few thousand entries.
+AUTO_MIN_TILES = 32768
+AUTO_MIN_STORED_PER_TILE = 2048
+AUTO_MIN_TILE_ENTRIES = 512
 
 # numpy mirror of the C struct apc_tile (64 bytes)
 TILE_DTYPE = np.dtype([
@@ -137,6 +145,7 @@ class CostTables:
     dup_entry_begin: np.ndarray = None  # entry offsets of the duplicates, grouped by canonical edge
     edge_dup_begin: np.ndarray = None
     edge_dup_count: np.ndarray = None
+    tiling: dict = None  # tile size and copies per tiled edge of the current tiling
 
     _DTYPES = {
         "tensor_rank": np.int32, "tensor_itemsize": np.int32, "tensor_shape": np.int64,
@@ -231,21 +240,38 @@ class CostTables:
             out.append(h.digest())
         return out
 
-    def build_tiles(self, tile_entries: int = DEFAULT_TILE_ENTRIES, dedupe: bool = False,
-                    max_copies: int = 8) -> None:
+    def build_tiles(self, tile_entries: Optional[int] = None, dedupe: bool = False, max_copies: int = 8,
+                    signatures=None) -> None:
         """Cuts every edge matrix into rectangles of about ``tile_entries`` entries:
         whole rows when a row fits the LDS column budget, column chunks otherwise.  With
         ``dedupe`` only the first of every group of identical edges is tiled; its tiles
         store their values to all copies.  (Call it after the strategy table is final:
         the compute-cost inputs are part of an edge's identity.)  One tiled edge serves at
         most ``max_copies - 1`` duplicates, so a long run of identical edges still spreads
-        over many workgroups."""
+        over many workgroups.  ``tile_entries=None`` chooses tile size and copies per tiled
+        edge from the table (``tiling`` records the choice)."""
+        if tile_entries is None:
+            sigs = self.edge_signatures() if dedupe and self.n_edges else None
+            te, mc = APC_TILE_MAX_ROWS * APC_TILE_MAX_COLS, int(max_copies)
+            while True:
+                self.build_tiles(te, dedupe, mc, signatures=sigs)
+                n = self.n_tiles
+                if n == 0 or n >= AUTO_MIN_TILES or self.n_entries / n <= AUTO_MIN_STORED_PER_TILE:
+                    break
+                if dedupe and mc > 2:
+                    mc //= 2
+                elif te > AUTO_MIN_TILE_ENTRIES:
+                    te //= 2
+                else:
+                    break
+            return
+        self.tiling = {"tile_entries": int(tile_entries), "max_copies": int(max_copies) if dedupe else 1}
         ns = self.edge_n_src.astype(np.int64)
         nt = self.edge_n_tgt.astype(np.int64)
         canonical = np.arange(self.n_edges, dtype=np.int64)
         if dedupe and self.n_edges:
             first: dict = {}  # signature -> [canonical edge, copies it already serves]
-            for e, sig in enumerate(self.edge_signatures()):
+            for e, sig in enumerate(signatures if signatures is not None else self.edge_signatures()):
                 slot = first.get(sig)
                 if slot is None or slot[1] >= min(APC_TILE_MAX_DUPS, max(int(max_copies) - 1, 0)):
                     first[sig] = [e, 0]  # a new canonical edge (also when the previous one is full)

@@ -26,6 +26,7 @@ There is no CPU path for the tables: without a HIP device construction raises.
 
 from __future__ import annotations
 
+import logging
 import math
 import operator
 import time
@@ -42,6 +43,8 @@ from .graphs.cost_inputs import fill_flops_and_bytes
 from .graphs.encode import EncodedGraph, all_input_nodes, encode_graph
 from .graphs.strategies import StrategyEnumerator
 from .ilp import BinaryProgram, next_name
+
+logger = logging.getLogger(__name__)
 
 
 class DeviceBackend:
@@ -60,7 +63,7 @@ class DeviceBackend:
             out = self.dev.run_spec_tables()
             return out["local_shape"].cpu().numpy(), out["local_stride"].cpu().numpy()
 
-    def upload_strategy_inputs(self, tables, tile_entries=2048, dedupe=True, max_copies=8):
+    def upload_strategy_inputs(self, tables, tile_entries=None, dedupe=True, max_copies=8):
         """The strategy table is final: tile the edges (identical edges once) and send both."""
         tables.build_tiles(tile_entries, dedupe=dedupe, max_copies=max_copies)
         tables.validate(self.dev.params)
@@ -79,6 +82,7 @@ class DeviceBackend:
         d.build_all()
         torch.cuda.synchronize(d.device)
         self.timings["kernels_s"] = time.perf_counter() - t0
+        logger.info("%s %.3f s", "kernels_s", self.timings["kernels_s"])
         t0 = time.perf_counter()
         out = {
             "comm": d.comm.cpu().numpy(),
@@ -87,6 +91,7 @@ class DeviceBackend:
             "compute_per_arg": d.compute_cost_per_arg.cpu().numpy(),
         }
         self.timings["copy_back_s"] = time.perf_counter() - t0
+        logger.info("%s %.3f s", "copy_back_s", self.timings["copy_back_s"])
         return out
 
     def row_min(self, row_ptr):
@@ -204,9 +209,10 @@ class ShardingOptimizer:
     device = "cuda:0"
     backend_cls = DeviceBackend
     solver_time_limit: Optional[float] = None
-    # tiling of the edge matrices: entries per tile, whether identical edges (repeated layers)
-    # are evaluated once, and how many copies one evaluated edge may serve
-    tile_entries = 2048
+    # tiling of the edge matrices: entries per tile (None: chosen from the table), whether
+    # identical edges (repeated layers) are evaluated once, and how many copies one evaluated
+    # edge may serve at most
+    tile_entries = None
     dedupe = True
     max_copies = 8
 
@@ -221,6 +227,7 @@ class ShardingOptimizer:
         t0 = time.perf_counter()
         self.strats = self.build_sharding_metadata()
         self.timings["enumerate_s"] = time.perf_counter() - t0
+        logger.info("%s %.3f s", "enumerate_s", self.timings["enumerate_s"])
 
         self.node_representative = {}
         if repeated_subgraphs:
@@ -229,6 +236,7 @@ class ShardingOptimizer:
             t0 = time.perf_counter()
             self.node_representative = cluster_nodes(self.graph, self.strats)
             self.timings["cluster_s"] = time.perf_counter() - t0
+            logger.info("%s %.3f s", "cluster_s", self.timings["cluster_s"])
         self.ds, self.num_inp_out, self.num_args = self.build_ds()
         self.validate()
         self.cluster_links = ClusterLinks(self)
@@ -262,20 +270,24 @@ class ShardingOptimizer:
         self.encoded: EncodedGraph = encode_graph(self.graph, self.strats, tuple(self.mesh.shape),
                                                   self._grad_param_nodes())
         self.timings["encode_s"] = time.perf_counter() - t0
+        logger.info("%s %.3f s", "encode_s", self.timings["encode_s"])
         self.params = self.cost_model_params()
         tb = self.encoded.tables
         t0 = time.perf_counter()
         self.backend = self.backend_cls(tb, self.params, self.device)
         local_shape, local_stride = self.backend.local_shapes()
         self.timings["upload_and_shapes_s"] = time.perf_counter() - t0
+        logger.info("%s %.3f s", "upload_and_shapes_s", self.timings["upload_and_shapes_s"])
         t0 = time.perf_counter()
         self.cost_input_stats = {}
         fill_flops_and_bytes(self.encoded, self.strats, local_shape, local_stride, self.cost_input_stats)
         self.backend.upload_strategy_inputs(tb, self.tile_entries, self.dedupe, self.max_copies)
         self.timings["flops_bytes_s"] = time.perf_counter() - t0
+        logger.info("%s %.3f s", "flops_bytes_s", self.timings["flops_bytes_s"])
         t0 = time.perf_counter()
         out = self.backend.build()
         self.timings["tables_s"] = time.perf_counter() - t0
+        logger.info("%s %.3f s", "tables_s", self.timings["tables_s"])
         self.timings.update({f"backend_{k}": v for k, v in getattr(self.backend, "timings", {}).items()})
         self.comm_cost = out["comm"]
         self.transition_cost = out["transition"]
@@ -287,6 +299,7 @@ class ShardingOptimizer:
         t0 = time.perf_counter()
         self._write_back_redistribute_cost()
         self.timings["write_back_s"] = time.perf_counter() - t0
+        logger.info("%s %.3f s", "write_back_s", self.timings["write_back_s"])
         return CostRecords(self), self.encoded.num_inp_out, self.encoded.num_args
 
     def create_cluster_links(self):

@@ -47,7 +47,7 @@ def parse_args():
     ap.add_argument("--workload", default="llama3_8b", choices=["llama3_8b", "llama3_70b", "block_1k", "stress"])
     ap.add_argument("--layers", type=int, default=None, help="override the number of decoder layers")
     ap.add_argument("--stress-nodes", type=int, default=200_000)
-    ap.add_argument("--tile-entries", type=int, default=None)
+    ap.add_argument("--tile-entries", type=int, default=None, help="entries per tile (default: chosen from the table)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU-baseline sample duration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-solve", action="store_true", help="skip the ILP leg of the plan wall-time")
@@ -100,7 +100,7 @@ def build_workload(args):
             return torch.randint(0, cfg.vocab_size, (batch, seq))
 
     class Optimizer(ShardingOptimizer):
-        tile_entries = args.tile_entries or 2048
+        tile_entries = args.tile_entries
         dedupe = not args.no_dedupe
         max_copies = args.max_copies
 
@@ -128,6 +128,10 @@ def solve_plan(planner, args):
     nd = planner.mesh.ndim
     x_sharding = (Shard(0),) + (Replicate(),) * (nd - 1)
     out_sharding = (Shard(0), Shard(2)) if (nd == 2 and args.workload != "block_1k") else x_sharding
+    if args.workload == "block_1k":
+        # batch 8 does not divide the 64-rank mesh, so no batch-sharded placement exists (the
+        # default constraint would raise, as the reference's does): pin the sequence dim instead
+        x_sharding = out_sharding = (Shard(1),)
     planner.add_input_constraints([x_sharding])
     planner.add_output_constraints([out_sharding])
     constraints_s = time.perf_counter() - t0
@@ -177,6 +181,11 @@ def cpu_baseline(tables, params, target_seconds):
 
 def main():
     args = parse_args()
+    # stage-by-stage progress of the (long, CPU-side) set-up goes to stderr
+    import logging
+
+    logging.basicConfig(stream=sys.stderr, level=logging.INFO, format="[bench %(relativeCreated)8.0f ms] %(message)s")
+    log = logging.getLogger("bench")
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; cost tables shard by edge range without any exchange step, "
               "but no multi-GPU path is part of it. Run with --gpus 1.", file=sys.stderr)
@@ -212,6 +221,7 @@ def main():
         if args.tile_entries:
             tables.build_tiles(args.tile_entries)
         dev = DeviceCostTables(tables, params, device="cuda:0")
+    log.info("tables resident: %d entries, %d tiles", tables.n_entries, tables.n_tiles)
     step = dev.prepare_step(row_min=True)
     torch.cuda.synchronize()
     host_timings["upload_and_prepare_s"] = time.perf_counter() - t0
@@ -256,6 +266,7 @@ def main():
     copy_back_s = time.perf_counter() - t0
     del host_out
 
+    log.info("timed region done: %.3f ms/step", wall_plain / K * 1e3)
     E = tables.n_entries
     alg_bytes = tables.algorithmic_bytes(comm=True, transition=True, cost=True)
     t_kernel = kernel_ms["redistribute_tables"] * 1e-3
@@ -275,7 +286,7 @@ def main():
         "dtype": "f64",
         "data": "synthetic",
         "config": {**desc, "edges": tables.n_edges, "strategies": tables.n_strategies, "specs": tables.n_specs,
-                   "entries": E, "tiles": tables.n_tiles,
+                   "entries": E, "tiles": tables.n_tiles, "tiling": tables.tiling,
                    "edges_deduplicated": int((tables.edge_canonical != np.arange(tables.n_edges)).sum()), "device_row": params.device_name,
                    "devices_per_host": 8, "step": "tensor_tables + spec_tables + compute_costs + "
                                                    "redistribute_tables(comm, transition, cost) + segmented_min(rows)"},
@@ -297,6 +308,7 @@ def main():
     if planner is not None:
         plan = {"stages_s": {k: round(v, 4) for k, v in host_timings.items()}}
         if not args.no_solve:
+            log.info("solving the ILP: %d variables", planner.sharding_optimizer.n_variables)
             plan.update(solve_plan(planner, args))
         table_stage = host_timings.get("optimizer_tables_s", 0.0)
         other = host_timings.get("capture_s", 0.0) + host_timings.get("optimizer_s", 0.0) - table_stage \
