@@ -35,7 +35,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 # and only reported for exactly that table: (entries, tiles, algorithmic bytes) must match.
 MEASURED_TRAFFIC_BYTES = {
     (1_821_368, 1_616, 32_348_914): (670.7 * 2.000 + 31_430.3) * 1024,             # llama3_8b, mesh (32, 8)
-    (464_235_576, 498_134, 8_003_825_874): (164_953.0 * 2.000 + 7_724_841.2) * 1024,  # stress, mesh (16, 8, 4)
+    (73_251_434, 40_727, 1_255_915_920): (12_302.2 * 2.000 + 1_230_763.9) * 1024,   # llama3_70b, mesh (8, 8, 8)
+    (464_235_576, 426_918, 8_003_825_874): (162_205.4 * 2.000 + 7_735_258.4) * 1024,  # stress, mesh (16, 8, 4)
 }
 
 
