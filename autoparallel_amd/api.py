@@ -26,7 +26,7 @@ class AutoParallelPlanner:
     optimizer_cls = ShardingOptimizer
 
     def __init__(self, model, input_fn, mesh, param_dtype=None, reduce_dtype=None, repeated_subgraphs=False,
-                 device="cpu"):
+                 device="cpu", dynamo=False):
         self.model = model
         self.input_fn = input_fn
         self.mesh = mesh
@@ -34,6 +34,7 @@ class AutoParallelPlanner:
         self.reduce_dtype = reduce_dtype
         self.repeated_subgraphs = repeated_subgraphs
         self.trace_device = device
+        self.dynamo = dynamo  # capture the forward with Dynamo first: needed for local_map regions
         self.timings = {}
         self._ctx = None
         self.input_constraints = None
@@ -42,7 +43,7 @@ class AutoParallelPlanner:
     def __enter__(self):
         t0 = time.perf_counter()
         self._ctx = capture_joint_graph(self.model, self.input_fn, param_dtype=self.param_dtype,
-                                        device=self.trace_device)
+                                        device=self.trace_device, dynamo=self.dynamo)
         self.gm, self.joint_with_descriptors = self._ctx.__enter__()
         self.timings["capture_s"] = time.perf_counter() - t0
         logger.info("%s %.3f s", "capture_s", self.timings["capture_s"])

@@ -480,7 +480,9 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
     st.colh[j] = make_uint2(codes, info);
     if (t != t0 || t < 0) mixed = true;
   }
-  for (int j = tid; j < rows; j += nthreads) {
+  // (threads taken from the far end: with two wavefronts one stages the producer specs while
+  // the other stages the consumer specs)
+  for (int j = nthreads - 1 - tid; j < rows; j += nthreads) {
     const int ts = tile.tgt_begin + tile.row_begin + j;
     const uint32_t tg = a.spec_codes[ts];
     // info: bit0 valid spec, bits 1 + 5i .. : 8 x class of mesh dim i, bit 30 every dim is a Shard

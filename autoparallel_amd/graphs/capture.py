@@ -119,12 +119,36 @@ def add_alias_nodes(gm: torch.fx.GraphModule) -> torch.fx.GraphModule:
     return gm
 
 
+def dynamo_capture(model: nn.Module, inputs: tuple) -> torch.fx.GraphModule:
+    """The model's forward as a Dynamo-captured graph module whose parameters keep their
+    fully qualified names, with every ``local_map``-decorated function kept as one
+    higher-order-op call instead of being traced through (api.py:152-192).  The joint
+    export of that module then carries a forward and a backward ``call_local_map`` node per
+    region, tagged with the region's declared placements (``meta["local_map_kwargs"]``)."""
+    from torch._dynamo.functional_export import _dynamo_graph_capture_for_export
+    from torch._dynamo.variables.higher_order_ops import LocalMapWrappedHigherOrderVariable
+    from torch._higher_order_ops import local_map as local_map_module
+    from torch.export._trace import _restore_state_dict
+
+    def forward(*args):
+        return model(*args)
+
+    with LocalMapWrappedHigherOrderVariable.enable(), local_map_module.defer_inlining(), \
+            torch._dynamo.utils._disable_saved_tensors_hooks_during_tracing(), \
+            torch._dynamo.config.patch(install_free_tensors=True):
+        gm = _dynamo_graph_capture_for_export(forward)(*inputs)
+        _restore_state_dict(model, gm)
+    return gm
+
+
 @contextlib.contextmanager
 def capture_joint_graph(model: nn.Module, input_fn, param_dtype: torch.dtype | None = None, device="cpu",
-                        add_aliases: bool = True):
+                        add_aliases: bool = True, dynamo: bool = False):
     """Context manager yielding ``(gm, joint_with_descriptors)`` for ``model`` (built on
     the meta device) and ``input_fn`` (called under the fake mode; returns a tensor or a
-    tuple of tensors).  The fake mode stays usable inside the ``with`` block."""
+    tuple of tensors).  The fake mode stays usable inside the ``with`` block.  ``dynamo``
+    captures the forward with Dynamo first (needed for models with ``local_map`` regions,
+    which plain AOT tracing would inline)."""
     from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
 
     fake_mode = FakeTensorMode()
@@ -136,6 +160,12 @@ def capture_joint_graph(model: nn.Module, input_fn, param_dtype: torch.dtype | N
     if not isinstance(inputs, tuple):
         inputs = (inputs,)
     with contextlib.ExitStack() as stack:
+        if dynamo:
+            from torch._higher_order_ops import local_map as local_map_module
+
+            # the joint export must not inline the regions either
+            stack.enter_context(local_map_module.defer_inlining())
+            model = dynamo_capture(model, inputs)
         joint = aot_export_joint_with_descriptors(stack, model, inputs, decompositions=decomposition_table())
         gm = joint.graph_module
         for node in gm.graph.nodes:

@@ -34,7 +34,7 @@ import operator
 import torch
 from torch.distributed.tensor._dtensor_spec import DTensorSpec, TensorMeta
 from torch.distributed.tensor._op_schema import OpSchema, OpSpec, OpStrategy, RuntimeSchemaInfo, TupleStrategy
-from torch.distributed.tensor.placement_types import Replicate, Shard
+from torch.distributed.tensor.placement_types import Placement, Replicate, Shard
 from torch.utils._pytree import tree_flatten, tree_map_only
 
 logger = logging.getLogger(__name__)
@@ -195,8 +195,9 @@ class StrategyEnumerator:
                     strats[node] = self._placeholder(val)
                 elif node.op == "call_function":
                     if node.meta.get("local_map_kwargs"):
-                        raise NotImplementedError("local_map regions are not supported by this enumerator yet")
-                    strats[node] = self._call_function(node, strats)
+                        strats[node] = self._local_map(node, strats)
+                    else:
+                        strats[node] = self._call_function(node, strats)
                 elif node.op == "output":
                     strats[node] = tree_map_only(torch.fx.Node, lambda x: strats[x], node.args)
                 else:
@@ -204,6 +205,50 @@ class StrategyEnumerator:
         return strats
 
     # ------------------------------------------------------------------------------------
+    def _local_map(self, node, strats) -> OpStrategy:
+        """A ``local_map`` region (forward or backward call of the higher-order op) has exactly
+        one strategy: the placements its author declared (optimize_sharding.py:174-196,
+        utils.py:195-313).  Leading arguments beyond the declared ones are activations saved
+        by the forward call and are replicated, as are outputs beyond the declared ones;
+        ``None`` / SymInt slots carry no spec.  The cost rows are placeholders: the cost
+        kernels recompute every entry from the specs."""
+        kw = node.meta["local_map_kwargs"]
+        if kw.get("in_placements") is None or kw.get("out_placements") is None:
+            raise NotImplementedError(f"{node}: local_map regions need in_placements and out_placements")
+        if kw.get("in_grad_placements") is not None:
+            raise NotImplementedError(f"{node}: local_map in_grad_placements are not supported")
+        if kw.get("device_mesh") not in (self.mesh, None):
+            raise NotImplementedError(f"{node}: local_map region declared on another device mesh")
+        if node.kwargs:
+            raise NotImplementedError(f"{node}: keyword arguments of a local_map call")
+        mesh = self.mesh
+        replicated = tuple(Replicate() for _ in range(mesh.ndim))
+
+        def spec_of(example, placements):
+            if example is None or placements is None or not isinstance(example, torch.Tensor):
+                return None
+            if isinstance(placements, Placement):
+                placements = (placements,)
+            return DTensorSpec(mesh=mesh, placements=tuple(placements), tensor_meta=_tensor_meta(example))
+
+        args = [a.meta["val"] if isinstance(a, torch.fx.Node) else a for a in node.args]
+        in_placements = list(kw["in_placements"])
+        n_saved = len(args) - len(in_placements)
+        if n_saved < 0:
+            raise RuntimeError(f"{node}: {len(in_placements)} input placements for {len(args)} arguments")
+        in_specs = [spec_of(a, replicated) for a in args[:n_saved]]
+        in_specs += [spec_of(a, p) for a, p in zip(args[n_saved:], in_placements)]
+        val = node.meta["val"]
+        outs = list(val) if isinstance(val, (list, tuple)) else [val]
+        out_placements = list(kw["out_placements"])
+        out_specs = [spec_of(o, p) for o, p in zip(outs, out_placements)]
+        out_specs += [spec_of(o, replicated) for o in outs[len(out_placements):]]
+        rows = []
+        for a in node.args:
+            producer = strats[a] if isinstance(a, torch.fx.Node) else None
+            rows.append(_zero_row(producer) if isinstance(producer, OpStrategy) else [0.0])
+        return OpStrategy([OpSpec(tuple(out_specs), input_specs=tuple(in_specs), redistribute_cost=rows)])
+
     def _signature(self, strategy) -> int:
         """A small integer naming the list of output specs of an OpStrategy."""
         if isinstance(strategy, OpStrategy):

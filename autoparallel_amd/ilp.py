@@ -33,6 +33,9 @@ class BinaryProgram:
         self._ub: list = []
         self._names: list = []
         self.upper = np.ones(self.n_vars, np.float64)  # variable upper bounds (0 = forced off)
+        # 1 = the variable must be integral, 0 = continuous in [0, upper] (a planner may leave
+        # variables continuous whose integrality follows from that of others)
+        self.integrality = np.ones(self.n_vars, np.float64)
         self.objective = np.zeros(self.n_vars, np.float64)
         self.status = None
         self.x = None
@@ -125,7 +128,7 @@ class BinaryProgram:
         if mip_rel_gap is not None:
             options["mip_rel_gap"] = float(mip_rel_gap)
         constraints = [LinearConstraint(a, lb, ub)] if self._names else []
-        res = milp(self.objective, integrality=np.ones(self.n_vars), bounds=Bounds(np.zeros(self.n_vars), self.upper),
+        res = milp(self.objective, integrality=self.integrality, bounds=Bounds(np.zeros(self.n_vars), self.upper),
                    constraints=constraints, options=options)
         self.solve_seconds = time.time() - t0
         self.raw = res

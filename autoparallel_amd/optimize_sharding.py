@@ -215,6 +215,12 @@ class ShardingOptimizer:
     tile_entries = None
     dedupe = True
     max_copies = 8
+    # ILP formulation: besides the reference's one binary per cost entry, one binary per (node,
+    # strategy) tied to the entry variables of that strategy's row.  Only these need to be
+    # declared integral: with a node's and its producers' choices fixed to unit vectors the
+    # row / column sum constraints leave exactly one feasible (integral) value for every entry
+    # variable.  Same feasible plans and optimum, far fewer branching variables for the solver.
+    node_choice_variables = True
 
     def __init__(self, gm, mesh, rescale_grad_comm_cost_for_mp=1.0, repeated_subgraphs=False):
         self.gm = gm
@@ -241,7 +247,7 @@ class ShardingOptimizer:
         self.validate()
         self.cluster_links = ClusterLinks(self)
         self.create_cluster_links()
-        self.prob = BinaryProgram(self.n_variables, "AutoParallel")
+        self.prob = BinaryProgram(self.n_variables + self.n_choice_variables, "AutoParallel")
         self.res = None
         self.add_default_constraints()
 
@@ -324,6 +330,19 @@ class ShardingOptimizer:
         self.var_of_entry = inverse.astype(np.int64)
         self.n_variables = len(uniq)
         self._linked_entry = var != ident
+        # choice variables: one per (node, strategy), shared with the node's representative
+        self.n_choice_variables = 0
+        self.choice_var_of_strategy = None
+        if self.node_choice_variables:
+            sb = self.encoded.strat_begin
+            choice = np.arange(tb.n_strategies, dtype=np.int64)
+            for node, rep in self.node_representative.items():
+                s1, s0 = self.node_map[node], self.node_map[rep]
+                n = len(self.strats[node].strategies)
+                choice[sb[s1]:sb[s1] + n] = np.arange(sb[s0], sb[s0] + n)
+            uniq_c, inverse_c = np.unique(choice, return_inverse=True)
+            self.choice_var_of_strategy = self.n_variables + inverse_c.astype(np.int64)
+            self.n_choice_variables = len(uniq_c)
 
     def _write_back_redistribute_cost(self):
         tb = self.encoded.tables
@@ -410,7 +429,29 @@ class ShardingOptimizer:
         self.prob.force_zero(self.var_of_entry[bad])
         self.inf_entries = bad
 
+    def add_choice_link_constraint(self):
+        """choice[node, strategy] = sum of the entry variables of that strategy's row of the
+        node's first argument; entry variables become continuous."""
+        tb = self.encoded.tables
+        cols, vals, lens = [], [], []
+        for s_i, node in enumerate(self.nodes):
+            if node.op == "output":
+                continue
+            b, nt, ns = self._edge(s_i, 0)
+            sb = self.encoded.strat_begin[s_i]
+            entries = self.var_of_entry[b + np.arange(nt)[:, None] * ns + np.arange(ns)[None, :]]
+            choice = self.choice_var_of_strategy[sb + np.arange(nt)][:, None]
+            cols.append(np.concatenate([entries, choice], axis=1).ravel())
+            vals.append(np.tile(np.concatenate([np.ones(ns), [-1.0]]), nt))
+            lens.append(np.full(nt, ns + 1))
+        if cols:
+            self.prob.add_rows(np.concatenate(cols), np.concatenate(vals), np.concatenate(lens), 0.0, 0.0,
+                               "choice_link")
+        self.prob.integrality[:self.n_variables] = 0.0
+
     def add_default_constraints(self):
+        if self.node_choice_variables:
+            self.add_choice_link_constraint()
         self.add_unique_decision_constraint()
         self.add_same_output_across_args_constraint()
         self.add_output_input_consistent_constraint()

@@ -8,6 +8,7 @@ The CPU tests build the tables with the oracle (test backend); the GPU tests bui
 with the HIP kernels and additionally require bit-identical tables and the identical
 plan and objective from the same solver."""
 
+import math
 import warnings
 
 import numpy as np
@@ -37,7 +38,8 @@ def meshes(fake_pg):
     with warnings.catch_warnings():
         warnings.simplefilter("ignore")
         return {"1d": init_device_mesh("cpu", (256,), mesh_dim_names=("dp",)),
-                "2d": init_device_mesh("cpu", (32, 8), mesh_dim_names=("dp", "tp"))}
+                "2d": init_device_mesh("cpu", (32, 8), mesh_dim_names=("dp", "tp")),
+                "3d": init_device_mesh("cpu", (8, 8, 4), mesh_dim_names=("dp", "tp", "cp"))}
 
 
 def _plan(planner_cls, mesh, kind, high_mem):
@@ -130,6 +132,72 @@ def test_reference_golden_plans_2d_with_oracle_tables(meshes, kind):
     assert "total_cost" in log and "Violated constraints: []" in log
 
 
+def _plan_local_map(planner_cls, mesh):
+    """tests/test_optimize_placement.py:425-452"""
+    model_fn, input_fn = make_model_and_inputs(mesh, "local_map_block")
+    with torch.device("meta"):
+        model = model_fn()
+    with planner_cls(model, input_fn, mesh, dynamo=True) as autop:
+        autop.add_parameter_memory_constraint(low=None, high=None)
+        x_sharding = (Shard(0), Replicate(), Shard(1))
+        autop.add_input_constraints([x_sharding])
+        autop.add_output_constraints([x_sharding])
+        placement = autop.optimize_placement()
+        return autop, placement
+
+
+def _check_local_map(autop, placement):
+    """The expectations of tests/test_optimize_placement.py:454-493.  The number of
+    activations the forward call saves depends on the attention kernel the trace
+    dispatches to (the reference counts 7 on a CUDA device); their placement does not."""
+    regions = [n for n in autop.gm.graph.nodes if "local_map_kwargs" in n.meta]
+    assert len(regions) == 2, "expected a forward and a backward call"
+    fw, bw = placement[regions[0]], placement[regions[1]]
+    rep = (Replicate(), Replicate(), Replicate())
+    q, k, v = fw.input_specs
+    assert q.placements == (Shard(0), Shard(1), Shard(2))
+    assert k.placements == v.placements == (Shard(0), Shard(1), Replicate())
+    out, *saved = fw.output_specs
+    assert out.placements == (Shard(0), Shard(1), Shard(2)) and len(saved) >= 3
+    assert all(s.placements == rep for s in saved if s is not None)
+    *saved_in, grad_out = bw.input_specs
+    assert len(saved_in) == len(saved)
+    assert grad_out.placements == (Shard(0), Shard(1), Shard(2))
+    assert all(s.placements == rep for s in saved_in if s is not None)
+    gq, gk, gv = bw.output_specs
+    assert gq.placements == (Shard(0), Shard(1), Shard(2))
+    assert gk.placements == gv.placements == (Shard(0), Shard(1), Replicate())
+
+
+def test_local_map_placements_are_respected_with_oracle_tables(meshes):
+    autop, placement = _plan_local_map(OraclePlanner, meshes["3d"])
+    _check_local_map(autop, placement)
+    assert not autop.sharding_optimizer.prob.violated_constraints()
+    # the plan honours the pinned input / output placement around the region
+    from torch._functorch._aot_autograd.fx_utils import get_plain_input_and_grad_nodes
+
+    ((x, grad_x),) = get_plain_input_and_grad_nodes(autop.gm.graph).values()
+    assert placement[x].output_specs.placements == (Shard(0), Replicate(), Shard(1))
+    assert placement[grad_x].output_specs.placements == (Shard(0), Replicate(), Shard(1))
+
+
+def test_parameter_smaller_than_the_mesh_stays_replicated(meshes):
+    """tests/test_optimize_placement.py:496-533: a parameter with fewer elements than the
+    mesh has ranks is left out of the memory constraint and ends up replicated."""
+    mesh = meshes["1d"]
+    model_fn, input_fn = make_model_and_inputs(mesh, "small_param")
+    with torch.device("meta"):
+        model = model_fn()
+    with OraclePlanner(model, input_fn, mesh) as autop:
+        autop.add_input_constraints([(Shard(0),)])
+        autop.add_parameter_memory_constraint()
+        placement = autop.optimize_placement()
+        params = list(get_param_nodes(autop.gm.graph))
+        assert len(params) == 1
+        for node in params:
+            assert placement[node].output_specs.placements == (Replicate(),)
+
+
 def test_unsolvable_problem_raises(meshes):
     model_fn, input_fn = make_model_and_inputs(meshes["2d"], "ffn")
     with torch.device("meta"):
@@ -171,3 +239,36 @@ def test_device_tables_give_identical_tables_plan_and_objective(gpu_device, mesh
     dm, da = d.row_minima()
     om, oa = o.row_minima()
     assert np.array_equal(dm, om) and np.array_equal(da, oa)
+
+
+@pytest.mark.parametrize("kind,mesh_key", [("ffn", "2d"), ("block", "1d")])
+def test_node_choice_variables_do_not_change_the_optimum(meshes, kind, mesh_key):
+    """Declaring only the per-(node, strategy) variables integral is a reformulation: the
+    reference's all-binary program has the same optimum."""
+
+    class AllBinaryOptimizer(OracleOptimizer):
+        node_choice_variables = False
+
+    class AllBinaryPlanner(AutoParallelPlanner):
+        optimizer_cls = AllBinaryOptimizer
+
+    a, plan_a = _plan(OraclePlanner, meshes[mesh_key], kind, None)
+    b, plan_b = _plan(AllBinaryPlanner, meshes[mesh_key], kind, None)
+    oa, ob = a.sharding_optimizer, b.sharding_optimizer
+    assert oa.n_choice_variables > 0 and ob.n_choice_variables == 0
+    assert oa.prob.n_vars == oa.n_variables + oa.n_choice_variables and ob.prob.n_vars == ob.n_variables
+    assert math.isclose(oa.objective_value(), ob.objective_value(), rel_tol=1e-12)
+    assert not oa.prob.violated_constraints() and not ob.prob.violated_constraints()
+
+
+@pytest.mark.gpu
+def test_local_map_plan_from_device_tables(gpu_device, meshes):
+    dev_autop, dev_plan = _plan_local_map(AutoParallelPlanner, meshes["3d"])
+    ora_autop, ora_plan = _plan_local_map(OraclePlanner, meshes["3d"])
+    d, o = dev_autop.sharding_optimizer, ora_autop.sharding_optimizer
+    assert type(d.backend).__name__ == "DeviceBackend"
+    assert np.array_equal(d.comm_cost, o.comm_cost)
+    assert np.array_equal(d.transition_cost, o.transition_cost)
+    assert np.array_equal(d.cost, o.cost)
+    assert d.res == o.res and d.objective_value() == o.objective_value()
+    _check_local_map(dev_autop, dev_plan)
