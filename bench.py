@@ -45,7 +45,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="llama3_8b", choices=["llama3_8b", "llama3_70b", "block_1k", "stress"])
+    ap.add_argument("--workload", default="llama3_8b", choices=["llama3_8b", "llama3_70b", "dsv3_moe", "block_1k", "stress"])
     ap.add_argument("--layers", type=int, default=None, help="override the number of decoder layers")
     ap.add_argument("--stress-nodes", type=int, default=200_000)
     ap.add_argument("--tile-entries", type=int, default=None, help="entries per tile (default: chosen from the table)")
@@ -78,27 +78,15 @@ def build_workload(args):
 
     # traced workloads go through the product path: capture -> ShardingOptimizer (which
     # enumerates, clusters, encodes, builds the device tables and copies them back)
-    import dataclasses
-
     import torch
 
     from autoparallel_amd.api import AutoParallelPlanner
     from autoparallel_amd.graphs import workloads
-    from autoparallel_amd.graphs.llama3 import Llama, SingleBlock
     from autoparallel_amd.optimize_sharding import ShardingOptimizer
 
-    cfg, mesh_sizes, batch, seq = workloads.WORKLOADS[args.workload]
-    if args.layers is not None:
-        cfg = dataclasses.replace(cfg, n_layers=args.layers)
+    mesh_sizes = workloads.WORKLOADS[args.workload][1]
     mesh = workloads.logical_mesh(mesh_sizes)
-    with torch.device("meta"):
-        model = SingleBlock(cfg) if args.workload == "block_1k" else Llama(cfg)
-    if args.workload == "block_1k":
-        def input_fn():
-            return torch.randn(batch, seq, cfg.dim, dtype=torch.bfloat16, requires_grad=True)
-    else:
-        def input_fn():
-            return torch.randint(0, cfg.vocab_size, (batch, seq))
+    model, input_fn, workload_desc, needs_dynamo = workloads.build_model(args.workload, mesh, n_layers=args.layers)
 
     class Optimizer(ShardingOptimizer):
         tile_entries = args.tile_entries
@@ -109,12 +97,10 @@ def build_workload(args):
         optimizer_cls = Optimizer
 
     planner = Planner(model, input_fn, mesh, param_dtype=torch.bfloat16, reduce_dtype=torch.float32,
-                      repeated_subgraphs=not args.no_clustering)
+                      repeated_subgraphs=not args.no_clustering, dynamo=needs_dynamo)
     planner.__enter__()
     opt = planner.sharding_optimizer
-    desc = {"workload": f"{args.workload} joint fwd+bwd graph ({cfg.n_layers} layers, dim {cfg.dim}, "
-                        f"batch {batch}, seq {seq}, bf16 params / fp32 reduce), logical mesh {tuple(mesh_sizes)}",
-            "mesh": list(mesh_sizes), "graph_nodes": len(opt.nodes), "ilp_variables": opt.n_variables,
+    desc = {"workload": workload_desc, "mesh": list(mesh_sizes), "graph_nodes": len(opt.nodes), "ilp_variables": opt.n_variables,
             "clustered_nodes": len(opt.node_representative)}
     return opt.encoded.tables, opt.params, desc, opt.backend.dev, planner, dict(planner.timings)
 
@@ -129,10 +115,10 @@ def solve_plan(planner, args):
     nd = planner.mesh.ndim
     x_sharding = (Shard(0),) + (Replicate(),) * (nd - 1)
     out_sharding = (Shard(0), Shard(2)) if (nd == 2 and args.workload != "block_1k") else x_sharding
-    if args.workload == "block_1k":
-        # batch 8 does not divide the 64-rank mesh, so no batch-sharded placement exists (the
-        # default constraint would raise, as the reference's does): pin the sequence dim instead
-        x_sharding = out_sharding = (Shard(1),)
+    if args.workload in ("block_1k", "dsv3_moe"):
+        # the batch (8 / 16) does not divide the mesh's first dim, so no batch-sharded placement
+        # exists (the default constraint would raise, as the reference's does): pin the sequence
+        x_sharding = out_sharding = (Shard(1),) + (Replicate(),) * (nd - 1)
     planner.add_input_constraints([x_sharding])
     planner.add_output_constraints([out_sharding])
     constraints_s = time.perf_counter() - t0

@@ -13,6 +13,7 @@ import torch
 
 from autoparallel_amd.api import AutoParallelPlanner
 from autoparallel_amd.graphs import workloads
+from autoparallel_amd.graphs.dsv3 import DeepSeekV3, DeepSeekV3Config
 from autoparallel_amd.graphs.llama3 import LLAMA3_8B, LLAMA3_70B, BLOCK_1K, Llama, LlamaConfig, SingleBlock
 from autoparallel_amd.optimize_sharding import ShardingOptimizer
 from oracle_backend import OracleBackend
@@ -28,17 +29,27 @@ class OraclePlanner(AutoParallelPlanner):
 
 TINY = LlamaConfig(dim=512, n_layers=3, n_heads=8, n_kv_heads=4, vocab_size=2048, ffn_dim_multiplier=1.0,
                    multiple_of=256, max_seq_len=256)
+# the DeepSeek-V3 style configuration with every width divided down: same ops, same graph shape
+TINY_MOE = DeepSeekV3Config(dim=256, n_layers=3, n_dense_layers=1, n_heads=8, q_lora_rank=64, kv_lora_rank=32,
+                            qk_nope_head_dim=16, qk_rope_head_dim=8, v_head_dim=16, inter_dim=512, moe_inter_dim=64,
+                            n_routed_experts=64, top_k=4, vocab_size=1024, max_seq_len=512)
 
 CASES = {
     # name: (config, mesh, batch, seq)
     "block_1k_mesh64": (BLOCK_1K, (64,), 8 * 8, 2048),  # batch x8 so that it divides the 64-rank mesh
     "llama3_8b_1layer_mesh32x8": (dataclasses.replace(LLAMA3_8B, n_layers=1), (32, 8), 32, 8192),
     "llama3_70b_1layer_mesh8x8x8": (dataclasses.replace(LLAMA3_70B, n_layers=1), (8, 8, 8), 64, 8192),
+    "dsv3_moe_tiny_mesh64x4": (TINY_MOE, (64, 4), 16, 512),  # batch 16 < 64 ranks: tokens shard along the sequence
 }
 
 
 def _planner(planner_cls, cfg, mesh_sizes, batch, seq, repeated_subgraphs=False, block=False):
     mesh = workloads.logical_mesh(mesh_sizes)
+    if isinstance(cfg, DeepSeekV3Config):
+        model, input_fn, _, dynamo = workloads.build_model("dsv3_moe", mesh, batch=batch, seq=seq, config=cfg)
+        assert dynamo
+        return planner_cls(model, input_fn, mesh, param_dtype=torch.bfloat16, reduce_dtype=torch.float32,
+                           repeated_subgraphs=repeated_subgraphs, dynamo=True)
     with torch.device("meta"):
         model = SingleBlock(cfg) if block else Llama(cfg)
     if block:
@@ -95,6 +106,34 @@ def test_tiny_llama_tables_and_clustering(fake_pg):
         for node, rep in opt.node_representative.items():
             assert str(plan[node]) == str(plan[rep])
         assert not opt.prob.violated_constraints()
+
+
+def test_tiny_moe_regions_and_plan(fake_pg):
+    """The mixture-of-experts decoder: every routed-expert region is one forward and one
+    backward node with the single strategy its author declared; the graph plans."""
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    with _planner(OraclePlanner, TINY_MOE, (8, 4), 16, 64, repeated_subgraphs=True) as autop:
+        opt = autop.sharding_optimizer
+        regions = [n for n in autop.gm.graph.nodes if "local_map_kwargs" in n.meta]
+        assert len(regions) == 2 * (TINY_MOE.n_layers - TINY_MOE.n_dense_layers)
+        for node in regions:
+            assert len(opt.strats[node].strategies) == 1
+        tokens, experts = (Shard(1), Shard(1)), (Shard(0), Replicate())
+        for fw in regions[: len(regions) // 2]:
+            spec = opt.strats[fw].strategies[0]
+            assert [s.placements for s in spec.input_specs] == [tokens] * 3 + [experts] * 3 + [tokens]
+            assert spec.output_specs[0].placements == tokens
+            assert all(s is None or s.placements == (Replicate(), Replicate()) for s in spec.output_specs[1:])
+        # the two identical MoE layers were linked
+        assert len(opt.node_representative) > 0 and opt.n_variables < opt.encoded.tables.n_entries
+        autop.add_parameter_memory_constraint(low=None, high=None)
+        autop.add_input_constraints([(Shard(1), Replicate())])
+        autop.add_output_constraints([(Shard(1), Replicate())])
+        plan = autop.optimize_placement()
+        assert not opt.prob.violated_constraints()
+        for node in regions:
+            assert str(plan[node]) == str(opt.strats[node].strategies[0])
 
 
 @pytest.mark.gpu
