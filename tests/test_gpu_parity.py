@@ -256,3 +256,32 @@ def test_full_size_stress_properties(gpu_device):
     seg_of_entry = torch.repeat_interleave(torch.arange(rp.numel() - 1, device=gpu_device)[:200_000],
                                            (rp[1:] - rp[:-1])[:200_000])
     assert bool((cost[: seg_of_entry.numel()] >= mins[seg_of_entry]).all())
+
+
+def test_graph_replay_of_one_pass_matches_eager(gpu_device):
+    """One pass recorded as a HIP graph (independent kernels on parallel branches) gives the
+    eager results on every replay, with eager work and synchronisations between replays."""
+    mesh = (8, 4, 2)
+    tb = stress_dag(seed=5, n_nodes=3000, mesh_sizes=mesh, frac_nonspec_nodes=0.02, frac_noncontiguous=0.2)
+    d = DeviceCostTables(tb, CostModelParams.from_mesh(mesh, rescale=2.2), device=gpu_device)
+    step = d.prepare_step(row_min=True)
+    for launch in step.values():
+        launch()
+    torch.cuda.synchronize()
+    outputs = {"comm": d.comm, "transition": d.transition, "cost": d.cost, "row_min": d.row_min,
+               "row_argmin": d.row_argmin, "compute": d.compute_cost, "per_arg": d.compute_cost_per_arg,
+               "bytes": d.tensor_bytes}
+    want = {k: v.clone() for k, v in outputs.items()}
+    enc = tb.as_dict()
+    op = po.make_params(mesh, rescale=2.2)
+    oracle = c_oracle.build_tables(enc, op, per_arg=c_oracle.compute_costs(enc, op)[1])
+    assert np.array_equal(want["cost"].cpu().numpy(), oracle["cost"])
+    graph = d.capture_step_graph(step)
+    for replay in range(4):
+        for v in outputs.values():
+            v.zero_()  # eager work between replays; also proves the replay rewrites everything
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for k, v in outputs.items():
+            assert torch.equal(v, want[k]), (replay, k)
