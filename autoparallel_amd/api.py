@@ -14,8 +14,6 @@ from __future__ import annotations
 import logging
 import time
 
-import torch
-
 from .graphs.capture import capture_joint_graph
 from .optimize_sharding import ShardingOptimizer
 

@@ -9,7 +9,6 @@ built library) construction raises: there is no CPU path.
 from __future__ import annotations
 
 import ctypes
-import os
 
 import numpy as np
 import torch
@@ -197,7 +196,7 @@ class DeviceCostTables:
         self.run_tensor_tables()
         spec = self.run_spec_tables()
         self.run_compute_costs()
-        self.alloc_outputs(True, os.environ.get('APC_EXP_NO_TRANS') is None, True)
+        self.alloc_outputs(True, True, True)
         lib, P, cp = self.lib, self._p, ctypes.byref(self.c_params)
         stream = self._stream()
         tb = self.tables

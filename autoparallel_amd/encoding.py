@@ -36,7 +36,7 @@ from typing import Optional
 import numpy as np
 
 from . import _native
-from ._native import APC_MAX_MESH, APC_MAX_RANK, APC_TILE_MAX_COLS, APC_TILE_MAX_DUPS, APC_TILE_MAX_ROWS
+from ._native import APC_MAX_RANK, APC_TILE_MAX_COLS, APC_TILE_MAX_DUPS, APC_TILE_MAX_ROWS
 
 REPLICATE = 0x00
 PARTIAL_SUM = 0x40

@@ -20,7 +20,6 @@ from __future__ import annotations
 import hashlib
 
 import torch
-from torch.distributed.tensor._dtensor_spec import DTensorSpec
 from torch.utils._pytree import tree_flatten
 
 from .encode import all_input_nodes

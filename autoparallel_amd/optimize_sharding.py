@@ -28,7 +28,6 @@ from __future__ import annotations
 
 import logging
 import math
-import operator
 import time
 from collections.abc import Mapping
 from typing import Optional

@@ -2,7 +2,6 @@
 host logic (encoding, ILP) can be exercised without a GPU and so GPU-built tables can be
 compared with oracle-built ones through the same solver.  Never used by the product."""
 
-import numpy as np
 
 from oracle import c_oracle
 from oracle import cost_oracle as po

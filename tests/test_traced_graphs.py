@@ -5,7 +5,6 @@ CPU: strategy enumeration / encoding / clustering invariants with oracle-built t
 GPU: device-built tables bit-identical to oracle-built ones on every configuration."""
 
 import dataclasses
-import warnings
 
 import numpy as np
 import pytest
@@ -13,7 +12,7 @@ import torch
 
 from autoparallel_amd.api import AutoParallelPlanner
 from autoparallel_amd.graphs import workloads
-from autoparallel_amd.graphs.dsv3 import DeepSeekV3, DeepSeekV3Config
+from autoparallel_amd.graphs.dsv3 import DeepSeekV3Config
 from autoparallel_amd.graphs.llama3 import LLAMA3_8B, LLAMA3_70B, BLOCK_1K, Llama, LlamaConfig, SingleBlock
 from autoparallel_amd.optimize_sharding import ShardingOptimizer
 from oracle_backend import OracleBackend
