@@ -205,9 +205,9 @@ __global__ __launch_bounds__(kBlock) void spec_tables_kernel(
     int64_t *__restrict__ lshape, int64_t *__restrict__ lstride, int64_t *__restrict__ lnumel,
     int64_t *__restrict__ lbytes) {
   // each thread derives one spec; the two [kBlock][8] result blocks are transposed through LDS
-  // so that the workgroup writes them as two contiguous 16 KB runs
-  __shared__ int64_t s_shape[kBlock * (APC_MAX_RANK + 1)];
-  __shared__ int64_t s_stride[kBlock * (APC_MAX_RANK + 1)];
+  // (one buffer, used for the shapes and then for the strides) so that the workgroup writes
+  // them as two contiguous 16 KB runs
+  __shared__ int64_t s_rows[kBlock * (APC_MAX_RANK + 1)];
   const int64_t base = (int64_t)blockIdx.x * kBlock;
   const int64_t s = base + threadIdx.x;
   int64_t sh[APC_MAX_RANK], st[APC_MAX_RANK];
@@ -251,18 +251,18 @@ __global__ __launch_bounds__(kBlock) void spec_tables_kernel(
     lnumel[s] = ne;
     lbytes[s] = nb;
   }
-#pragma unroll
-  for (int i = 0; i < APC_MAX_RANK; ++i) {
-    s_shape[threadIdx.x * (APC_MAX_RANK + 1) + i] = sh[i];
-    s_stride[threadIdx.x * (APC_MAX_RANK + 1) + i] = st[i];
-  }
-  __syncthreads();
   const int64_t live = (n - base < kBlock ? n - base : kBlock) * APC_MAX_RANK;
-  for (int k = threadIdx.x; k < live; k += kBlock) {
-    const int row = k / APC_MAX_RANK, col = k % APC_MAX_RANK;
-    lshape[base * APC_MAX_RANK + k] = s_shape[row * (APC_MAX_RANK + 1) + col];
-    lstride[base * APC_MAX_RANK + k] = s_stride[row * (APC_MAX_RANK + 1) + col];
-  }
+#pragma unroll
+  for (int i = 0; i < APC_MAX_RANK; ++i) s_rows[threadIdx.x * (APC_MAX_RANK + 1) + i] = sh[i];
+  __syncthreads();
+  for (int k = threadIdx.x; k < live; k += kBlock)
+    lshape[base * APC_MAX_RANK + k] = s_rows[(k / APC_MAX_RANK) * (APC_MAX_RANK + 1) + k % APC_MAX_RANK];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < APC_MAX_RANK; ++i) s_rows[threadIdx.x * (APC_MAX_RANK + 1) + i] = st[i];
+  __syncthreads();
+  for (int k = threadIdx.x; k < live; k += kBlock)
+    lstride[base * APC_MAX_RANK + k] = s_rows[(k / APC_MAX_RANK) * (APC_MAX_RANK + 1) + k % APC_MAX_RANK];
 }
 
 // ------------------------------------------------------------------------------------------

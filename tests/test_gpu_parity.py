@@ -285,3 +285,35 @@ def test_graph_replay_of_one_pass_matches_eager(gpu_device):
         torch.cuda.synchronize()
         for k, v in outputs.items():
             assert torch.equal(v, want[k]), (replay, k)
+
+
+@pytest.mark.parametrize("mesh", [(6,), (4, 8), (16, 2, 4), (2, 2, 2, 2)])
+@pytest.mark.parametrize("contiguous", [True, False])
+def test_every_placement_pair(gpu_device, mesh, contiguous):
+    """Brute force over the placement algebra: every producer placement against every consumer
+    placement (Replicate, Partial(sum), Partial(avg), Shard of each tensor dim, on every mesh
+    dim; a sample of 300 x 300 on the 4-D mesh), for a contiguous and a transposed tensor, with
+    and without the gradient rescale.  Kernel == C oracle bit for bit on all of them, == the
+    scalar Python oracle on the 1-D and 2-D meshes."""
+    import itertools
+
+    M = len(mesh)
+    options = [0, partial_code(0), partial_code(1), shard_code(0), shard_code(1), shard_code(2)]
+    combos = list(itertools.product(options, repeat=M))
+    if len(combos) > 300:
+        rng = np.random.default_rng(7)
+        keep = rng.choice(len(combos), 300, replace=False)
+        combos = [combos[i] for i in sorted(keep)]
+    shape = [96, 64, 32]
+    stride = [2048, 32, 1] if contiguous else [1, 96, 6144]
+    for flags, rescale in ((0, 1.0), (1, 2.2)):
+        tb = _two_node_tables(mesh, shape, stride, 2, combos, combos, flags=flags)
+        assert tb.n_entries == len(combos) ** 2
+        d, want = _run_and_compare(tb, mesh, rescale, gpu_device)
+        comm = d.comm.cpu().numpy().reshape(len(combos), len(combos))
+        assert (np.diag(comm) == 0.0).all()  # identical placements cost nothing
+        if M <= 2:
+            py = po.build_tables(tb.as_dict(), po.make_params(mesh, rescale=rescale))
+            assert np.array_equal(d.comm.cpu().numpy(), np.asarray(py["comm"]))
+            assert np.array_equal(d.cost.cpu().numpy(), np.asarray(py["cost"]))
+            assert np.array_equal(d.transition.cpu().numpy(), np.asarray(py["transition"], dtype=np.uint8))
