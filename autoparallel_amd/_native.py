@@ -64,6 +64,7 @@ EXPORTS = (
     "apc_tensor_tables",
     "apc_spec_tables",
     "apc_compute_costs",
+    "apc_input_tables",
     "apc_redistribute_tables",
     "apc_segmented_min",
 )

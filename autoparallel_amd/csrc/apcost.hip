@@ -169,13 +169,21 @@ __device__ __forceinline__ int64_t xcd_chunked_unit(int shift) {
 // ------------------------------------------------------------------------------------------
 // a7: bytes + contiguity per tensor
 // ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void tensor_tables_kernel(int64_t n, const int32_t *__restrict__ rank,
-                                                               const int32_t *__restrict__ itemsize,
-                                                               const int64_t *__restrict__ shape,
-                                                               const int64_t *__restrict__ stride,
-                                                               int64_t *__restrict__ bytes,
-                                                               uint8_t *__restrict__ cont) {
-  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+struct TensorTableArgs {
+  int64_t n;
+  const int32_t *rank, *itemsize;
+  const int64_t *shape, *stride;
+  int64_t *bytes;
+  uint8_t *cont;
+};
+
+__device__ __forceinline__ void tensor_tables_block(int64_t block, const TensorTableArgs &a) {
+  const int64_t n = a.n;
+  const int32_t *__restrict__ rank = a.rank, *__restrict__ itemsize = a.itemsize;
+  const int64_t *__restrict__ shape = a.shape, *__restrict__ stride = a.stride;
+  int64_t *__restrict__ bytes = a.bytes;
+  uint8_t *__restrict__ cont = a.cont;
+  const int64_t t = block * kBlock + threadIdx.x;
   if (t >= n) return;
   const int r = rank[t];
   const int64_t *sh = shape + t * APC_MAX_RANK;
@@ -195,20 +203,34 @@ __global__ __launch_bounds__(kBlock) void tensor_tables_kernel(int64_t n, const 
   cont[t] = ok ? 1 : 0;
 }
 
+__global__ __launch_bounds__(kBlock) void tensor_tables_kernel(TensorTableArgs a) {
+  tensor_tables_block(blockIdx.x, a);
+}
+
 // ------------------------------------------------------------------------------------------
 // a8: local shard shape / stride / counts per spec
 // ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void spec_tables_kernel(
-    apc_params p, int64_t n, const uint32_t *__restrict__ codes, const int32_t *__restrict__ tensor,
-    const int32_t *__restrict__ rank, const int32_t *__restrict__ itemsize,
-    const int64_t *__restrict__ shape, const int64_t *__restrict__ stride, int64_t *__restrict__ shards,
-    int64_t *__restrict__ lshape, int64_t *__restrict__ lstride, int64_t *__restrict__ lnumel,
-    int64_t *__restrict__ lbytes) {
+struct SpecTableArgs {
+  int64_t n;
+  const uint32_t *codes;
+  const int32_t *tensor, *rank, *itemsize;
+  const int64_t *shape, *stride;
+  int64_t *shards, *lshape, *lstride, *lnumel, *lbytes;
+};
+
+// s_rows: kBlock * (APC_MAX_RANK + 1) values of LDS
+__device__ __forceinline__ void spec_tables_block(int64_t block, const apc_params &p, const SpecTableArgs &a,
+                                                  int64_t *s_rows) {
+  const int64_t n = a.n;
+  const uint32_t *__restrict__ codes = a.codes;
+  const int32_t *__restrict__ tensor = a.tensor, *__restrict__ rank = a.rank, *__restrict__ itemsize = a.itemsize;
+  const int64_t *__restrict__ shape = a.shape, *__restrict__ stride = a.stride;
+  int64_t *__restrict__ shards = a.shards, *__restrict__ lshape = a.lshape, *__restrict__ lstride = a.lstride;
+  int64_t *__restrict__ lnumel = a.lnumel, *__restrict__ lbytes = a.lbytes;
   // each thread derives one spec; the two [kBlock][8] result blocks are transposed through LDS
   // (one buffer, used for the shapes and then for the strides) so that the workgroup writes
   // them as two contiguous 16 KB runs
-  __shared__ int64_t s_rows[kBlock * (APC_MAX_RANK + 1)];
-  const int64_t base = (int64_t)blockIdx.x * kBlock;
+  const int64_t base = block * kBlock;
   const int64_t s = base + threadIdx.x;
   int64_t sh[APC_MAX_RANK], st[APC_MAX_RANK];
 #pragma unroll
@@ -265,15 +287,33 @@ __global__ __launch_bounds__(kBlock) void spec_tables_kernel(
     lstride[base * APC_MAX_RANK + k] = s_rows[(k / APC_MAX_RANK) * (APC_MAX_RANK + 1) + k % APC_MAX_RANK];
 }
 
+__global__ __launch_bounds__(kBlock) void spec_tables_kernel(apc_params p, SpecTableArgs a) {
+  __shared__ int64_t s_rows[kBlock * (APC_MAX_RANK + 1)];
+  spec_tables_block(blockIdx.x, p, a, s_rows);
+}
+
 // ------------------------------------------------------------------------------------------
 // a9/a10: compute-cost tail per (node, strategy)
 // ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void compute_costs_kernel(
-    apc_params p, int64_t n, const int64_t *__restrict__ flops, const int64_t *__restrict__ rw_bytes,
-    const int8_t *__restrict__ dtype, const uint8_t *__restrict__ zero_cost,
-    const int32_t *__restrict__ num_args, double *__restrict__ compute, double *__restrict__ per_arg,
-    int32_t *__restrict__ error_flag) {
-  const int64_t s = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+struct ComputeCostArgs {
+  int64_t n;
+  const int64_t *flops, *rw_bytes;
+  const int8_t *dtype;
+  const uint8_t *zero_cost;
+  const int32_t *num_args;
+  double *compute, *per_arg;
+  int32_t *error_flag;
+};
+
+__device__ __forceinline__ void compute_costs_block(int64_t block, const apc_params &p, const ComputeCostArgs &a) {
+  const int64_t n = a.n;
+  const int64_t *__restrict__ flops = a.flops, *__restrict__ rw_bytes = a.rw_bytes;
+  const int8_t *__restrict__ dtype = a.dtype;
+  const uint8_t *__restrict__ zero_cost = a.zero_cost;
+  const int32_t *__restrict__ num_args = a.num_args;
+  double *__restrict__ compute = a.compute, *__restrict__ per_arg = a.per_arg;
+  int32_t *__restrict__ error_flag = a.error_flag;
+  const int64_t s = block * kBlock + threadIdx.x;
   if (s >= n) return;
   double c = 0.0;
   if (!zero_cost[s]) {
@@ -296,6 +336,23 @@ __global__ __launch_bounds__(kBlock) void compute_costs_kernel(
   }
   if (compute) compute[s] = c;
   if (per_arg) per_arg[s] = c / (double)num_args[s];
+}
+
+__global__ __launch_bounds__(kBlock) void compute_costs_kernel(apc_params p, ComputeCostArgs a) {
+  compute_costs_block(blockIdx.x, p, a);
+}
+
+// The three tables above in one launch: workgroups [0, spec_blocks) take the spec table (the
+// largest), the next tensor_blocks the tensor table, the rest the compute costs.  None of the
+// three reads another's output.
+__global__ __launch_bounds__(kBlock) void input_tables_kernel(apc_params p, TensorTableArgs t, SpecTableArgs sp,
+                                                              ComputeCostArgs c, int64_t spec_blocks,
+                                                              int64_t tensor_blocks) {
+  __shared__ int64_t s_rows[kBlock * (APC_MAX_RANK + 1)];
+  const int64_t b = blockIdx.x;
+  if (b < spec_blocks) spec_tables_block(b, p, sp, s_rows);
+  else if (b < spec_blocks + tensor_blocks) tensor_tables_block(b - spec_blocks, t);
+  else compute_costs_block(b - spec_blocks - tensor_blocks, p, c);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -914,8 +971,8 @@ int apc_tensor_tables(int64_t n, const int32_t *rank, const int32_t *itemsize, c
   if (n < 0) return fail(-1, "n_tensors < 0");
   if (n == 0) return 0;
   if (!rank || !itemsize || !shape || !stride || !bytes || !cont) return fail(-1, "apc_tensor_tables: NULL array");
-  hipLaunchKernelGGL(tensor_tables_kernel, dim3(blocks_for(n, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, n,
-                     rank, itemsize, shape, stride, bytes, cont);
+  hipLaunchKernelGGL(tensor_tables_kernel, dim3(blocks_for(n, kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
+                     TensorTableArgs{n, rank, itemsize, shape, stride, bytes, cont});
   return check_launch("apc_tensor_tables");
 }
 
@@ -930,7 +987,8 @@ int apc_spec_tables(const apc_params *params, int64_t n, const uint32_t *codes, 
       !lbytes)
     return fail(-1, "apc_spec_tables: NULL array");
   hipLaunchKernelGGL(spec_tables_kernel, dim3(blocks_for(n, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, *params,
-                     n, codes, tensor, rank, itemsize, shape, stride, shards, lshape, lstride, lnumel, lbytes);
+                     SpecTableArgs{n, codes, tensor, rank, itemsize, shape, stride, shards, lshape, lstride, lnumel,
+                                   lbytes});
   return check_launch("apc_spec_tables");
 }
 
@@ -942,8 +1000,38 @@ int apc_compute_costs(const apc_params *params, int64_t n, const int64_t *flops,
   if (n == 0) return 0;
   if (!flops || !rw_bytes || !dtype || !zero_cost || !num_args) return fail(-1, "apc_compute_costs: NULL input");
   hipLaunchKernelGGL(compute_costs_kernel, dim3(blocks_for(n, kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
-                     *params, n, flops, rw_bytes, dtype, zero_cost, num_args, compute, per_arg, error_flag);
+                     *params,
+                     ComputeCostArgs{n, flops, rw_bytes, dtype, zero_cost, num_args, compute, per_arg, error_flag});
   return check_launch("apc_compute_costs");
+}
+
+int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t *rank, const int32_t *itemsize,
+                     const int64_t *shape, const int64_t *stride, int64_t *tensor_bytes, uint8_t *tensor_contiguous,
+                     int64_t n_specs, const uint32_t *spec_codes, const int32_t *spec_tensor, int64_t *num_shards,
+                     int64_t *local_shape, int64_t *local_stride, int64_t *local_numel, int64_t *local_bytes,
+                     int64_t n_strategies, const int64_t *flops, const int64_t *rw_bytes, const int8_t *dtype,
+                     const uint8_t *zero_cost, const int32_t *num_args, double *compute, double *per_arg,
+                     int32_t *error_flag, void *stream) {
+  if (int rc = check_params(params)) return rc;
+  if (n_tensors < 0 || n_specs < 0 || n_strategies < 0) return fail(-1, "apc_input_tables: negative count");
+  if (n_tensors > 0 && (!rank || !itemsize || !shape || !stride || !tensor_bytes || !tensor_contiguous))
+    return fail(-1, "apc_input_tables: NULL tensor array");
+  if (n_specs > 0 && (!spec_codes || !spec_tensor || !rank || !itemsize || !shape || !stride || !num_shards ||
+                      !local_shape || !local_stride || !local_numel || !local_bytes))
+    return fail(-1, "apc_input_tables: NULL spec array");
+  if (n_strategies > 0 && (!flops || !rw_bytes || !dtype || !zero_cost || !num_args))
+    return fail(-1, "apc_input_tables: NULL strategy array");
+  const int64_t sb = blocks_for(n_specs, kBlock), tb = blocks_for(n_tensors, kBlock), cb = blocks_for(n_strategies, kBlock);
+  if (sb + tb + cb == 0) return 0;
+  if (sb + tb + cb > INT32_MAX) return fail(-1, "apc_input_tables: too many rows for one launch");
+  hipLaunchKernelGGL(input_tables_kernel, dim3((unsigned)(sb + tb + cb)), dim3(kBlock), 0, (hipStream_t)stream, *params,
+                     TensorTableArgs{n_tensors, rank, itemsize, shape, stride, tensor_bytes, tensor_contiguous},
+                     SpecTableArgs{n_specs, spec_codes, spec_tensor, rank, itemsize, shape, stride, num_shards,
+                                   local_shape, local_stride, local_numel, local_bytes},
+                     ComputeCostArgs{n_strategies, flops, rw_bytes, dtype, zero_cost, num_args, compute, per_arg,
+                                     error_flag},
+                     sb, tb);
+  return check_launch("apc_input_tables");
 }
 
 int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes, const uint8_t *tensor_contiguous,

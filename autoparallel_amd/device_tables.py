@@ -189,10 +189,12 @@ class DeviceCostTables:
 
     # ---- one full device-side pass with pre-bound arguments -------------------------------------
     @_guarded
-    def prepare_step(self, row_min=True):
+    def prepare_step(self, row_min=True, fused_inputs=False):
         """Allocates every output once and returns ``{kernel name: zero-argument launcher}``
         in launch order.  A launcher only enqueues (no allocation, no synchronisation), so a
-        timed loop measures the kernels and not Python argument marshalling."""
+        timed loop measures the kernels and not Python argument marshalling.  With
+        ``fused_inputs`` the tensor, spec and compute-cost tables are one launch
+        (``input_tables``) instead of three."""
         self.run_tensor_tables()
         spec = self.run_spec_tables()
         self.run_compute_costs()
@@ -224,12 +226,16 @@ class DeviceCostTables:
                     _native.check(rc, what)
             return launch
 
-        step = {
-            "tensor_tables": bind(lib.apc_tensor_tables, a_tensor, "apc_tensor_tables"),
-            "spec_tables": bind(lib.apc_spec_tables, a_spec, "apc_spec_tables"),
-            "compute_costs": bind(lib.apc_compute_costs, a_compute, "apc_compute_costs"),
-            "redistribute_tables": bind(lib.apc_redistribute_tables, a_tables, "apc_redistribute_tables"),
-        }
+        if fused_inputs:
+            a_inputs = (cp,) + a_tensor[:-1] + (a_spec[1], a_spec[2], a_spec[3]) + a_spec[8:-1] + a_compute[1:]
+            step = {"input_tables": bind(lib.apc_input_tables, a_inputs, "apc_input_tables")}
+        else:
+            step = {
+                "tensor_tables": bind(lib.apc_tensor_tables, a_tensor, "apc_tensor_tables"),
+                "spec_tables": bind(lib.apc_spec_tables, a_spec, "apc_spec_tables"),
+                "compute_costs": bind(lib.apc_compute_costs, a_compute, "apc_compute_costs"),
+            }
+        step["redistribute_tables"] = bind(lib.apc_redistribute_tables, a_tables, "apc_redistribute_tables")
         if row_min:
             row_ptr = torch.from_numpy(tb.row_ptr()).to(self.device)
             n_seg = row_ptr.numel() - 1
@@ -258,9 +264,12 @@ class DeviceCostTables:
             main = torch.cuda.current_stream()
             for b in branches:
                 b.wait_stream(main)
-            step["spec_tables"](ctypes.c_void_p(main.cuda_stream))
-            step["tensor_tables"](ctypes.c_void_p(branches[0].cuda_stream))
-            step["compute_costs"](ctypes.c_void_p(branches[1].cuda_stream))
+            if "input_tables" in step:
+                step["input_tables"](ctypes.c_void_p(main.cuda_stream))
+            else:
+                step["spec_tables"](ctypes.c_void_p(main.cuda_stream))
+                step["tensor_tables"](ctypes.c_void_p(branches[0].cuda_stream))
+                step["compute_costs"](ctypes.c_void_p(branches[1].cuda_stream))
             for b in branches:
                 main.wait_stream(b)
             step["redistribute_tables"](ctypes.c_void_p(main.cuda_stream))

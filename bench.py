@@ -55,6 +55,8 @@ def parse_args():
     ap.add_argument("--no-clustering", action="store_true", help="one ILP variable per entry (no variable sharing)")
     ap.add_argument("--no-dedupe", action="store_true", help="tile every edge even if an identical one exists")
     ap.add_argument("--max-copies", type=int, default=8, help="identical edges served by one tiled edge")
+    ap.add_argument("--separate-input-kernels", action="store_true",
+                    help="launch the tensor, spec and compute-cost tables as three kernels instead of one")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy three times (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -209,7 +211,7 @@ def main():
             tables.build_tiles(args.tile_entries)
         dev = DeviceCostTables(tables, params, device="cuda:0")
     log.info("tables resident: %d entries, %d tiles", tables.n_entries, tables.n_tiles)
-    step = dev.prepare_step(row_min=True)
+    step = dev.prepare_step(row_min=True, fused_inputs=not args.separate_input_kernels)
     torch.cuda.synchronize()
     host_timings["upload_and_prepare_s"] = time.perf_counter() - t0
     host_timings["setup_total_s"] = time.perf_counter() - t_setup
@@ -275,8 +277,10 @@ def main():
         "config": {**desc, "edges": tables.n_edges, "strategies": tables.n_strategies, "specs": tables.n_specs,
                    "entries": E, "tiles": tables.n_tiles, "tiling": tables.tiling,
                    "edges_deduplicated": int((tables.edge_canonical != np.arange(tables.n_edges)).sum()), "device_row": params.device_name,
-                   "devices_per_host": 8, "step": "tensor_tables + spec_tables + compute_costs + "
-                                                   "redistribute_tables(comm, transition, cost) + segmented_min(rows)"},
+                   "devices_per_host": 8,
+                   "step": ("tensor_tables + spec_tables + compute_costs" if args.separate_input_kernels else
+                            "input_tables(tensor + spec + compute-cost tables, one launch)") +
+                           " + redistribute_tables(comm, transition, cost) + segmented_min(rows)"},
         "roofline": {"bound": "hbm", "kernel": "redistribute_tiles_kernel", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get((E, tables.n_tiles, alg_bytes)),

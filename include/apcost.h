@@ -154,6 +154,20 @@ int apc_compute_costs(const apc_params *params, int64_t n_strategies, const int6
                       const int32_t *num_args, double *compute_cost, double *compute_cost_per_arg,
                       int32_t *error_flag, void *stream);
 
+/* apc_tensor_tables + apc_spec_tables + apc_compute_costs in ONE launch (none of the three
+ * reads another's output): same arguments, same results, two launches fewer.  For a caller that
+ * already holds the per-strategy flop / byte counts, e.g. when the tables of a graph are
+ * rebuilt under another cost model.  (A planner that still has to infer those counts from the
+ * local shard shapes, compute_estimation.py:244-300, calls the three entry points in turn.) */
+int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
+                     const int32_t *tensor_itemsize, const int64_t *tensor_shape, const int64_t *tensor_stride,
+                     int64_t *tensor_bytes, uint8_t *tensor_contiguous, int64_t n_specs, const uint32_t *spec_codes,
+                     const int32_t *spec_tensor, int64_t *num_shards, int64_t *local_shape, int64_t *local_stride,
+                     int64_t *local_numel, int64_t *local_bytes, int64_t n_strategies, const int64_t *flops,
+                     const int64_t *rw_bytes, const int8_t *dtype_code, const uint8_t *zero_cost,
+                     const int32_t *num_args, double *compute_cost, double *compute_cost_per_arg,
+                     int32_t *error_flag, void *stream);
+
 /* The redistribution-cost matrices of every edge, plus the assembled ILP cost.
  * Replaces the two inner loops of ShardingOptimizer.build_ds
  * (optimize_sharding.py:306-379): estimate_strategy_comms_cost /

@@ -317,3 +317,33 @@ def test_every_placement_pair(gpu_device, mesh, contiguous):
             assert np.array_equal(d.comm.cpu().numpy(), np.asarray(py["comm"]))
             assert np.array_equal(d.cost.cpu().numpy(), np.asarray(py["cost"]))
             assert np.array_equal(d.transition.cpu().numpy(), np.asarray(py["transition"], dtype=np.uint8))
+
+
+def test_fused_input_tables_match_the_three_entry_points(gpu_device):
+    mesh = (16, 8, 4)
+    tb = stress_dag(seed=9, n_nodes=2500, mesh_sizes=mesh, frac_nonspec_nodes=0.03, frac_noncontiguous=0.2)
+    p = CostModelParams.from_mesh(mesh, rescale=2.2)
+    names = ("tensor_bytes", "tensor_contiguous", "compute_cost", "compute_cost_per_arg", "comm", "transition", "cost",
+             "row_min", "row_argmin")
+    results = []
+    for fused in (False, True):
+        d = DeviceCostTables(tb, p, device=gpu_device)
+        step = d.prepare_step(row_min=True, fused_inputs=fused)
+        assert ("input_tables" in step) == fused and len(step) == (3 if fused else 5)
+        for name in names:
+            getattr(d, name).zero_()
+        spec = d._step_keepalive[1]
+        for v in spec.values():
+            v.zero_()
+        for launch in step.values():
+            launch()
+        torch.cuda.synchronize()
+        out = {name: getattr(d, name).cpu().numpy() for name in names}
+        out.update({f"spec_{k}": v.cpu().numpy() for k, v in spec.items()})
+        results.append(out)
+    for key in results[0]:
+        assert np.array_equal(results[0][key], results[1][key]), key
+    enc = tb.as_dict()
+    assert np.array_equal(results[1]["tensor_bytes"], c_oracle.tensor_tables(enc)[0])
+    assert np.array_equal(results[1]["spec_local_shape"], c_oracle.spec_tables(enc, mesh)[1])
+    assert (results[1]["cost"] != 0).any()
