@@ -789,16 +789,27 @@ __global__ __launch_bounds__(kBlock) void segmented_min_kernel(const double *__r
       arg = j;
     }
   };
-  // four independent loads in flight per lane, taken in index order (first minimum wins)
-  int64_t j = lo + sub;
-  for (; j + 3 * G < hi; j += 4 * G) {
-    const double v0 = values[j], v1 = values[j + G], v2 = values[j + 2 * G], v3 = values[j + 3 * G];
-    take(v0, j);
-    take(v1, j + G);
-    take(v2, j + 2 * G);
-    take(v3, j + 3 * G);
+  // A lane reads pairs of consecutive values (one 16-byte load; segments start at any 8-byte
+  // offset, which global loads allow), two such loads in flight, taken in index order (first
+  // minimum wins); the G lanes of a group sweep 2 G consecutive values per load.
+  struct __attribute__((packed, aligned(8))) Pair {
+    double x, y;
+  };
+  int64_t j = lo + 2 * sub;
+  for (; j + 2 * G + 1 < hi; j += 4 * G) {
+    const Pair a = *reinterpret_cast<const Pair *>(values + j);
+    const Pair b = *reinterpret_cast<const Pair *>(values + j + 2 * G);
+    take(a.x, j);
+    take(a.y, j + 1);
+    take(b.x, j + 2 * G);
+    take(b.y, j + 2 * G + 1);
   }
-  for (; j < hi; j += G) take(values[j], j);
+  for (; j + 1 < hi; j += 2 * G) {
+    const Pair a = *reinterpret_cast<const Pair *>(values + j);
+    take(a.x, j);
+    take(a.y, j + 1);
+  }
+  if (j < hi) take(values[j], j);
   // lexicographic (value, index) min inside the group; lanes that saw nothing lose
 #pragma unroll
   for (int off = G / 2; off > 0; off >>= 1) {
