@@ -93,33 +93,46 @@ def _two_node_tables(mesh, shape, stride, itemsize, src_codes, tgt_codes, flags=
         edge_entry_begin=[0, ns * nt], edge_strat_begin=[ns], pt_values=[])
 
 
+def _golden():
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(__file__), "golden", "known_answers.json")) as f:
+        return json.load(f)
+
+
 def test_known_answer_values_on_device(gpu_device):
-    """The hand-derived values (mesh (32, 8), [4096, 4096] bf16) straight from the kernel."""
+    """The hand-derived values (tests/golden/known_answers.json) straight from the kernel."""
     R, P, S0, S1 = 0, partial_code(), shard_code(0), shard_code(1)
+    named = {"R": R, "P": P, "S0": S0, "S1": S1}
+    g = _golden()
+    mesh = tuple(g["environment"]["mesh"])
+    for case in g["redistribute_cost_us"]:
+        src, tgt = tuple(named[x] for x in case["src"]), tuple(named[x] for x in case["tgt"])
+        tb = _two_node_tables(mesh, case["shape"], case["stride"], case["itemsize"], [src], [tgt])
+        d = DeviceCostTables(tb, CostModelParams.from_mesh(mesh), device=gpu_device)
+        comm, trans, _ = d.build_all()
+        assert comm.cpu().numpy()[0] == case["value"], case["note"]
+        assert trans.cpu().numpy()[0] == 1
+    # one matrix with the special cases around them
     src = [(S0, S0), (P, P), (S0, S1), (R, R), (S0, R)]
     tgt = [(R, S0), (R, R), (S0, S0), (S0, R), (S0, S1), (P, R)]
-    tb = _two_node_tables((32, 8), [4096, 4096], [4096, 1], 2, src, tgt)
-    d = DeviceCostTables(tb, CostModelParams.from_mesh((32, 8)), device=gpu_device)
+    tb = _two_node_tables(mesh, [4096, 4096], [4096, 1], 2, src, tgt)
+    d = DeviceCostTables(tb, CostModelParams.from_mesh(mesh), device=gpu_device)
     comm, trans, _ = d.build_all()
     m = comm.cpu().numpy().reshape(len(tgt), len(src))
-    assert m[0, 0] == 286.43246022079404  # (S0,S0) -> (R,S0)
-    assert m[1, 0] == 609.0198034363015  # (S0,S0) -> (R,R)
-    assert m[2, 1] == 609.0198034363015  # (P,P) -> (S0,S0): flipped order
-    assert m[3, 2] == 27.543354475484605  # (S0,S1) -> (S0,R)
-    assert m[4, 0] == 67.08959654717788  # (S0,S0) -> (S0,S1)
+    assert m[0, 0] == 286.43246022079404 and m[2, 1] == 609.0198034363015 and m[3, 2] == 27.543354475484605
     assert m[2, 0] == 0.0 and m[0, 3] == 0.0  # identity, replicated source
     assert math.isinf(m[5, 3]) and math.isinf(m[5, 0])  # -> Partial banned
     t = trans.cpu().numpy().reshape(len(tgt), len(src))
     assert t[2, 0] == 0 and t[0, 0] == 1 and t[3, 4] == 0
-    # fp32 [8192, 4096] all-reduce on the inter-host dim
-    tb = _two_node_tables((32, 8), [8192, 4096], [4096, 1], 4, [(P, R)], [(R, R)])
-    d = DeviceCostTables(tb, CostModelParams.from_mesh((32, 8)), device=gpu_device)
-    assert d.build_all()[0].cpu().numpy()[0] == 12726.477454130818
 
 
 def test_compute_cost_known_answer_and_assembly(gpu_device):
     S0 = shard_code(0)
-    flops, rw = 68719476736, 67108864
+    kat = _golden()["compute_cost"]
+    flops, rw = kat["flops"], kat["read_write_bytes"]
+    assert kat["cost_us"] == 99.26256931388127
     tb = _two_node_tables((32, 8), [4096, 4096], [4096, 1], 2, [(S0, S0)], [(0, S0)], flags=1, num_args=2,
                           flops=flops, rw=rw)
     d = DeviceCostTables(tb, CostModelParams.from_mesh((32, 8), rescale=2.2), device=gpu_device)

@@ -104,17 +104,29 @@ def _cost(src, tgt, shape=KAT_SHAPE, stride=KAT_STRIDE, itemsize=2, mesh=(32, 8)
     return po.estimate_strategy_comms_cost(src, tgt, shape, stride, itemsize, po.make_params(mesh))
 
 
+def _golden():
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(__file__), "golden", "known_answers.json")) as f:
+        return json.load(f)
+
+
+_NAMED = {"R": R, "P": P, "S0": S0, "S1": S1}
+
+
 def test_known_answers_2d_mesh():
-    # hand-derived from the published formulas, mesh (32, 8), 8 devices/host, H100 row,
-    # [4096, 4096] bf16 contiguous
-    assert _cost((S0, S0), (R, S0)) == 286.43246022079404
-    assert _cost((S0, S0), (R, R)) == 609.0198034363015
-    assert _cost((P, P), (S0, S0)) == 609.0198034363015  # walks mesh dim 1 first
-    p = po.make_params((32, 8))
-    assert po.redistribute_cost((P, P), (S0, S0), KAT_SHAPE, KAT_STRIDE, 2, p, [0, 1]) == 1679.9030362418368
-    assert _cost((S0, S1), (S0, R)) == 27.543354475484605  # all-gather + 7 us reshuffle floor
-    assert _cost((S0, S0), (S0, S1)) == 67.08959654717788  # all-to-all x5 + one copy
-    assert _cost((P, R), (R, R), [8192, 4096], [4096, 1], 4) == 12726.477454130818
+    # hand-derived from the published formulas, mesh (32, 8), 8 devices/host, H100 row
+    g = _golden()
+    mesh = tuple(g["environment"]["mesh"])
+    for case in g["redistribute_cost_us"]:
+        src, tgt = tuple(_NAMED[x] for x in case["src"]), tuple(_NAMED[x] for x in case["tgt"])
+        assert _cost(src, tgt, case["shape"], case["stride"], case["itemsize"], mesh) == case["value"], case["note"]
+    u = g["unflipped_order_us"]
+    p = po.make_params(mesh)
+    assert po.redistribute_cost(tuple(_NAMED[x] for x in u["src"]), tuple(_NAMED[x] for x in u["tgt"]), u["shape"],
+                                u["stride"], u["itemsize"], p, u["order"]) == u["value"]
+    assert p.bw[0] == g["inter_host_bandwidth_GBps"]
 
 
 def test_hand_expanded_allgather_value():
