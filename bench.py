@@ -285,6 +285,7 @@ def main():
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get((E, tables.n_tiles, alg_bytes)),
                      "algorithmic_bytes_per_launch": alg_bytes,
+                     "bytes_written_per_entry": {"comm_f64": 8, "transition_u8": 1, "cost_f64": 8},
                      "avg_launch_us": t_kernel * 1e6, "min_launch_us": kernel_ms_min["redistribute_tables"] * 1e3,
                      "timing": "HIP events around every launch of the kernel inside the timed region"},
         "kernel_us": {k: v * 1e3 for k, v in kernel_ms.items()},
