@@ -226,3 +226,25 @@ def test_oracle_and_product_agree_on_constants():
         assert a.bw == b.bw and a.lat == b.lat and a.hbm_bw == b.hbm_bw and tuple(a.gpu_flops) == tuple(b.gpu_flops)
     assert po.shard(3) == shard_code(3) and po.partial(2) == partial_code(2)
     assert po.DTYPE_CODES == __import__("autoparallel_amd.cost_model", fromlist=["x"]).DTYPE_CODES
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    """No library, no product: loading raises (there is no CPU path to fall back to), and so
+    does everything built on it."""
+    import subprocess
+    import sys
+
+    code = (
+        "import sys\n"
+        "from autoparallel_amd import _native\n"
+        "try:\n"
+        "    _native.lib()\n"
+        "except RuntimeError as e:\n"
+        "    assert 'missing' in str(e), e\n"
+        "    sys.exit(42)\n"
+        "sys.exit(0)\n"
+    )
+    env = dict(os.environ, APCOST_LIBRARY=str(tmp_path / "no_such_libapcost.so"))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True)
+    assert proc.returncode == 42, proc.stderr[-2000:]
