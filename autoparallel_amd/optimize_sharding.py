@@ -197,7 +197,7 @@ class ClusterLinks(Mapping):
                 yield key
 
     def __len__(self):
-        return int(self._o._linked_entry.sum())
+        return self._o.n_linked_entries
 
 
 class ShardingOptimizer:
@@ -309,39 +309,55 @@ class ShardingOptimizer:
 
     def create_cluster_links(self):
         """Entries of a linked node share the ILP variables of its representative's entries
-        (same argument, same strategy pair)."""
+        (same argument, same strategy pair).  Variables are numbered edge by edge over the
+        edges that are their own representative; a linked edge takes its representative's
+        block of numbers."""
         tb = self.encoded.tables
-        ident = np.arange(tb.n_entries, dtype=np.int64)
-        self._identity_vars = ident
-        var = ident.copy()
+        n_edges = tb.n_edges
+        begin = tb.edge_entry_begin.astype(np.int64)
+        sizes = begin[1:] - begin[:-1]
+        edge_rep = np.arange(n_edges, dtype=np.int64)
         for node, rep in self.node_representative.items():
             s1, s0 = self.node_map[node], self.node_map[rep]
             assert self.num_args[s1] == self.num_args[s0], f"clustering linked {node} and {rep} with different arity"
             for argi in range(self.num_args[s1]):
-                b1, nt1, ns1 = self._edge(s1, argi)
-                b0, nt0, ns0 = self._edge(s0, argi)
-                assert (nt1, ns1) == (nt0, ns0), (
+                e1, e0 = self.encoded.edge_of[(s1, argi)], self.encoded.edge_of[(s0, argi)]
+                assert (tb.edge_n_tgt[e1], tb.edge_n_src[e1]) == (tb.edge_n_tgt[e0], tb.edge_n_src[e0]), (
                     f"Problem with graph clustering: {rep} and {node} don't have the same number of input/output "
                     "placements. Please report a bug")
-                var[b1:b1 + nt1 * ns1] = np.arange(b0, b0 + nt0 * ns0)
-        # compact variable ids: one per distinct representative entry
-        uniq, inverse = np.unique(var, return_inverse=True)
-        self.var_of_entry = inverse.astype(np.int64)
-        self.n_variables = len(uniq)
-        self._linked_entry = var != ident
+                edge_rep[e1] = e0
+        while not np.array_equal(edge_rep[edge_rep], edge_rep):  # representatives are roots already; be safe
+            edge_rep = edge_rep[edge_rep]
+        is_root = edge_rep == np.arange(n_edges)
+        base = np.zeros(n_edges, np.int64)
+        base[is_root] = np.cumsum(sizes[is_root]) - sizes[is_root]
+        self.edge_var_base = base[edge_rep]
+        self.edge_is_representative = is_root
+        self.var_of_entry = np.repeat(self.edge_var_base - begin[:-1], sizes) + np.arange(tb.n_entries, dtype=np.int64)
+        self.n_variables = int(sizes[is_root].sum())
+        self.n_linked_entries = int(sizes[~is_root].sum())
         # choice variables: one per (node, strategy), shared with the node's representative
         self.n_choice_variables = 0
         self.choice_var_of_strategy = None
+        self.node_choice_base = {}
         if self.node_choice_variables:
             sb = self.encoded.strat_begin
-            choice = np.arange(tb.n_strategies, dtype=np.int64)
+            choice = np.zeros(tb.n_strategies, np.int64)
+            next_free = self.n_variables
+            for s_i, node in enumerate(self.nodes):
+                if node.op == "output" or node in self.node_representative:
+                    continue
+                n = len(self.strats[node].strategies)
+                self.node_choice_base[s_i] = next_free
+                choice[sb[s_i]:sb[s_i] + n] = np.arange(next_free, next_free + n)
+                next_free += n
             for node, rep in self.node_representative.items():
                 s1, s0 = self.node_map[node], self.node_map[rep]
                 n = len(self.strats[node].strategies)
-                choice[sb[s1]:sb[s1] + n] = np.arange(sb[s0], sb[s0] + n)
-            uniq_c, inverse_c = np.unique(choice, return_inverse=True)
-            self.choice_var_of_strategy = self.n_variables + inverse_c.astype(np.int64)
-            self.n_choice_variables = len(uniq_c)
+                self.node_choice_base[s1] = self.node_choice_base[s0]
+                choice[sb[s1]:sb[s1] + n] = choice[sb[s0]:sb[s0] + n]
+            self.choice_var_of_strategy = choice
+            self.n_choice_variables = next_free - self.n_variables
 
     def _write_back_redistribute_cost(self):
         tb = self.encoded.tables
@@ -372,54 +388,72 @@ class ShardingOptimizer:
         return int(tb.edge_entry_begin[e]), int(tb.edge_n_tgt[e]), int(tb.edge_n_src[e])
 
     # ---- default constraints (optimize_sharding.py:402-542) --------------------------------
+    # Linked nodes share variable blocks, so most constraints of a repeated layer are literally
+    # the rows of its representative layer.  A row is determined by the variable blocks (and
+    # shapes) it is built from; every emitter below skips a combination it has already emitted
+    # instead of materialising the row and leaving it to the solver front-end to drop.
     def add_unique_decision_constraint(self):
         """For every (node, argument): exactly one (output, input) strategy pair."""
         tb = self.encoded.tables
-        lens = tb.edge_entry_begin[1:] - tb.edge_entry_begin[:-1]
-        self.prob.add_rows(self.var_of_entry, 1.0, lens, 1.0, 1.0, "unique_decision")
+        sizes = (tb.edge_entry_begin[1:] - tb.edge_entry_begin[:-1])[self.edge_is_representative]
+        self.prob.add_rows(np.arange(self.n_variables, dtype=np.int64), 1.0, sizes, 1.0, 1.0, "unique_decision")
+
+    def _edge_vars(self, s_i, argi):
+        """(variable block start, consumer strategies, producer strategies) of one edge."""
+        e = self.encoded.edge_of[(s_i, argi)]
+        tb = self.encoded.tables
+        return int(self.edge_var_base[e]), int(tb.edge_n_tgt[e]), int(tb.edge_n_src[e])
 
     def add_same_output_across_args_constraint(self):
         """All arguments of a node agree on the node's output strategy."""
-        cols, vals, lens = [], [], []
+        cols, vals, lens, seen = [], [], [], set()
         for s_i, node in enumerate(self.nodes):
             if node.op != "call_function" or len(self._all_input_nodes(node)) <= 1:
                 continue
-            b0, nt, ns0 = self._edge(s_i, 0)
+            b0, nt, ns0 = self._edge_vars(s_i, 0)
             for argi in range(1, len(self._all_input_nodes(node))):
-                ba, nta, nsa = self._edge(s_i, argi)
+                ba, nta, nsa = self._edge_vars(s_i, argi)
                 assert nta == nt
+                key = (b0, ba, nt, ns0, nsa)
+                if key in seen:
+                    continue
+                seen.add(key)
                 first = b0 + np.arange(nt)[:, None] * ns0 + np.arange(ns0)[None, :]
                 other = ba + np.arange(nt)[:, None] * nsa + np.arange(nsa)[None, :]
                 cols.append(np.concatenate([first, other], axis=1).ravel())
                 vals.append(np.tile(np.concatenate([np.ones(ns0), -np.ones(nsa)]), nt))
                 lens.append(np.full(nt, ns0 + nsa))
         if cols:
-            self.prob.add_rows(self.var_of_entry[np.concatenate(cols)], np.concatenate(vals), np.concatenate(lens),
-                               0.0, 0.0, "same_across_args")
+            self.prob.add_rows(np.concatenate(cols), np.concatenate(vals), np.concatenate(lens), 0.0, 0.0,
+                               "same_across_args")
 
     def add_output_input_consistent_constraint(self):
         """The producer's chosen output strategy is the column its consumers read."""
-        cols, vals, lens = [], [], []
+        cols, vals, lens, seen = [], [], [], set()
         for s_i, node in enumerate(self.nodes):
             if node.op == "output":
                 continue
-            bp, ntp, nsp = self._edge(s_i, 0)
+            bp, ntp, nsp = self._edge_vars(s_i, 0)
             for user in node.users:
                 if user.op == "output":
                     continue
                 s_j = self.node_map[user]
                 argj = [i for i, n in enumerate(user.all_input_nodes) if n == node]
                 assert len(argj) == 1
-                bc, ntc, nsc = self._edge(s_j, argj[0])
+                bc, ntc, nsc = self._edge_vars(s_j, argj[0])
                 assert nsc == ntp, f"{node} has {ntp} strategies, {user} arg {argj[0]} reads {nsc}"
+                key = (bp, bc, ntp, nsp, ntc)
+                if key in seen:
+                    continue
+                seen.add(key)
                 prod = bp + np.arange(ntp)[:, None] * nsp + np.arange(nsp)[None, :]  # row o of producer
                 cons = bc + np.arange(ntc)[None, :] * nsc + np.arange(nsc)[:, None]  # column o of consumer
                 cols.append(np.concatenate([prod, cons], axis=1).ravel())
                 vals.append(np.tile(np.concatenate([np.ones(nsp), -np.ones(ntc)]), ntp))
                 lens.append(np.full(ntp, nsp + ntc))
         if cols:
-            self.prob.add_rows(self.var_of_entry[np.concatenate(cols)], np.concatenate(vals), np.concatenate(lens),
-                               0.0, 0.0, "output_input_consistent")
+            self.prob.add_rows(np.concatenate(cols), np.concatenate(vals), np.concatenate(lens), 0.0, 0.0,
+                               "output_input_consistent")
 
     def add_inf_cost_constraint(self):
         """Non-finite costs become 10000 and their variable is forced to 0."""
@@ -431,15 +465,17 @@ class ShardingOptimizer:
     def add_choice_link_constraint(self):
         """choice[node, strategy] = sum of the entry variables of that strategy's row of the
         node's first argument; entry variables become continuous."""
-        tb = self.encoded.tables
-        cols, vals, lens = [], [], []
+        cols, vals, lens, seen = [], [], [], set()
         for s_i, node in enumerate(self.nodes):
             if node.op == "output":
                 continue
-            b, nt, ns = self._edge(s_i, 0)
-            sb = self.encoded.strat_begin[s_i]
-            entries = self.var_of_entry[b + np.arange(nt)[:, None] * ns + np.arange(ns)[None, :]]
-            choice = self.choice_var_of_strategy[sb + np.arange(nt)][:, None]
+            b, nt, ns = self._edge_vars(s_i, 0)
+            cb = self.node_choice_base[s_i]
+            if (b, cb) in seen:
+                continue
+            seen.add((b, cb))
+            entries = b + np.arange(nt)[:, None] * ns + np.arange(ns)[None, :]
+            choice = (cb + np.arange(nt))[:, None]
             cols.append(np.concatenate([entries, choice], axis=1).ravel())
             vals.append(np.tile(np.concatenate([np.ones(ns), [-1.0]]), nt))
             lens.append(np.full(nt, ns + 1))
@@ -458,8 +494,8 @@ class ShardingOptimizer:
 
     # ---- solve (optimize_sharding.py:648-701) ------------------------------------------------
     def get_solution(self, verbose=False):
-        obj = np.zeros(self.prob.n_vars)
-        np.add.at(obj, self.var_of_entry, self.cost)  # duplicate variables: costs add up
+        # linked entries share a variable: their costs add up
+        obj = np.bincount(self.var_of_entry, weights=self.cost, minlength=self.prob.n_vars).astype(np.float64)
         self.prob.objective = obj
         status = self.prob.solve(verbose=verbose, time_limit=self.solver_time_limit)
         if status == -1:
