@@ -365,9 +365,8 @@ __global__ __launch_bounds__(kBlock) void input_tables_kernel(apc_params p, Tens
 // different tensors, and the 2-D (Partial, Partial) -> all-Shard order flip.
 //
 // One workgroup per tile.  (A variant in which a workgroup walked a run of tiles, one
-// wavefront staging tile t+1 while the others computed tile t, was measured slower: the
-// staging of a tile is a chain of two dependent loads, and many short workgroups overlap
-// those chains better than one staging wavefront per workgroup does.)
+// wavefront staging tile t+1 while the others computed tile t, was measured slower than
+// many short workgroups.)
 // ------------------------------------------------------------------------------------------
 
 struct TableArgs {
@@ -443,9 +442,9 @@ struct TileStage {
   alignas(16) uint32_t act[APC_TILE_MAX_COLS * ActionRows<M>::kWords];  // one action row per mesh dim
   uint2 row[APC_TILE_MAX_ROWS];   // consumer specs: x = codes, y = info
   double cpa[APC_TILE_MAX_ROWS];  // compute cost / num_args of the consumer strategies
-  int64_t dup[APC_TILE_MAX_DUPS];  // entry offsets of identical edges, relative to this edge
+  int64_t dup[APC_TILE_MAX_DUPS];  // first entries of the identical edges
   double gb_unsharded;  // bytes / 1024^3 of the tile's tensor
-  int mixed;            // some spec is not a DTensorSpec on the tile's tensor: generic loop
+  int mixed[4];         // per staging wavefront: some spec is not a DTensorSpec on the tile's tensor (generic loop)
   int cont;             // the tile's tensor is contiguous
 };
 
@@ -467,8 +466,38 @@ __device__ __forceinline__ TileView view_of(const apc_tile &tile) {
                   tile.flags,           tile.dup_count,    tile.src_begin, tile.entry_begin, tile.pt_begin};
 }
 
-// Stages tile `tile` with `nthreads` cooperating threads (this thread is `tid`).  The caller
-// synchronises before the stage is read.  Only global loads and LDS writes: no stores.
+// Element `i` (a per-lane index below M) of one of the per-mesh-dim arrays of the kernel
+// parameters, as a select chain over scalar registers.  (Indexing the array by a lane value
+// makes the compiler read the kernel arguments through vector memory, and a vector load
+// waits behind every store the compute unit has in flight.)
+template <int M, typename T, int N>
+__device__ __forceinline__ T pick(const T (&v)[N], int i) {
+  static_assert(M <= N, "array shorter than the mesh");
+  T e[M];  // every element is read (scalar loads) before the selects, so they stay selects
+#pragma unroll
+  for (int k = 0; k < M; ++k) e[k] = v[k];
+  T r = e[0];
+#pragma unroll
+  for (int k = 1; k < M; ++k) r = i == k ? e[k] : r;
+  return r;
+}
+
+// ring_r on a per-lane mesh dim d, with hops = hop_scale * (mesh_size[d] - 1).
+template <int M>
+__device__ __forceinline__ double ring_at(double gb, const apc_params &p, int d, int hop_scale) {
+  const int n = pick<M>(p.mesh_size, d);
+  const double hops = (double)(hop_scale * (n - 1));
+  const double latency = p.base_latency + hops * pick<M>(p.lat, d);
+  const double bw = div_by(div_by(gb * hops, (double)n, pick<M>(p.inv_mesh, d)), pick<M>(p.bw, d), pick<M>(p.inv_bw, d));
+  return latency + bw * 1e6;
+}
+
+// Stages tile `tile` with `nthreads` (>= 64) cooperating threads (this thread is `tid`).  The
+// caller synchronises before the stage is read.  Only global loads and LDS writes: no stores.
+// Every vector load of the tile is issued first, in one round, and the state terms are
+// computed from scalar operands while the loads are in flight: under a store-bound kernel
+// each dependent round of vector loads queues behind the stores of the other workgroups of
+// the compute unit, so the number of rounds, not of loads, is what staging costs.
 template <int M>
 __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs &a, const apc_tile &tile,
                                            TileStage<M> &st, int tid, int nthreads) {
@@ -479,6 +508,36 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   const bool no_producer = (tile.flags & APC_EDGE_NO_PRODUCER) != 0;
   const bool terms_wanted = t0 >= 0 && !no_producer;
   bool mixed = !terms_wanted;
+  // ---- the round of vector loads ------------------------------------------------------------
+  // producer spec tid, consumer spec nthreads - 1 - tid (taken from the far end: with two
+  // wavefronts one loads the producer specs while the other loads the consumer specs).
+  // Threads past the tile's specs load its first spec again: unconditional loads, whose
+  // values are first touched after the state terms.
+  const int jc = tid, jr = nthreads - 1 - tid;
+  const bool has_col = jc < cols, has_row = jr < rows;
+  const int sp = tile.src_begin + tile.col_begin + (has_col ? jc : 0);
+  const int ts = tile.tgt_begin + tile.row_begin + (has_row ? jr : 0);
+  const int col_tensor = a.spec_tensor[sp];
+  const uint32_t col_codes = a.spec_codes[sp];
+  const uint32_t row_codes = a.spec_codes[ts];
+  const int row_tensor = a.spec_tensor[ts];
+  double row_cpa = 0.0;
+  if (a.per_arg) row_cpa = a.per_arg[tile.strat_begin + tile.row_begin + (has_row ? jr : 0)];
+  // (dup_count <= APC_TILE_MAX_DUPS < 2 * nthreads)
+  const bool has_dup0 = tid < tile.dup_count, has_dup1 = tid + nthreads < tile.dup_count;
+  int64_t dup0 = 0, dup1 = 0;
+  if (has_dup0) dup0 = a.dup_entry_begin[tile.dup_begin + tid];
+  if (has_dup1) dup1 = a.dup_entry_begin[tile.dup_begin + tid + nthreads];
+  // the contiguity byte of the tile's tensor, read as the aligned word around it (which lies
+  // in the byte's own page): a wave-uniform word goes through the scalar cache
+  uint32_t contiguous = 1;
+  if (terms_wanted) {
+    const uint8_t *flag = a.tensor_contiguous + t0;
+    const uint32_t lane = (uint32_t)(reinterpret_cast<uintptr_t>(flag) & 3);
+    const uint32_t word = *reinterpret_cast<const uint32_t *>(flag - lane);
+    contiguous = (word >> (8 * lane)) & 0xFFu;
+  }
+  // ---- state terms (scalar operands only) ---------------------------------------------------
   if (terms_wanted) {
     // every collective / read-write term the tile can need, once per running-bytes state, in
     // the reference's operation order (collective_runtime_estimation.py:66-68, :86, :128;
@@ -488,7 +547,11 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
       const int level = 31 - __clz((k >> M) + 1);
       const int rem = k - (((1 << level) - 1) << M);
       const int mask = rem >> level, hist = rem & ((1 << level) - 1);
-      double gb = div_by(fbytes, p.shards[mask], p.inv_shards[mask]) * 0x1p-30;  // / 1024 / 1024 / 1024
+      double shards = 1.0;  // exact: a product of mesh sizes (torch _dtensor_spec.py:555-561)
+#pragma unroll
+      for (int i = 0; i < M; ++i)
+        if ((mask >> i) & 1) shards *= (double)p.mesh_size[i];
+      double gb = fbytes / shards * 0x1p-30;  // / 1024 / 1024 / 1024
 #pragma unroll
       for (int i = 0; i < M; ++i) {
         if (i < level && ((hist >> i) & 1)) {
@@ -497,10 +560,10 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
         }
       }
       double ag = 0.0, rs = 0.0, ar = 0.0;
-      if (level >= 1) ag = ring_r(gb, p, level - 1, p.mesh_size[level - 1] - 1);
+      if (level >= 1) ag = ring_at<M>(gb, p, level - 1, 1);
       if (level < M) {
-        rs = ring_r(gb, p, level, p.mesh_size[level] - 1);
-        ar = ring_r(gb, p, level, 2 * (p.mesh_size[level] - 1));
+        rs = ring_at<M>(gb, p, level, 1);
+        ar = ring_at<M>(gb, p, level, 2);
       }
       double a2a = rs;
       a2a *= p.a2a_scale;
@@ -511,52 +574,45 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
       st.terms[4 * NS + k] = a2a;
       st.terms[5 * NS + k] = rw_time_r(gb * 2 * 1073741824.0, p);
     }
-    if (tid == 0) {
-      st.gb_unsharded = fbytes / 1024 / 1024 / 1024;
-      st.cont = a.tensor_contiguous[t0] != 0;
-    }
+    if (tid == 0) st.gb_unsharded = fbytes / 1024 / 1024 / 1024;
   } else if (tid == 0) {
     st.gb_unsharded = 0.0;
-    st.cont = 1;
   }
-  for (int j = tid; j < tile.dup_count; j += nthreads)
-    st.dup[j] = a.dup_entry_begin[tile.dup_begin + j] - tile.entry_begin;
-  for (int j = tid; j < cols; j += nthreads) {
-    const int sp = tile.src_begin + tile.col_begin + j;
-    const int t = a.spec_tensor[sp];
-    const uint32_t codes = a.spec_codes[sp];
+  // ---- what the loads brought, to LDS ---------------------------------------------------------
+  if (tid == 0) st.cont = contiguous != 0;
+  if (has_dup0) st.dup[tid] = dup0;
+  if (has_dup1) st.dup[tid + nthreads] = dup1;
+  if (has_col) {
     // info: bit0 valid spec, bit1 fully replicated, bits 4.. mask of sharded mesh dims
-    uint32_t info = (t >= 0 ? 1u : 0u) | (codes == 0u ? 2u : 0u);
+    uint32_t info = (col_tensor >= 0 ? 1u : 0u) | (col_codes == 0u ? 2u : 0u);
 #pragma unroll
     for (int i = 0; i < M; ++i) {
-      const uint32_t c = (codes >> (8 * i)) & 0xFF;
+      const uint32_t c = (col_codes >> (8 * i)) & 0xFF;
       const int cls = placement_class(c);
       info |= (cls >= 2 ? 1u : 0u) << (4 + i);
-      st.act[j * AW + i] = cls == 0 ? pair_row(0) : cls == 1 ? pair_row(1) : cls == 2 ? pair_row(2) : pair_row(3);
+      st.act[jc * AW + i] = cls == 0 ? pair_row(0) : cls == 1 ? pair_row(1) : cls == 2 ? pair_row(2) : pair_row(3);
     }
-    st.colh[j] = make_uint2(codes, info);
-    if (t != t0 || t < 0) mixed = true;
+    st.colh[jc] = make_uint2(col_codes, info);
+    if (col_tensor != t0 || col_tensor < 0) mixed = true;
   }
-  // (threads taken from the far end: with two wavefronts one stages the producer specs while
-  // the other stages the consumer specs)
-  for (int j = nthreads - 1 - tid; j < rows; j += nthreads) {
-    const int ts = tile.tgt_begin + tile.row_begin + j;
-    const uint32_t tg = a.spec_codes[ts];
+  if (has_row) {
     // info: bit0 valid spec, bits 1 + 5i .. : 8 x class of mesh dim i, bit 30 every dim is a Shard
-    uint32_t info = a.spec_tensor[ts] >= 0 ? 1u : 0u;
+    uint32_t info = row_tensor >= 0 ? 1u : 0u;
     bool all_shard = true;
 #pragma unroll
     for (int i = 0; i < M; ++i) {
-      const uint32_t t = (tg >> (8 * i)) & 0xFF;
+      const uint32_t t = (row_codes >> (8 * i)) & 0xFF;
       info |= (uint32_t)(placement_class(t) * 8) << (1 + 5 * i);
       all_shard &= kind_of(t) == 2;
     }
     if (all_shard) info |= 1u << 30;
     if (!(info & 1u)) mixed = true;  // a consumer spec that is not a DTensorSpec
-    st.row[j] = make_uint2(tg, info);
-    st.cpa[j] = a.per_arg ? a.per_arg[tile.strat_begin + tile.row_begin + j] : 0.0;
+    st.row[jr] = make_uint2(row_codes, info);
+    st.cpa[jr] = row_cpa;
   }
-  if (mixed) st.mixed = 1;  // cleared by the caller before staging
+  // one flag per wavefront, written unconditionally: nothing to clear beforehand
+  const bool wave_mixed = __ballot(mixed) != 0;
+  if ((tid & 63) == 0) st.mixed[tid >> 6] = wave_mixed ? 1 : 0;
 }
 
 // One entry of a tile whose producer specs all name one tensor (column c, row r of the tile).
@@ -635,6 +691,7 @@ struct TileOut {
   double *comm;
   uint8_t *trans;
   double *cost;
+  int64_t entry_begin;  // first entry of the tile's edge (an identical edge's values sit at its own first entry)
 };
 
 // Stores one entry's values to its edge and to every identical edge.  ALL: every output
@@ -647,7 +704,7 @@ __device__ __forceinline__ void store_entry(const TileOut &o, int dup_count, con
   if (ALL || o.trans) o.trans[local] = (uint8_t)trans;
   if (ALL || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost) + off8) = total;
   for (int d = 0; d < dup_count; ++d) {
-    const int64_t delta = uniform_i64(s_dup[d]);
+    const int64_t delta = uniform_i64(s_dup[d]) - o.entry_begin;
     if (ALL || o.comm) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.comm + delta) + off8) = comm;
     if (ALL || o.trans) (o.trans + delta)[local] = (uint8_t)trans;
     if (ALL || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost + delta) + off8) = total;
@@ -669,7 +726,7 @@ __device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const 
   if (first < 0) first += nthreads;
   int r = first / v.cols, c = first - r * v.cols;
   const TileOut out{a.comm_out ? a.comm_out + tile_base : nullptr, a.trans_out ? a.trans_out + tile_base : nullptr,
-                    a.cost_out ? a.cost_out + tile_base : nullptr};
+                    a.cost_out ? a.cost_out + tile_base : nullptr, v.entry_begin};
   for (int idx = first; idx < n; idx += nthreads) {
     double comm, total;
     int trans;
@@ -718,7 +775,7 @@ __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const 
     if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
     if (a.cost_out) a.cost_out[o] = total;
     for (int d = 0; d < v.dup_count; ++d) {
-      const int64_t od = o + st.dup[d];
+      const int64_t od = o + (st.dup[d] - v.entry_begin);
       if (a.comm_out) a.comm_out[od] = comm;
       if (a.trans_out) a.trans_out[od] = (uint8_t)trans;
       if (a.cost_out) a.cost_out[od] = total;
@@ -736,7 +793,9 @@ __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const 
 template <int M>
 __device__ __forceinline__ void tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M> &st,
                                              const TileView &v, int tid, int nthreads) {
-  if (uniform_i32(st.mixed)) {
+  int mixed = st.mixed[0];
+  for (int w = 1; w < nthreads / 64; ++w) mixed |= st.mixed[w];
+  if (uniform_i32(mixed)) {
     generic_tile_entries<M>(p, a, st, v, tid, nthreads);
     return;
   }
@@ -759,9 +818,10 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
   __shared__ TileStage<M> s_stage;
   const int64_t tile_id = xcd_chunked_unit(xcd_shift);
   if (tile_id >= n_tiles) return;
+  static_assert(kTileThreads == 64 || kTileThreads == 128 || kTileThreads == 256, "wavefronts per tile: 1, 2 or 4");
+  static_assert(kTileThreads >= APC_TILE_MAX_COLS && kTileThreads >= APC_TILE_MAX_ROWS &&
+                2 * kTileThreads > APC_TILE_MAX_DUPS, "one staging round covers a tile");
   const apc_tile tile = a.tiles[tile_id];
-  if (threadIdx.x == 0) s_stage.mixed = 0;
-  __syncthreads();
   stage_tile<M>(p, a, tile, s_stage, threadIdx.x, kTileThreads);
   __syncthreads();
   tile_entries<M>(p, a, s_stage, view_of(tile), threadIdx.x, kTileThreads);
@@ -1061,14 +1121,17 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
               tiles,        dup_entry_begin,   comm_out,   trans_out,   cost_out};
   const int nt = (int)n_tiles, xs = xcd_shift();
   hipStream_t s = (hipStream_t)stream;
-  // small matrices (traced graphs): one wavefront per tile; larger ones: two wavefronts share a
-  // tile's staged inputs.  (n_entries counts the copies written for de-duplicated edges too:
-  // work per tile either way.)
+  // Wavefronts per tile by the mean number of values a tile stores (n_entries counts the
+  // copies written for de-duplicated edges too: work per tile either way): one below 512,
+  // two up to 1536, four above.  Measured on tables of 290 .. 1800 values per tile: more
+  // wavefronts drain a long tile sooner, fewer leave more tiles resident per compute unit.
   const dim3 grid((unsigned)(((n_tiles + (1 << xs) - 1) >> xs) << xs));  // rounded up for xcd_chunked_unit
-  int threads = n_entries / n_tiles >= 512 ? 128 : 64;
+  const int64_t per_tile = n_entries / n_tiles;
+  int threads = per_tile >= 1536 ? 256 : per_tile >= 512 ? 128 : 64;
   if (const char *env = getenv("APC_TILE_THREADS")) threads = atoi(env);  // tuning override
 #define APC_LAUNCH(M_)                                                                                         \
-  if (threads >= 128) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 128>), grid, dim3(128), 0, s, *params, a, nt, xs); \
+  if (threads >= 256) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 256>), grid, dim3(256), 0, s, *params, a, nt, xs); \
+  else if (threads >= 128) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 128>), grid, dim3(128), 0, s, *params, a, nt, xs); \
   else hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 64>), grid, dim3(64), 0, s, *params, a, nt, xs)
   switch (params->mesh_ndim) {
     case 1: APC_LAUNCH(1); break;

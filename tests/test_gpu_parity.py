@@ -188,6 +188,22 @@ def test_deduplicated_edges_receive_identical_values(gpu_device):
         _run_and_compare(tb, mesh, 2.2, gpu_device)
 
 
+@pytest.mark.parametrize("threads", [64, 128, 256])
+def test_wavefronts_per_tile_do_not_change_results(gpu_device, threads, monkeypatch):
+    """The launcher picks one, two or four wavefronts per tile from the table's mean tile
+    size; each choice (forced here through the tuning override, read at every launch) must
+    give the oracle's bits, with and without identical edges stored to several copies."""
+    from test_abi_and_encoding import twin_graph
+
+    monkeypatch.setenv("APC_TILE_THREADS", str(threads))
+    for mesh in [(32, 8), (16, 8, 4)]:
+        tb = stress_dag(seed=9, n_nodes=500, mesh_sizes=mesh, frac_nonspec_nodes=0.02, frac_noncontiguous=0.2)
+        _run_and_compare(tb, mesh, 2.2, gpu_device)
+        tw = twin_graph(stress_dag(seed=10, n_nodes=300, mesh_sizes=mesh, frac_nonspec_nodes=0.02))
+        tw.build_tiles(2048, dedupe=True)
+        _run_and_compare(tw, mesh, 2.2, gpu_device)
+
+
 def test_tile_size_does_not_change_results(gpu_device):
     mesh = (16, 8, 4)
     base = None
