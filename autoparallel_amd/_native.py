@@ -67,6 +67,7 @@ EXPORTS = (
     "apc_input_tables",
     "apc_redistribute_tables",
     "apc_segmented_min",
+    "apc_strategy_bounds",
 )
 
 _lib = None

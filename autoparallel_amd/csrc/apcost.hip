@@ -897,6 +897,31 @@ int xcd_shift() {
   return shift;
 }
 
+// ------------------------------------------------------------------------------------------
+// a14: optimistic cost of every (node, strategy): the sum over the node's edges of that
+// consumer strategy's row minimum.  A plan pays, on every edge, at least the minimum of the
+// row of the strategy its consumer takes, so min over a node's strategies, summed over the
+// nodes, bounds the ILP objective from below, and the per-node argmin is the greedy choice a
+// warm start begins from.  One thread per strategy; a node's edges are added in the order of
+// edges_by_node (deterministic sum).
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void strategy_bounds_kernel(int64_t n_strategies,
+                                                                 const int32_t *__restrict__ strat_node,
+                                                                 const int64_t *__restrict__ node_strat_begin,
+                                                                 const int64_t *__restrict__ node_edge_begin,
+                                                                 const int32_t *__restrict__ edges_by_node,
+                                                                 const int64_t *__restrict__ edge_row_begin,
+                                                                 const double *__restrict__ row_min,
+                                                                 double *__restrict__ bound) {
+  const int64_t s = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (s >= n_strategies) return;
+  const int n = strat_node[s];
+  const int64_t k = s - node_strat_begin[n];
+  double sum = 0.0;
+  for (int64_t j = node_edge_begin[n]; j < node_edge_begin[n + 1]; ++j) sum += row_min[edge_row_begin[edges_by_node[j]] + k];
+  bound[s] = sum;
+}
+
 inline unsigned blocks_for(int64_t n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
 
 template <int G>
@@ -1168,6 +1193,20 @@ int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_se
     default: return fail(-1, "segment group width %d is not a power of two up to 64", g);
   }
   return check_launch("apc_segmented_min");
+}
+
+int apc_strategy_bounds(int64_t n_strategies, const int32_t *strat_node, const int64_t *node_strat_begin,
+                        const int64_t *node_edge_begin, const int32_t *edges_by_node, const int64_t *edge_row_begin,
+                        const double *row_min, double *bound, void *stream) {
+  if (n_strategies < 0) return fail(-1, "negative count");
+  if (n_strategies == 0) return 0;
+  if (!strat_node || !node_strat_begin || !node_edge_begin || !edge_row_begin || !row_min || !bound)
+    return fail(-1, "apc_strategy_bounds: NULL array");  // (edges_by_node may be NULL when no node has an edge)
+  if ((n_strategies + kBlock - 1) / kBlock > INT32_MAX) return fail(-1, "n_strategies %lld too large", (long long)n_strategies);
+  hipLaunchKernelGGL(strategy_bounds_kernel, dim3(blocks_for(n_strategies, kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
+                     n_strategies, strat_node, node_strat_begin, node_edge_begin, edges_by_node, edge_row_begin, row_min,
+                     bound);
+  return check_launch("apc_strategy_bounds");
 }
 
 }  // extern "C"

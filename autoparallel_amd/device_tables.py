@@ -303,3 +303,31 @@ class DeviceCostTables:
                                             self._stream())
         _native.check(rc, "apc_segmented_min")
         return mins, args
+
+    def strategy_bounds(self, row_min: torch.Tensor) -> torch.Tensor:
+        """Per-(node, strategy) sum of the row minima of the node's edges (``row_min`` in the
+        order of ``CostTables.row_ptr()``)."""
+        t = self.tables
+        if row_min.dtype != torch.float64 or not row_min.is_contiguous():
+            raise TypeError("strategy_bounds takes a contiguous float64 array of row minima")
+        if row_min.numel() != int(t.edge_n_tgt.astype(np.int64).sum()):
+            raise ValueError("row_min must hold one value per matrix row")
+        if getattr(self, "_bound_index", None) is None:
+            self._bound_index = {k: _to_device(v, self.device) for k, v in t.strategy_bound_index().items()}
+            self._bound_index["node_strat_begin"] = _to_device(np.ascontiguousarray(t.node_strat_begin, np.int64), self.device)
+        ix = self._bound_index
+        bound = self._empty((t.n_strategies,), torch.float64)
+        with torch.cuda.device(self.device):
+            rc = self.lib.apc_strategy_bounds(ctypes.c_int64(t.n_strategies), self._p(ix["strat_node"]),
+                                              self._p(ix["node_strat_begin"]), self._p(ix["node_edge_begin"]),
+                                              self._p(ix["edges_by_node"]), self._p(ix["edge_row_begin"]),
+                                              self._p(row_min), self._p(bound), self._stream())
+        _native.check(rc, "apc_strategy_bounds")
+        return bound
+
+    def greedy_strategies(self, row_min: torch.Tensor):
+        """-> (bound per strategy, min per node, argmin per node): the cheapest strategy of every
+        node when each of its edges is charged its row minimum."""
+        bound = self.strategy_bounds(row_min)
+        node_min, node_arg = self.segmented_min(bound, self._bound_index["node_strat_begin"], check=False)
+        return bound, node_min, node_arg

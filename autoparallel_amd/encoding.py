@@ -405,6 +405,28 @@ class CostTables:
         return out
 
     # ---- derived index arrays ------------------------------------------------------------
+    def strategy_bound_index(self) -> dict:
+        """Index arrays of the per-strategy lower bounds (C entry ``apc_strategy_bounds``):
+        the node of every strategy, every node's edges (as consumer) in edge order, and the
+        first matrix row of every edge in the order of ``row_ptr()``."""
+        n_nodes = self.n_nodes
+        n_strat = np.diff(self.node_strat_begin).astype(np.int64)
+        node = self.edge_node.astype(np.int64)
+        if self.n_edges and (node.min() < 0 or node.max() >= n_nodes):
+            raise RuntimeError("edge_node outside the node table")
+        if not np.array_equal(self.edge_n_tgt.astype(np.int64), n_strat[node]):
+            raise RuntimeError("an edge's row count differs from its consumer node's strategy count")
+        order = np.argsort(node, kind="stable")
+        node_edge_begin = np.zeros(n_nodes + 1, np.int64)
+        np.cumsum(np.bincount(node, minlength=n_nodes), out=node_edge_begin[1:])
+        edge_row_begin = np.cumsum(self.edge_n_tgt.astype(np.int64)) - self.edge_n_tgt
+        return {
+            "strat_node": _i32(np.repeat(np.arange(n_nodes, dtype=np.int64), n_strat)),
+            "node_edge_begin": node_edge_begin,
+            "edges_by_node": _i32(order),
+            "edge_row_begin": _i64(edge_row_begin),
+        }
+
     def row_ptr(self) -> np.ndarray:
         """CSR pointer of matrix rows over the entry array: one segment per
         (edge, consumer strategy), length = that edge's producer count."""

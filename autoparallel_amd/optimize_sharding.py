@@ -100,6 +100,14 @@ class DeviceBackend:
             mins, args = self.dev.segmented_min(self.dev.cost, row_ptr)
             return mins.cpu().numpy(), args.cpu().numpy()
 
+    def greedy(self, row_ptr):
+        """-> (bound per strategy, min per node, argmin per node) from the row minima of the cost table"""
+        from .device_tables import _real_tensors
+
+        with _real_tensors():
+            mins, _ = self.dev.segmented_min(self.dev.cost, row_ptr)
+            return tuple(x.cpu().numpy() for x in self.dev.greedy_strategies(mins))
+
 
 class CostRecords(Mapping):
     """``ds``: (s_i, argi, ss, ii) -> record, backed by the flat result arrays."""
@@ -694,6 +702,25 @@ class ShardingOptimizer:
     def row_minima(self):
         """min / first-argmin over producer strategies for every (edge, consumer strategy)."""
         return self.backend.row_min(self.encoded.tables.row_ptr())
+
+    def edge_minima(self):
+        """min / first-argmin (flattened consumer-strategy-major index) of every edge's whole matrix."""
+        return self.backend.row_min(self.encoded.tables.edge_entry_begin)
+
+    def greedy_strategies(self):
+        """-> ({node: strategy index}, lower bound).  Every node takes the strategy that is
+        cheapest when each of its input edges is charged the row minimum of that strategy.
+        The choices of neighbouring nodes need not agree, so this is a starting point, not a
+        plan; the sum of the per-node minima is a lower bound of every plan's objective (user
+        constraints only remove plans).  No counterpart in the reference, which hands the
+        table to the solver directly (optimize_sharding.py:648-659)."""
+        _, node_min, node_arg = self.backend.greedy(self.encoded.tables.row_ptr())
+        # (a node without strategies, the graph's output node, has argmin -1 and adds nothing)
+        choice = {node: int(node_arg[i]) for i, node in enumerate(self.encoded.nodes) if node_arg[i] >= 0}
+        return choice, math.fsum(m for m, a in zip(node_min.tolist(), node_arg.tolist()) if a >= 0)
+
+    def lower_bound(self) -> float:
+        return self.greedy_strategies()[1]
 
     # ---- structural checks (optimize_sharding.py:908-958) -------------------------------------------
     def validate(self):

@@ -126,9 +126,12 @@ def solve_plan(planner, args):
     constraints_s = time.perf_counter() - t0
     planner.optimize_placement()
     opt = planner.sharding_optimizer
+    t0 = time.perf_counter()
+    _, lower_bound = opt.greedy_strategies()  # row minima -> per-strategy bounds -> per-node minima, on the device
+    bound_s = time.perf_counter() - t0
     return {"constraints_s": constraints_s, "solve_s": planner.timings["solve_s"],
             "objective": opt.objective_value(), "ilp_rows": getattr(opt.prob, "rows_after_dedupe", None),
-            "ilp_variables": opt.n_variables}
+            "ilp_variables": opt.n_variables, "lower_bound_from_row_minima": lower_bound, "lower_bound_s": bound_s}
 
 
 def cpu_baseline(tables, params, target_seconds):

@@ -191,6 +191,19 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
 int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_segments, int64_t n_values,
                       double *seg_min, int32_t *seg_argmin, void *stream);
 
+/* Optimistic cost of every (node, strategy): bound[s] = sum, over the edges e of the node that
+ * owns strategy s (edges_by_node[node_edge_begin[n] .. node_edge_begin[n + 1]), added in that
+ * order), of row_min[edge_row_begin[e] + (s - node_strat_begin[n])], where row_min holds the
+ * row minima of the cost matrices (apc_segmented_min over the rows) and edge_row_begin[e] is
+ * the first row of edge e.  Every plan pays at least the row minimum of its consumer's
+ * strategy on every edge, so apc_segmented_min of bound over node_strat_begin gives a lower
+ * bound of the ILP objective (the sum of the minima) and a greedy strategy per node (the
+ * argmin).  No counterpart in the reference (optimize_sharding.py:648-659 goes straight to
+ * the solver): used for pruning and warm start.  The caller checks the index arrays. */
+int apc_strategy_bounds(int64_t n_strategies, const int32_t *strat_node, const int64_t *node_strat_begin,
+                        const int64_t *node_edge_begin, const int32_t *edges_by_node, const int64_t *edge_row_begin,
+                        const double *row_min, double *bound, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

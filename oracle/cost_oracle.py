@@ -470,3 +470,28 @@ def segmented_min(values, seg_ptr):
         mins.append(best)
         args.append(arg)
     return mins, args
+
+
+def strategy_bounds(enc: dict, row_min):
+    """Optimistic cost of every (node, strategy): the sum, over the node's edges in edge
+    order, of that consumer strategy's row minimum (``row_min`` ordered by edge, then consumer
+    strategy).  No reference counterpart (a14); pinned by brute force over all plans of tiny
+    graphs: min over a node's strategies, summed over nodes, never exceeds the best plan."""
+    nsb = [int(x) for x in enc["node_strat_begin"]]
+    bound = [0.0] * nsb[-1]
+    row = 0
+    for e in range(len(enc["edge_node"])):
+        n, nt = int(enc["edge_node"][e]), int(enc["edge_n_tgt"][e])
+        assert nt == nsb[n + 1] - nsb[n], "an edge has one row per strategy of its consumer"
+        for k in range(nt):
+            bound[nsb[n] + k] += float(row_min[row + k])
+        row += nt
+    return bound
+
+
+def greedy_strategies(enc: dict, row_min):
+    """-> (bound per strategy, min per node, first argmin per node, lower bound of any plan's
+    cost); a node without strategies (the graph's output node) has argmin -1 and adds nothing."""
+    bound = strategy_bounds(enc, row_min)
+    mins, args = segmented_min(bound, enc["node_strat_begin"])
+    return bound, mins, args, math.fsum(m for m, a in zip(mins, args) if a >= 0)

@@ -34,3 +34,10 @@ class OracleBackend:
 
     def row_min(self, row_ptr):
         return c_oracle.segmented_min(self.cost, row_ptr)
+
+    def greedy(self, row_ptr):
+        import numpy as np
+
+        mins, _ = c_oracle.segmented_min(self.cost, row_ptr)
+        bound, node_min, node_arg, _ = po.greedy_strategies(self.tables.as_dict(), mins)
+        return np.asarray(bound), np.asarray(node_min), np.asarray(node_arg)

@@ -245,6 +245,26 @@ def test_row_min_of_cost_tables(gpu_device):
     assert np.array_equal(mins.cpu().numpy(), wm) and np.array_equal(args.cpu().numpy(), wa)
 
 
+@pytest.mark.parametrize("mesh", [(32, 8), (16, 8, 4)])
+def test_strategy_bounds_and_greedy_strategies_match_oracle(gpu_device, mesh):
+    """Per-strategy sums of row minima and the per-node (min, argmin): same bits as the oracle
+    (a node's edges are added in edge order on both sides)."""
+    tb = stress_dag(seed=13, n_nodes=800, mesh_sizes=mesh, frac_nonspec_nodes=0.02)
+    d, want = _run_and_compare(tb, mesh, 2.2, gpu_device)
+    row_min, _ = d.segmented_min(d.cost, tb.row_ptr())
+    bound, node_min, node_arg = d.greedy_strategies(row_min)
+    torch.cuda.synchronize()
+    enc = tb.as_dict()
+    want_rows, _ = c_oracle.segmented_min(want["cost"], tb.row_ptr())
+    wb, wm, wa, _ = po.greedy_strategies(enc, want_rows)
+    assert np.array_equal(bound.cpu().numpy(), np.asarray(wb))
+    assert np.array_equal(node_min.cpu().numpy(), np.asarray(wm))
+    assert np.array_equal(node_arg.cpu().numpy(), np.asarray(wa))
+    # wrong sizes are refused before any launch
+    with pytest.raises(ValueError):
+        d.strategy_bounds(row_min[:-1].contiguous())
+
+
 def test_full_size_stress_properties(gpu_device):
     """The raw-throughput workload at a size the CPU cannot check entry by entry in test
     time: size-independent properties instead.  (a) the diagonal property: wherever the

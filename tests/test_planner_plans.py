@@ -239,6 +239,10 @@ def test_device_tables_give_identical_tables_plan_and_objective(gpu_device, mesh
     dm, da = d.row_minima()
     om, oa = o.row_minima()
     assert np.array_equal(dm, om) and np.array_equal(da, oa)
+    # so do the greedy strategies and the lower bound built on them, which the optimum respects
+    (dc, dlb), (oc, olb) = d.greedy_strategies(), o.greedy_strategies()
+    assert dlb == olb and {n.name: k for n, k in dc.items()} == {n.name: k for n, k in oc.items()}
+    assert dlb <= d.objective_value() * (1 + 1e-12)
 
 
 @pytest.mark.parametrize("kind,mesh_key", [("ffn", "2d"), ("block", "1d")])
