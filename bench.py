@@ -34,9 +34,9 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 # from inside this process, so the figure is the one of the profiled run of the same command
 # and only reported for exactly that table: (entries, tiles, algorithmic bytes) must match.
 MEASURED_TRAFFIC_BYTES = {
-    (1_821_368, 1_616, 32_348_914): (679.3 * 2.000 + 31_411.9) * 1024,             # llama3_8b, mesh (32, 8)
-    (73_251_434, 40_727, 1_255_915_920): (12_442.3 * 2.000 + 1_233_261.1) * 1024,   # llama3_70b, mesh (8, 8, 8)
-    (464_235_576, 426_918, 8_003_825_874): (162_390.3 * 2.000 + 7_739_954.5) * 1024,  # stress, mesh (16, 8, 4)
+    (1_821_368, 1_616, 32_348_914): (674.1 * 2.000 + 31_426.0) * 1024,             # llama3_8b, mesh (32, 8)
+    (73_251_434, 40_727, 1_255_915_920): (12_334.7 * 2.000 + 1_220_980.7) * 1024,   # llama3_70b, mesh (8, 8, 8)
+    (464_235_576, 426_918, 8_003_825_874): (159_699.9 * 2.000 + 7_760_701.8) * 1024,  # stress, mesh (16, 8, 4)
 }
 
 
