@@ -207,6 +207,24 @@ __global__ __launch_bounds__(kBlock) void tensor_tables_kernel(TensorTableArgs a
   tensor_tables_block(blockIdx.x, a);
 }
 
+// ceil(x / m) for x >= 0 and a mesh size m whose correctly rounded reciprocal y is known.
+// Below 2^52 the quotient is taken in fp64 (both operands exact, div_by rounds once, so the
+// truncated value is off by at most one) and corrected by the exact integer remainder: a
+// dozen instructions against the ~120 of a 64-bit integer division, which made this kernel
+// VALU-bound.  Larger values take the integer division.
+__device__ __forceinline__ int64_t ceil_div_by(int64_t x, int32_t m, double y) {
+  const int64_t num = x + m - 1;
+  if (num >> 52) return num / m;
+  int64_t q = (int64_t)div_by((double)num, (double)m, y);
+  int64_t rem = num - q * m;
+  if (rem < 0) {
+    q -= 1;
+    rem += m;
+  }
+  if (rem >= m) q += 1;
+  return q;
+}
+
 // ------------------------------------------------------------------------------------------
 // a8: local shard shape / stride / counts per spec
 // ------------------------------------------------------------------------------------------
@@ -219,6 +237,18 @@ struct SpecTableArgs {
 };
 
 // s_rows: kBlock * (APC_MAX_RANK + 1) values of LDS
+// Writes the first `live` values (a multiple of APC_MAX_RANK) of the workgroup's staged rows
+// (APC_MAX_RANK + 1 slots per row in LDS) to `out` as one contiguous run, two values (one
+// 16-byte store) per lane: rows hold an even number of values, so a pair never straddles rows.
+__device__ __forceinline__ void write_rows(int64_t *__restrict__ out, const int64_t *s_rows, int64_t live) {
+  typedef int64_t pair_t __attribute__((ext_vector_type(2)));
+  for (int k = 2 * threadIdx.x; k < live; k += 2 * kBlock) {
+    const int64_t *src = s_rows + (k / APC_MAX_RANK) * (APC_MAX_RANK + 1) + k % APC_MAX_RANK;
+    pair_t v = {src[0], src[1]};
+    *reinterpret_cast<pair_t *>(out + k) = v;
+  }
+}
+
 __device__ __forceinline__ void spec_tables_block(int64_t block, const apc_params &p, const SpecTableArgs &a,
                                                   int64_t *s_rows) {
   const int64_t n = a.n;
@@ -227,64 +257,68 @@ __device__ __forceinline__ void spec_tables_block(int64_t block, const apc_param
   const int64_t *__restrict__ shape = a.shape, *__restrict__ stride = a.stride;
   int64_t *__restrict__ shards = a.shards, *__restrict__ lshape = a.lshape, *__restrict__ lstride = a.lstride;
   int64_t *__restrict__ lnumel = a.lnumel, *__restrict__ lbytes = a.lbytes;
-  // each thread derives one spec; the two [kBlock][8] result blocks are transposed through LDS
-  // (one buffer, used for the shapes and then for the strides) so that the workgroup writes
-  // them as two contiguous 16 KB runs
+  // Each thread derives one spec in its own row of an LDS buffer (the Shard dim indexes the
+  // row, so no register array is indexed by a lane value), first the shape and then, in the
+  // same buffer, the stride; the workgroup writes each [kBlock][8] result block out as one
+  // contiguous 16 KB run.
   const int64_t base = block * kBlock;
   const int64_t s = base + threadIdx.x;
-  int64_t sh[APC_MAX_RANK], st[APC_MAX_RANK];
-#pragma unroll
-  for (int i = 0; i < APC_MAX_RANK; ++i) sh[i] = st[i] = 0;
-  int64_t nsh = 0, ne = 0, nb = 0;
+  int64_t *row = s_rows + threadIdx.x * (APC_MAX_RANK + 1);
+  const int64_t live = (n - base < kBlock ? n - base : kBlock) * APC_MAX_RANK;
+  int t = -1, r = 0;
+  uint32_t pc = 0;
   if (s < n) {
-    const int t = tensor[s];
+    t = tensor[s];
     if (t >= 0) {
-      const int r = rank[t];
+      r = rank[t];
+      pc = codes[s];
+    }
+  }
+  // (every load is issued before the first store: a load behind stores waits for them)
+  int64_t st[APC_MAX_RANK];
 #pragma unroll
-      for (int i = 0; i < APC_MAX_RANK; ++i) {
-        if (i < r) {
-          sh[i] = shape[(int64_t)t * APC_MAX_RANK + i];
-          st[i] = stride[(int64_t)t * APC_MAX_RANK + i];
-        }
-      }
-      nsh = 1;
-      const uint32_t pc = codes[s];
-      for (int i = 0; i < p.mesh_ndim; ++i) {
-        const uint32_t c = (pc >> (8 * i)) & 0xFF;
-        if (kind_of(c) == 2) {
-          const int d = dim_of(c);
-          const int64_t m = p.mesh_size[i];
-          nsh *= m;
-          // compile-time indices keep sh/st in registers
-#pragma unroll
-          for (int j = 0; j < APC_MAX_RANK; ++j) {
-            if (j == d) sh[j] = (sh[j] + m - 1) / m;
-            if (j == d - 1 && d - 1 > 0) st[j] = (st[j] + m - 1) / m;  // compute_estimation.py:225-228
-          }
-        }
-      }
+  for (int i = 0; i < APC_MAX_RANK; ++i) {
+    row[i] = i < r ? shape[(int64_t)t * APC_MAX_RANK + i] : 0;
+    st[i] = i < r ? stride[(int64_t)t * APC_MAX_RANK + i] : 0;
+  }
+  const int64_t item = t >= 0 ? itemsize[t] : 0;
+  int64_t nsh = t >= 0 ? 1 : 0;
+  for (int i = 0; i < p.mesh_ndim; ++i) {
+    const uint32_t c = (pc >> (8 * i)) & 0xFF;
+    if (kind_of(c) == 2) {
+      const int d = dim_of(c);
+      nsh *= p.mesh_size[i];
+      if (d < APC_MAX_RANK) row[d] = ceil_div_by(row[d], p.mesh_size[i], p.inv_mesh[i]);
+    }
+  }
+  if (s < n) {
+    int64_t ne = 0, nb = 0;
+    if (t >= 0) {
       ne = 1;
 #pragma unroll
       for (int i = 0; i < APC_MAX_RANK; ++i)
-        if (i < r) ne *= sh[i];
-      nb = ne * itemsize[t];
+        if (i < r) ne *= row[i];
+      nb = ne * item;
     }
     shards[s] = nsh;
     lnumel[s] = ne;
     lbytes[s] = nb;
   }
-  const int64_t live = (n - base < kBlock ? n - base : kBlock) * APC_MAX_RANK;
-#pragma unroll
-  for (int i = 0; i < APC_MAX_RANK; ++i) s_rows[threadIdx.x * (APC_MAX_RANK + 1) + i] = sh[i];
   __syncthreads();
-  for (int k = threadIdx.x; k < live; k += kBlock)
-    lshape[base * APC_MAX_RANK + k] = s_rows[(k / APC_MAX_RANK) * (APC_MAX_RANK + 1) + k % APC_MAX_RANK];
+  write_rows(lshape + base * APC_MAX_RANK, s_rows, live);
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < APC_MAX_RANK; ++i) s_rows[threadIdx.x * (APC_MAX_RANK + 1) + i] = st[i];
+  for (int i = 0; i < APC_MAX_RANK; ++i) row[i] = st[i];
+  for (int i = 0; i < p.mesh_ndim; ++i) {
+    const uint32_t c = (pc >> (8 * i)) & 0xFF;
+    if (kind_of(c) == 2) {
+      const int d = dim_of(c);
+      if (d - 1 > 0 && d - 1 < APC_MAX_RANK)  // compute_estimation.py:225-228
+        row[d - 1] = ceil_div_by(row[d - 1], p.mesh_size[i], p.inv_mesh[i]);
+    }
+  }
   __syncthreads();
-  for (int k = threadIdx.x; k < live; k += kBlock)
-    lstride[base * APC_MAX_RANK + k] = s_rows[(k / APC_MAX_RANK) * (APC_MAX_RANK + 1) + k % APC_MAX_RANK];
+  write_rows(lstride + base * APC_MAX_RANK, s_rows, live);
 }
 
 __global__ __launch_bounds__(kBlock) void spec_tables_kernel(apc_params p, SpecTableArgs a) {
