@@ -41,8 +41,6 @@ class ApcParams(ctypes.Structure):
         ("inv_mesh", ctypes.c_double * APC_MAX_MESH),
         ("inv_hbm_bw", ctypes.c_double),
         ("inv_rw_eff", ctypes.c_double),
-        ("shards", ctypes.c_double * (1 << APC_MAX_MESH)),
-        ("inv_shards", ctypes.c_double * (1 << APC_MAX_MESH)),
     ]
 
 

@@ -142,11 +142,4 @@ class CostModelParams:
             c.inv_mesh[i] = 1.0 / float(self.mesh_sizes[i])
         c.inv_hbm_bw = 1.0 / self.hbm_bw
         c.inv_rw_eff = 1.0 / self.rw_eff
-        for mask in range(1 << self.ndim):
-            shards = 1.0
-            for i in range(self.ndim):
-                if (mask >> i) & 1:
-                    shards *= float(self.mesh_sizes[i])
-            c.shards[mask] = shards
-            c.inv_shards[mask] = 1.0 / shards
         return c

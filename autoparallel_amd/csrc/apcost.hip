@@ -978,13 +978,6 @@ int check_params(const apc_params *p) {
   }
   if (p->inv_hbm_bw != 1.0 / p->hbm_bw || p->inv_rw_eff != 1.0 / p->rw_eff)
     return fail(-1, "inv_hbm_bw / inv_rw_eff are not 1.0 / hbm_bw, 1.0 / rw_eff");
-  for (int mask = 0; mask < (1 << p->mesh_ndim); ++mask) {
-    double shards = 1.0;
-    for (int i = 0; i < p->mesh_ndim; ++i)
-      if ((mask >> i) & 1) shards *= (double)p->mesh_size[i];
-    if (p->shards[mask] != shards || p->inv_shards[mask] != 1.0 / shards)
-      return fail(-1, "shards[%d] / inv_shards[%d] do not match the mesh", mask, mask);
-  }
   return 0;
 }
 

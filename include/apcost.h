@@ -104,8 +104,6 @@ typedef struct apc_params {
   double inv_mesh[APC_MAX_MESH]; /* 1.0 / mesh_size[i] */
   double inv_hbm_bw;             /* 1.0 / hbm_bw */
   double inv_rw_eff;             /* 1.0 / rw_eff */
-  double shards[1 << APC_MAX_MESH];     /* product of mesh_size[i] over the bits of the index */
-  double inv_shards[1 << APC_MAX_MESH]; /* 1.0 / shards[mask] */
 } apc_params;
 
 int apc_version(void);

@@ -29,13 +29,27 @@ def test_library_exports_every_declared_symbol():
     assert lib.apc_version() == 1
 
 
-def test_params_struct_layout_matches_header():
-    # 4 + 16 (+4 pad) + 32 + 32 + 7*8 + 64 + 4 (+4 pad)
-    assert ctypes.sizeof(_native.ApcTile) == 64 and _native.ApcTile.entry_begin.offset == 40
-    # 216 bytes of model parameters + 4 + 4 + 1 + 1 + 16 + 16 derived doubles
-    assert ctypes.sizeof(_native.ApcParams) == 216 + 42 * 8
-    assert _native.ApcParams.bw.offset == 24 and _native.ApcParams.gpu_flops.offset == 144
-    assert _native.ApcParams.inv_bw.offset == 216
+def test_params_struct_layout_matches_header(tmp_path):
+    """The ctypes mirrors against the C compiler's own layout of include/apcost.h."""
+    import subprocess
+
+    fields_p = [name for name, _ in _native.ApcParams._fields_]
+    fields_t = [name for name, _ in _native.ApcTile._fields_]
+    src = tmp_path / "layout.c"
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "apcost.h"', 'int main(void) {',
+             '  printf("%zu %zu\\n", sizeof(apc_params), sizeof(apc_tile));']
+    lines += [f'  printf("%zu\\n", offsetof(apc_params, {f}));' for f in fields_p]
+    lines += [f'  printf("%zu\\n", offsetof(apc_tile, {f}));' for f in fields_t]
+    lines += ['  return 0;', '}']
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include"),
+                    "-o", str(exe), str(src)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert [int(out[0]), int(out[1])] == [ctypes.sizeof(_native.ApcParams), ctypes.sizeof(_native.ApcTile)]
+    want = [getattr(_native.ApcParams, f).offset for f in fields_p] + [getattr(_native.ApcTile, f).offset for f in fields_t]
+    assert [int(x) for x in out[2:]] == want
+    assert ctypes.sizeof(_native.ApcTile) == 64  # one record per scalar 64-byte load
 
 
 def test_placement_codes_round_trip():
