@@ -550,9 +550,33 @@ class StrategyEnumerator:
 
         return propagate_single_input_strategy(schema)
 
-    def _split_tensor(self, schema):
-        raise NotImplementedError(
-            "aten.split.Tensor: the per-spec split rule this override relied on no longer exists in torch")
+    def _split_tensor(self, schema) -> OpStrategy:
+        """propagation_rules.py:649-671.  The reference applies torch's per-spec split rule (in
+        the torch it pins; the function is gone from current torch, so what it did is restated
+        here) to every strategy of the producer: a producer with a Partial placement is not
+        supported, one sharded on the split dim yields no strategy (the old rule asked for a
+        redistribution instead), any other keeps its placements on every piece.  A kept
+        strategy accepts only the producer strategy it came from (cost 0, all others inf)."""
+        args = schema.args_schema
+        producer, size = args[0], args[1]
+        dim = args[2] if len(args) > 2 else 0
+        out = []
+        for i, s in enumerate(producer.strategies):
+            src = s.output_spec
+            if any(p.is_partial() for p in src.placements):
+                raise NotImplementedError(f"splitting distributed tensor with Partial placement is not implemented: {src}")
+            d = dim + src.ndim if dim < 0 else dim
+            if any(p.is_shard(d) for p in src.placements):
+                continue
+            n = src.tensor_meta.shape[d]
+            pieces = len(size) if isinstance(size, (list, tuple)) else max(-(-n // size), 1)
+            outs = tuple(DTensorSpec(self.mesh, src.placements) for _ in range(pieces))
+            spec = OpSpec(outs, input_specs=(src,))
+            row = [math.inf] * len(producer.strategies)
+            row[i] = 0.0
+            spec.redistribute_cost = [row]
+            out.append(spec)
+        return OpStrategy(out)
 
     def _sdpa(self, schema) -> OpStrategy:
         out = self._registered(schema.op, schema)

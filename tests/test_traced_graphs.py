@@ -163,3 +163,45 @@ def test_device_tables_match_oracle_on_benchmark_configurations(gpu_device, fake
             assert np.array_equal(d[name], o[name]), name
     # something was actually costed: finite positive comm and compute costs exist
     assert (d["comm"][np.isfinite(d["comm"])] > 0).any() and (d["per_arg"] > 0).any()
+
+
+def test_split_tensor_rule(fake_pg):
+    """aten.split.Tensor (propagation_rules.py:649-671): a producer strategy sharded on the
+    split dim yields none, any other keeps its placements on every piece and accepts only the
+    producer strategy it came from; a Partial producer is refused as the reference's rule did."""
+    import math
+
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.distributed.tensor._op_schema import OpSpec, OpStrategy
+    from torch.distributed.tensor._dtensor_spec import DTensorSpec
+    from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
+
+    from autoparallel_amd.graphs.strategies import StrategyEnumerator, _tensor_meta
+
+    mesh = init_device_mesh("cpu", (4, 2), mesh_dim_names=("dp", "tp"))
+    enum = StrategyEnumerator(mesh)
+    with torch.device("meta"):
+        x = torch.empty(8, 12, 16)
+    producer = enum._placeholder(x)
+    aten = torch.ops.aten
+    out = enum.placement_options(aten.split.Tensor, [producer, 4, 1], [x, 4, 1], {})
+    kept = [i for i, s in enumerate(producer.strategies) if not any(p.is_shard(1) for p in s.output_spec.placements)]
+    assert len(kept) < len(producer.strategies) and len(out.strategies) == len(kept)
+    for s, i in zip(out.strategies, kept):
+        src = producer.strategies[i].output_spec
+        assert len(s.output_specs) == 3  # 12 / 4 pieces
+        for piece in s.output_specs:
+            assert piece.placements == src.placements and tuple(piece.tensor_meta.shape) == (8, 4, 16)
+        assert s.input_specs[0].placements == src.placements
+        row = s.redistribute_cost[0]
+        assert row[i] == 0.0 and all(math.isinf(c) for j, c in enumerate(row) if j != i)
+    # ragged sizes given as a list, negative dim
+    out = enum.placement_options(aten.split.Tensor, [producer, 5, -1], [x, 5, -1], {})
+    assert all([tuple(p.tensor_meta.shape) for p in s.output_specs] == [(8, 12, 5)] * 3 + [(8, 12, 1)] for s in out.strategies)
+    assert not any(any(p.is_shard(2) for p in s.output_specs[0].placements) for s in out.strategies)
+    # a Partial producer
+    tm = _tensor_meta(x)
+    partial = DTensorSpec(mesh, (Partial("sum"), Replicate()), tensor_meta=tm)
+    with pytest.raises(NotImplementedError, match="Partial"):
+        enum.placement_options(aten.split.Tensor, [OpStrategy([OpSpec(partial, input_specs=[partial], redistribute_cost=[[0.0]])]), 4, 1],
+                               [x, 4, 1], {})
