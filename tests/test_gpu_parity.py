@@ -93,6 +93,49 @@ def _two_node_tables(mesh, shape, stride, itemsize, src_codes, tgt_codes, flags=
         edge_entry_begin=[0, ns * nt], edge_strat_begin=[ns], pt_values=[])
 
 
+@pytest.mark.parametrize("mesh", [(3, 5, 7), (64, 2), (6, 1, 1000003)])
+def test_local_shapes_of_very_large_dims(gpu_device, mesh):
+    """The shard-shape kernel divides through the mesh size's reciprocal with an integer
+    correction below 2^52 and with the integer division above: dims and strides chosen at
+    multiples of the mesh sizes +-1, near 2^52 and far above it, against Python integers."""
+    M = len(mesh)
+    rng = np.random.default_rng(5)
+    dims = []
+    for m in mesh:
+        for k in (1, 2, 3, 1000, 2**20 + 1, 2**40 // m, 2**51 // m):
+            dims += [k * m - 1, k * m, k * m + 1]
+    dims += [2**52 - 1, 2**52, 2**52 + 1, 2**52 - 64, 1, 2, 0]
+    shapes, strides = [], []
+    for i, d in enumerate(dims):
+        # rank 3, the large value as shape[1] (bytes stay below 2^53: the other dims are 1) and,
+        # independently, stride[1] (the one Shard(2) divides) up to 2^62 (strides are not bounded by the bytes)
+        big = int(rng.integers(2**52, 2**62)) if i % 3 == 0 else d
+        shapes.append([1, d, 1] + [0] * 5)
+        strides.append([dims[(i * 5 + 1) % len(dims)], big if i % 3 == 0 else dims[(i * 7 + 3) % len(dims)], 1] + [0] * 5)
+    T = len(shapes)
+    codes, tensor = [], []
+    shard_sets = [[shard_code(1)] * M, [shard_code(2)] * M, [shard_code(1), 0, shard_code(2)][:M] + [0] * max(0, M - 3),
+                  [shard_code(0)] * M]
+    for t in range(T):
+        for c in shard_sets:
+            codes.append(pack_codes(c[:M]))
+            tensor.append(t)
+    n = len(codes)
+    tb = CostTables(
+        mesh_sizes=mesh, tensor_rank=[3] * T, tensor_itemsize=[1] * T, tensor_shape=shapes, tensor_stride=strides,
+        spec_codes=codes, spec_tensor=tensor, strat_flops=[0] * n, strat_rw_bytes=[0] * n, strat_dtype=[3] * n,
+        strat_zero_cost=[1] * n, strat_num_args=[1] * n, node_strat_begin=[0, n], edge_node=[], edge_arg=[],
+        edge_src_begin=[], edge_n_src=[], edge_tgt_begin=[], edge_n_tgt=[], edge_flags=[], edge_pt_begin=[],
+        edge_entry_begin=[0], edge_strat_begin=[], pt_values=[])
+    d = DeviceCostTables(tb, CostModelParams.from_mesh(mesh), device=gpu_device, validate=False)
+    got = d.run_spec_tables()
+    torch.cuda.synchronize()
+    want = po.spec_tables(tb.as_dict(), mesh)
+    for key, w in zip(("num_shards", "local_shape", "local_stride", "local_numel", "local_bytes"), want):
+        # (local numel / bytes of the 2^52-sized dims exceed nothing: the other dims are 1)
+        assert np.array_equal(got[key].cpu().numpy(), np.asarray(w, dtype=np.int64)), key
+
+
 def _golden():
     import json
     import os
