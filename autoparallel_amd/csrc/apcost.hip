@@ -885,12 +885,26 @@ __global__ __launch_bounds__(kBlock) void segmented_min_kernel(const double *__r
     }
   };
   // A lane reads pairs of consecutive values (one 16-byte load; segments start at any 8-byte
-  // offset, which global loads allow), two such loads in flight, taken in index order (first
+  // offset, which global loads allow), four such loads in flight (two on a short remainder), taken in index order (first
   // minimum wins); the G lanes of a group sweep 2 G consecutive values per load.
   struct __attribute__((packed, aligned(8))) Pair {
     double x, y;
   };
   int64_t j = lo + 2 * sub;
+  for (; j + 6 * G + 1 < hi; j += 8 * G) {
+    const Pair a = *reinterpret_cast<const Pair *>(values + j);
+    const Pair b = *reinterpret_cast<const Pair *>(values + j + 2 * G);
+    const Pair c = *reinterpret_cast<const Pair *>(values + j + 4 * G);
+    const Pair d = *reinterpret_cast<const Pair *>(values + j + 6 * G);
+    take(a.x, j);
+    take(a.y, j + 1);
+    take(b.x, j + 2 * G);
+    take(b.y, j + 2 * G + 1);
+    take(c.x, j + 4 * G);
+    take(c.y, j + 4 * G + 1);
+    take(d.x, j + 6 * G);
+    take(d.y, j + 6 * G + 1);
+  }
   for (; j + 2 * G + 1 < hi; j += 4 * G) {
     const Pair a = *reinterpret_cast<const Pair *>(values + j);
     const Pair b = *reinterpret_cast<const Pair *>(values + j + 2 * G);
