@@ -14,6 +14,8 @@ from __future__ import annotations
 import logging
 import time
 
+import torch
+
 from .graphs.capture import capture_joint_graph
 from .optimize_sharding import ShardingOptimizer
 
@@ -22,6 +24,7 @@ logger = logging.getLogger(__name__)
 
 class AutoParallelPlanner:
     optimizer_cls = ShardingOptimizer
+    active = False  # api.py:251-308: False before the with block, True inside, None after
 
     def __init__(self, model, input_fn, mesh, param_dtype=None, reduce_dtype=None, repeated_subgraphs=False,
                  device="cpu", dynamo=False):
@@ -38,7 +41,15 @@ class AutoParallelPlanner:
         self.input_constraints = None
         self.output_constraints = None
 
+    def _assert_entered(self):
+        # api.py:300-308
+        if self.active is False:
+            raise RuntimeError("You must use AutoParallel as a context manager: with AutoParallel() as p: ...")
+        if self.active is None:
+            raise RuntimeError("AutoParallel is not reentrant, please file a bug report if you need this functionality")
+
     def __enter__(self):
+        assert self.active is False
         t0 = time.perf_counter()
         self._ctx = capture_joint_graph(self.model, self.input_fn, param_dtype=self.param_dtype,
                                         device=self.trace_device, dynamo=self.dynamo)
@@ -59,12 +70,15 @@ class AutoParallelPlanner:
         self.timings["optimizer_s"] = time.perf_counter() - t0
         logger.info("%s %.3f s", "optimizer_s", self.timings["optimizer_s"])
         self.timings.update({f"optimizer_{k}": v for k, v in self.sharding_optimizer.timings.items()})
+        self.active = True
         return self
 
     def __exit__(self, *exc):
+        self.active = None
         return self._ctx.__exit__(*exc)
 
     def add_parameter_memory_constraint(self, low=None, high=None):
+        self._assert_entered()
         if low is None:
             low = 0.0
         if high is None:
@@ -73,16 +87,19 @@ class AutoParallelPlanner:
         self.sharding_optimizer.add_parameter_memory_constraint(low, high)
 
     def add_input_constraints(self, constraints):
+        self._assert_entered()
         assert self.input_constraints is None, "Input constraints have already been set"
         self.sharding_optimizer.add_sharded_input_constraint(constraints)
         self.input_constraints = constraints if constraints is not None else ()
 
     def add_output_constraints(self, constraints):
+        self._assert_entered()
         assert self.output_constraints is None, "Output constraints have already been set"
         self.sharding_optimizer.add_sharded_output_constraint(constraints)
         self.output_constraints = constraints if constraints is not None else ()
 
     def optimize_placement(self, verbose=False):
+        self._assert_entered()
         if self.input_constraints is None:
             self.add_input_constraints(None)
         if self.output_constraints is None:
@@ -96,3 +113,68 @@ class AutoParallelPlanner:
         if self.sharding_optimizer.prob.status == -1:
             raise RuntimeError("Didn't find solution")
         return self.sharding_placement
+
+
+class _ModelWithLoss(torch.nn.Module):
+    """forward(*model_inputs, target) -> loss_fn(model(*model_inputs), target) (api.py:329-332)."""
+
+    def __init__(self, model, loss_fn):
+        super().__init__()
+        self.model = model
+        self.loss_fn = loss_fn
+
+    def forward(self, *args):
+        *model_inputs, target = args
+        return self.loss_fn(self.model(*model_inputs), target)
+
+
+class AutoParallel(AutoParallelPlanner):
+    """The reference's entry point with its constructor (api.py:195-253), for the planning
+    half of its life cycle: ``with AutoParallel(model, input_fn, mesh, mp_policy) as autop:``
+    then the constraint methods and ``optimize_placement()``.  ``mp_policy`` is torch's
+    ``MixedPrecisionPolicy`` (``reduce_dtype`` defaults to ``param_dtype`` as in
+    cast_parametrization.py:116-125); ``repeated_subgraphs`` travels in ``**kwargs`` as in the
+    reference.  The arguments that only matter once a plan is applied (``compile``,
+    ``enable_ac``, ``ac_stage_size_in_GiB``, ``reshard_after_forward``) are kept as
+    attributes; applying a plan is outside this package and ``apply_placement`` says so."""
+
+    def __init__(self, model, input_fn, mesh, mp_policy=None, compile: bool = False, enable_ac: bool = True,
+                 ac_stage_size_in_GiB="auto", reshard_after_forward: bool = True, dynamic: bool = False,
+                 loss_fn=None, **kwargs):
+        if dynamic:
+            raise NotImplementedError("dynamic shapes are not planned by this package")
+        param_dtype = reduce_dtype = None
+        if mp_policy is not None:
+            param_dtype = mp_policy.param_dtype
+            reduce_dtype = mp_policy.reduce_dtype or param_dtype
+        self.mp_policy = mp_policy
+        self.kwargs = kwargs
+        self.compile = compile
+        self.enable_ac = enable_ac
+        self.ac_stage_size_in_GiB = ac_stage_size_in_GiB
+        self.reshard_after_forward = reshard_after_forward
+        self.loss_fn = loss_fn
+        if loss_fn is not None:
+            user_input_fn = input_fn
+
+            def input_fn():
+                raw = user_input_fn()
+                if not (isinstance(raw, tuple) and len(raw) == 2):
+                    raise ValueError("When loss_fn is provided, input_fn must return (inputs, target) "
+                                     "where inputs can be a single tensor or tuple of tensors")
+                model_inputs, target = raw
+                if not isinstance(model_inputs, tuple):
+                    model_inputs = (model_inputs,)
+                return (*model_inputs, target)
+
+            model = _ModelWithLoss(model, loss_fn)
+        super().__init__(model, input_fn, mesh, param_dtype=param_dtype, reduce_dtype=reduce_dtype,
+                         repeated_subgraphs=kwargs.get("repeated_subgraphs", False),
+                         dynamo=kwargs.get("dynamo", False))
+
+    def optimize_placement(self, verbose=True):
+        return super().optimize_placement(verbose=verbose)
+
+    def apply_placement(self, sharding_placement=None):
+        raise NotImplementedError("applying a plan (re-tracing with collectives, api.py:447-602) is outside this package: "
+                                  "hand optimize_placement()'s result to the reference's apply_placement")

@@ -276,3 +276,45 @@ def test_local_map_plan_from_device_tables(gpu_device, meshes):
     assert np.array_equal(d.cost, o.cost)
     assert d.res == o.res and d.objective_value() == o.objective_value()
     _check_local_map(dev_autop, dev_plan)
+
+
+def test_reference_entry_point_signature(meshes):
+    """``AutoParallel`` with the reference's constructor (api.py:202-253): mixed-precision policy,
+    loss function with (inputs, target), context-manager discipline, plan on the (32, 8) mesh."""
+    from torch.distributed.fsdp import MixedPrecisionPolicy
+
+    from autoparallel_amd.api import AutoParallel
+
+    class OracleAutoParallel(AutoParallel):
+        optimizer_cls = OracleOptimizer
+
+    mesh = meshes["2d"]
+    bs, dim = 64 * mesh.shape[0], 1024
+    with torch.device("meta"):
+        model = torch.nn.Linear(dim, dim)
+
+    def input_fn():
+        return torch.randn(bs, dim)
+
+    def with_target():
+        return input_fn(), torch.randn(bs, dim)
+
+    autop = OracleAutoParallel(model, with_target, mesh, MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=torch.float32),
+                               loss_fn=torch.nn.functional.mse_loss, repeated_subgraphs=True)
+    with pytest.raises(RuntimeError, match="context manager"):
+        autop.add_parameter_memory_constraint()
+    with autop:
+        assert autop.sharding_optimizer.rescale_grad_comm_cost_for_mp == pytest.approx(4 / 2 * 1.1)
+        autop.add_parameter_memory_constraint(low=None, high=None)
+        autop.add_input_constraints([(Shard(0), Replicate())] * 2)
+        autop.add_output_constraints([(Replicate(), Replicate())])  # the loss is a scalar: no batch dim to shard
+        placement = autop.optimize_placement(verbose=False)
+        params = get_param_nodes(autop.gm.graph)
+        assert len(params) == 2 and all(placement[n].output_specs.tensor_meta.dtype == torch.float32 for n in params)
+        with pytest.raises(NotImplementedError, match="outside this package"):
+            autop.apply_placement(placement)
+    with pytest.raises(RuntimeError, match="not reentrant"):
+        autop.optimize_placement()
+    with pytest.raises(ValueError, match="input_fn must return"):
+        with OracleAutoParallel(model, input_fn, mesh, loss_fn=torch.nn.functional.mse_loss):
+            pass
