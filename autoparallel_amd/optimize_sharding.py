@@ -228,6 +228,7 @@ class ShardingOptimizer:
     # row / column sum constraints leave exactly one feasible (integral) value for every entry
     # variable.  Same feasible plans and optimum, far fewer branching variables for the solver.
     node_choice_variables = True
+    compact_constraints = True  # with choice variables: the structural constraints written through them
 
     def __init__(self, gm, mesh, rescale_grad_comm_cost_for_mp=1.0, repeated_subgraphs=False):
         self.gm = gm
@@ -492,7 +493,70 @@ class ShardingOptimizer:
                                "choice_link")
         self.prob.integrality[:self.n_variables] = 0.0
 
+    def add_compact_constraints(self):
+        """The feasible plans of the reference's three structural constraints, written through
+        the per-(node, strategy) choice variables y instead of entry variables against entry
+        variables:
+          * every node takes one strategy: sum_s y[n, s] = 1;
+          * every edge's matrix row sums are its consumer's choice:
+            sum_ii x[e, ss, ii] = y[consumer, ss]  (unique decision per edge, agreement of a
+            node's arguments and the choice link, optimize_sharding.py:402-455, in one family);
+          * the columns a consumer reads are its producer's choice:
+            sum_ss x[e, ss, o] = y[producer, o]  for exactly the (producer, user, argument
+            index) triples the reference couples (optimize_sharding.py:457-520, including its
+            use of the user's de-duplicated input list as the argument index).
+        Row sums equal to y make the reference's producer-row = consumer-column equation the
+        third family, so the feasible set is the same; the rows are shorter (a consistency
+        row no longer carries the producer's whole first matrix), about half as many nonzeros,
+        and nothing is left for the solver's presolve to discover as redundant."""
+        seen = set()
+        one_cols, one_lens = [], []
+        cols, vals, lens = [], [], []
+        for s_i, node in enumerate(self.nodes):
+            if node.op == "output":
+                continue
+            cb = self.node_choice_base[s_i]
+            n = len(self.strats[node].strategies)
+            if ("one", cb) not in seen:
+                seen.add(("one", cb))
+                one_cols.append(cb + np.arange(n))
+                one_lens.append(n)
+            for argi in range(self.num_args[s_i]):
+                b, nt, ns = self._edge_vars(s_i, argi)
+                assert nt == n
+                if ("row", b, cb) in seen:
+                    continue
+                seen.add(("row", b, cb))
+                entries = b + np.arange(nt)[:, None] * ns + np.arange(ns)[None, :]
+                cols.append(np.concatenate([entries, (cb + np.arange(nt))[:, None]], axis=1).ravel())
+                vals.append(np.tile(np.concatenate([np.ones(ns), [-1.0]]), nt))
+                lens.append(np.full(nt, ns + 1))
+            for user in node.users:
+                if user.op == "output":
+                    continue
+                s_j = self.node_map[user]
+                argj = [i for i, x in enumerate(user.all_input_nodes) if x == node]
+                assert len(argj) == 1
+                bc, ntc, nsc = self._edge_vars(s_j, argj[0])
+                assert nsc == n, f"{node} has {n} strategies, {user} arg {argj[0]} reads {nsc}"
+                if ("col", bc, cb) in seen:
+                    continue
+                seen.add(("col", bc, cb))
+                entries = bc + np.arange(ntc)[None, :] * nsc + np.arange(nsc)[:, None]  # column o of the consumer
+                cols.append(np.concatenate([entries, (cb + np.arange(nsc))[:, None]], axis=1).ravel())
+                vals.append(np.tile(np.concatenate([np.ones(ntc), [-1.0]]), nsc))
+                lens.append(np.full(nsc, ntc + 1))
+        if one_cols:
+            self.prob.add_rows(np.concatenate(one_cols), 1.0, np.asarray(one_lens), 1.0, 1.0, "one_strategy")
+        if cols:
+            self.prob.add_rows(np.concatenate(cols), np.concatenate(vals), np.concatenate(lens), 0.0, 0.0, "choice_link")
+        self.prob.integrality[:self.n_variables] = 0.0
+
     def add_default_constraints(self):
+        if self.node_choice_variables and self.compact_constraints:
+            self.add_compact_constraints()
+            self.add_inf_cost_constraint()
+            return
         if self.node_choice_variables:
             self.add_choice_link_constraint()
         self.add_unique_decision_constraint()
