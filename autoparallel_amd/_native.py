@@ -64,6 +64,7 @@ EXPORTS = (
     "apc_compute_costs",
     "apc_input_tables",
     "apc_redistribute_tables",
+    "apc_build_tables",
     "apc_segmented_min",
     "apc_strategy_bounds",
 )

@@ -166,6 +166,21 @@ __device__ __forceinline__ int64_t xcd_chunked_unit(int shift) {
   return (int64_t)(blockIdx.x & ((1u << shift) - 1)) * per + (blockIdx.x >> shift);
 }
 
+// Element `i` (a per-lane index below M) of one of the arrays of the kernel parameters, as a select chain over scalar registers.  (Indexing the array by a lane value
+// makes the compiler read the kernel arguments through vector memory, and a vector load
+// waits behind every store the compute unit has in flight.)
+template <int M, typename T, int N>
+__device__ __forceinline__ T pick(const T (&v)[N], int i) {
+  static_assert(M <= N, "array shorter than the mesh");
+  T e[M];  // every element is read (scalar loads) before the selects, so they stay selects
+#pragma unroll
+  for (int k = 0; k < M; ++k) e[k] = v[k];
+  T r = e[0];
+#pragma unroll
+  for (int k = 1; k < M; ++k) r = i == k ? e[k] : r;
+  return r;
+}
+
 // ------------------------------------------------------------------------------------------
 // a7: bytes + contiguity per tensor
 // ------------------------------------------------------------------------------------------
@@ -177,34 +192,46 @@ struct TensorTableArgs {
   uint8_t *cont;
 };
 
-__device__ __forceinline__ void tensor_tables_block(int64_t block, const TensorTableArgs &a) {
-  const int64_t n = a.n;
-  const int32_t *__restrict__ rank = a.rank, *__restrict__ itemsize = a.itemsize;
-  const int64_t *__restrict__ shape = a.shape, *__restrict__ stride = a.stride;
-  int64_t *__restrict__ bytes = a.bytes;
-  uint8_t *__restrict__ cont = a.cont;
-  const int64_t t = block * kBlock + threadIdx.x;
-  if (t >= n) return;
-  const int r = rank[t];
-  const int64_t *sh = shape + t * APC_MAX_RANK;
-  const int64_t *st = stride + t * APC_MAX_RANK;
-  int64_t nbytes = itemsize[t];
+// Bytes and contiguity of one tensor row (torch _collective_utils.py:230-232,
+// _prims_common/__init__.py:252-292).
+__device__ __forceinline__ void tensor_bytes_and_contiguity(int r, int64_t itemsize, const int64_t *sh, const int64_t *st,
+                                                            int64_t &nbytes, bool &contiguous) {
+  // the whole (zero-padded) rows are read at once, before the scan: one round of loads
+  // instead of one per dim
+  int64_t x[APC_MAX_RANK], y[APC_MAX_RANK];
+#pragma unroll
+  for (int i = 0; i < APC_MAX_RANK; ++i) {
+    x[i] = sh[i];
+    y[i] = st[i];
+  }
+  nbytes = itemsize;
   int64_t expected = 1, expected_max = 1;
   bool ok = true;
-  for (int i = r - 1; i >= 0; --i) {
-    const int64_t x = sh[i], y = st[i];
-    nbytes *= x;
-    if (x == 1) continue;
-    if (y != expected && y != expected_max) ok = false;
-    expected_max *= (x > 1 ? x : 1);
-    expected *= x;
+#pragma unroll
+  for (int i = APC_MAX_RANK - 1; i >= 0; --i) {
+    if (i >= r) continue;
+    nbytes *= x[i];
+    if (x[i] == 1) continue;
+    if (y[i] != expected && y[i] != expected_max) ok = false;
+    expected_max *= (x[i] > 1 ? x[i] : 1);
+    expected *= x[i];
   }
-  bytes[t] = nbytes;
-  cont[t] = ok ? 1 : 0;
+  contiguous = ok;
+}
+
+template <int BS>
+__device__ __forceinline__ void tensor_tables_block(int64_t block, const TensorTableArgs &a) {
+  const int64_t t = block * BS + threadIdx.x;
+  if (t >= a.n) return;
+  int64_t nbytes;
+  bool ok;
+  tensor_bytes_and_contiguity(a.rank[t], a.itemsize[t], a.shape + t * APC_MAX_RANK, a.stride + t * APC_MAX_RANK, nbytes, ok);
+  a.bytes[t] = nbytes;
+  a.cont[t] = ok ? 1 : 0;
 }
 
 __global__ __launch_bounds__(kBlock) void tensor_tables_kernel(TensorTableArgs a) {
-  tensor_tables_block(blockIdx.x, a);
+  tensor_tables_block<kBlock>(blockIdx.x, a);
 }
 
 // ceil(x / m) for x >= 0 and a mesh size m whose correctly rounded reciprocal y is known.
@@ -240,15 +267,17 @@ struct SpecTableArgs {
 // Writes the first `live` values (a multiple of APC_MAX_RANK) of the workgroup's staged rows
 // (APC_MAX_RANK + 1 slots per row in LDS) to `out` as one contiguous run, two values (one
 // 16-byte store) per lane: rows hold an even number of values, so a pair never straddles rows.
+template <int BS>
 __device__ __forceinline__ void write_rows(int64_t *__restrict__ out, const int64_t *s_rows, int64_t live) {
   typedef int64_t pair_t __attribute__((ext_vector_type(2)));
-  for (int k = 2 * threadIdx.x; k < live; k += 2 * kBlock) {
+  for (int k = 2 * threadIdx.x; k < live; k += 2 * BS) {
     const int64_t *src = s_rows + (k / APC_MAX_RANK) * (APC_MAX_RANK + 1) + k % APC_MAX_RANK;
     pair_t v = {src[0], src[1]};
     *reinterpret_cast<pair_t *>(out + k) = v;
   }
 }
 
+template <int BS>
 __device__ __forceinline__ void spec_tables_block(int64_t block, const apc_params &p, const SpecTableArgs &a,
                                                   int64_t *s_rows) {
   const int64_t n = a.n;
@@ -259,12 +288,12 @@ __device__ __forceinline__ void spec_tables_block(int64_t block, const apc_param
   int64_t *__restrict__ lnumel = a.lnumel, *__restrict__ lbytes = a.lbytes;
   // Each thread derives one spec in its own row of an LDS buffer (the Shard dim indexes the
   // row, so no register array is indexed by a lane value), first the shape and then, in the
-  // same buffer, the stride; the workgroup writes each [kBlock][8] result block out as one
-  // contiguous 16 KB run.
-  const int64_t base = block * kBlock;
+  // same buffer, the stride; the workgroup (BS threads) writes each [BS][8] result block out
+  // as one contiguous run.
+  const int64_t base = block * BS;
   const int64_t s = base + threadIdx.x;
   int64_t *row = s_rows + threadIdx.x * (APC_MAX_RANK + 1);
-  const int64_t live = (n - base < kBlock ? n - base : kBlock) * APC_MAX_RANK;
+  const int64_t live = (n - base < BS ? n - base : BS) * APC_MAX_RANK;
   int t = -1, r = 0;
   uint32_t pc = 0;
   if (s < n) {
@@ -305,7 +334,7 @@ __device__ __forceinline__ void spec_tables_block(int64_t block, const apc_param
     lbytes[s] = nb;
   }
   __syncthreads();
-  write_rows(lshape + base * APC_MAX_RANK, s_rows, live);
+  write_rows<BS>(lshape + base * APC_MAX_RANK, s_rows, live);
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < APC_MAX_RANK; ++i) row[i] = st[i];
@@ -318,12 +347,12 @@ __device__ __forceinline__ void spec_tables_block(int64_t block, const apc_param
     }
   }
   __syncthreads();
-  write_rows(lstride + base * APC_MAX_RANK, s_rows, live);
+  write_rows<BS>(lstride + base * APC_MAX_RANK, s_rows, live);
 }
 
 __global__ __launch_bounds__(kBlock) void spec_tables_kernel(apc_params p, SpecTableArgs a) {
   __shared__ int64_t s_rows[kBlock * (APC_MAX_RANK + 1)];
-  spec_tables_block(blockIdx.x, p, a, s_rows);
+  spec_tables_block<kBlock>(blockIdx.x, p, a, s_rows);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -339,41 +368,37 @@ struct ComputeCostArgs {
   int32_t *error_flag;
 };
 
-__device__ __forceinline__ void compute_costs_block(int64_t block, const apc_params &p, const ComputeCostArgs &a) {
-  const int64_t n = a.n;
-  const int64_t *__restrict__ flops = a.flops, *__restrict__ rw_bytes = a.rw_bytes;
-  const int8_t *__restrict__ dtype = a.dtype;
-  const uint8_t *__restrict__ zero_cost = a.zero_cost;
-  const int32_t *__restrict__ num_args = a.num_args;
-  double *__restrict__ compute = a.compute, *__restrict__ per_arg = a.per_arg;
-  int32_t *__restrict__ error_flag = a.error_flag;
-  const int64_t s = block * kBlock + threadIdx.x;
-  if (s >= n) return;
-  double c = 0.0;
-  if (!zero_cost[s]) {
-    const double rw = rw_time((double)rw_bytes[s], p);
-    const int64_t f = flops[s];
-    if (f == 0) {
-      c = rw;
-    } else {
-      const int dt = dtype[s];
-      const double gf = (dt >= 0 && dt < APC_MAX_DTYPES) ? p.gpu_flops[dt] : 0.0;
-      if (gf == 0.0) {
-        if (error_flag) *error_flag = 1;  // compute_estimation.py:198-201 raises ValueError
-        c = NAN;
-      } else {
-        double t = (double)f / gf * 1e6;
-        t = t / p.compute_eff;
-        c = t > rw ? t : rw;
-      }
-    }
+// Compute cost of one strategy (compute_estimation.py:334-365); `unsupported` is set when the
+// strategy has flops and its dtype has no throughput on the device row (the result is NaN).
+__device__ __forceinline__ double compute_cost_of(const apc_params &p, bool zero_cost, int64_t rw_bytes, int64_t flops,
+                                                  int dt, bool &unsupported) {
+  unsupported = false;
+  if (zero_cost) return 0.0;
+  const double rw = rw_time((double)rw_bytes, p);
+  if (flops == 0) return rw;
+  const double gf = (dt >= 0 && dt < APC_MAX_DTYPES) ? pick<APC_MAX_DTYPES>(p.gpu_flops, dt) : 0.0;
+  if (gf == 0.0) {
+    unsupported = true;  // compute_estimation.py:198-201 raises ValueError
+    return NAN;
   }
-  if (compute) compute[s] = c;
-  if (per_arg) per_arg[s] = c / (double)num_args[s];
+  double t = (double)flops / gf * 1e6;
+  t = t / p.compute_eff;
+  return t > rw ? t : rw;
+}
+
+template <int BS>
+__device__ __forceinline__ void compute_costs_block(int64_t block, const apc_params &p, const ComputeCostArgs &a) {
+  const int64_t s = block * BS + threadIdx.x;
+  if (s >= a.n) return;
+  bool unsupported;
+  const double c = compute_cost_of(p, a.zero_cost[s] != 0, a.rw_bytes[s], a.flops[s], a.dtype[s], unsupported);
+  if (unsupported && a.error_flag) *a.error_flag = 1;
+  if (a.compute) a.compute[s] = c;
+  if (a.per_arg) a.per_arg[s] = c / (double)a.num_args[s];
 }
 
 __global__ __launch_bounds__(kBlock) void compute_costs_kernel(apc_params p, ComputeCostArgs a) {
-  compute_costs_block(blockIdx.x, p, a);
+  compute_costs_block<kBlock>(blockIdx.x, p, a);
 }
 
 // The three tables above in one launch: workgroups [0, spec_blocks) take the spec table (the
@@ -384,9 +409,9 @@ __global__ __launch_bounds__(kBlock) void input_tables_kernel(apc_params p, Tens
                                                               int64_t tensor_blocks) {
   __shared__ int64_t s_rows[kBlock * (APC_MAX_RANK + 1)];
   const int64_t b = blockIdx.x;
-  if (b < spec_blocks) spec_tables_block(b, p, sp, s_rows);
-  else if (b < spec_blocks + tensor_blocks) tensor_tables_block(b - spec_blocks, t);
-  else compute_costs_block(b - spec_blocks - tensor_blocks, p, c);
+  if (b < spec_blocks) spec_tables_block<kBlock>(b, p, sp, s_rows);
+  else if (b < spec_blocks + tensor_blocks) tensor_tables_block<kBlock>(b - spec_blocks, t);
+  else compute_costs_block<kBlock>(b - spec_blocks - tensor_blocks, p, c);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -416,7 +441,30 @@ struct TableArgs {
   double *comm_out;
   uint8_t *trans_out;
   double *cost_out;
+  // When the tensor and compute-cost tables are produced by the same launch (build_tables_kernel)
+  // a tile cannot read them: tensor_bytes / tensor_contiguous / per_arg are NULL and the tile
+  // derives the few values it needs from the tables those are computed from.
+  const int32_t *rank, *itemsize;
+  const int64_t *shape, *stride;
+  const int64_t *flops, *rw_bytes;
+  const int8_t *dtype;
+  const uint8_t *zero_cost;
+  const int32_t *num_args;
 };
+
+// Bytes and contiguity of tensor t: read from the tensor table, or (DERIVE) derived from its
+// shape row.  A compile-time choice: as a run-time one it cost the tile kernel a third of
+// its registers.
+template <bool DERIVE>
+__device__ __forceinline__ void tensor_info(const TableArgs &a, int t, int64_t &nbytes, bool &contiguous) {
+  if (!DERIVE) {
+    nbytes = a.tensor_bytes[t];
+    contiguous = a.tensor_contiguous[t] != 0;
+  } else {
+    tensor_bytes_and_contiguity(a.rank[t], a.itemsize[t], a.shape + (int64_t)t * APC_MAX_RANK,
+                                a.stride + (int64_t)t * APC_MAX_RANK, nbytes, contiguous);
+  }
+}
 
 // What one mesh dim contributes, by (producer class, consumer class) with classes
 // 0 Replicate, 1 Partial, 2 Shard(0), 3 Shard(d != 0); only consulted when the two placement
@@ -501,22 +549,6 @@ __device__ __forceinline__ TileView view_of(const apc_tile &tile) {
                   tile.flags,           tile.dup_count,    tile.src_begin, tile.entry_begin, tile.pt_begin};
 }
 
-// Element `i` (a per-lane index below M) of one of the per-mesh-dim arrays of the kernel
-// parameters, as a select chain over scalar registers.  (Indexing the array by a lane value
-// makes the compiler read the kernel arguments through vector memory, and a vector load
-// waits behind every store the compute unit has in flight.)
-template <int M, typename T, int N>
-__device__ __forceinline__ T pick(const T (&v)[N], int i) {
-  static_assert(M <= N, "array shorter than the mesh");
-  T e[M];  // every element is read (scalar loads) before the selects, so they stay selects
-#pragma unroll
-  for (int k = 0; k < M; ++k) e[k] = v[k];
-  T r = e[0];
-#pragma unroll
-  for (int k = 1; k < M; ++k) r = i == k ? e[k] : r;
-  return r;
-}
-
 // ring_r on a per-lane mesh dim d, with hops = hop_scale * (mesh_size[d] - 1).
 template <int M>
 __device__ __forceinline__ double ring_at(double gb, const apc_params &p, int d, int hop_scale) {
@@ -533,7 +565,7 @@ __device__ __forceinline__ double ring_at(double gb, const apc_params &p, int d,
 // computed from scalar operands while the loads are in flight: under a store-bound kernel
 // each dependent round of vector loads queues behind the stores of the other workgroups of
 // the compute unit, so the number of rounds, not of loads, is what staging costs.
-template <int M>
+template <int M, bool DERIVE>
 __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs &a, const apc_tile &tile,
                                            TileStage<M> &st, int tid, int nthreads) {
   constexpr int NS = States<M>::kCount;
@@ -556,8 +588,19 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   const uint32_t col_codes = a.spec_codes[sp];
   const uint32_t row_codes = a.spec_codes[ts];
   const int row_tensor = a.spec_tensor[ts];
+  const int sr = tile.strat_begin + tile.row_begin + (has_row ? jr : 0);
   double row_cpa = 0.0;
-  if (a.per_arg) row_cpa = a.per_arg[tile.strat_begin + tile.row_begin + (has_row ? jr : 0)];
+  int64_t row_flops = 0, row_rw = 0;
+  int row_dtype = 0, row_zero = 1, row_args = 1;
+  if (!DERIVE) {
+    if (a.per_arg) row_cpa = a.per_arg[sr];
+  } else {
+    row_flops = a.flops[sr];
+    row_rw = a.rw_bytes[sr];
+    row_dtype = a.dtype[sr];
+    row_zero = a.zero_cost[sr];
+    row_args = a.num_args[sr];
+  }
   // (dup_count <= APC_TILE_MAX_DUPS < 2 * nthreads)
   const bool has_dup0 = tid < tile.dup_count, has_dup1 = tid + nthreads < tile.dup_count;
   int64_t dup0 = 0, dup1 = 0;
@@ -566,18 +609,26 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   // the contiguity byte of the tile's tensor, read as the aligned word around it (which lies
   // in the byte's own page): a wave-uniform word goes through the scalar cache
   uint32_t contiguous = 1;
+  int64_t tensor_nbytes = 0;
   if (terms_wanted) {
-    const uint8_t *flag = a.tensor_contiguous + t0;
-    const uint32_t lane = (uint32_t)(reinterpret_cast<uintptr_t>(flag) & 3);
-    const uint32_t word = *reinterpret_cast<const uint32_t *>(flag - lane);
-    contiguous = (word >> (8 * lane)) & 0xFFu;
+    if (!DERIVE) {
+      const uint8_t *flag = a.tensor_contiguous + t0;
+      const uint32_t lane = (uint32_t)(reinterpret_cast<uintptr_t>(flag) & 3);
+      const uint32_t word = *reinterpret_cast<const uint32_t *>(flag - lane);
+      contiguous = (word >> (8 * lane)) & 0xFFu;
+      tensor_nbytes = a.tensor_bytes[t0];
+    } else {  // (t0 is wave-uniform: scalar loads and scalar arithmetic)
+      bool ok;
+      tensor_info<true>(a, t0, tensor_nbytes, ok);
+      contiguous = ok ? 1u : 0u;
+    }
   }
   // ---- state terms (scalar operands only) ---------------------------------------------------
   if (terms_wanted) {
     // every collective / read-write term the tile can need, once per running-bytes state, in
     // the reference's operation order (collective_runtime_estimation.py:66-68, :86, :128;
     // torch _collective_utils.py:281-313; compute_estimation.py:302-314)
-    const double fbytes = (double)a.tensor_bytes[t0];
+    const double fbytes = (double)tensor_nbytes;
     for (int k = tid; k < NS; k += nthreads) {
       const int level = 31 - __clz((k >> M) + 1);
       const int rem = k - (((1 << level) - 1) << M);
@@ -643,6 +694,10 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
     if (all_shard) info |= 1u << 30;
     if (!(info & 1u)) mixed = true;  // a consumer spec that is not a DTensorSpec
     st.row[jr] = make_uint2(row_codes, info);
+    if (DERIVE) {  // the value compute_costs_block writes for this strategy
+      bool unsupported;
+      row_cpa = compute_cost_of(p, row_zero != 0, row_rw, row_flops, row_dtype, unsupported) / (double)row_args;
+    }
     st.cpa[jr] = row_cpa;
   }
   // one flag per wavefront, written unconditionally: nothing to clear beforehand
@@ -778,7 +833,7 @@ __device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const 
 }
 
 // Generic loop: pass-through edges and edges whose producer specs name different tensors.
-template <int M>
+template <int M, bool DERIVE>
 __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M> &st,
                                                      const TileView &v, int tid, int nthreads) {
   const int n = v.rows * v.cols;
@@ -800,8 +855,11 @@ __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const 
 #pragma unroll
       for (int i = 0; i < M; ++i)
         if (kind_of((src >> (8 * i)) & 0xFF) == 2) shards *= p.mesh_size[i];
-      const double gb = (double)a.tensor_bytes[sten] / (double)shards / 1024 / 1024 / 1024;
-      comm = entry_cost<M>(src, tgt, gb, a.tensor_contiguous[sten] != 0, p);
+      int64_t sten_bytes;
+      bool sten_contiguous;
+      tensor_info<DERIVE>(a, sten, sten_bytes, sten_contiguous);
+      const double gb = (double)sten_bytes / (double)shards / 1024 / 1024 / 1024;
+      comm = entry_cost<M>(src, tgt, gb, sten_contiguous, p);
     }
     if (v.flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;
     const int64_t o = v.entry_begin + local;
@@ -825,13 +883,13 @@ __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const 
 }
 
 // All entries of a staged tile.
-template <int M>
+template <int M, bool DERIVE>
 __device__ __forceinline__ void tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M> &st,
                                              const TileView &v, int tid, int nthreads) {
   int mixed = st.mixed[0];
   for (int w = 1; w < nthreads / 64; ++w) mixed |= st.mixed[w];
   if (uniform_i32(mixed)) {
-    generic_tile_entries<M>(p, a, st, v, tid, nthreads);
+    generic_tile_entries<M, DERIVE>(p, a, st, v, tid, nthreads);
     return;
   }
   const bool rescale = (v.flags & APC_EDGE_GRAD_RESCALE) != 0;
@@ -857,9 +915,44 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
   static_assert(kTileThreads >= APC_TILE_MAX_COLS && kTileThreads >= APC_TILE_MAX_ROWS &&
                 2 * kTileThreads > APC_TILE_MAX_DUPS, "one staging round covers a tile");
   const apc_tile tile = a.tiles[tile_id];
-  stage_tile<M>(p, a, tile, s_stage, threadIdx.x, kTileThreads);
+  stage_tile<M, false>(p, a, tile, s_stage, threadIdx.x, kTileThreads);
   __syncthreads();
-  tile_entries<M>(p, a, s_stage, view_of(tile), threadIdx.x, kTileThreads);
+  tile_entries<M, false>(p, a, s_stage, view_of(tile), threadIdx.x, kTileThreads);
+}
+
+// Every table of a pass in one launch: workgroups [0, tile_blocks) take the tiles of the
+// redistribution-cost matrices (tile_blocks = n_tiles rounded up to the XCD chunking), the
+// next spec_blocks the spec table, then the tensor table, then the compute costs, kThreads rows
+// per workgroup.  No workgroup reads what another writes: a tile derives its tensor's byte
+// count and contiguity and its consumer strategies' compute costs with the functions the
+// table workgroups use (TableArgs), so the values are the same bits.  One launch instead of
+// two spares a table of a few tens of MB one ramp-up and one drain of the chip, which at that
+// size are a third of each kernel.
+template <int M, int kThreads>
+__global__ __launch_bounds__(kThreads) void build_tables_kernel(apc_params p, TableArgs a, TensorTableArgs t,
+                                                                SpecTableArgs sp, ComputeCostArgs c, int n_tiles,
+                                                                int64_t tile_blocks, int64_t spec_blocks,
+                                                                int64_t tensor_blocks, int xcd_shift) {
+  constexpr size_t kRowBytes = (size_t)kThreads * (APC_MAX_RANK + 1) * sizeof(int64_t);
+  constexpr size_t kLds = sizeof(TileStage<M>) > kRowBytes ? sizeof(TileStage<M>) : kRowBytes;
+  __shared__ __align__(16) unsigned char s_raw[kLds];
+  static_assert(kThreads == 64 || kThreads == 128 || kThreads == 256, "wavefronts per workgroup: 1, 2 or 4");
+  const int64_t b = blockIdx.x;
+  if (b < tile_blocks) {
+    const int64_t per = tile_blocks >> xcd_shift;
+    const int64_t tile_id = (b & ((1 << xcd_shift) - 1)) * per + (b >> xcd_shift);
+    if (tile_id >= n_tiles) return;
+    TileStage<M> &stage = *reinterpret_cast<TileStage<M> *>(s_raw);
+    const apc_tile tile = a.tiles[tile_id];
+    stage_tile<M, true>(p, a, tile, stage, threadIdx.x, kThreads);
+    __syncthreads();
+    tile_entries<M, true>(p, a, stage, view_of(tile), threadIdx.x, kThreads);
+    return;
+  }
+  const int64_t tb = b - tile_blocks;
+  if (tb < spec_blocks) spec_tables_block<kThreads>(tb, p, sp, reinterpret_cast<int64_t *>(s_raw));
+  else if (tb < spec_blocks + tensor_blocks) tensor_tables_block<kThreads>(tb - spec_blocks, t);
+  else compute_costs_block<kThreads>(tb - spec_blocks - tensor_blocks, p, c);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1185,7 +1278,8 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
     return fail(-1, "apc_redistribute_tables: NULL table");
   if (cost_out && !per_arg) return fail(-1, "cost_out needs compute_cost_per_arg");
   TableArgs a{tensor_bytes, tensor_contiguous, spec_codes, spec_tensor, pt_values, per_arg,
-              tiles,        dup_entry_begin,   comm_out,   trans_out,   cost_out};
+              tiles,        dup_entry_begin,   comm_out,   trans_out,   cost_out,
+              nullptr,      nullptr,           nullptr,    nullptr,     nullptr, nullptr, nullptr, nullptr, nullptr};
   const int nt = (int)n_tiles, xs = xcd_shift();
   hipStream_t s = (hipStream_t)stream;
   // Wavefronts per tile by the mean number of values a tile stores (n_entries counts the
@@ -1208,6 +1302,66 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
   }
 #undef APC_LAUNCH
   return check_launch("apc_redistribute_tables");
+}
+
+int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t *rank, const int32_t *itemsize,
+                     const int64_t *shape, const int64_t *stride, int64_t *tensor_bytes, uint8_t *tensor_contiguous,
+                     int64_t n_specs, const uint32_t *spec_codes, const int32_t *spec_tensor, int64_t *num_shards,
+                     int64_t *local_shape, int64_t *local_stride, int64_t *local_numel, int64_t *local_bytes,
+                     int64_t n_strategies, const int64_t *flops, const int64_t *rw_bytes, const int8_t *dtype,
+                     const uint8_t *zero_cost, const int32_t *num_args, double *compute, double *per_arg,
+                     int32_t *error_flag, const double *pt_values, int64_t n_tiles, const apc_tile *tiles,
+                     const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *trans_out,
+                     double *cost_out, void *stream) {
+  if (int rc = check_params(params)) return rc;
+  if (n_tensors < 0 || n_specs < 0 || n_strategies < 0 || n_entries < 0) return fail(-1, "apc_build_tables: negative count");
+  if (n_tiles < 0 || n_tiles > (1 << 30)) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
+  if (n_tensors > 0 && (!rank || !itemsize || !shape || !stride || !tensor_bytes || !tensor_contiguous))
+    return fail(-1, "apc_build_tables: NULL tensor array");
+  const bool spec_table = num_shards || local_shape || local_stride || local_numel || local_bytes;
+  if (spec_table && n_specs > 0 && (!spec_codes || !spec_tensor || !num_shards || !local_shape || !local_stride ||
+                                    !local_numel || !local_bytes))
+    return fail(-1, "apc_build_tables: the spec table needs all five of its outputs");
+  if (n_strategies > 0 && (!flops || !rw_bytes || !dtype || !zero_cost || !num_args))
+    return fail(-1, "apc_build_tables: NULL strategy array");
+  if (n_tiles > 0 && (!spec_codes || !spec_tensor || !tiles || !rank || !itemsize || !shape || !stride))
+    return fail(-1, "apc_build_tables: NULL table");
+  const int xs = xcd_shift();
+  int threads = 256;
+  if (n_tiles > 0) {
+    const int64_t per_tile = n_entries / n_tiles;
+    threads = per_tile >= 1536 ? 256 : per_tile >= 512 ? 128 : 64;
+  }
+  if (const char *env = getenv("APC_TILE_THREADS")) threads = atoi(env);  // tuning override
+  threads = threads >= 256 ? 256 : threads >= 128 ? 128 : 64;
+  const int64_t tile_blocks = ((n_tiles + (1 << xs) - 1) >> xs) << xs;
+  const int64_t sb = spec_table ? blocks_for(n_specs, threads) : 0, tb = blocks_for(n_tensors, threads),
+                cb = blocks_for(n_strategies, threads);
+  const int64_t blocks = tile_blocks + sb + tb + cb;
+  if (blocks == 0) return 0;
+  if (blocks > INT32_MAX) return fail(-1, "apc_build_tables: too many rows for one launch");
+  // the tiles read neither the tensor table nor the compute costs (written by this launch)
+  TableArgs a{nullptr, nullptr, spec_codes, spec_tensor, pt_values, nullptr, tiles, dup_entry_begin,
+              comm_out, trans_out, cost_out, rank, itemsize, shape, stride, flops, rw_bytes, dtype, zero_cost, num_args};
+  const TensorTableArgs ta{n_tensors, rank, itemsize, shape, stride, tensor_bytes, tensor_contiguous};
+  const SpecTableArgs sa{n_specs, spec_codes, spec_tensor, rank, itemsize, shape, stride, num_shards,
+                         local_shape, local_stride, local_numel, local_bytes};
+  const ComputeCostArgs ca{n_strategies, flops, rw_bytes, dtype, zero_cost, num_args, compute, per_arg, error_flag};
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)blocks);
+  const int nt = (int)n_tiles;
+#define APC_LAUNCH_ALL(M_)                                                                                              \
+  if (threads == 256) hipLaunchKernelGGL((build_tables_kernel<M_, 256>), grid, dim3(256), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
+  else if (threads == 128) hipLaunchKernelGGL((build_tables_kernel<M_, 128>), grid, dim3(128), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
+  else hipLaunchKernelGGL((build_tables_kernel<M_, 64>), grid, dim3(64), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs)
+  switch (params->mesh_ndim) {
+    case 1: APC_LAUNCH_ALL(1); break;
+    case 2: APC_LAUNCH_ALL(2); break;
+    case 3: APC_LAUNCH_ALL(3); break;
+    default: APC_LAUNCH_ALL(4); break;
+  }
+#undef APC_LAUNCH_ALL
+  return check_launch("apc_build_tables");
 }
 
 int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_seg, int64_t n_values, double *mins,

@@ -188,13 +188,24 @@ class DeviceCostTables:
         return self.run_redistribute_tables()
 
     # ---- one full device-side pass with pre-bound arguments -------------------------------------
+    # A pass over a table this small is bound by the ramp-up and drain of every launch, and
+    # one launch for all tables wins (Llama-3-8B on a (32, 8) mesh, 78 MB: 25 us against 30 us
+    # per pass); above it the tiles' own derivation of what they would otherwise read costs
+    # more than a launch (measured crossover between 90 MB and 170 MB of tables).
+    ONE_LAUNCH_MAX_BYTES = 128 << 20
+
     @_guarded
-    def prepare_step(self, row_min=True, fused_inputs=False):
+    def prepare_step(self, row_min=True, fused_inputs=False, one_launch=None):
         """Allocates every output once and returns ``{kernel name: zero-argument launcher}``
         in launch order.  A launcher only enqueues (no allocation, no synchronisation), so a
         timed loop measures the kernels and not Python argument marshalling.  With
         ``fused_inputs`` the tensor, spec and compute-cost tables are one launch
-        (``input_tables``) instead of three."""
+        (``input_tables``) instead of three; with ``one_launch`` they and the cost matrices
+        are one (``build_tables``); ``one_launch=None`` takes one launch for tables up to
+        ``ONE_LAUNCH_MAX_BYTES`` when ``fused_inputs`` is set."""
+        if one_launch is None:
+            total = self.tables.algorithmic_bytes() + self.tables.algorithmic_bytes_input_tables()
+            one_launch = bool(fused_inputs) and total <= self.ONE_LAUNCH_MAX_BYTES
         self.run_tensor_tables()
         spec = self.run_spec_tables()
         self.run_compute_costs()
@@ -226,7 +237,11 @@ class DeviceCostTables:
                     _native.check(rc, what)
             return launch
 
-        if fused_inputs:
+        if one_launch:
+            a_all = (cp,) + a_tensor[:-1] + (a_spec[1], a_spec[2], a_spec[3]) + a_spec[8:-1] + a_compute[1:-1] + \
+                (a_tables[5],) + a_tables[7:]
+            step = {"build_tables": bind(lib.apc_build_tables, a_all, "apc_build_tables")}
+        elif fused_inputs:
             a_inputs = (cp,) + a_tensor[:-1] + (a_spec[1], a_spec[2], a_spec[3]) + a_spec[8:-1] + a_compute[1:]
             step = {"input_tables": bind(lib.apc_input_tables, a_inputs, "apc_input_tables")}
         else:
@@ -235,7 +250,8 @@ class DeviceCostTables:
                 "spec_tables": bind(lib.apc_spec_tables, a_spec, "apc_spec_tables"),
                 "compute_costs": bind(lib.apc_compute_costs, a_compute, "apc_compute_costs"),
             }
-        step["redistribute_tables"] = bind(lib.apc_redistribute_tables, a_tables, "apc_redistribute_tables")
+        if not one_launch:
+            step["redistribute_tables"] = bind(lib.apc_redistribute_tables, a_tables, "apc_redistribute_tables")
         if row_min:
             row_ptr = torch.from_numpy(tb.row_ptr()).to(self.device)
             n_seg = row_ptr.numel() - 1

@@ -212,6 +212,13 @@ class CostTables:
         per_edge = (self.edge_n_src.astype(np.int64) + self.edge_n_tgt.astype(np.int64)) * m + 64
         return per_entry * self.n_entries + int(per_edge.sum())
 
+    def algorithmic_bytes_input_tables(self) -> int:
+        """Bytes the tensor, spec and compute-cost tables must move at minimum: per tensor 136 B
+        read (rank, itemsize, shape, stride) and 9 B written; per spec 8 B read and 152 B
+        written (shard count, local shape and stride, local element and byte counts); per
+        strategy 22 B read and 16 B written."""
+        return 145 * self.n_tensors + 160 * self.n_specs + 38 * self.n_strategies
+
     # ---- tiles -------------------------------------------------------------------------
     def edge_signatures(self) -> list:
         """One digest per edge over everything its matrix depends on: both spec lists

@@ -55,8 +55,10 @@ def parse_args():
     ap.add_argument("--no-clustering", action="store_true", help="one ILP variable per entry (no variable sharing)")
     ap.add_argument("--no-dedupe", action="store_true", help="tile every edge even if an identical one exists")
     ap.add_argument("--max-copies", type=int, default=8, help="identical edges served by one tiled edge")
-    ap.add_argument("--separate-input-kernels", action="store_true",
-                    help="launch the tensor, spec and compute-cost tables as three kernels instead of one")
+    ap.add_argument("--table-launches", type=int, default=None, choices=[1, 2, 4],
+                    help="launches that build the tables of a pass: 1 = everything in one (apc_build_tables), "
+                         "2 = input tables, then cost matrices, 4 = tensor, spec and compute-cost tables on their own "
+                         "(default: 1 for tables up to 128 MiB, else 2)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy three times (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -214,7 +216,9 @@ def main():
             tables.build_tiles(args.tile_entries)
         dev = DeviceCostTables(tables, params, device="cuda:0")
     log.info("tables resident: %d entries, %d tiles", tables.n_entries, tables.n_tiles)
-    step = dev.prepare_step(row_min=True, fused_inputs=not args.separate_input_kernels)
+    step = dev.prepare_step(row_min=True, fused_inputs=args.table_launches != 4,
+                            one_launch=None if args.table_launches is None else args.table_launches == 1)
+    args.table_launches = 1 if "build_tables" in step else 2 if "input_tables" in step else 4
     torch.cuda.synchronize()
     host_timings["upload_and_prepare_s"] = time.perf_counter() - t0
     host_timings["setup_total_s"] = time.perf_counter() - t_setup
@@ -260,8 +264,12 @@ def main():
 
     log.info("timed region done: %.3f ms/step", wall_plain / K * 1e3)
     E = tables.n_entries
+    # the launch that writes the cost matrices; in one-launch mode it also writes the input tables
+    main = "build_tables" if args.table_launches == 1 else "redistribute_tables"
     alg_bytes = tables.algorithmic_bytes(comm=True, transition=True, cost=True)
-    t_kernel = kernel_ms["redistribute_tables"] * 1e-3
+    if args.table_launches == 1:
+        alg_bytes += tables.algorithmic_bytes_input_tables()
+    t_kernel = kernel_ms[main] * 1e-3
     achieved = alg_bytes / t_kernel / 1e9
     ms_per_step = wall_plain / K * 1e3
     result = {
@@ -281,15 +289,19 @@ def main():
                    "entries": E, "tiles": tables.n_tiles, "tiling": tables.tiling,
                    "edges_deduplicated": int((tables.edge_canonical != np.arange(tables.n_edges)).sum()), "device_row": params.device_name,
                    "devices_per_host": 8,
-                   "step": ("tensor_tables + spec_tables + compute_costs" if args.separate_input_kernels else
-                            "input_tables(tensor + spec + compute-cost tables, one launch)") +
-                           " + redistribute_tables(comm, transition, cost) + segmented_min(rows)"},
-        "roofline": {"bound": "hbm", "kernel": "redistribute_tiles_kernel", "achieved": achieved,
+                   "step": {1: "build_tables(tensor, spec and compute-cost tables + comm, transition, cost: one launch)",
+                            2: "input_tables(tensor + spec + compute-cost tables, one launch) + "
+                               "redistribute_tables(comm, transition, cost)",
+                            4: "tensor_tables + spec_tables + compute_costs + redistribute_tables(comm, transition, cost)"
+                            }[args.table_launches] + " + segmented_min(rows)"},
+        "roofline": {"bound": "hbm", "kernel": "build_tables_kernel" if args.table_launches == 1 else "redistribute_tiles_kernel",
+                     "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get((E, tables.n_tiles, alg_bytes)),
+                     "algorithmic_bytes_input_tables": tables.algorithmic_bytes_input_tables() if args.table_launches == 1 else 0,
                      "algorithmic_bytes_per_launch": alg_bytes,
                      "bytes_written_per_entry": {"comm_f64": 8, "transition_u8": 1, "cost_f64": 8},
-                     "avg_launch_us": t_kernel * 1e6, "min_launch_us": kernel_ms_min["redistribute_tables"] * 1e3,
+                     "avg_launch_us": t_kernel * 1e6, "min_launch_us": kernel_ms_min[main] * 1e3,
                      "timing": "HIP events around every launch of the kernel inside the timed region"},
         "kernel_us": {k: v * 1e3 for k, v in kernel_ms.items()},
         "ms_per_step_with_events": wall / K * 1e3,

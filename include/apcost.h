@@ -181,6 +181,26 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
                             const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out,
                             uint8_t *transition_out, double *cost_out, void *stream);
 
+/* Every table of a pass in ONE launch: apc_input_tables + apc_redistribute_tables (same
+ * arguments, same results: the union of the reference lines those replace).  The workgroups
+ * that tile the cost matrices do not read tensor_bytes / tensor_contiguous /
+ * compute_cost_per_arg, which other workgroups of the same launch are writing: they derive the
+ * values they need from the tensor and strategy tables with the same device functions.  A
+ * table of a few tens of MB (one transformer graph on a 2-D mesh) spends a third of each
+ * launch ramping the chip up and draining it; this saves one of each.  The five spec-table
+ * outputs may all be NULL (the spec table is then skipped: a planner computes it first and
+ * alone, because the flop / byte counts passed here depend on it). */
+int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
+                     const int32_t *tensor_itemsize, const int64_t *tensor_shape, const int64_t *tensor_stride,
+                     int64_t *tensor_bytes, uint8_t *tensor_contiguous, int64_t n_specs, const uint32_t *spec_codes,
+                     const int32_t *spec_tensor, int64_t *num_shards, int64_t *local_shape, int64_t *local_stride,
+                     int64_t *local_numel, int64_t *local_bytes, int64_t n_strategies, const int64_t *flops,
+                     const int64_t *rw_bytes, const int8_t *dtype_code, const uint8_t *zero_cost,
+                     const int32_t *num_args, double *compute_cost, double *compute_cost_per_arg,
+                     int32_t *error_flag, const double *pt_values, int64_t n_tiles, const apc_tile *tiles,
+                     const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *transition_out,
+                     double *cost_out, void *stream);
+
 /* Segmented minimum with first-argmin (relative to the segment start); empty
  * segments give (+inf, -1).  No counterpart in the reference (which hands the full
  * table to the ILP solver, optimize_sharding.py:648-659): used for pruning and

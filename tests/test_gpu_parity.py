@@ -439,3 +439,47 @@ def test_fused_input_tables_match_the_three_entry_points(gpu_device):
     assert np.array_equal(results[1]["tensor_bytes"], c_oracle.tensor_tables(enc)[0])
     assert np.array_equal(results[1]["spec_local_shape"], c_oracle.spec_tables(enc, mesh)[1])
     assert (results[1]["cost"] != 0).any()
+
+
+@pytest.mark.parametrize("mesh,threads", [((32, 8), None), ((16, 8, 4), None), ((16, 8, 4), 64), ((16, 8, 4), 256), ((2, 3, 2, 2), None)])
+def test_one_launch_build_matches_the_separate_entry_points(gpu_device, mesh, threads, monkeypatch):
+    """apc_build_tables (tiles that derive tensor bytes, contiguity and compute costs themselves,
+    beside the workgroups that write those tables) against the launch-by-launch pass and the
+    oracle: every output array, bit for bit; with identical edges stored to several copies,
+    non-contiguous tensors and specs that are not DTensorSpecs in the mix."""
+    from test_abi_and_encoding import twin_graph
+
+    if threads:
+        monkeypatch.setenv("APC_TILE_THREADS", str(threads))
+    tb = twin_graph(stress_dag(seed=17, n_nodes=900, mesh_sizes=mesh, frac_nonspec_nodes=0.03, frac_noncontiguous=0.2))
+    tb.build_tiles(1024, dedupe=True)
+    p = CostModelParams.from_mesh(mesh, rescale=2.2)
+    names = ("tensor_bytes", "tensor_contiguous", "compute_cost", "compute_cost_per_arg", "comm", "transition", "cost",
+             "row_min", "row_argmin")
+    results = []
+    for one_launch in (False, True):
+        d = DeviceCostTables(tb, p, device=gpu_device)
+        step = d.prepare_step(row_min=True, fused_inputs=True, one_launch=one_launch)
+        assert list(step) == (["build_tables", "segmented_min"] if one_launch else
+                              ["input_tables", "redistribute_tables", "segmented_min"])
+        for name in names:
+            getattr(d, name).zero_()
+        spec = d._step_keepalive[1]
+        for v in spec.values():
+            v.zero_()
+        for launch in step.values():
+            launch()
+        torch.cuda.synchronize()
+        out = {name: getattr(d, name).cpu().numpy() for name in names}
+        out.update({f"spec_{k}": v.cpu().numpy() for k, v in spec.items()})
+        results.append(out)
+    for key in results[0]:
+        assert np.array_equal(results[0][key], results[1][key]), key
+    enc = tb.as_dict()
+    op = po.make_params(mesh, rescale=2.2)
+    want_cc, want_pa = c_oracle.compute_costs(enc, op)
+    want = c_oracle.build_tables(enc, op, per_arg=want_pa)
+    _assert_costs(results[1]["cost"], want["cost"], "cost")
+    _assert_costs(results[1]["comm"], want["comm"], "comm")
+    assert np.array_equal(results[1]["transition"], want["transition"])
+    _assert_costs(results[1]["compute_cost"], want_cc, "compute_cost")
