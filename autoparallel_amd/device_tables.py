@@ -280,7 +280,9 @@ class DeviceCostTables:
             main = torch.cuda.current_stream()
             for b in branches:
                 b.wait_stream(main)
-            if "input_tables" in step:
+            if "build_tables" in step:
+                step["build_tables"](ctypes.c_void_p(main.cuda_stream))
+            elif "input_tables" in step:
                 step["input_tables"](ctypes.c_void_p(main.cuda_stream))
             else:
                 step["spec_tables"](ctypes.c_void_p(main.cuda_stream))
@@ -288,7 +290,8 @@ class DeviceCostTables:
                 step["compute_costs"](ctypes.c_void_p(branches[1].cuda_stream))
             for b in branches:
                 main.wait_stream(b)
-            step["redistribute_tables"](ctypes.c_void_p(main.cuda_stream))
+            if "redistribute_tables" in step:
+                step["redistribute_tables"](ctypes.c_void_p(main.cuda_stream))
             if "segmented_min" in step:
                 step["segmented_min"](ctypes.c_void_p(main.cuda_stream))
         self._step_keepalive.append(branches)

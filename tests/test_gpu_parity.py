@@ -350,13 +350,16 @@ def test_full_size_stress_properties(gpu_device):
     assert bool((cost[: seg_of_entry.numel()] >= mins[seg_of_entry]).all())
 
 
-def test_graph_replay_of_one_pass_matches_eager(gpu_device):
-    """One pass recorded as a HIP graph (independent kernels on parallel branches) gives the
-    eager results on every replay, with eager work and synchronisations between replays."""
+@pytest.mark.parametrize("launches", [5, 2])
+def test_graph_replay_of_one_pass_matches_eager(gpu_device, launches):
+    """One pass recorded as a HIP graph (five launches with the independent kernels on parallel
+    branches, or the one-launch build + row minima) gives the eager results on every replay,
+    with eager work and synchronisations between replays."""
     mesh = (8, 4, 2)
     tb = stress_dag(seed=5, n_nodes=3000, mesh_sizes=mesh, frac_nonspec_nodes=0.02, frac_noncontiguous=0.2)
     d = DeviceCostTables(tb, CostModelParams.from_mesh(mesh, rescale=2.2), device=gpu_device)
-    step = d.prepare_step(row_min=True)
+    step = d.prepare_step(row_min=True, fused_inputs=launches == 2, one_launch=launches == 2)
+    assert len(step) == launches
     for launch in step.values():
         launch()
     torch.cuda.synchronize()
@@ -420,7 +423,7 @@ def test_fused_input_tables_match_the_three_entry_points(gpu_device):
     results = []
     for fused in (False, True):
         d = DeviceCostTables(tb, p, device=gpu_device)
-        step = d.prepare_step(row_min=True, fused_inputs=fused)
+        step = d.prepare_step(row_min=True, fused_inputs=fused, one_launch=False)
         assert ("input_tables" in step) == fused and len(step) == (3 if fused else 5)
         for name in names:
             getattr(d, name).zero_()
