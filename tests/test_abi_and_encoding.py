@@ -178,6 +178,7 @@ def test_validator_accepts_generated_tables():
     (lambda t: t.edge_entry_begin.__setitem__(2, int(t.edge_entry_begin[2]) + 1), "entry_begin"),
     (lambda t: t.edge_src_begin.__setitem__(1, t.n_specs), "producer spec range"),
     (lambda t: t.edge_strat_begin.__setitem__(1, t.n_strategies), "strategy rows"),
+    (lambda t: t.edge_n_src.__setitem__(1, (1 << 22) + 1), "strategies"),
     (lambda t: t.tile_row_count.__setitem__(0, 10**4), "rows"),
     (lambda t: t.tile_col_begin.__setitem__(0, -1), "cols"),
 ])
