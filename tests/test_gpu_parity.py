@@ -486,3 +486,47 @@ def test_one_launch_build_matches_the_separate_entry_points(gpu_device, mesh, th
     _assert_costs(results[1]["comm"], want["comm"], "comm")
     assert np.array_equal(results[1]["transition"], want["transition"])
     _assert_costs(results[1]["compute_cost"], want_cc, "compute_cost")
+
+
+def test_randomized_configurations(gpu_device, monkeypatch):
+    """A seeded sweep over what the launchers choose between: mesh rank, strategy counts up to
+    130 (column-chunked tiles), tile size, identical-edge copies, wavefronts per tile, one or two
+    table launches, gradient rescale; every output against the C oracle, bit for bit."""
+    from test_abi_and_encoding import twin_graph
+
+    rng = np.random.default_rng(2024)
+    meshes = [(64,), (32, 8), (8, 8, 8), (5, 3, 2), (2, 3, 2, 2), (128, 2)]
+    for it in range(12):
+        mesh = meshes[it % len(meshes)]
+        maxs = int(rng.choice([8, 40, 64, 130]))
+        tb = stress_dag(seed=int(rng.integers(1, 10**6)), n_nodes=int(rng.integers(50, 600)), mesh_sizes=mesh,
+                        max_strategies=maxs, min_strategies=min(4, maxs),
+                        frac_nonspec_nodes=float(rng.choice([0.0, 0.02, 0.1])),
+                        frac_noncontiguous=float(rng.choice([0.0, 0.2, 0.6])),
+                        frac_grad_nodes=float(rng.choice([0.0, 0.05, 0.3])))
+        if rng.random() < 0.5:
+            tb = twin_graph(tb)
+        copies = int(rng.choice([1, 2, 8]))
+        tb.build_tiles(int(rng.choice([64, 300, 1024, 4096])), dedupe=copies > 1, max_copies=copies)
+        threads = str(rng.choice(["", "64", "128", "256"]))
+        if threads:
+            monkeypatch.setenv("APC_TILE_THREADS", threads)
+        else:
+            monkeypatch.delenv("APC_TILE_THREADS", raising=False)
+        one_launch = bool(rng.random() < 0.5)
+        rescale = float(rng.choice([1.0, 2.2]))
+        d = DeviceCostTables(tb, CostModelParams.from_mesh(mesh, rescale=rescale), device=gpu_device)
+        step = d.prepare_step(row_min=True, fused_inputs=True, one_launch=one_launch)
+        for launch in step.values():
+            launch()
+        torch.cuda.synchronize()
+        enc, op = tb.as_dict(), po.make_params(mesh, rescale=rescale)
+        want_cc, want_pa = c_oracle.compute_costs(enc, op)
+        want = c_oracle.build_tables(enc, op, per_arg=want_pa)
+        want_min, want_arg = c_oracle.segmented_min(want["cost"], tb.row_ptr())
+        what = f"case {it}: mesh {mesh}, {maxs} strategies, {copies} copies, threads {threads or 'auto'}, one launch {one_launch}"
+        _assert_costs(d.comm.cpu().numpy(), want["comm"], what + " comm")
+        _assert_costs(d.cost.cpu().numpy(), want["cost"], what + " cost")
+        assert np.array_equal(d.transition.cpu().numpy(), want["transition"]), what
+        _assert_costs(d.compute_cost.cpu().numpy(), want_cc, what + " compute_cost")
+        assert np.array_equal(d.row_min.cpu().numpy(), want_min) and np.array_equal(d.row_argmin.cpu().numpy(), want_arg), what
