@@ -318,3 +318,45 @@ def test_reference_entry_point_signature(meshes):
     with pytest.raises(ValueError, match="input_fn must return"):
         with OracleAutoParallel(model, input_fn, mesh, loss_fn=torch.nn.functional.mse_loss):
             pass
+
+
+class _PartlyFrozen(torch.nn.Module):
+    """Trainable weights, a frozen weight and a buffer (the planning half of the reference's
+    tests/test_ordered_sharding.py:90-188: parameters whose gradient node is None)."""
+
+    def __init__(self, dim, all_frozen=False):
+        super().__init__()
+        self.first = torch.nn.Linear(dim, dim, bias=False)
+        self.frozen = torch.nn.Parameter(torch.randn(dim, dim), requires_grad=False)
+        self.register_buffer("offset", torch.randn(dim))
+        self.last = torch.nn.Linear(dim, dim, bias=False)
+        if all_frozen:
+            for p in self.parameters():
+                p.requires_grad = False
+
+    def forward(self, x):
+        x = self.first(x)
+        x = x + torch.mm(x, self.frozen)
+        x = x + self.offset
+        return self.last(x)
+
+
+@pytest.mark.parametrize("all_frozen", [False, True])
+def test_plans_with_parameters_that_have_no_gradient(meshes, all_frozen):
+    from torch._functorch._aot_autograd.fx_utils import get_param_and_grad_nodes
+
+    mesh, dim = meshes["2d"], 128
+    with torch.device("meta"):
+        model = _PartlyFrozen(dim, all_frozen)
+    with OraclePlanner(model, lambda: torch.randn(512, dim, requires_grad=True), mesh) as autop:
+        autop.add_parameter_memory_constraint(low=0, high=None)
+        placement = autop.optimize_placement()
+        pairs = list(get_param_and_grad_nodes(autop.gm.graph).values())
+        assert len(pairs) == 3
+        assert any(grad is None for _, grad in pairs)
+        assert all(grad is None for _, grad in pairs) == all_frozen
+        for param, grad in pairs:  # a parameter and its gradient (where it has one) are placed alike
+            assert param in placement
+            if grad is not None:
+                assert placement[param].output_specs.placements == placement[grad].output_specs.placements
+        assert not autop.sharding_optimizer.prob.violated_constraints()
