@@ -753,14 +753,18 @@ class ShardingOptimizer:
         return code
 
     def print_costs_for_node(self, node, arg=0, **kwargs):
+        """Prints the redistribution-cost matrix of ``node``'s ``arg``-th input edge: a row per
+        strategy of ``node``, a column per strategy of the input (optimize_sharding.py:633-646),
+        taken from the flat array the kernels filled."""
         from tabulate import tabulate
         from torch.distributed.tensor._op_schema import _pretty_print_spec
 
-        tgt = self.strats[node]
-        src = self.strats[self._all_input_nodes(node)[arg]]
-        headers = [""] + [_pretty_print_spec(x.output_specs) for x in src.strategies]
-        costs = [[str(x)] + x.redistribute_cost[arg] for x in tgt.strategies]
-        print(tabulate(costs, headers=headers, **kwargs))
+        begin, n_rows, n_cols = self._edge(self.node_map[node], arg)
+        matrix = self.comm_cost[begin:begin + n_rows * n_cols].reshape(n_rows, n_cols)
+        producer = self._all_input_nodes(node)[arg]
+        header = [""] + [_pretty_print_spec(s.output_specs) for s in self.strats[producer].strategies]
+        body = [[str(s), *matrix[i].tolist()] for i, s in enumerate(self.strats[node].strategies)]
+        print(tabulate(body, headers=header, **kwargs))
 
     # ---- warm-start helpers built on the segmented min kernel -------------------------------------
     def row_minima(self):

@@ -360,3 +360,19 @@ def test_plans_with_parameters_that_have_no_gradient(meshes, all_frozen):
             if grad is not None:
                 assert placement[param].output_specs.placements == placement[grad].output_specs.placements
         assert not autop.sharding_optimizer.prob.violated_constraints()
+
+
+
+def test_print_costs_for_node(meshes, capsys):
+    autop, _ = _plan(OraclePlanner, meshes["2d"], "ffn", None)
+    opt = autop.sharding_optimizer
+    mm = autop.gm.graph.find_nodes(op="call_function", target=torch.ops.aten.mm.default)[0]
+    opt.print_costs_for_node(mm, arg=1, floatfmt=".3f")
+    out = capsys.readouterr().out.splitlines()
+    n_rows = len(opt.strats[mm].strategies)
+    n_cols = len(opt.strats[opt._all_input_nodes(mm)[1]].strategies)
+    assert len(out) == 2 + n_rows  # header, rule, one line per strategy of the node
+    s_i = opt.node_map[mm]
+    first = opt.ds[(s_i, 1, 0, 0)]["comm_cost"]
+    assert f"{first:.3f}" in out[2]
+    assert len(out[0].split("  ")) >= n_cols
