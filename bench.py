@@ -36,8 +36,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 MEASURED_TRAFFIC_BYTES = {
     (1_821_368, 1_616, 80_507_252): (3_038.8 * 2.000 + 74_539.1) * 1024,           # llama3_8b, mesh (32, 8), all tables in one launch
     (1_821_368, 1_616, 32_348_914): (674.1 * 2.000 + 31_426.0) * 1024,             # the same, --table-launches 2
-    (73_251_434, 40_727, 1_255_915_920): (12_334.7 * 2.000 + 1_220_980.7) * 1024,   # llama3_70b, mesh (8, 8, 8)
-    (464_235_576, 426_918, 8_003_825_874): (159_699.9 * 2.000 + 7_760_701.8) * 1024,  # stress, mesh (16, 8, 4)
+    (73_251_434, 40_727, 1_255_915_920): (12_325.7 * 2.000 + 1_220_870.3) * 1024,   # llama3_70b, mesh (8, 8, 8)
+    (464_235_576, 426_918, 8_003_825_874): (160_762.9 * 2.000 + 7_760_997.7) * 1024,  # stress, mesh (16, 8, 4)
 }
 
 
