@@ -41,5 +41,26 @@ def build_library(verbose: bool = False) -> str:
     return LIB_PATH
 
 
+ABI_CONSUMER_SOURCE = os.path.join(_ROOT, "tests", "abi_consumer.cpp")
+ABI_CONSUMER_PATH = os.path.join(_ROOT, "tests", "abi_consumer")
+
+
+def build_abi_consumer(verbose: bool = False) -> str:
+    """The C++ program that uses the library through include/apcost.h alone (no Python, no
+    torch): proof that the boundary is a plain C ABI.  A GPU test runs it."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, "--offload-arch=gfx950", "-O1", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           f"-I{INCLUDE}", "-o", ABI_CONSUMER_PATH,
+           ABI_CONSUMER_SOURCE, f"-L{_PKG}", "-lapcost", "-Wl,-rpath,$ORIGIN/../autoparallel_amd"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        err = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l)
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
+    return ABI_CONSUMER_PATH
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_abi_consumer(verbose=True))

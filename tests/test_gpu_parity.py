@@ -530,3 +530,17 @@ def test_randomized_configurations(gpu_device, monkeypatch):
         assert np.array_equal(d.transition.cpu().numpy(), want["transition"]), what
         _assert_costs(d.compute_cost.cpu().numpy(), want_cc, what + " compute_cost")
         assert np.array_equal(d.row_min.cpu().numpy(), want_min) and np.array_equal(d.row_argmin.cpu().numpy(), want_arg), what
+
+
+def test_cpp_consumer_of_the_c_abi(gpu_device):
+    """tests/abi_consumer.cpp: a C++ program that includes include/apcost.h, links the library
+    and checks the hand-derived known answers itself (no Python, no torch in that process)."""
+    import os
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "abi_consumer")
+    if not os.path.exists(exe):
+        pytest.fail(f"{exe} is missing: build it with `python -m autoparallel_amd._build`")
+    run = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "abi consumer ok" in run.stdout
