@@ -216,6 +216,9 @@ class ShardingOptimizer:
     device = "cuda:0"
     backend_cls = DeviceBackend
     solver_time_limit: Optional[float] = None
+    # relative gap at which the solver may stop: 0 = prove optimality (the reference's CBC default);
+    # None = the solver's own default (1e-4)
+    solver_rel_gap: Optional[float] = 0.0
     # tiling of the edge matrices: entries per tile (None: chosen from the table), whether
     # identical edges (repeated layers) are evaluated once, and how many copies one evaluated
     # edge may serve at most
@@ -569,7 +572,7 @@ class ShardingOptimizer:
         # linked entries share a variable: their costs add up
         obj = np.bincount(self.var_of_entry, weights=self.cost, minlength=self.prob.n_vars).astype(np.float64)
         self.prob.objective = obj
-        status = self.prob.solve(verbose=verbose, time_limit=self.solver_time_limit)
+        status = self.prob.solve(verbose=verbose, time_limit=self.solver_time_limit, mip_rel_gap=self.solver_rel_gap)
         if status == -1:
             print(self.get_violated_constraints_log())
             raise RuntimeError("Unsolvable problem")
