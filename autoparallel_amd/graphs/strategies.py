@@ -276,7 +276,9 @@ class StrategyEnumerator:
     def _fresh_copy(strategy: OpStrategy) -> OpStrategy:
         out = []
         for s in strategy.strategies:
-            rc = None if s.redistribute_cost is None else [list(row) for row in s.redistribute_cost]
+            # the outer list is the node's own (rows are replaced per argument when the computed
+            # costs are written back); the rows themselves are shared read-only with the memo
+            rc = None if s.redistribute_cost is None else list(s.redistribute_cost)
             out.append(OpSpec(s.output_specs, input_specs=s.input_specs, redistribute_cost=rc))
         return OpStrategy(out)
 
