@@ -234,6 +234,20 @@ class ShardingOptimizer:
     compact_constraints = True  # with choice variables: the structural constraints written through them
 
     def __init__(self, gm, mesh, rescale_grad_comm_cost_for_mp=1.0, repeated_subgraphs=False):
+        # Construction allocates millions of small long-lived objects (strategies, cost rows)
+        # and no reference cycles worth collecting: the cyclic collector's full passes over
+        # them were a fifth of the construction time on the 70B graph.
+        import gc
+
+        was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            self._construct(gm, mesh, rescale_grad_comm_cost_for_mp, repeated_subgraphs)
+        finally:
+            if was_enabled:
+                gc.enable()
+
+    def _construct(self, gm, mesh, rescale_grad_comm_cost_for_mp, repeated_subgraphs):
         self.gm = gm
         self.graph = gm.graph
         self.nodes = list(self.graph.nodes)
