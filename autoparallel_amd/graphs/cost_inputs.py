@@ -49,6 +49,7 @@ def fill_flops_and_bytes(encoded, strats, local_shape: np.ndarray, local_stride:
     outputs of the spec-table kernel."""
     tb = encoded.tables
     memo: dict = {}
+    node_memo: dict = {}  # node key -> first strategy row of the node that was evaluated
     n_eval = 0
     for s_i, node in enumerate(encoded.nodes):
         if node.op == "output":
@@ -82,6 +83,18 @@ def fill_flops_and_bytes(encoded, strats, local_shape: np.ndarray, local_stride:
         if mode is None:
             out_val = node.meta.get("val")
             mode = getattr(out_val, "fake_mode", None) if isinstance(out_val, torch.Tensor) else None
+        # a node of a repeated layer has the rows of its first occurrence: same op, constants,
+        # dtypes and local shapes / strides of every strategy
+        node_key = (node.target, const_key, dtypes, tuple(ranks), n,
+                    tuple(local_shape[spec_rows[k]:spec_rows[k] + n, :r].tobytes() +
+                          local_stride[spec_rows[k]:spec_rows[k] + n, :r].tobytes() for k, r in enumerate(ranks)))
+        seen = node_memo.get(node_key)
+        if seen is not None:
+            tb.strat_flops[base:base + n] = tb.strat_flops[seen:seen + n]
+            tb.strat_rw_bytes[base:base + n] = tb.strat_rw_bytes[seen:seen + n]
+            tb.strat_dtype[base:base + n] = tb.strat_dtype[seen:seen + n]
+            continue
+        node_memo[node_key] = base
         for ss in range(n):
             shapes = []
             for k, r in enumerate(ranks):
