@@ -261,17 +261,19 @@ struct SpecTableArgs {
   const int32_t *tensor, *rank, *itemsize;
   const int64_t *shape, *stride;
   int64_t *shards, *lshape, *lstride, *lnumel, *lbytes;
+  int width;  // values per row of lshape / lstride: even, 2 .. APC_MAX_RANK, >= every tensor's rank
 };
 
 // s_rows: kBlock * (APC_MAX_RANK + 1) values of LDS
-// Writes the first `live` values (a multiple of APC_MAX_RANK) of the workgroup's staged rows
-// (APC_MAX_RANK + 1 slots per row in LDS) to `out` as one contiguous run, two values (one
-// 16-byte store) per lane: rows hold an even number of values, so a pair never straddles rows.
+// Writes the staged rows of the workgroup (APC_MAX_RANK + 1 slots per row in LDS) to `out`, the
+// first `width` values of each row, `live` values in all (rows x width), as one contiguous run,
+// two values (one 16-byte store) per lane: width is even, so a pair never straddles rows.
 template <int BS>
-__device__ __forceinline__ void write_rows(int64_t *__restrict__ out, const int64_t *s_rows, int64_t live) {
+__device__ __forceinline__ void write_rows(int64_t *__restrict__ out, const int64_t *s_rows, int live, int width) {
   typedef int64_t pair_t __attribute__((ext_vector_type(2)));
   for (int k = 2 * threadIdx.x; k < live; k += 2 * BS) {
-    const int64_t *src = s_rows + (k / APC_MAX_RANK) * (APC_MAX_RANK + 1) + k % APC_MAX_RANK;
+    const int r = k / width, c = k - r * width;
+    const int64_t *src = s_rows + r * (APC_MAX_RANK + 1) + c;
     pair_t v = {src[0], src[1]};
     *reinterpret_cast<pair_t *>(out + k) = v;
   }
@@ -293,7 +295,8 @@ __device__ __forceinline__ void spec_tables_block(int64_t block, const apc_param
   const int64_t base = block * BS;
   const int64_t s = base + threadIdx.x;
   int64_t *row = s_rows + threadIdx.x * (APC_MAX_RANK + 1);
-  const int64_t live = (n - base < BS ? n - base : BS) * APC_MAX_RANK;
+  const int width = a.width;
+  const int live = (int)(n - base < BS ? n - base : BS) * width;
   int t = -1, r = 0;
   uint32_t pc = 0;
   if (s < n) {
@@ -334,7 +337,7 @@ __device__ __forceinline__ void spec_tables_block(int64_t block, const apc_param
     lbytes[s] = nb;
   }
   __syncthreads();
-  write_rows<BS>(lshape + base * APC_MAX_RANK, s_rows, live);
+  write_rows<BS>(lshape + base * width, s_rows, live, width);
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < APC_MAX_RANK; ++i) row[i] = st[i];
@@ -347,7 +350,7 @@ __device__ __forceinline__ void spec_tables_block(int64_t block, const apc_param
     }
   }
   __syncthreads();
-  write_rows<BS>(lstride + base * APC_MAX_RANK, s_rows, live);
+  write_rows<BS>(lstride + base * width, s_rows, live, width);
 }
 
 __global__ __launch_bounds__(kBlock) void spec_tables_kernel(apc_params p, SpecTableArgs a) {
@@ -1073,6 +1076,12 @@ void launch_segmented_min(const double *values, const int64_t *seg_ptr, int64_t 
                      seg_ptr, n_seg, mins, args);
 }
 
+int check_width(int width) {
+  if (width < 2 || width > APC_MAX_RANK || (width & 1))
+    return fail(-1, "shape_width %d must be even and in [2, %d]", width, APC_MAX_RANK);
+  return 0;
+}
+
 int check_params(const apc_params *p) {
   if (!p) return fail(-1, "params is NULL");
   if (p->mesh_ndim < 1 || p->mesh_ndim > APC_MAX_MESH)
@@ -1209,9 +1218,10 @@ int apc_tensor_tables(int64_t n, const int32_t *rank, const int32_t *itemsize, c
 
 int apc_spec_tables(const apc_params *params, int64_t n, const uint32_t *codes, const int32_t *tensor,
                     const int32_t *rank, const int32_t *itemsize, const int64_t *shape, const int64_t *stride,
-                    int64_t *shards, int64_t *lshape, int64_t *lstride, int64_t *lnumel, int64_t *lbytes,
-                    void *stream) {
+                    int64_t *shards, int64_t *lshape, int64_t *lstride, int32_t shape_width, int64_t *lnumel,
+                    int64_t *lbytes, void *stream) {
   if (int rc = check_params(params)) return rc;
+  if (int rc = check_width(shape_width)) return rc;
   if (n < 0) return fail(-1, "n_specs < 0");
   if (n == 0) return 0;
   if (!codes || !tensor || !rank || !itemsize || !shape || !stride || !shards || !lshape || !lstride || !lnumel ||
@@ -1219,7 +1229,7 @@ int apc_spec_tables(const apc_params *params, int64_t n, const uint32_t *codes, 
     return fail(-1, "apc_spec_tables: NULL array");
   hipLaunchKernelGGL(spec_tables_kernel, dim3(blocks_for(n, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, *params,
                      SpecTableArgs{n, codes, tensor, rank, itemsize, shape, stride, shards, lshape, lstride, lnumel,
-                                   lbytes});
+                                   lbytes, shape_width});
   return check_launch("apc_spec_tables");
 }
 
@@ -1239,11 +1249,12 @@ int apc_compute_costs(const apc_params *params, int64_t n, const int64_t *flops,
 int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t *rank, const int32_t *itemsize,
                      const int64_t *shape, const int64_t *stride, int64_t *tensor_bytes, uint8_t *tensor_contiguous,
                      int64_t n_specs, const uint32_t *spec_codes, const int32_t *spec_tensor, int64_t *num_shards,
-                     int64_t *local_shape, int64_t *local_stride, int64_t *local_numel, int64_t *local_bytes,
-                     int64_t n_strategies, const int64_t *flops, const int64_t *rw_bytes, const int8_t *dtype,
-                     const uint8_t *zero_cost, const int32_t *num_args, double *compute, double *per_arg,
-                     int32_t *error_flag, void *stream) {
+                     int64_t *local_shape, int64_t *local_stride, int32_t shape_width, int64_t *local_numel,
+                     int64_t *local_bytes, int64_t n_strategies, const int64_t *flops, const int64_t *rw_bytes,
+                     const int8_t *dtype, const uint8_t *zero_cost, const int32_t *num_args, double *compute,
+                     double *per_arg, int32_t *error_flag, void *stream) {
   if (int rc = check_params(params)) return rc;
+  if (int rc = check_width(shape_width)) return rc;
   if (n_tensors < 0 || n_specs < 0 || n_strategies < 0) return fail(-1, "apc_input_tables: negative count");
   if (n_tensors > 0 && (!rank || !itemsize || !shape || !stride || !tensor_bytes || !tensor_contiguous))
     return fail(-1, "apc_input_tables: NULL tensor array");
@@ -1258,7 +1269,7 @@ int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t 
   hipLaunchKernelGGL(input_tables_kernel, dim3((unsigned)(sb + tb + cb)), dim3(kBlock), 0, (hipStream_t)stream, *params,
                      TensorTableArgs{n_tensors, rank, itemsize, shape, stride, tensor_bytes, tensor_contiguous},
                      SpecTableArgs{n_specs, spec_codes, spec_tensor, rank, itemsize, shape, stride, num_shards,
-                                   local_shape, local_stride, local_numel, local_bytes},
+                                   local_shape, local_stride, local_numel, local_bytes, shape_width},
                      ComputeCostArgs{n_strategies, flops, rw_bytes, dtype, zero_cost, num_args, compute, per_arg,
                                      error_flag},
                      sb, tb);
@@ -1307,10 +1318,10 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
 int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t *rank, const int32_t *itemsize,
                      const int64_t *shape, const int64_t *stride, int64_t *tensor_bytes, uint8_t *tensor_contiguous,
                      int64_t n_specs, const uint32_t *spec_codes, const int32_t *spec_tensor, int64_t *num_shards,
-                     int64_t *local_shape, int64_t *local_stride, int64_t *local_numel, int64_t *local_bytes,
-                     int64_t n_strategies, const int64_t *flops, const int64_t *rw_bytes, const int8_t *dtype,
-                     const uint8_t *zero_cost, const int32_t *num_args, double *compute, double *per_arg,
-                     int32_t *error_flag, const double *pt_values, int64_t n_tiles, const apc_tile *tiles,
+                     int64_t *local_shape, int64_t *local_stride, int32_t shape_width, int64_t *local_numel,
+                     int64_t *local_bytes, int64_t n_strategies, const int64_t *flops, const int64_t *rw_bytes,
+                     const int8_t *dtype, const uint8_t *zero_cost, const int32_t *num_args, double *compute,
+                     double *per_arg, int32_t *error_flag, const double *pt_values, int64_t n_tiles, const apc_tile *tiles,
                      const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *trans_out,
                      double *cost_out, void *stream) {
   if (int rc = check_params(params)) return rc;
@@ -1319,6 +1330,8 @@ int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t 
   if (n_tensors > 0 && (!rank || !itemsize || !shape || !stride || !tensor_bytes || !tensor_contiguous))
     return fail(-1, "apc_build_tables: NULL tensor array");
   const bool spec_table = num_shards || local_shape || local_stride || local_numel || local_bytes;
+  if (spec_table)
+    if (int rc = check_width(shape_width)) return rc;
   if (spec_table && n_specs > 0 && (!spec_codes || !spec_tensor || !num_shards || !local_shape || !local_stride ||
                                     !local_numel || !local_bytes))
     return fail(-1, "apc_build_tables: the spec table needs all five of its outputs");
@@ -1345,7 +1358,7 @@ int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t 
               comm_out, trans_out, cost_out, rank, itemsize, shape, stride, flops, rw_bytes, dtype, zero_cost, num_args};
   const TensorTableArgs ta{n_tensors, rank, itemsize, shape, stride, tensor_bytes, tensor_contiguous};
   const SpecTableArgs sa{n_specs, spec_codes, spec_tensor, rank, itemsize, shape, stride, num_shards,
-                         local_shape, local_stride, local_numel, local_bytes};
+                         local_shape, local_stride, local_numel, local_bytes, shape_width};
   const ComputeCostArgs ca{n_strategies, flops, rw_bytes, dtype, zero_cost, num_args, compute, per_arg, error_flag};
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)blocks);

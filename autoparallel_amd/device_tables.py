@@ -113,10 +113,11 @@ class DeviceCostTables:
     @_guarded
     def run_spec_tables(self):
         n = self.tables.n_specs
+        width = self.tables.shape_width()  # rows as wide as the largest rank needs, not APC_MAX_RANK
         out = {
             "num_shards": self._empty((n,), torch.int64),
-            "local_shape": self._empty((n, APC_MAX_RANK), torch.int64),
-            "local_stride": self._empty((n, APC_MAX_RANK), torch.int64),
+            "local_shape": self._empty((n, width), torch.int64),
+            "local_stride": self._empty((n, width), torch.int64),
             "local_numel": self._empty((n,), torch.int64),
             "local_bytes": self._empty((n,), torch.int64),
         }
@@ -125,8 +126,8 @@ class DeviceCostTables:
                 ctypes.byref(self.c_params), ctypes.c_int64(n), self._p("spec_codes"), self._p("spec_tensor"),
                 self._p("tensor_rank"), self._p("tensor_itemsize"), self._p("tensor_shape"),
                 self._p("tensor_stride"), self._p(out["num_shards"]), self._p(out["local_shape"]),
-                self._p(out["local_stride"]), self._p(out["local_numel"]), self._p(out["local_bytes"]),
-                self._stream())
+                self._p(out["local_stride"]), ctypes.c_int32(width), self._p(out["local_numel"]),
+                self._p(out["local_bytes"]), self._stream())
         _native.check(rc, "apc_spec_tables")
         self.spec_out = out
         return out
@@ -219,8 +220,8 @@ class DeviceCostTables:
                     P("tensor_stride"), P(self.tensor_bytes), P(self.tensor_contiguous), stream)
         a_spec = (cp, ctypes.c_int64(tb.n_specs), P("spec_codes"), P("spec_tensor"), P("tensor_rank"),
                   P("tensor_itemsize"), P("tensor_shape"), P("tensor_stride"), P(spec["num_shards"]),
-                  P(spec["local_shape"]), P(spec["local_stride"]), P(spec["local_numel"]), P(spec["local_bytes"]),
-                  stream)
+                  P(spec["local_shape"]), P(spec["local_stride"]), ctypes.c_int32(spec["local_shape"].shape[1]),
+                  P(spec["local_numel"]), P(spec["local_bytes"]), stream)
         a_compute = (cp, ctypes.c_int64(tb.n_strategies), P("strat_flops"), P("strat_rw_bytes"), P("strat_dtype"),
                      P("strat_zero_cost"), P("strat_num_args"), P(self.compute_cost), P(self.compute_cost_per_arg),
                      P(err), stream)

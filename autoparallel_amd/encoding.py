@@ -212,12 +212,18 @@ class CostTables:
         per_edge = (self.edge_n_src.astype(np.int64) + self.edge_n_tgt.astype(np.int64)) * m + 64
         return per_entry * self.n_entries + int(per_edge.sum())
 
+    def shape_width(self) -> int:
+        """Values per row of the local shape / stride tables: the largest tensor rank, rounded up
+        to even (rows leave the kernel as 16-byte pairs), at least 2."""
+        top = int(self.tensor_rank.max()) if self.n_tensors else 0
+        return max(2, top + (top & 1))
+
     def algorithmic_bytes_input_tables(self) -> int:
         """Bytes the tensor, spec and compute-cost tables must move at minimum: per tensor 136 B
-        read (rank, itemsize, shape, stride) and 9 B written; per spec 8 B read and 152 B
-        written (shard count, local shape and stride, local element and byte counts); per
-        strategy 22 B read and 16 B written."""
-        return 145 * self.n_tensors + 160 * self.n_specs + 38 * self.n_strategies
+        read (rank, itemsize, shape, stride) and 9 B written; per spec 8 B read and 24 B + two
+        rows of ``shape_width()`` values written (shard count, local element and byte counts,
+        local shape and stride); per strategy 22 B read and 16 B written."""
+        return 145 * self.n_tensors + (32 + 16 * self.shape_width()) * self.n_specs + 38 * self.n_strategies
 
     # ---- tiles -------------------------------------------------------------------------
     def edge_signatures(self) -> list:

@@ -45,7 +45,7 @@ def _const_key(x):
 
 def fill_flops_and_bytes(encoded, strats, local_shape: np.ndarray, local_stride: np.ndarray, stats=None) -> None:
     """Writes strat_flops / strat_rw_bytes / strat_dtype / strat_zero_cost of
-    ``encoded.tables`` in place.  ``local_shape`` / ``local_stride`` are the [n_specs, 8]
+    ``encoded.tables`` in place.  ``local_shape`` / ``local_stride`` are the [n_specs, width]
     outputs of the spec-table kernel."""
     tb = encoded.tables
     memo: dict = {}

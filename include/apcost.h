@@ -135,12 +135,14 @@ int apc_tensor_tables(int64_t n_tensors, const int32_t *tensor_rank, const int32
 /* Local shard shape / stride / element and byte counts and shard count per spec.
  * Replaces _get_sharded_shape_stride (compute_estimation.py:211-229) and
  * DTensorSpec.num_shards (torch distributed/tensor/_dtensor_spec.py:555-561).
- * local_shape / local_stride are [n_specs][APC_MAX_RANK], zero padded. */
+ * local_shape / local_stride are [n_specs][shape_width], zero padded: shape_width is even, at
+ * most APC_MAX_RANK and at least the largest tensor rank (the caller's choice: rows of rank-4
+ * tables padded to 8 would double the bytes this table writes). */
 int apc_spec_tables(const apc_params *params, int64_t n_specs, const uint32_t *spec_codes,
                     const int32_t *spec_tensor, const int32_t *tensor_rank, const int32_t *tensor_itemsize,
                     const int64_t *tensor_shape, const int64_t *tensor_stride, int64_t *num_shards,
-                    int64_t *local_shape, int64_t *local_stride, int64_t *local_numel, int64_t *local_bytes,
-                    void *stream);
+                    int64_t *local_shape, int64_t *local_stride, int32_t shape_width, int64_t *local_numel,
+                    int64_t *local_bytes, void *stream);
 
 /* Per-(node, strategy) compute cost and compute cost / num_args.
  * Replaces the arithmetic tail of estimate_strategy_runtime_cost
@@ -161,10 +163,10 @@ int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t 
                      const int32_t *tensor_itemsize, const int64_t *tensor_shape, const int64_t *tensor_stride,
                      int64_t *tensor_bytes, uint8_t *tensor_contiguous, int64_t n_specs, const uint32_t *spec_codes,
                      const int32_t *spec_tensor, int64_t *num_shards, int64_t *local_shape, int64_t *local_stride,
-                     int64_t *local_numel, int64_t *local_bytes, int64_t n_strategies, const int64_t *flops,
-                     const int64_t *rw_bytes, const int8_t *dtype_code, const uint8_t *zero_cost,
-                     const int32_t *num_args, double *compute_cost, double *compute_cost_per_arg,
-                     int32_t *error_flag, void *stream);
+                     int32_t shape_width, int64_t *local_numel, int64_t *local_bytes, int64_t n_strategies,
+                     const int64_t *flops, const int64_t *rw_bytes, const int8_t *dtype_code,
+                     const uint8_t *zero_cost, const int32_t *num_args, double *compute_cost,
+                     double *compute_cost_per_arg, int32_t *error_flag, void *stream);
 
 /* The redistribution-cost matrices of every edge, plus the assembled ILP cost.
  * Replaces the two inner loops of ShardingOptimizer.build_ds
@@ -194,10 +196,11 @@ int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t 
                      const int32_t *tensor_itemsize, const int64_t *tensor_shape, const int64_t *tensor_stride,
                      int64_t *tensor_bytes, uint8_t *tensor_contiguous, int64_t n_specs, const uint32_t *spec_codes,
                      const int32_t *spec_tensor, int64_t *num_shards, int64_t *local_shape, int64_t *local_stride,
-                     int64_t *local_numel, int64_t *local_bytes, int64_t n_strategies, const int64_t *flops,
-                     const int64_t *rw_bytes, const int8_t *dtype_code, const uint8_t *zero_cost,
-                     const int32_t *num_args, double *compute_cost, double *compute_cost_per_arg,
-                     int32_t *error_flag, const double *pt_values, int64_t n_tiles, const apc_tile *tiles,
+                     int32_t shape_width, int64_t *local_numel, int64_t *local_bytes, int64_t n_strategies,
+                     const int64_t *flops, const int64_t *rw_bytes, const int8_t *dtype_code,
+                     const uint8_t *zero_cost, const int32_t *num_args, double *compute_cost,
+                     double *compute_cost_per_arg, int32_t *error_flag, const double *pt_values, int64_t n_tiles,
+                     const apc_tile *tiles,
                      const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *transition_out,
                      double *cost_out, void *stream);
 

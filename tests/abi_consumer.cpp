@@ -121,8 +121,9 @@ int main() {
   HIP_OK(hipMalloc(&d_bytes, 8));
   HIP_OK(hipMalloc(&d_cont, 16));
   HIP_OK(hipMalloc(&d_shards, 4 * 8));
-  HIP_OK(hipMalloc(&d_lshape, 4 * APC_MAX_RANK * 8));
-  HIP_OK(hipMalloc(&d_lstride, 4 * APC_MAX_RANK * 8));
+  const int width = 2;  // values per row of the local shape / stride tables: the tensor's rank
+  HIP_OK(hipMalloc(&d_lshape, 4 * width * 8));
+  HIP_OK(hipMalloc(&d_lstride, 4 * width * 8));
   HIP_OK(hipMalloc(&d_lnumel, 4 * 8));
   HIP_OK(hipMalloc(&d_lbytes, 4 * 8));
   HIP_OK(hipMalloc(&d_compute, 4 * 8));
@@ -144,14 +145,14 @@ int main() {
 
   // every table of the pass in one launch, then the minimum of the whole matrix
   APC_OK(apc_build_tables(&p, 1, d_rank, d_item, d_shape, d_stride, d_bytes, d_cont, 4, d_codes, d_spec_tensor, d_shards,
-                          d_lshape, d_lstride, d_lnumel, d_lbytes, 4, d_flops, d_rw, d_dtype, d_zero, d_args, d_compute,
+                          d_lshape, d_lstride, width, d_lnumel, d_lbytes, 4, d_flops, d_rw, d_dtype, d_zero, d_args, d_compute,
                           d_per_arg, d_err, nullptr, 1, d_tiles, nullptr, 3, d_comm, d_trans, d_cost, nullptr));
   APC_OK(apc_segmented_min(d_cost, d_seg, 1, 3, d_min, d_arg, nullptr));
   HIP_OK(hipDeviceSynchronize());
 
   double comm[3], cost[3], seg_min = 0.0;
   uint8_t trans[3];
-  int64_t bytes = 0, lshape[4 * APC_MAX_RANK];
+  int64_t bytes = 0, lshape[4 * 2];
   int32_t seg_arg = -1;
   HIP_OK(hipMemcpy(comm, d_comm, sizeof(comm), hipMemcpyDeviceToHost));
   HIP_OK(hipMemcpy(cost, d_cost, sizeof(cost), hipMemcpyDeviceToHost));
@@ -172,7 +173,7 @@ int main() {
   }
   bad += bytes != 4096LL * 4096 * 2;
   bad += lshape[0] != 4096 / 32 / 8 || lshape[1] != 4096;                        // (S0, S0): dim 0 split twice
-  bad += lshape[3 * APC_MAX_RANK] != 4096 / 32 || lshape[3 * APC_MAX_RANK + 1] != 4096 / 8;  // (S0, S1)
+  bad += lshape[3 * width] != 4096 / 32 || lshape[3 * width + 1] != 4096 / 8;  // (S0, S1)
   bad += seg_min != want[2] + 1.0 || seg_arg != 2;
   std::printf(bad ? "abi consumer: %d MISMATCHES\n" : "abi consumer ok\n", bad);
   return bad ? 1 : 0;

@@ -32,6 +32,15 @@ def _assert_costs(got: np.ndarray, want: np.ndarray, what: str):
     assert np.array_equal(got, want), f"{what}: not bit-identical ({int((got != want).sum())} entries differ)"
 
 
+def _same_rows(got: np.ndarray, want) -> bool:
+    """Device rows are ``shape_width()`` wide, the oracle's 8: equal where both exist, zero beyond."""
+    want = np.asarray(want, dtype=np.int64)
+    if got.ndim == 1:
+        return np.array_equal(got, want)
+    w = got.shape[1]
+    return np.array_equal(got, want[:, :w]) and not want[:, w:].any()
+
+
 def _run_and_compare(tb: CostTables, mesh, rescale, device):
     p = CostModelParams.from_mesh(mesh, rescale=rescale)
     op = po.make_params(mesh, rescale=rescale)
@@ -61,7 +70,8 @@ def test_tables_match_oracle_on_seeded_dags(gpu_device, mesh):
     got = d.run_spec_tables()
     for key, w in zip(("num_shards", "local_shape", "local_stride", "local_numel", "local_bytes"),
                       c_oracle.spec_tables(enc, mesh)):
-        assert np.array_equal(got[key].cpu().numpy(), w), key
+        assert _same_rows(got[key].cpu().numpy(), w), key
+    assert got["local_shape"].shape[1] == tb.shape_width() <= 8
 
 
 def test_python_oracle_agrees_on_a_small_case(gpu_device):
@@ -133,7 +143,8 @@ def test_local_shapes_of_very_large_dims(gpu_device, mesh):
     want = po.spec_tables(tb.as_dict(), mesh)
     for key, w in zip(("num_shards", "local_shape", "local_stride", "local_numel", "local_bytes"), want):
         # (local numel / bytes of the 2^52-sized dims exceed nothing: the other dims are 1)
-        assert np.array_equal(got[key].cpu().numpy(), np.asarray(w, dtype=np.int64)), key
+        assert _same_rows(got[key].cpu().numpy(), w), key
+    assert got["local_shape"].shape[1] == 4  # rank 3, rounded up to even
 
 
 def _golden():
@@ -440,7 +451,7 @@ def test_fused_input_tables_match_the_three_entry_points(gpu_device):
         assert np.array_equal(results[0][key], results[1][key]), key
     enc = tb.as_dict()
     assert np.array_equal(results[1]["tensor_bytes"], c_oracle.tensor_tables(enc)[0])
-    assert np.array_equal(results[1]["spec_local_shape"], c_oracle.spec_tables(enc, mesh)[1])
+    assert _same_rows(results[1]["spec_local_shape"], c_oracle.spec_tables(enc, mesh)[1])
     assert (results[1]["cost"] != 0).any()
 
 
