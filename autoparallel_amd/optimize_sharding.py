@@ -87,6 +87,7 @@ class DeviceBackend:
             "comm": d.comm.cpu().numpy(),
             "transition": d.transition.cpu().numpy(),
             "cost": d.cost.cpu().numpy(),
+            "compute": d.compute_cost.cpu().numpy(),
             "compute_per_arg": d.compute_cost_per_arg.cpu().numpy(),
         }
         self.timings["copy_back_s"] = time.perf_counter() - t0
@@ -323,6 +324,7 @@ class ShardingOptimizer:
         self.comm_cost = out["comm"]
         self.transition_cost = out["transition"]
         self.cost = out["cost"].copy()
+        self.compute_cost = out["compute"]  # per (node, strategy), before the division by num_args
         self.compute_cost_per_arg = out["compute_per_arg"]
         self.var_of_entry = np.arange(tb.n_entries, dtype=np.int64)
         # the recomputed costs are written back into OpSpec.redistribute_cost, which

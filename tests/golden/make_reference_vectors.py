@@ -1,0 +1,173 @@
+"""Writes ``reference_compute_costs.json``: the compute cost of every (node, strategy) of
+four traced graphs as the reference's own ``estimate_strategy_runtime_cost``
+(autoparallel/compute_estimation.py:334-365) returns it.  That function runs each operator on
+fake tensors of the sharded argument shapes, so its result depends on what every operator's
+meta kernel and flop formula return: no closed form pins it for operators other than mm.
+
+Runs only where /root/reference exists (never on a GPU box, never from a test).  Only
+``autoparallel.compute_estimation`` is imported: it needs nothing but torch.  The reference's
+strategy enumeration (``autoparallel.utils`` / ``propagation_rules`` / ``dtensor_util``) does
+not import under the installed torch (``register_op_strategy`` has left
+``torch.distributed.tensor._ops.utils``), and no stand-in was written for it.  So the graphs
+and the strategy lists are this repository's own (capture + ``StrategyEnumerator``): they are
+the INPUT of the vectors, stored beside the costs so that a test can tell a changed input from
+a changed result.
+
+The environment is the one the reference's planner tests patch in
+(tests/test_optimize_placement.py:141-142): 8 devices per host, device name "H100".
+
+    python tests/golden/make_reference_vectors.py
+"""
+
+import json
+import os
+import sys
+import warnings
+from unittest.mock import patch
+
+import torch
+from torch.utils._pytree import tree_flatten
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+REFERENCE = "/root/reference"  # put on sys.path by main() only: the helpers above it are imported by a test
+
+CASES = [
+    # (name, model kind or workload, mesh)
+    ("ffn_32x8", "ffn", (32, 8)),
+    ("block_32x8", "block", (32, 8)),
+    ("llama3_8b_1layer_32x8", "llama3_8b", (32, 8)),
+    ("llama3_70b_1layer_8x8x8", "llama3_70b", (8, 8, 8)),
+]
+
+
+def placement_code(p) -> str:
+    if p.is_replicate():
+        return "R"
+    if p.is_partial():
+        return "P" if p.reduce_op == "sum" else f"P[{p.reduce_op}]"
+    name = type(p).__name__
+    return f"S{p.dim}" if name == "Shard" else f"{name}{p.dim}"
+
+
+def spec_code(spec) -> str:
+    if spec is None:
+        return "-"
+    if isinstance(spec, (tuple, list)):
+        return "(" + ";".join(spec_code(s) for s in spec) + ")"
+    return "".join(placement_code(p) for p in spec.placements) if len(spec.placements) else "()"
+
+
+def strategy_code(s) -> str:
+    ins = ",".join(spec_code(x) for x in (s.input_specs or ()))
+    return f"{ins}->{spec_code(s.output_specs)}"
+
+
+def node_signature(node) -> str:
+    """Operator and argument shapes / strides / dtypes: what the reference's functions saw."""
+    if node.op == "placeholder":
+        v = node.meta["val"]
+        return f"placeholder {tuple(v.shape)} {tuple(v.stride())} {v.dtype}"
+
+    def one(x):
+        if isinstance(x, torch.fx.Node):
+            v = x.meta["val"]
+            if isinstance(v, torch.Tensor):
+                return f"T{tuple(v.shape)}{tuple(v.stride())}{str(v.dtype).replace('torch.', '')}"
+            return "V"
+        return repr(x)
+
+    flat, _ = tree_flatten((node.args, node.kwargs))
+    return f"{node.target} " + " ".join(one(x) for x in flat)
+
+
+def make_graph(kind, mesh):
+    from autoparallel_amd.graphs.capture import capture_joint_graph
+
+    if kind.startswith("llama3"):
+        # one decoder layer of the benchmark model at its full shapes, bf16 parameter casts
+        from autoparallel_amd.graphs.workloads import build_model
+
+        model, input_fn, _, _ = build_model(kind, mesh, n_layers=1)
+        return capture_joint_graph(model, input_fn, param_dtype=torch.bfloat16, device="cpu", dynamo=False)
+    from models import make_model_and_inputs
+
+    model_fn, input_fn = make_model_and_inputs(mesh, kind)
+    with torch.device("meta"):
+        model = model_fn()
+    return capture_joint_graph(model, input_fn, param_dtype=None, device="cpu", dynamo=False)
+
+
+def reference_tables(gm, mesh):
+    from autoparallel.compute_estimation import estimate_strategy_runtime_cost
+
+    from autoparallel_amd.graphs.strategies import enumerate_strategies
+
+    strats, _ = enumerate_strategies(gm, mesh)
+    records = []
+    for node in gm.graph.nodes:
+        if node.op == "output":
+            continue
+        strategies = strats[node].strategies
+        costs = [float(estimate_strategy_runtime_cost(node, s)) for s in strategies]
+        records.append((node.name, node_signature(node), [strategy_code(s) for s in strategies],
+                        [c.hex() for c in costs]))  # float.hex keeps every bit
+    return records
+
+
+def pack(records):
+    """Nodes of one kind repeat, and so do strategy lists and cost values: every distinct
+    strategy list and every distinct cost value is stored once and named by its index.
+    node = [name, signature index, strategy-list index, [cost-value index per strategy]]."""
+    signatures, lists, values, nodes = {}, {}, {}, []
+
+    def intern(table, key):
+        return table.setdefault(key, len(table))
+
+    for name, sig, codes, costs in records:
+        nodes.append([name, intern(signatures, sig), intern(lists, tuple(codes)),
+                      [intern(values, c) for c in costs]])
+    return {"signatures": list(signatures), "strategy_lists": [list(x) for x in lists],
+            "cost_values_us": list(values), "nodes": nodes}
+
+
+def main():
+    import torch.distributed as dist
+    from torch.distributed.device_mesh import _mesh_resources, init_device_mesh
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    assert os.path.isdir(REFERENCE), "the reference is not present here: the committed vectors are used as they are"
+    sys.path.insert(0, REFERENCE)
+    dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=512)
+    out = {"provenance": "written by tests/golden/make_reference_vectors.py from the reference's "
+                         "estimate_strategy_runtime_cost (autoparallel/compute_estimation.py:334-365), "
+                         f"torch {torch.__version__}",
+           "environment": {"devices_per_host": 8, "device_name": "H100"},
+           "cases": {}}
+    for name, kind, mesh_sizes in CASES:
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            mesh = init_device_mesh("cpu", mesh_sizes)
+        ctx = make_graph(kind, mesh)
+        gm, _ = ctx.__enter__()
+        try:
+            with patch("torch.cuda.device_count", lambda: 8), \
+                    patch("torch.cuda.get_device_name", lambda device=None: "H100"), \
+                    patch.object(type(_mesh_resources), "num_devices_per_host", lambda self, device_type: 8):
+                records = reference_tables(gm, mesh)
+        finally:
+            ctx.__exit__(None, None, None)
+        out["cases"][name] = {"kind": kind, "mesh": list(mesh_sizes), **pack(records)}
+        print(name, len(records), "nodes,", sum(len(r[2]) for r in records), "strategies,",
+              len(out["cases"][name]["strategy_lists"]), "distinct lists,",
+              len(out["cases"][name]["cost_values_us"]), "distinct costs", flush=True)
+    path = os.path.join(HERE, "reference_compute_costs.json")
+    with open(path, "w") as f:
+        json.dump(out, f, separators=(",", ":"))
+    print(path, os.path.getsize(path), "bytes")
+
+
+if __name__ == "__main__":
+    main()

@@ -28,6 +28,7 @@ class OracleBackend:
         enc = self.tables.as_dict()
         compute, per_arg = c_oracle.compute_costs(enc, self.params)
         out = c_oracle.build_tables(enc, self.params, per_arg=per_arg)
+        out["compute"] = compute
         out["compute_per_arg"] = per_arg
         self.cost = out["cost"]
         return out

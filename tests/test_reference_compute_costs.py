@@ -1,0 +1,93 @@
+"""Compute-cost parity against vectors written by the reference itself.
+
+``tests/golden/reference_compute_costs.json`` holds, for every (node, strategy) of four traced
+graphs (the reference tests' FFN and transformer block on (32, 8); one decoder layer of
+Llama-3-8B on (32, 8) and of Llama-3-70B on (8, 8, 8), at the benchmark shapes), what the
+reference's ``estimate_strategy_runtime_cost`` (autoparallel/compute_estimation.py:334-365)
+returned for it: the operator run on fake tensors of the sharded shapes under torch's flop
+counter.  Here the same number comes from the shard-shape table, one shape-function run per
+distinct key, and the compute-cost kernel (CPU test: the oracle's restatement of the tail);
+equality is exact.  The graphs and strategy lists are this repository's own; the fixture stores
+them as the vectors' inputs and the test first checks that they are unchanged."""
+
+import json
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from autoparallel_amd.api import AutoParallelPlanner
+from autoparallel_amd.graphs import workloads
+from autoparallel_amd.optimize_sharding import ShardingOptimizer
+from models import make_model_and_inputs
+from oracle_backend import OracleBackend
+
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+from make_reference_vectors import node_signature, strategy_code  # noqa: E402  (pure helpers; imports no reference code)
+
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_compute_costs.json")) as f:
+    FIXTURE = json.load(f)
+
+
+class OracleOptimizer(ShardingOptimizer):
+    backend_cls = OracleBackend
+
+
+class OraclePlanner(AutoParallelPlanner):
+    optimizer_cls = OracleOptimizer
+
+
+def _planner(planner_cls, case):
+    kind, mesh_sizes = case["kind"], tuple(case["mesh"])
+    mesh = workloads.logical_mesh(mesh_sizes)
+    if kind.startswith("llama3"):
+        model, input_fn, _, _ = workloads.build_model(kind, mesh, n_layers=1)
+        # no reduce dtype: the gradient rescale does not touch compute costs
+        return planner_cls(model, input_fn, mesh, param_dtype=torch.bfloat16)
+    model_fn, input_fn = make_model_and_inputs(mesh, kind)
+    with torch.device("meta"):
+        model = model_fn()
+    return planner_cls(model, input_fn, mesh)
+
+
+def _check(planner_cls, name):
+    case = FIXTURE["cases"][name]
+    values = [float.fromhex(x) for x in case["cost_values_us"]]
+    with _planner(planner_cls, case) as p:
+        o = p.sharding_optimizer
+        assert (o.params.device_name, o.devices_per_host) == ("H100", 8) == \
+            (FIXTURE["environment"]["device_name"], FIXTURE["environment"]["devices_per_host"])
+        nodes = [n for n in o.graph.nodes if n.op != "output"]
+        assert len(nodes) == len(case["nodes"])
+        n_checked = n_positive = 0
+        for node, (want_name, sig_i, list_i, cost_is) in zip(nodes, case["nodes"]):
+            # the vectors' inputs: same node, operator, argument shapes and strategy list
+            assert node.name == want_name
+            assert node_signature(node) == case["signatures"][sig_i], node
+            strategies = o.strats[node].strategies
+            assert [strategy_code(s) for s in strategies] == case["strategy_lists"][list_i], node
+            # the vectors' outputs
+            begin = o.encoded.strat_begin[o.node_map[node]]
+            got = o.compute_cost[begin:begin + len(strategies)]
+            want = np.array([values[i] for i in cost_is])
+            assert np.array_equal(got, want), (node, got, want)
+            num_args = o.num_args[o.node_map[node]]
+            if num_args:  # optimize_sharding.py:371-373: each argument's entries carry compute / num_args
+                assert np.array_equal(o.compute_cost_per_arg[begin:begin + len(strategies)], want / num_args), node
+            n_checked += len(strategies)
+            n_positive += int((want > 0).sum())
+        assert n_checked == o.encoded.tables.n_strategies and n_positive > n_checked // 10  # views, placeholders and getitem cost nothing
+        return type(o.backend).__name__
+
+
+@pytest.mark.parametrize("name", list(FIXTURE["cases"]))
+def test_oracle_compute_costs_equal_the_reference_vectors(fake_pg, name):
+    assert _check(OraclePlanner, name) == "OracleBackend"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(FIXTURE["cases"]))
+def test_device_compute_costs_equal_the_reference_vectors(gpu_device, fake_pg, name):
+    assert _check(AutoParallelPlanner, name) == "DeviceBackend"
