@@ -55,6 +55,13 @@ class ApcTile(ctypes.Structure):
     ]
 
 
+class ApcRowMinima(ctypes.Structure):
+    _fields_ = [
+        ("edge_row_begin", ctypes.c_void_p), ("dup_row_begin", ctypes.c_void_p),
+        ("row_min", ctypes.c_void_p), ("row_argmin", ctypes.c_void_p),
+    ]
+
+
 EXPORTS = (
     "apc_version",
     "apc_last_error",
@@ -65,6 +72,8 @@ EXPORTS = (
     "apc_input_tables",
     "apc_redistribute_tables",
     "apc_build_tables",
+    "apc_redistribute_tables_row_min",
+    "apc_build_tables_row_min",
     "apc_segmented_min",
     "apc_strategy_bounds",
 )

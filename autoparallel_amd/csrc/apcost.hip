@@ -18,6 +18,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 #include "apcost.h"
 
@@ -453,6 +454,13 @@ struct TableArgs {
   const int8_t *dtype;
   const uint8_t *zero_cost;
   const int32_t *num_args;
+  // Row minima written by the tiles themselves (NULL: not wanted).  Matrix rows are numbered
+  // edge by edge (edge_row_begin[e] + consumer strategy); dup_row_begin[k] is the first row of
+  // the identical edge whose first entry is dup_entry_begin[k].
+  const int64_t *edge_row_begin;
+  const int64_t *dup_row_begin;
+  double *row_min_out;
+  int32_t *row_arg_out;
 };
 
 // Bytes and contiguity of tensor t: read from the tensor table, or (DERIVE) derived from its
@@ -519,8 +527,21 @@ struct ActionRows {
 };
 
 // Everything the entry loops need about one tile, in LDS.
-template <int M>
-struct TileStage {
+// What a tile that also takes its row minima keeps in LDS beside the rest (a launch that does
+// not want them is a different instantiation and does not pay for the space).
+struct RowMinStage {
+  int64_t dup_row[APC_TILE_MAX_DUPS];  // first matrix rows of the identical edges
+  // A row of at most 64 entries meets at most two of the 64-entry chunks the wavefronts
+  // walk.  Slot 0 takes the part that holds the row's first column, slot 1 the part that
+  // starts a chunk: one writer per slot, no atomics.
+  double rmin[2][APC_TILE_MAX_ROWS];
+  int rarg[2][APC_TILE_MAX_ROWS];
+  int64_t row_out;  // first matrix row of the tile's edge
+};
+struct NoRowMinStage {};
+
+template <int M, bool RM>
+struct TileStage : std::conditional_t<RM, RowMinStage, NoRowMinStage> {
   // term arrays: [0] zeros, [1] all-gather, [2] reduce-scatter, [3] all-reduce,
   // [4] all-to-all (= reduce-scatter shaped term x a2a_scale, :22-32), [5] read+write
   double terms[kLdsTermArrays * States<M>::kCount];
@@ -568,9 +589,9 @@ __device__ __forceinline__ double ring_at(double gb, const apc_params &p, int d,
 // computed from scalar operands while the loads are in flight: under a store-bound kernel
 // each dependent round of vector loads queues behind the stores of the other workgroups of
 // the compute unit, so the number of rounds, not of loads, is what staging costs.
-template <int M, bool DERIVE>
+template <int M, bool DERIVE, bool RM>
 __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs &a, const apc_tile &tile,
-                                           TileStage<M> &st, int tid, int nthreads) {
+                                           TileStage<M, RM> &st, int tid, int nthreads) {
   constexpr int NS = States<M>::kCount;
   constexpr int AW = ActionRows<M>::kWords;
   const int rows = tile.counts & 0xFFFF, cols = tile.counts >> 16;
@@ -609,6 +630,12 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   int64_t dup0 = 0, dup1 = 0;
   if (has_dup0) dup0 = a.dup_entry_begin[tile.dup_begin + tid];
   if (has_dup1) dup1 = a.dup_entry_begin[tile.dup_begin + tid + nthreads];
+  int64_t dup_row0 = 0, dup_row1 = 0, row_out = 0;
+  if constexpr (RM) {
+    if (has_dup0) dup_row0 = a.dup_row_begin[tile.dup_begin + tid];
+    if (has_dup1) dup_row1 = a.dup_row_begin[tile.dup_begin + tid + nthreads];
+    row_out = a.edge_row_begin[tile.edge];  // wave-uniform: a scalar load
+  }
   // the contiguity byte of the tile's tensor, read as the aligned word around it (which lies
   // in the byte's own page): a wave-uniform word goes through the scalar cache
   uint32_t contiguous = 1;
@@ -671,6 +698,12 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   if (tid == 0) st.cont = contiguous != 0;
   if (has_dup0) st.dup[tid] = dup0;
   if (has_dup1) st.dup[tid + nthreads] = dup1;
+  if constexpr (RM) {
+    if (has_dup0) st.dup_row[tid] = dup_row0;
+    if (has_dup1) st.dup_row[tid + nthreads] = dup_row1;
+    if (tid < APC_TILE_MAX_ROWS) st.rmin[1][tid] = __builtin_inf();  // (slot 0 of every row is always written)
+    if (tid == 0) st.row_out = row_out;
+  }
   if (has_col) {
     // info: bit0 valid spec, bit1 fully replicated, bits 4.. mask of sharded mesh dims
     uint32_t info = (col_tensor >= 0 ? 1u : 0u) | (col_codes == 0u ? 2u : 0u);
@@ -711,8 +744,8 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
 // One entry of a tile whose producer specs all name one tensor (column c, row r of the tile).
 // Straight-line code: all lookups of an entry are independent of its fp additions, so they
 // are issued together; no vector memory loads.
-template <int M, bool CONT, bool RESCALE>
-__device__ __forceinline__ void uniform_entry(const apc_params &p, const TileStage<M> &st, int r, int c,
+template <int M, bool CONT, bool RESCALE, bool RM>
+__device__ __forceinline__ void uniform_entry(const apc_params &p, const TileStage<M, RM> &st, int r, int c,
                                               double &comm_o, double &total_o, int &trans_o) {
   constexpr int NS = States<M>::kCount;
   const uint2 colv = st.colh[c];
@@ -804,10 +837,96 @@ __device__ __forceinline__ void store_entry(const TileOut &o, int dup_count, con
   }
 }
 
+// Row minima inside the tile kernel.  The 64 lanes of a wavefront hold 64 consecutive entries
+// of the tile (inactive lanes: +inf), row after row.  A segmented minimum by doubling leaves, in
+// the first lane of every run of one row, the minimum of the run and the first column that has
+// it; that lane writes the row's slot.  `c` is the lane's column, `cols` the row length.
+__device__ __forceinline__ void row_min_chunk(double (&rmin)[2][APC_TILE_MAX_ROWS], int (&rarg)[2][APC_TILE_MAX_ROWS],
+                                              bool active, double value, int r, int c, int cols, int lane) {
+  double m = active ? value : __builtin_inf();
+  int mc = c;
+  for (int off = 1; off < 64 && off < cols; off <<= 1) {  // (cols is wave-uniform)
+    const double om = __shfl_down(m, off, 64);
+    const int oc = __shfl_down(mc, off, 64);
+    // the lane `off` further on holds an entry of the same row (entries are consecutive)
+    if (lane + off < 64 && c + off < cols && om < m) {  // strict: ties keep the lower column
+      m = om;
+      mc = oc;
+    }
+  }
+  if (active && (c == 0 || lane == 0)) {
+    const int slot = c == 0 ? 0 : 1;
+    rmin[slot][r] = m;
+    rarg[slot][r] = mc;
+  }
+}
+
+// After every wavefront of the tile has written its slots: one thread per row joins the two
+// parts and stores minimum and first argmin to the row of the tile's edge and of every
+// identical edge.  (Called by every thread of the workgroup.)
+template <int M>
+__device__ __forceinline__ void row_min_finish(const TableArgs &a, TileStage<M, true> &st, const TileView &v, int tid) {
+  __syncthreads();
+  if (tid >= v.rows) return;
+  double m = st.rmin[0][tid];
+  int mc = st.rarg[0][tid];
+  const double m1 = st.rmin[1][tid];
+  if (m1 < m) {  // the later part wins only if strictly smaller
+    m = m1;
+    mc = st.rarg[1][tid];
+  }
+  const int64_t row = st.row_out + v.row_begin + tid;
+  a.row_min_out[row] = m;
+  a.row_arg_out[row] = v.col_begin + mc;
+  for (int d = 0; d < v.dup_count; ++d) {
+    const int64_t rd = st.dup_row[d] + v.row_begin + tid;
+    a.row_min_out[rd] = m;
+    a.row_arg_out[rd] = v.col_begin + mc;
+  }
+}
+
+// The entry loop of a tile that holds whole rows, with the row minima: the walk of
+// uniform_tile_entries, except that every lane of a wavefront makes the same number of
+// passes (a lane in front of the tile's first entry idles in the first pass instead of
+// wrapping round), so that the lanes of one pass hold consecutive entries.
+template <int M, bool CONT, bool RESCALE>
+__device__ __forceinline__ void uniform_tile_entries_row_min(const apc_params &p, const TableArgs &a, TileStage<M, true> &st,
+                                                             const TileView &v, int tid, int nthreads) {
+  const int n = v.rows * v.cols;
+  const int dr = nthreads / v.cols, dc = nthreads - dr * v.cols;
+  const int64_t tile_base = v.entry_begin + (int64_t)v.row_begin * v.n_src + v.col_begin;
+  const int shift = (int)(tile_base & 63);
+  const int lane = tid & 63;
+  int idx = tid - shift;
+  const int first = idx < 0 ? idx + nthreads : idx;
+  int r = first / v.cols, c = first - r * v.cols;
+  const TileOut out{a.comm_out + tile_base, a.trans_out + tile_base, a.cost_out + tile_base, v.entry_begin};
+  for (int wave_first = tid - lane - shift; wave_first < n; wave_first += nthreads, idx += nthreads) {
+    const bool active = idx >= 0 && idx < n;
+    double comm, total = 0.0;
+    int trans;
+    if (active) {
+      uniform_entry<M, CONT, RESCALE>(p, st, r, c, comm, total, trans);
+      store_entry<true>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
+                        trans);
+    }
+    row_min_chunk(st.rmin, st.rarg, active, total, r, c, v.cols, lane);
+    if (active) {
+      c += dc;
+      r += dr;
+      if (c >= v.cols) {
+        c -= v.cols;
+        r += 1;
+      }
+    }
+  }
+  row_min_finish<M>(a, st, v, tid);
+}
+
 // The per-entry loop of such a tile for `nthreads` threads (this one is `tid`): a flattened
 // (row, column) walk, so a wavefront writes 64 consecutive entries.
-template <int M, bool CONT, bool RESCALE, bool ALL>
-__device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M> &st,
+template <int M, bool CONT, bool RESCALE, bool ALL, bool RM>
+__device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M, RM> &st,
                                                      const TileView &v, int tid, int nthreads) {
   const int n = v.rows * v.cols;
   const int dr = nthreads / v.cols, dc = nthreads - dr * v.cols;
@@ -836,70 +955,97 @@ __device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const 
 }
 
 // Generic loop: pass-through edges and edges whose producer specs name different tensors.
-template <int M, bool DERIVE>
-__device__ __forceinline__ void generic_tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M> &st,
+// ROW_MIN (tiles of whole rows only): every lane of a wavefront makes the same number of
+// passes and the row minima are taken on the way.
+template <int M, bool DERIVE, bool ROW_MIN, bool RM>
+__device__ __forceinline__ void generic_tile_entries(const apc_params &p, const TableArgs &a, TileStage<M, RM> &st,
                                                      const TileView &v, int tid, int nthreads) {
   const int n = v.rows * v.cols;
+  const int lane = tid & 63;
   int r = tid / v.cols, c = tid - r * v.cols;
   const int dr = nthreads / v.cols, dc = nthreads - dr * v.cols;
   const bool no_producer = (v.flags & APC_EDGE_NO_PRODUCER) != 0;
-  for (int idx = tid; idx < n; idx += nthreads) {
-    const int64_t local = (int64_t)(v.row_begin + r) * v.n_src + (v.col_begin + c);
-    double comm;
-    int trans = 0;
-    const uint32_t src = st.colh[c].x, cinfo = st.colh[c].y;
-    const uint32_t tgt = st.row[r].x, tinfo = st.row[r].y;
-    if (no_producer || !(cinfo & tinfo & 1u)) {
-      comm = a.pt_values[v.pt_begin + local];
-    } else {
-      trans = (src != tgt) ? p.transition_scale : 0;
-      const int sten = a.spec_tensor[v.src_begin + v.col_begin + c];
-      int64_t shards = 1;
+  for (int idx = tid; ROW_MIN ? idx - lane < n : idx < n; idx += nthreads) {
+    const bool active = !ROW_MIN || idx < n;
+    double total = 0.0;
+    if (active) {
+      const int64_t local = (int64_t)(v.row_begin + r) * v.n_src + (v.col_begin + c);
+      double comm;
+      int trans = 0;
+      const uint32_t src = st.colh[c].x, cinfo = st.colh[c].y;
+      const uint32_t tgt = st.row[r].x, tinfo = st.row[r].y;
+      if (no_producer || !(cinfo & tinfo & 1u)) {
+        comm = a.pt_values[v.pt_begin + local];
+      } else {
+        trans = (src != tgt) ? p.transition_scale : 0;
+        const int sten = a.spec_tensor[v.src_begin + v.col_begin + c];
+        int64_t shards = 1;
 #pragma unroll
-      for (int i = 0; i < M; ++i)
-        if (kind_of((src >> (8 * i)) & 0xFF) == 2) shards *= p.mesh_size[i];
-      int64_t sten_bytes;
-      bool sten_contiguous;
-      tensor_info<DERIVE>(a, sten, sten_bytes, sten_contiguous);
-      const double gb = (double)sten_bytes / (double)shards / 1024 / 1024 / 1024;
-      comm = entry_cost<M>(src, tgt, gb, sten_contiguous, p);
+        for (int i = 0; i < M; ++i)
+          if (kind_of((src >> (8 * i)) & 0xFF) == 2) shards *= p.mesh_size[i];
+        int64_t sten_bytes;
+        bool sten_contiguous;
+        tensor_info<DERIVE>(a, sten, sten_bytes, sten_contiguous);
+        const double gb = (double)sten_bytes / (double)shards / 1024 / 1024 / 1024;
+        comm = entry_cost<M>(src, tgt, gb, sten_contiguous, p);
+      }
+      if (v.flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;
+      const int64_t o = v.entry_begin + local;
+      total = comm + st.cpa[r] + (double)trans;
+      if (a.comm_out) a.comm_out[o] = comm;
+      if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
+      if (a.cost_out) a.cost_out[o] = total;
+      for (int d = 0; d < v.dup_count; ++d) {
+        const int64_t od = o + (st.dup[d] - v.entry_begin);
+        if (a.comm_out) a.comm_out[od] = comm;
+        if (a.trans_out) a.trans_out[od] = (uint8_t)trans;
+        if (a.cost_out) a.cost_out[od] = total;
+      }
     }
-    if (v.flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;
-    const int64_t o = v.entry_begin + local;
-    const double total = comm + st.cpa[r] + (double)trans;
-    if (a.comm_out) a.comm_out[o] = comm;
-    if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
-    if (a.cost_out) a.cost_out[o] = total;
-    for (int d = 0; d < v.dup_count; ++d) {
-      const int64_t od = o + (st.dup[d] - v.entry_begin);
-      if (a.comm_out) a.comm_out[od] = comm;
-      if (a.trans_out) a.trans_out[od] = (uint8_t)trans;
-      if (a.cost_out) a.cost_out[od] = total;
-    }
-    c += dc;
-    r += dr;
-    if (c >= v.cols) {
-      c -= v.cols;
-      r += 1;
+    if constexpr (ROW_MIN && RM) row_min_chunk(st.rmin, st.rarg, active, total, r, c, v.cols, lane);
+    if (active) {
+      c += dc;
+      r += dr;
+      if (c >= v.cols) {
+        c -= v.cols;
+        r += 1;
+      }
     }
   }
+  if constexpr (ROW_MIN && RM) row_min_finish<M>(a, st, v, tid);
 }
 
-// All entries of a staged tile.
-template <int M, bool DERIVE>
-__device__ __forceinline__ void tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M> &st,
+// All entries of a staged tile.  Row minima are taken when the caller wants them and the tile
+// holds whole rows (which the host arranges for every tile of a table before asking).
+template <int M, bool DERIVE, bool RM>
+__device__ __forceinline__ void tile_entries(const apc_params &p, const TableArgs &a, TileStage<M, RM> &st,
                                              const TileView &v, int tid, int nthreads) {
   int mixed = st.mixed[0];
   for (int w = 1; w < nthreads / 64; ++w) mixed |= st.mixed[w];
+  const bool all = a.comm_out && a.trans_out && a.cost_out;
+  const bool row_minima = RM && all && v.cols == v.n_src;
   if (uniform_i32(mixed)) {
-    generic_tile_entries<M, DERIVE>(p, a, st, v, tid, nthreads);
+    if constexpr (RM) {
+      if (row_minima) {
+        generic_tile_entries<M, DERIVE, true>(p, a, st, v, tid, nthreads);
+        return;
+      }
+    }
+    generic_tile_entries<M, DERIVE, false>(p, a, st, v, tid, nthreads);
     return;
   }
   const bool rescale = (v.flags & APC_EDGE_GRAD_RESCALE) != 0;
-  const bool all = a.comm_out && a.trans_out && a.cost_out;
-#define APC_TILE_LOOP(CONT_, RESCALE_)                                               \
-  if (all) uniform_tile_entries<M, CONT_, RESCALE_, true>(p, a, st, v, tid, nthreads); \
-  else uniform_tile_entries<M, CONT_, RESCALE_, false>(p, a, st, v, tid, nthreads)
+#define APC_TILE_LOOP(CONT_, RESCALE_)                                                            \
+  do {                                                                                            \
+    if constexpr (RM) {                                                                           \
+      if (row_minima) {                                                                           \
+        uniform_tile_entries_row_min<M, CONT_, RESCALE_>(p, a, st, v, tid, nthreads);             \
+        break;                                                                                    \
+      }                                                                                           \
+    }                                                                                             \
+    if (all) uniform_tile_entries<M, CONT_, RESCALE_, true>(p, a, st, v, tid, nthreads);          \
+    else uniform_tile_entries<M, CONT_, RESCALE_, false>(p, a, st, v, tid, nthreads);             \
+  } while (0)
   if (uniform_i32(st.cont)) {
     if (rescale) { APC_TILE_LOOP(true, true); } else { APC_TILE_LOOP(true, false); }
   } else {
@@ -908,10 +1054,10 @@ __device__ __forceinline__ void tile_entries(const apc_params &p, const TableArg
 #undef APC_TILE_LOOP
 }
 
-template <int M, int kTileThreads>
+template <int M, int kTileThreads, bool RM>
 __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_params p, TableArgs a, int n_tiles,
                                                                           int xcd_shift) {
-  __shared__ TileStage<M> s_stage;
+  __shared__ TileStage<M, RM> s_stage;
   const int64_t tile_id = xcd_chunked_unit(xcd_shift);
   if (tile_id >= n_tiles) return;
   static_assert(kTileThreads == 64 || kTileThreads == 128 || kTileThreads == 256, "wavefronts per tile: 1, 2 or 4");
@@ -931,13 +1077,13 @@ __global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_pa
 // table workgroups use (TableArgs), so the values are the same bits.  One launch instead of
 // two spares a table of a few tens of MB one ramp-up and one drain of the chip, which at that
 // size are a third of each kernel.
-template <int M, int kThreads>
+template <int M, int kThreads, bool RM>
 __global__ __launch_bounds__(kThreads) void build_tables_kernel(apc_params p, TableArgs a, TensorTableArgs t,
                                                                 SpecTableArgs sp, ComputeCostArgs c, int n_tiles,
                                                                 int64_t tile_blocks, int64_t spec_blocks,
                                                                 int64_t tensor_blocks, int xcd_shift) {
   constexpr size_t kRowBytes = (size_t)kThreads * (APC_MAX_RANK + 1) * sizeof(int64_t);
-  constexpr size_t kLds = sizeof(TileStage<M>) > kRowBytes ? sizeof(TileStage<M>) : kRowBytes;
+  constexpr size_t kLds = sizeof(TileStage<M, RM>) > kRowBytes ? sizeof(TileStage<M, RM>) : kRowBytes;
   __shared__ __align__(16) unsigned char s_raw[kLds];
   static_assert(kThreads == 64 || kThreads == 128 || kThreads == 256, "wavefronts per workgroup: 1, 2 or 4");
   const int64_t b = blockIdx.x;
@@ -945,7 +1091,7 @@ __global__ __launch_bounds__(kThreads) void build_tables_kernel(apc_params p, Ta
     const int64_t per = tile_blocks >> xcd_shift;
     const int64_t tile_id = (b & ((1 << xcd_shift) - 1)) * per + (b >> xcd_shift);
     if (tile_id >= n_tiles) return;
-    TileStage<M> &stage = *reinterpret_cast<TileStage<M> *>(s_raw);
+    TileStage<M, RM> &stage = *reinterpret_cast<TileStage<M, RM> *>(s_raw);
     const apc_tile tile = a.tiles[tile_id];
     stage_tile<M, true>(p, a, tile, stage, threadIdx.x, kThreads);
     __syncthreads();
@@ -1276,12 +1422,27 @@ int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t 
   return check_launch("apc_input_tables");
 }
 
-int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes, const uint8_t *tensor_contiguous,
-                            const uint32_t *spec_codes, const int32_t *spec_tensor, const double *pt_values,
-                            const double *per_arg, int64_t n_tiles, const apc_tile *tiles,
-                            const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *trans_out,
-                            double *cost_out, void *stream) {
+}  // extern "C"
+
+// Row minima need all three outputs and, when some tile serves identical edges, their rows.
+static int check_row_minima(const apc_row_minima *rows, const double *comm_out, const uint8_t *trans_out,
+                            const double *cost_out, const int64_t *dup_entry_begin, const char *who) {
+  if (!rows) return 0;
+  if (!rows->edge_row_begin || !rows->row_min || !rows->row_argmin) return fail(-1, "%s: NULL row-minimum array", who);
+  if (dup_entry_begin && !rows->dup_row_begin) return fail(-1, "%s: identical edges need dup_row_begin", who);
+  if (!comm_out || !trans_out || !cost_out) return fail(-1, "%s: row minima need comm_out, transition_out and cost_out", who);
+  return 0;
+}
+
+static int redistribute_tables_impl(const apc_params *params, const int64_t *tensor_bytes,
+                                    const uint8_t *tensor_contiguous, const uint32_t *spec_codes,
+                                    const int32_t *spec_tensor, const double *pt_values, const double *per_arg,
+                                    int64_t n_tiles, const apc_tile *tiles, const int64_t *dup_entry_begin,
+                                    int64_t n_entries, double *comm_out, uint8_t *trans_out, double *cost_out,
+                                    const apc_row_minima *rows, void *stream) {
   if (int rc = check_params(params)) return rc;
+  if (int rc = check_row_minima(rows, comm_out, trans_out, cost_out, dup_entry_begin, "apc_redistribute_tables_row_min"))
+    return rc;
   if (n_tiles < 0 || n_tiles > (1 << 30)) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tiles == 0) return 0;
   if (n_entries < 0) return fail(-1, "n_entries < 0");
@@ -1290,7 +1451,9 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
   if (cost_out && !per_arg) return fail(-1, "cost_out needs compute_cost_per_arg");
   TableArgs a{tensor_bytes, tensor_contiguous, spec_codes, spec_tensor, pt_values, per_arg,
               tiles,        dup_entry_begin,   comm_out,   trans_out,   cost_out,
-              nullptr,      nullptr,           nullptr,    nullptr,     nullptr, nullptr, nullptr, nullptr, nullptr};
+              nullptr,      nullptr,           nullptr,    nullptr,     nullptr, nullptr, nullptr, nullptr, nullptr,
+              rows ? rows->edge_row_begin : nullptr, rows ? rows->dup_row_begin : nullptr,
+              rows ? rows->row_min : nullptr, rows ? rows->row_argmin : nullptr};
   const int nt = (int)n_tiles, xs = xcd_shift();
   hipStream_t s = (hipStream_t)stream;
   // Wavefronts per tile by the mean number of values a tile stores (n_entries counts the
@@ -1301,21 +1464,24 @@ int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_byte
   const int64_t per_tile = n_entries / n_tiles;
   int threads = per_tile >= 1536 ? 256 : per_tile >= 512 ? 128 : 64;
   if (const char *env = getenv("APC_TILE_THREADS")) threads = atoi(env);  // tuning override
-#define APC_LAUNCH(M_)                                                                                         \
-  if (threads >= 256) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 256>), grid, dim3(256), 0, s, *params, a, nt, xs); \
-  else if (threads >= 128) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 128>), grid, dim3(128), 0, s, *params, a, nt, xs); \
-  else hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 64>), grid, dim3(64), 0, s, *params, a, nt, xs)
+#define APC_LAUNCH_RM(M_, RM_)                                                                                  \
+  if (threads >= 256) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 256, RM_>), grid, dim3(256), 0, s, *params, a, nt, xs); \
+  else if (threads >= 128) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 128, RM_>), grid, dim3(128), 0, s, *params, a, nt, xs); \
+  else hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 64, RM_>), grid, dim3(64), 0, s, *params, a, nt, xs)
+#define APC_LAUNCH(M_)                        \
+  if (rows) { APC_LAUNCH_RM(M_, true); } else { APC_LAUNCH_RM(M_, false); }
   switch (params->mesh_ndim) {
     case 1: APC_LAUNCH(1); break;
     case 2: APC_LAUNCH(2); break;
     case 3: APC_LAUNCH(3); break;
     default: APC_LAUNCH(4); break;
   }
+#undef APC_LAUNCH_RM
 #undef APC_LAUNCH
   return check_launch("apc_redistribute_tables");
 }
 
-int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t *rank, const int32_t *itemsize,
+static int build_tables_impl(const apc_params *params, int64_t n_tensors, const int32_t *rank, const int32_t *itemsize,
                      const int64_t *shape, const int64_t *stride, int64_t *tensor_bytes, uint8_t *tensor_contiguous,
                      int64_t n_specs, const uint32_t *spec_codes, const int32_t *spec_tensor, int64_t *num_shards,
                      int64_t *local_shape, int64_t *local_stride, int32_t shape_width, int64_t *local_numel,
@@ -1323,8 +1489,9 @@ int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t 
                      const int8_t *dtype, const uint8_t *zero_cost, const int32_t *num_args, double *compute,
                      double *per_arg, int32_t *error_flag, const double *pt_values, int64_t n_tiles, const apc_tile *tiles,
                      const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *trans_out,
-                     double *cost_out, void *stream) {
+                     double *cost_out, const apc_row_minima *rows, void *stream) {
   if (int rc = check_params(params)) return rc;
+  if (int rc = check_row_minima(rows, comm_out, trans_out, cost_out, dup_entry_begin, "apc_build_tables_row_min")) return rc;
   if (n_tensors < 0 || n_specs < 0 || n_strategies < 0 || n_entries < 0) return fail(-1, "apc_build_tables: negative count");
   if (n_tiles < 0 || n_tiles > (1 << 30)) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tensors > 0 && (!rank || !itemsize || !shape || !stride || !tensor_bytes || !tensor_contiguous))
@@ -1355,7 +1522,9 @@ int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t 
   if (blocks > INT32_MAX) return fail(-1, "apc_build_tables: too many rows for one launch");
   // the tiles read neither the tensor table nor the compute costs (written by this launch)
   TableArgs a{nullptr, nullptr, spec_codes, spec_tensor, pt_values, nullptr, tiles, dup_entry_begin,
-              comm_out, trans_out, cost_out, rank, itemsize, shape, stride, flops, rw_bytes, dtype, zero_cost, num_args};
+              comm_out, trans_out, cost_out, rank, itemsize, shape, stride, flops, rw_bytes, dtype, zero_cost, num_args,
+              rows ? rows->edge_row_begin : nullptr, rows ? rows->dup_row_begin : nullptr,
+              rows ? rows->row_min : nullptr, rows ? rows->row_argmin : nullptr};
   const TensorTableArgs ta{n_tensors, rank, itemsize, shape, stride, tensor_bytes, tensor_contiguous};
   const SpecTableArgs sa{n_specs, spec_codes, spec_tensor, rank, itemsize, shape, stride, num_shards,
                          local_shape, local_stride, local_numel, local_bytes, shape_width};
@@ -1363,19 +1532,71 @@ int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t 
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)blocks);
   const int nt = (int)n_tiles;
-#define APC_LAUNCH_ALL(M_)                                                                                              \
-  if (threads == 256) hipLaunchKernelGGL((build_tables_kernel<M_, 256>), grid, dim3(256), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
-  else if (threads == 128) hipLaunchKernelGGL((build_tables_kernel<M_, 128>), grid, dim3(128), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
-  else hipLaunchKernelGGL((build_tables_kernel<M_, 64>), grid, dim3(64), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs)
+#define APC_LAUNCH_ALL_RM(M_, RM_)                                                                                      \
+  if (threads == 256) hipLaunchKernelGGL((build_tables_kernel<M_, 256, RM_>), grid, dim3(256), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
+  else if (threads == 128) hipLaunchKernelGGL((build_tables_kernel<M_, 128, RM_>), grid, dim3(128), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
+  else hipLaunchKernelGGL((build_tables_kernel<M_, 64, RM_>), grid, dim3(64), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs)
+#define APC_LAUNCH_ALL(M_)                    \
+  if (rows) { APC_LAUNCH_ALL_RM(M_, true); } else { APC_LAUNCH_ALL_RM(M_, false); }
   switch (params->mesh_ndim) {
     case 1: APC_LAUNCH_ALL(1); break;
     case 2: APC_LAUNCH_ALL(2); break;
     case 3: APC_LAUNCH_ALL(3); break;
     default: APC_LAUNCH_ALL(4); break;
   }
+#undef APC_LAUNCH_ALL_RM
 #undef APC_LAUNCH_ALL
   return check_launch("apc_build_tables");
 }
+
+extern "C" {
+
+int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes, const uint8_t *tensor_contiguous,
+                            const uint32_t *spec_codes, const int32_t *spec_tensor, const double *pt_values,
+                            const double *per_arg, int64_t n_tiles, const apc_tile *tiles,
+                            const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *trans_out,
+                            double *cost_out, void *stream) {
+  return redistribute_tables_impl(params, tensor_bytes, tensor_contiguous, spec_codes, spec_tensor, pt_values, per_arg,
+                                  n_tiles, tiles, dup_entry_begin, n_entries, comm_out, trans_out, cost_out, nullptr,
+                                  stream);
+}
+
+int apc_redistribute_tables_row_min(const apc_params *params, const int64_t *tensor_bytes,
+                                    const uint8_t *tensor_contiguous, const uint32_t *spec_codes,
+                                    const int32_t *spec_tensor, const double *pt_values, const double *per_arg,
+                                    int64_t n_tiles, const apc_tile *tiles, const int64_t *dup_entry_begin,
+                                    int64_t n_entries, double *comm_out, uint8_t *trans_out, double *cost_out,
+                                    const apc_row_minima *rows, void *stream) {
+  if (!rows) return fail(-1, "apc_redistribute_tables_row_min: NULL rows");
+  return redistribute_tables_impl(params, tensor_bytes, tensor_contiguous, spec_codes, spec_tensor, pt_values, per_arg,
+                                  n_tiles, tiles, dup_entry_begin, n_entries, comm_out, trans_out, cost_out, rows, stream);
+}
+
+#define APC_BUILD_TABLES_PARAMS                                                                                         \
+  const apc_params *params, int64_t n_tensors, const int32_t *rank, const int32_t *itemsize, const int64_t *shape,      \
+      const int64_t *stride, int64_t *tensor_bytes, uint8_t *tensor_contiguous, int64_t n_specs,                        \
+      const uint32_t *spec_codes, const int32_t *spec_tensor, int64_t *num_shards, int64_t *local_shape,                \
+      int64_t *local_stride, int32_t shape_width, int64_t *local_numel, int64_t *local_bytes, int64_t n_strategies,     \
+      const int64_t *flops, const int64_t *rw_bytes, const int8_t *dtype, const uint8_t *zero_cost,                     \
+      const int32_t *num_args, double *compute, double *per_arg, int32_t *error_flag, const double *pt_values,          \
+      int64_t n_tiles, const apc_tile *tiles, const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out,      \
+      uint8_t *trans_out, double *cost_out
+#define APC_BUILD_TABLES_ARGS                                                                                           \
+  params, n_tensors, rank, itemsize, shape, stride, tensor_bytes, tensor_contiguous, n_specs, spec_codes, spec_tensor,  \
+      num_shards, local_shape, local_stride, shape_width, local_numel, local_bytes, n_strategies, flops, rw_bytes,      \
+      dtype, zero_cost, num_args, compute, per_arg, error_flag, pt_values, n_tiles, tiles, dup_entry_begin, n_entries,  \
+      comm_out, trans_out, cost_out
+
+int apc_build_tables(APC_BUILD_TABLES_PARAMS, void *stream) {
+  return build_tables_impl(APC_BUILD_TABLES_ARGS, nullptr, stream);
+}
+
+int apc_build_tables_row_min(APC_BUILD_TABLES_PARAMS, const apc_row_minima *rows, void *stream) {
+  if (!rows) return fail(-1, "apc_build_tables_row_min: NULL rows");
+  return build_tables_impl(APC_BUILD_TABLES_ARGS, rows, stream);
+}
+#undef APC_BUILD_TABLES_PARAMS
+#undef APC_BUILD_TABLES_ARGS
 
 int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_seg, int64_t n_values, double *mins,
                       int32_t *args, void *stream) {

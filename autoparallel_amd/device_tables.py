@@ -23,6 +23,7 @@ _UPLOAD = (
     "strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "strat_num_args",
     "edge_src_begin", "edge_n_src", "edge_tgt_begin", "edge_n_tgt", "edge_flags", "edge_pt_begin",
     "edge_entry_begin", "edge_strat_begin", "pt_values", "tile_records", "dup_entry_begin",
+    "dup_row_begin",
 )
 
 
@@ -76,6 +77,8 @@ class DeviceCostTables:
         self.comm = None
         self.transition = None
         self.cost = None
+        self.row_min = None  # minima / first argmins of the rows of ``cost``, when a table launch took them
+        self.row_argmin = None
 
     @_guarded
     def refresh(self, *names):
@@ -159,26 +162,43 @@ class DeviceCostTables:
         self.cost = self._empty((n,), torch.float64) if cost else None
 
     @_guarded
-    def launch_redistribute_tables(self):
+    def launch_redistribute_tables(self, row_min=False):
         """One enqueue of the table kernel over pre-allocated outputs (no allocation,
-        no synchronisation): the timed unit of the benchmark."""
-        with torch.cuda.device(self.device):
-            rc = self.lib.apc_redistribute_tables(
-                ctypes.byref(self.c_params), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
+        no synchronisation).  ``row_min``: the launch also writes ``row_min`` / ``row_argmin``
+        (allocated by ``run_redistribute_tables``)."""
+        args = (ctypes.byref(self.c_params), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
                 self._p("spec_codes"), self._p("spec_tensor"), self._p("pt_values"),
                 self._p(self.compute_cost_per_arg), ctypes.c_int64(self.tables.n_tiles), self._p("tile_records"),
-                self._p("dup_entry_begin"), ctypes.c_int64(self.tables.n_entries), self._p(self.comm), self._p(self.transition),
-                self._p(self.cost), self._stream())
+                self._p("dup_entry_begin"), ctypes.c_int64(self.tables.n_entries), self._p(self.comm),
+                self._p(self.transition), self._p(self.cost))
+        with torch.cuda.device(self.device):
+            if row_min:
+                edge_row_begin = _to_device(self.tables.edge_row_begin(), self.device)
+                rows = _native.ApcRowMinima(self._p(edge_row_begin), self._p("dup_row_begin"), self._p(self.row_min),
+                                            self._p(self.row_argmin))
+                rc = self.lib.apc_redistribute_tables_row_min(*args, ctypes.byref(rows), self._stream())
+                self._rows_keepalive = (edge_row_begin, rows)  # until the stream has run the launch
+            else:
+                rc = self.lib.apc_redistribute_tables(*args, self._stream())
         _native.check(rc, "apc_redistribute_tables")
 
     @_guarded
-    def run_redistribute_tables(self, comm=True, transition=True, cost=True):
+    def run_redistribute_tables(self, comm=True, transition=True, cost=True, row_min=None):
+        """``row_min``: also take the row minima of ``cost`` in the same launch (``None``: when all
+        three outputs are wanted and ``row_min_in_tiles_pays``)."""
         if self.tensor_bytes is None:
             self.run_tensor_tables()
         if cost and self.compute_cost_per_arg is None:
             self.run_compute_costs()
         self.alloc_outputs(comm, transition, cost)
-        self.launch_redistribute_tables()
+        if row_min is None:
+            row_min = bool(comm and transition and cost) and self.row_min_in_tiles_pays()
+        self.row_min = self.row_argmin = None
+        if row_min:
+            n_rows = int(self.tables.edge_n_tgt.astype(np.int64).sum())
+            self.row_min = self._empty((n_rows,), torch.float64)
+            self.row_argmin = self._empty((n_rows,), torch.int32)
+        self.launch_redistribute_tables(row_min=bool(row_min))
         return self.comm, self.transition, self.cost
 
     @_guarded
@@ -195,17 +215,40 @@ class DeviceCostTables:
     # more than a launch (measured crossover between 90 MB and 170 MB of tables).
     ONE_LAUNCH_MAX_BYTES = 128 << 20
 
+    def row_min_in_tiles_pays(self) -> bool:
+        """Whether the launch that writes the cost matrices should take the row minima itself.
+        Inside the tiles the minima cost arithmetic in the store loop, about 4.1 ps per entry a
+        tile computes (identical edges are computed, and reduced, once for all their copies); a
+        ``segmented_min`` launch costs about 4 us plus reading every stored entry back at about
+        4.5 TB/s.  Measured per pass, in tiles / separate: Llama-3-8B on (32, 8) 18.8 / 23.9 us
+        (33.4 / 31.7 us when every identical edge is computed on its own), the mixture of experts
+        15.7 / 17.7 us, the 464 M-entry stress table 3.77 / 3.37 ms."""
+        tb = self.tables
+        if not tb.rows_fit_tiles():
+            return False
+        computed = int((tb.tile_row_count.astype(np.int64) * tb.tile_col_count.astype(np.int64)).sum())
+        return computed * 4.1e-6 < 4.0 + 8.0 * tb.n_entries / 4.5e6
+
     @_guarded
-    def prepare_step(self, row_min=True, fused_inputs=False, one_launch=None):
+    def prepare_step(self, row_min=True, fused_inputs=False, one_launch=None, row_min_in_tiles=None):
         """Allocates every output once and returns ``{kernel name: zero-argument launcher}``
         in launch order.  A launcher only enqueues (no allocation, no synchronisation), so a
         timed loop measures the kernels and not Python argument marshalling.  With
         ``fused_inputs`` the tensor, spec and compute-cost tables are one launch
         (``input_tables``) instead of three; with ``one_launch`` they and the cost matrices
         are one (``build_tables``); ``one_launch=None`` takes one launch for tables up to
-        ``ONE_LAUNCH_MAX_BYTES`` when ``fused_inputs`` is set."""
+        ``ONE_LAUNCH_MAX_BYTES`` when ``fused_inputs`` is set.  ``row_min_in_tiles``: the launch
+        that writes the cost matrices takes the row minima too (no ``segmented_min`` launch, no
+        second read of the matrices); it needs every row inside one tile
+        (``CostTables.rows_fit_tiles``), and ``None`` takes it when ``row_min_in_tiles_pays``."""
+        fits = self.tables.rows_fit_tiles()
+        total = self.tables.algorithmic_bytes() + self.tables.algorithmic_bytes_input_tables()
+        if row_min_in_tiles is None:
+            row_min_in_tiles = self.row_min_in_tiles_pays()
+        row_min_in_tiles = bool(row_min_in_tiles) and bool(row_min)
+        if row_min_in_tiles and not fits:
+            raise ValueError("row minima inside the table launch need every matrix row inside one tile")
         if one_launch is None:
-            total = self.tables.algorithmic_bytes() + self.tables.algorithmic_bytes_input_tables()
             one_launch = bool(fused_inputs) and total <= self.ONE_LAUNCH_MAX_BYTES
         self.run_tensor_tables()
         spec = self.run_spec_tables()
@@ -238,10 +281,26 @@ class DeviceCostTables:
                     _native.check(rc, what)
             return launch
 
+        rows_arg = ()
+        if row_min:
+            n_rows = int(tb.edge_n_tgt.astype(np.int64).sum())
+            self.row_min = self._empty((n_rows,), torch.float64)
+            self.row_argmin = self._empty((n_rows,), torch.int32)
+        if row_min_in_tiles:
+            edge_row_begin = _to_device(tb.edge_row_begin(), self.device)
+            self._step_keepalive.append(edge_row_begin)
+            rows = _native.ApcRowMinima(P(edge_row_begin), P("dup_row_begin"), P(self.row_min), P(self.row_argmin))
+            self._step_keepalive.append(rows)
+            rows_arg = (ctypes.byref(rows),)
+        table_fn = (lib.apc_redistribute_tables_row_min, "apc_redistribute_tables_row_min") if row_min_in_tiles \
+            else (lib.apc_redistribute_tables, "apc_redistribute_tables")
+        all_fn = (lib.apc_build_tables_row_min, "apc_build_tables_row_min") if row_min_in_tiles \
+            else (lib.apc_build_tables, "apc_build_tables")
+        a_tables = a_tables[:-1] + rows_arg + (stream,)
         if one_launch:
             a_all = (cp,) + a_tensor[:-1] + (a_spec[1], a_spec[2], a_spec[3]) + a_spec[8:-1] + a_compute[1:-1] + \
                 (a_tables[5],) + a_tables[7:]
-            step = {"build_tables": bind(lib.apc_build_tables, a_all, "apc_build_tables")}
+            step = {"build_tables": bind(all_fn[0], a_all, all_fn[1])}
         elif fused_inputs:
             a_inputs = (cp,) + a_tensor[:-1] + (a_spec[1], a_spec[2], a_spec[3]) + a_spec[8:-1] + a_compute[1:]
             step = {"input_tables": bind(lib.apc_input_tables, a_inputs, "apc_input_tables")}
@@ -252,12 +311,11 @@ class DeviceCostTables:
                 "compute_costs": bind(lib.apc_compute_costs, a_compute, "apc_compute_costs"),
             }
         if not one_launch:
-            step["redistribute_tables"] = bind(lib.apc_redistribute_tables, a_tables, "apc_redistribute_tables")
-        if row_min:
+            step["redistribute_tables"] = bind(table_fn[0], a_tables, table_fn[1])
+        if row_min and not row_min_in_tiles:
             row_ptr = torch.from_numpy(tb.row_ptr()).to(self.device)
             n_seg = row_ptr.numel() - 1
-            self.row_min = self._empty((n_seg,), torch.float64)
-            self.row_argmin = self._empty((n_seg,), torch.int32)
+            assert n_seg == self.row_min.numel()
             self._step_keepalive.append(row_ptr)
             a_min = (P(self.cost), P(row_ptr), ctypes.c_int64(n_seg), ctypes.c_int64(tb.n_entries), P(self.row_min),
                      P(self.row_argmin), stream)

@@ -143,6 +143,7 @@ class CostTables:
     tile_records: np.ndarray = None
     edge_canonical: np.ndarray = None  # edge -> the identical edge that is tiled (itself unless de-duplicated)
     dup_entry_begin: np.ndarray = None  # entry offsets of the duplicates, grouped by canonical edge
+    dup_row_begin: np.ndarray = None  # their first matrix rows (rows numbered as in ``row_ptr()``)
     edge_dup_begin: np.ndarray = None
     edge_dup_count: np.ndarray = None
     tiling: dict = None  # tile size and copies per tiled edge of the current tiling
@@ -298,6 +299,7 @@ class CostTables:
         order = np.argsort(canonical[dup_edges], kind="stable")
         dup_edges = dup_edges[order]
         self.dup_entry_begin = _i64(self.edge_entry_begin[:-1][dup_edges]) if self.n_edges else _i64([])
+        self.dup_row_begin = _i64(self.edge_row_begin()[dup_edges]) if self.n_edges else _i64([])
         self.edge_dup_count = np.bincount(canonical[dup_edges], minlength=self.n_edges).astype(np.int64)
         self.edge_dup_begin = np.cumsum(self.edge_dup_count) - self.edge_dup_count
         live = (ns > 0) & (nt > 0) & ~is_dup
@@ -331,6 +333,7 @@ class CostTables:
         if self.edge_canonical is None or len(self.edge_canonical) != self.n_edges:
             self.edge_canonical = np.arange(self.n_edges, dtype=np.int64)
             self.dup_entry_begin = _i64([])
+            self.dup_row_begin = _i64([])
             self.edge_dup_count = np.zeros(self.n_edges, np.int64)
             self.edge_dup_begin = np.zeros(self.n_edges, np.int64)
         rec = np.zeros(len(te), TILE_DTYPE)
@@ -439,6 +442,23 @@ class CostTables:
             "edges_by_node": _i32(order),
             "edge_row_begin": _i64(edge_row_begin),
         }
+
+    def edge_row_begin(self) -> np.ndarray:
+        """First matrix row of every edge: rows are numbered edge by edge, one per consumer
+        strategy (the order of ``row_ptr()``)."""
+        nt = self.edge_n_tgt.astype(np.int64)
+        return _i64(np.cumsum(nt) - nt)
+
+    def rows_fit_tiles(self) -> bool:
+        """Every matrix row lies inside one tile (and none is empty), so the launch that writes
+        the cost matrices can take the row minima itself."""
+        ns = self.edge_n_src.astype(np.int64)
+        nt = self.edge_n_tgt.astype(np.int64)
+        with_rows = nt > 0
+        if not bool(((ns[with_rows] >= 1) & (ns[with_rows] <= APC_TILE_MAX_COLS)).all()):
+            return False
+        te = self.tile_edge.astype(np.int64)
+        return bool((self.tile_col_begin == 0).all() and (self.tile_col_count == ns[te]).all())
 
     def row_ptr(self) -> np.ndarray:
         """CSR pointer of matrix rows over the entry array: one segment per

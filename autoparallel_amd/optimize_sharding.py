@@ -67,7 +67,7 @@ class DeviceBackend:
         tables.build_tiles(tile_entries, dedupe=dedupe, max_copies=max_copies)
         tables.validate(self.dev.params)
         self.dev.refresh("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "tile_records",
-                         "dup_entry_begin")
+                         "dup_entry_begin", "dup_row_begin")
 
     def build(self):
         from .device_tables import _real_tensors
@@ -98,15 +98,25 @@ class DeviceBackend:
         from .device_tables import _real_tensors
 
         with _real_tensors():
+            if self._are_matrix_rows(row_ptr):  # the table launch already took them
+                return self.dev.row_min.cpu().numpy(), self.dev.row_argmin.cpu().numpy()
             mins, args = self.dev.segmented_min(self.dev.cost, row_ptr)
             return mins.cpu().numpy(), args.cpu().numpy()
+
+    def _are_matrix_rows(self, row_ptr) -> bool:
+        d = self.dev
+        return d.row_min is not None and len(row_ptr) == d.row_min.numel() + 1 and \
+            np.array_equal(row_ptr, d.tables.row_ptr())
 
     def greedy(self, row_ptr):
         """-> (bound per strategy, min per node, argmin per node) from the row minima of the cost table"""
         from .device_tables import _real_tensors
 
         with _real_tensors():
-            mins, _ = self.dev.segmented_min(self.dev.cost, row_ptr)
+            if self._are_matrix_rows(row_ptr):
+                mins = self.dev.row_min
+            else:
+                mins, _ = self.dev.segmented_min(self.dev.cost, row_ptr)
             return tuple(x.cpu().numpy() for x in self.dev.greedy_strategies(mins))
 
 

@@ -60,6 +60,10 @@ def parse_args():
                     help="launches that build the tables of a pass: 1 = everything in one (apc_build_tables), "
                          "2 = input tables, then cost matrices, 4 = tensor, spec and compute-cost tables on their own "
                          "(default: 1 for tables up to 128 MiB, else 2)")
+    ap.add_argument("--row-min", choices=["auto", "tiles", "separate"], default="auto",
+                    help="where the row minima of a pass are taken: by the launch that writes the cost matrices "
+                         "(tiles), by a segmented_min launch that reads them back (separate); auto = tiles whenever "
+                         "every matrix row lies inside one tile")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy three times (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -218,7 +222,9 @@ def main():
         dev = DeviceCostTables(tables, params, device="cuda:0")
     log.info("tables resident: %d entries, %d tiles", tables.n_entries, tables.n_tiles)
     step = dev.prepare_step(row_min=True, fused_inputs=args.table_launches != 4,
-                            one_launch=None if args.table_launches is None else args.table_launches == 1)
+                            one_launch=None if args.table_launches is None else args.table_launches == 1,
+                            row_min_in_tiles={"auto": None, "tiles": True, "separate": False}[args.row_min])
+    row_min_in_tiles = "segmented_min" not in step
     args.table_launches = 1 if "build_tables" in step else 2 if "input_tables" in step else 4
     torch.cuda.synchronize()
     host_timings["upload_and_prepare_s"] = time.perf_counter() - t0
@@ -270,6 +276,9 @@ def main():
     alg_bytes = tables.algorithmic_bytes(comm=True, transition=True, cost=True)
     if args.table_launches == 1:
         alg_bytes += tables.algorithmic_bytes_input_tables()
+    n_rows = int(tables.edge_n_tgt.astype(np.int64).sum())
+    if row_min_in_tiles:
+        alg_bytes += 12 * n_rows  # minimum f64 + argmin i32 per matrix row, written by the same launch
     t_kernel = kernel_ms[main] * 1e-3
     achieved = alg_bytes / t_kernel / 1e9
     ms_per_step = wall_plain / K * 1e3
@@ -294,7 +303,9 @@ def main():
                             2: "input_tables(tensor + spec + compute-cost tables, one launch) + "
                                "redistribute_tables(comm, transition, cost)",
                             4: "tensor_tables + spec_tables + compute_costs + redistribute_tables(comm, transition, cost)"
-                            }[args.table_launches] + " + segmented_min(rows)"},
+                            }[args.table_launches] +
+                           (", row minima taken by that launch" if row_min_in_tiles else " + segmented_min(rows)"),
+                   "matrix_rows": n_rows},
         "roofline": {"bound": "hbm", "kernel": "build_tables_kernel" if args.table_launches == 1 else "redistribute_tiles_kernel",
                      "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
@@ -302,6 +313,7 @@ def main():
                      "algorithmic_bytes_input_tables": tables.algorithmic_bytes_input_tables() if args.table_launches == 1 else 0,
                      "algorithmic_bytes_per_launch": alg_bytes,
                      "bytes_written_per_entry": {"comm_f64": 8, "transition_u8": 1, "cost_f64": 8},
+                     "bytes_written_per_matrix_row": 12 if row_min_in_tiles else 0,
                      "avg_launch_us": t_kernel * 1e6, "min_launch_us": kernel_ms_min[main] * 1e3,
                      "timing": "HIP events around every launch of the kernel inside the timed region"},
         "kernel_us": {k: v * 1e3 for k, v in kernel_ms.items()},

@@ -204,6 +204,46 @@ int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t 
                      const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *transition_out,
                      double *cost_out, void *stream);
 
+/* Row minima taken by the launch that writes the cost matrices: for every matrix row (edge,
+ * consumer strategy) the minimum of cost_out over the producer strategies and the first
+ * column that has it, i.e. what apc_segmented_min gives over the rows of cost_out, without
+ * reading the matrices again (and once per tiled edge, not once per identical copy).
+ * Rows are numbered edge by edge: row = edge_row_begin[edge] + consumer strategy.
+ * dup_row_begin[k] is the first row of the identical edge whose first entry is
+ * dup_entry_begin[k] (NULL when dup_entry_begin is).
+ * Precondition, for the caller to check: every edge with rows has between 1 and
+ * APC_TILE_MAX_COLS producer strategies and every tile holds whole rows (col_begin = 0,
+ * col_count = n_src); rows of tiles that do not are left unwritten.
+ * No counterpart in the reference (see apc_segmented_min). */
+typedef struct apc_row_minima {
+  const int64_t *edge_row_begin; /* [n_edges] */
+  const int64_t *dup_row_begin;  /* parallel to dup_entry_begin */
+  double *row_min;               /* [n_rows] */
+  int32_t *row_argmin;           /* [n_rows] */
+} apc_row_minima;
+
+/* apc_redistribute_tables with the row minima; all three outputs are required. */
+int apc_redistribute_tables_row_min(const apc_params *params, const int64_t *tensor_bytes,
+                                    const uint8_t *tensor_contiguous, const uint32_t *spec_codes,
+                                    const int32_t *spec_tensor, const double *pt_values,
+                                    const double *compute_cost_per_arg, int64_t n_tiles, const apc_tile *tiles,
+                                    const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out,
+                                    uint8_t *transition_out, double *cost_out, const apc_row_minima *rows,
+                                    void *stream);
+
+/* apc_build_tables with the row minima; all three outputs are required. */
+int apc_build_tables_row_min(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
+                             const int32_t *tensor_itemsize, const int64_t *tensor_shape,
+                             const int64_t *tensor_stride, int64_t *tensor_bytes, uint8_t *tensor_contiguous,
+                             int64_t n_specs, const uint32_t *spec_codes, const int32_t *spec_tensor,
+                             int64_t *num_shards, int64_t *local_shape, int64_t *local_stride, int32_t shape_width,
+                             int64_t *local_numel, int64_t *local_bytes, int64_t n_strategies, const int64_t *flops,
+                             const int64_t *rw_bytes, const int8_t *dtype_code, const uint8_t *zero_cost,
+                             const int32_t *num_args, double *compute_cost, double *compute_cost_per_arg,
+                             int32_t *error_flag, const double *pt_values, int64_t n_tiles, const apc_tile *tiles,
+                             const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out,
+                             uint8_t *transition_out, double *cost_out, const apc_row_minima *rows, void *stream);
+
 /* Segmented minimum with first-argmin (relative to the segment start); empty
  * segments give (+inf, -1).  No counterpart in the reference (which hands the full
  * table to the ILP solver, optimize_sharding.py:648-659): used for pruning and

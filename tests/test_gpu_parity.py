@@ -297,6 +297,11 @@ def test_row_min_of_cost_tables(gpu_device):
     mins, args = d.segmented_min(d.cost, rp)
     wm, wa = c_oracle.segmented_min(want["cost"], rp)
     assert np.array_equal(mins.cpu().numpy(), wm) and np.array_equal(args.cpu().numpy(), wa)
+    # a table this small has its row minima taken by the launch that wrote the matrices
+    assert d.row_min_in_tiles_pays() and d.row_min is not None
+    assert np.array_equal(d.row_min.cpu().numpy(), wm) and np.array_equal(d.row_argmin.cpu().numpy(), wa)
+    d.run_redistribute_tables(row_min=False)
+    assert d.row_min is None
 
 
 @pytest.mark.parametrize("mesh", [(32, 8), (16, 8, 4)])
@@ -361,15 +366,17 @@ def test_full_size_stress_properties(gpu_device):
     assert bool((cost[: seg_of_entry.numel()] >= mins[seg_of_entry]).all())
 
 
-@pytest.mark.parametrize("launches", [5, 2])
+@pytest.mark.parametrize("launches", [5, 2, 1])
 def test_graph_replay_of_one_pass_matches_eager(gpu_device, launches):
     """One pass recorded as a HIP graph (five launches with the independent kernels on parallel
-    branches, or the one-launch build + row minima) gives the eager results on every replay,
-    with eager work and synchronisations between replays."""
+    branches, the one-launch build + row minima, or the one launch that takes the row minima
+    too) gives the eager results on every replay, with eager work and synchronisations between
+    replays."""
     mesh = (8, 4, 2)
     tb = stress_dag(seed=5, n_nodes=3000, mesh_sizes=mesh, frac_nonspec_nodes=0.02, frac_noncontiguous=0.2)
     d = DeviceCostTables(tb, CostModelParams.from_mesh(mesh, rescale=2.2), device=gpu_device)
-    step = d.prepare_step(row_min=True, fused_inputs=launches == 2, one_launch=launches == 2)
+    step = d.prepare_step(row_min=True, fused_inputs=launches <= 2, one_launch=launches <= 2,
+                          row_min_in_tiles=launches == 1)
     assert len(step) == launches
     for launch in step.values():
         launch()
@@ -434,7 +441,7 @@ def test_fused_input_tables_match_the_three_entry_points(gpu_device):
     results = []
     for fused in (False, True):
         d = DeviceCostTables(tb, p, device=gpu_device)
-        step = d.prepare_step(row_min=True, fused_inputs=fused, one_launch=False)
+        step = d.prepare_step(row_min=True, fused_inputs=fused, one_launch=False, row_min_in_tiles=False)
         assert ("input_tables" in step) == fused and len(step) == (3 if fused else 5)
         for name in names:
             getattr(d, name).zero_()
@@ -471,11 +478,13 @@ def test_one_launch_build_matches_the_separate_entry_points(gpu_device, mesh, th
     names = ("tensor_bytes", "tensor_contiguous", "compute_cost", "compute_cost_per_arg", "comm", "transition", "cost",
              "row_min", "row_argmin")
     results = []
-    for one_launch in (False, True):
+    assert tb.rows_fit_tiles()
+    for one_launch, in_tiles in ((False, False), (True, False), (False, True), (True, True)):
+        # in_tiles: the launch that writes the matrices takes the row minima as well
         d = DeviceCostTables(tb, p, device=gpu_device)
-        step = d.prepare_step(row_min=True, fused_inputs=True, one_launch=one_launch)
-        assert list(step) == (["build_tables", "segmented_min"] if one_launch else
-                              ["input_tables", "redistribute_tables", "segmented_min"])
+        step = d.prepare_step(row_min=True, fused_inputs=True, one_launch=one_launch, row_min_in_tiles=in_tiles)
+        assert list(step) == (["build_tables"] if one_launch else ["input_tables", "redistribute_tables"]) + \
+            ([] if in_tiles else ["segmented_min"])
         for name in names:
             getattr(d, name).zero_()
         spec = d._step_keepalive[1]
@@ -487,8 +496,9 @@ def test_one_launch_build_matches_the_separate_entry_points(gpu_device, mesh, th
         out = {name: getattr(d, name).cpu().numpy() for name in names}
         out.update({f"spec_{k}": v.cpu().numpy() for k, v in spec.items()})
         results.append(out)
-    for key in results[0]:
-        assert np.array_equal(results[0][key], results[1][key]), key
+    for other in results[1:]:
+        for key in results[0]:
+            assert np.array_equal(results[0][key], other[key]), key
     enc = tb.as_dict()
     op = po.make_params(mesh, rescale=2.2)
     want_cc, want_pa = c_oracle.compute_costs(enc, op)
@@ -497,6 +507,8 @@ def test_one_launch_build_matches_the_separate_entry_points(gpu_device, mesh, th
     _assert_costs(results[1]["comm"], want["comm"], "comm")
     assert np.array_equal(results[1]["transition"], want["transition"])
     _assert_costs(results[1]["compute_cost"], want_cc, "compute_cost")
+    want_min, want_arg = c_oracle.segmented_min(want["cost"], tb.row_ptr())
+    assert np.array_equal(results[3]["row_min"], want_min) and np.array_equal(results[3]["row_argmin"], want_arg)
 
 
 def test_randomized_configurations(gpu_device, monkeypatch):
@@ -507,7 +519,7 @@ def test_randomized_configurations(gpu_device, monkeypatch):
 
     rng = np.random.default_rng(2024)
     meshes = [(64,), (32, 8), (8, 8, 8), (5, 3, 2), (2, 3, 2, 2), (128, 2)]
-    for it in range(12):
+    for it in range(16):
         mesh = meshes[it % len(meshes)]
         maxs = int(rng.choice([8, 40, 64, 130]))
         tb = stress_dag(seed=int(rng.integers(1, 10**6)), n_nodes=int(rng.integers(50, 600)), mesh_sizes=mesh,
@@ -527,7 +539,12 @@ def test_randomized_configurations(gpu_device, monkeypatch):
         one_launch = bool(rng.random() < 0.5)
         rescale = float(rng.choice([1.0, 2.2]))
         d = DeviceCostTables(tb, CostModelParams.from_mesh(mesh, rescale=rescale), device=gpu_device)
-        step = d.prepare_step(row_min=True, fused_inputs=True, one_launch=one_launch)
+        in_tiles = tb.rows_fit_tiles() and bool(rng.random() < 0.7)  # row minima taken by the table launch
+        assert tb.rows_fit_tiles() or maxs > 64
+        step = d.prepare_step(row_min=True, fused_inputs=True, one_launch=one_launch, row_min_in_tiles=in_tiles)
+        assert ("segmented_min" in step) != in_tiles
+        d.row_min.fill_(-1.0)
+        d.row_argmin.fill_(-7)
         for launch in step.values():
             launch()
         torch.cuda.synchronize()
@@ -535,7 +552,7 @@ def test_randomized_configurations(gpu_device, monkeypatch):
         want_cc, want_pa = c_oracle.compute_costs(enc, op)
         want = c_oracle.build_tables(enc, op, per_arg=want_pa)
         want_min, want_arg = c_oracle.segmented_min(want["cost"], tb.row_ptr())
-        what = f"case {it}: mesh {mesh}, {maxs} strategies, {copies} copies, threads {threads or 'auto'}, one launch {one_launch}"
+        what = f"case {it}: mesh {mesh}, {maxs} strategies, {copies} copies, threads {threads or 'auto'}, one launch {one_launch}, row minima in tiles {in_tiles}"
         _assert_costs(d.comm.cpu().numpy(), want["comm"], what + " comm")
         _assert_costs(d.cost.cpu().numpy(), want["cost"], what + " cost")
         assert np.array_equal(d.transition.cpu().numpy(), want["transition"]), what

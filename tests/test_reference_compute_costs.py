@@ -12,6 +12,7 @@ them as the vectors' inputs and the test first checks that they are unchanged.""
 
 import json
 import os
+import re
 import sys
 
 import numpy as np
@@ -29,6 +30,13 @@ from make_reference_vectors import node_signature, strategy_code  # noqa: E402  
 
 with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_compute_costs.json")) as f:
     FIXTURE = json.load(f)
+
+
+def _portable(signature: str) -> str:
+    """The random-number state that flash attention hands from forward to backward is a (2,)
+    uint64 tensor when traced without a GPU and two int64 scalars when traced with one: 16 bytes
+    either way, and nothing else in the graph depends on it."""
+    return re.sub(r"T\(2,\)\(1,\)uint64 T\(\)\(\)uint64|T\(\)\(\)int64 T\(\)\(\)int64", "RNG-STATE", signature)
 
 
 class OracleOptimizer(ShardingOptimizer):
@@ -65,7 +73,7 @@ def _check(planner_cls, name):
         for node, (want_name, sig_i, list_i, cost_is) in zip(nodes, case["nodes"]):
             # the vectors' inputs: same node, operator, argument shapes and strategy list
             assert node.name == want_name
-            assert node_signature(node) == case["signatures"][sig_i], node
+            assert _portable(node_signature(node)) == _portable(case["signatures"][sig_i]), node
             strategies = o.strats[node].strategies
             assert [strategy_code(s) for s in strategies] == case["strategy_lists"][list_i], node
             # the vectors' outputs
