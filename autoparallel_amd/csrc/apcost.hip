@@ -1441,10 +1441,10 @@ static int redistribute_tables_impl(const apc_params *params, const int64_t *ten
                                     int64_t n_entries, double *comm_out, uint8_t *trans_out, double *cost_out,
                                     const apc_row_minima *rows, void *stream) {
   if (int rc = check_params(params)) return rc;
-  if (int rc = check_row_minima(rows, comm_out, trans_out, cost_out, dup_entry_begin, "apc_redistribute_tables_row_min"))
-    return rc;
   if (n_tiles < 0 || n_tiles > (1 << 30)) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tiles == 0) return 0;
+  if (int rc = check_row_minima(rows, comm_out, trans_out, cost_out, dup_entry_begin, "apc_redistribute_tables_row_min"))
+    return rc;
   if (n_entries < 0) return fail(-1, "n_entries < 0");
   if (!tensor_bytes || !tensor_contiguous || !spec_codes || !spec_tensor || !tiles)
     return fail(-1, "apc_redistribute_tables: NULL table");
@@ -1491,7 +1491,8 @@ static int build_tables_impl(const apc_params *params, int64_t n_tensors, const 
                      const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *trans_out,
                      double *cost_out, const apc_row_minima *rows, void *stream) {
   if (int rc = check_params(params)) return rc;
-  if (int rc = check_row_minima(rows, comm_out, trans_out, cost_out, dup_entry_begin, "apc_build_tables_row_min")) return rc;
+  if (n_tiles > 0)
+    if (int rc = check_row_minima(rows, comm_out, trans_out, cost_out, dup_entry_begin, "apc_build_tables_row_min")) return rc;
   if (n_tensors < 0 || n_specs < 0 || n_strategies < 0 || n_entries < 0) return fail(-1, "apc_build_tables: negative count");
   if (n_tiles < 0 || n_tiles > (1 << 30)) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tensors > 0 && (!rank || !itemsize || !shape || !stride || !tensor_bytes || !tensor_contiguous))

@@ -224,7 +224,7 @@ class DeviceCostTables:
         (33.4 / 31.7 us when every identical edge is computed on its own), the mixture of experts
         15.7 / 17.7 us, the 464 M-entry stress table 3.77 / 3.37 ms."""
         tb = self.tables
-        if not tb.rows_fit_tiles():
+        if tb.n_tiles == 0 or not tb.rows_fit_tiles():
             return False
         computed = int((tb.tile_row_count.astype(np.int64) * tb.tile_col_count.astype(np.int64)).sum())
         return computed * 4.1e-6 < 4.0 + 8.0 * tb.n_entries / 4.5e6

@@ -291,7 +291,7 @@ def test_segmented_min_matches_oracle(gpu_device, max_len):
 
 def test_row_min_of_cost_tables(gpu_device):
     mesh = (32, 8)
-    tb = stress_dag(seed=9, n_nodes=800, mesh_sizes=mesh)
+    tb = stress_dag(seed=9, n_nodes=300, mesh_sizes=mesh)
     d, want = _run_and_compare(tb, mesh, 2.2, gpu_device)
     rp = tb.row_ptr()
     mins, args = d.segmented_min(d.cost, rp)
