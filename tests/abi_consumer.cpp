@@ -148,7 +148,26 @@ int main() {
                           d_lshape, d_lstride, width, d_lnumel, d_lbytes, 4, d_flops, d_rw, d_dtype, d_zero, d_args, d_compute,
                           d_per_arg, d_err, nullptr, 1, d_tiles, nullptr, 3, d_comm, d_trans, d_cost, nullptr));
   APC_OK(apc_segmented_min(d_cost, d_seg, 1, 3, d_min, d_arg, nullptr));
+  // the same pass with the minimum of every matrix row (three rows of one column) taken by the launch itself
+  const std::vector<int64_t> edge_row_begin{0};
+  double *d_row_min = nullptr;
+  int32_t *d_row_arg = nullptr;
+  HIP_OK(hipMalloc(&d_row_min, 3 * 8));
+  HIP_OK(hipMalloc(&d_row_arg, 3 * 4));
+  const apc_row_minima rows{to_device(edge_row_begin), nullptr, d_row_min, d_row_arg};
+  if (!rows.edge_row_begin) {
+    std::printf("device allocation failed\n");
+    return 2;
+  }
+  APC_OK(apc_build_tables_row_min(&p, 1, d_rank, d_item, d_shape, d_stride, d_bytes, d_cont, 4, d_codes, d_spec_tensor,
+                                  d_shards, d_lshape, d_lstride, width, d_lnumel, d_lbytes, 4, d_flops, d_rw, d_dtype,
+                                  d_zero, d_args, d_compute, d_per_arg, d_err, nullptr, 1, d_tiles, nullptr, 3, d_comm,
+                                  d_trans, d_cost, &rows, nullptr));
   HIP_OK(hipDeviceSynchronize());
+  double row_min[3];
+  int32_t row_arg[3];
+  HIP_OK(hipMemcpy(row_min, d_row_min, sizeof(row_min), hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(row_arg, d_row_arg, sizeof(row_arg), hipMemcpyDeviceToHost));
 
   double comm[3], cost[3], seg_min = 0.0;
   uint8_t trans[3];
@@ -175,6 +194,7 @@ int main() {
   bad += lshape[0] != 4096 / 32 / 8 || lshape[1] != 4096;                        // (S0, S0): dim 0 split twice
   bad += lshape[3 * width] != 4096 / 32 || lshape[3 * width + 1] != 4096 / 8;  // (S0, S1)
   bad += seg_min != want[2] + 1.0 || seg_arg != 2;
+  for (int i = 0; i < 3; ++i) bad += row_min[i] != want[i] + 1.0 || row_arg[i] != 0;
   std::printf(bad ? "abi consumer: %d MISMATCHES\n" : "abi consumer ok\n", bad);
   return bad ? 1 : 0;
 }
