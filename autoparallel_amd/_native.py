@@ -75,6 +75,7 @@ EXPORTS = (
     "apc_redistribute_tables_row_min",
     "apc_build_tables_row_min",
     "apc_segmented_min",
+    "apc_segmented_min_copies",
     "apc_strategy_bounds",
 )
 

@@ -1109,14 +1109,24 @@ __global__ __launch_bounds__(kThreads) void build_tables_kernel(apc_params p, Ta
 // chosen by the host from the mean segment length), so short segments do not leave most of
 // a wavefront idle.
 // ------------------------------------------------------------------------------------------
-template <int G>
+// Which segments to reduce and where else each result goes (SELECTED instantiation): segment
+// selected[i] is reduced and its result stored to itself and to copy_segments[copy_ptr[i] ..
+// copy_ptr[i + 1]), segments the caller knows to hold the same values.
+struct SegmentCopies {
+  const int64_t *selected;
+  const int64_t *copy_ptr;
+  const int64_t *copy_segments;
+};
+
+template <int G, bool SELECTED>
 __global__ __launch_bounds__(kBlock) void segmented_min_kernel(const double *__restrict__ values,
                                                                const int64_t *__restrict__ seg_ptr,
                                                                int64_t n_seg, double *__restrict__ mins,
-                                                               int32_t *__restrict__ args) {
+                                                               int32_t *__restrict__ args, SegmentCopies copies) {
   const int sub = threadIdx.x & (G - 1);
-  const int64_t seg = (int64_t)blockIdx.x * (kBlock / G) + (threadIdx.x / G);
-  const bool live = seg < n_seg;
+  const int64_t slot = (int64_t)blockIdx.x * (kBlock / G) + (threadIdx.x / G);
+  const bool live = slot < n_seg;  // (n_seg counts the selected segments when SELECTED)
+  const int64_t seg = SELECTED ? (live ? copies.selected[slot] : 0) : slot;
   const int64_t lo = live ? seg_ptr[seg] : 0, hi = live ? seg_ptr[seg + 1] : 0;
   double best = INFINITY;
   int64_t arg = INT64_MAX;  // absolute index; INT64_MAX = none seen
@@ -1173,8 +1183,16 @@ __global__ __launch_bounds__(kBlock) void segmented_min_kernel(const double *__r
     }
   }
   if (live && sub == 0) {
+    const int32_t rel = arg == INT64_MAX ? -1 : (int32_t)(arg - lo);
     mins[seg] = best;
-    args[seg] = arg == INT64_MAX ? -1 : (int32_t)(arg - lo);
+    args[seg] = rel;
+    if (SELECTED) {
+      for (int64_t k = copies.copy_ptr[slot], end = copies.copy_ptr[slot + 1]; k < end; ++k) {
+        const int64_t to = copies.copy_segments[k];
+        mins[to] = best;
+        args[to] = rel;
+      }
+    }
   }
 }
 
@@ -1217,9 +1235,13 @@ inline unsigned blocks_for(int64_t n, int per_block) { return (unsigned)((n + pe
 
 template <int G>
 void launch_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_seg, double *mins, int32_t *args,
-                          hipStream_t stream) {
-  hipLaunchKernelGGL(segmented_min_kernel<G>, dim3(blocks_for(n_seg, kBlock / G)), dim3(kBlock), 0, stream, values,
-                     seg_ptr, n_seg, mins, args);
+                          const SegmentCopies *copies, hipStream_t stream) {
+  if (copies)
+    hipLaunchKernelGGL((segmented_min_kernel<G, true>), dim3(blocks_for(n_seg, kBlock / G)), dim3(kBlock), 0, stream,
+                       values, seg_ptr, n_seg, mins, args, *copies);
+  else
+    hipLaunchKernelGGL((segmented_min_kernel<G, false>), dim3(blocks_for(n_seg, kBlock / G)), dim3(kBlock), 0, stream,
+                       values, seg_ptr, n_seg, mins, args, SegmentCopies{nullptr, nullptr, nullptr});
 }
 
 int check_width(int width) {
@@ -1599,11 +1621,13 @@ int apc_build_tables_row_min(APC_BUILD_TABLES_PARAMS, const apc_row_minima *rows
 #undef APC_BUILD_TABLES_PARAMS
 #undef APC_BUILD_TABLES_ARGS
 
-int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_seg, int64_t n_values, double *mins,
-                      int32_t *args, void *stream) {
+}  // extern "C"
+
+static int segmented_min_impl(const double *values, const int64_t *seg_ptr, int64_t n_seg, int64_t n_values, double *mins,
+                              int32_t *args, const SegmentCopies *copies, const char *who, void *stream) {
   if (n_seg < 0 || n_values < 0) return fail(-1, "negative count");
   if (n_seg == 0) return 0;
-  if (!seg_ptr || !mins || !args || (!values && n_values > 0)) return fail(-1, "apc_segmented_min: NULL array");
+  if (!seg_ptr || !mins || !args || (!values && n_values > 0)) return fail(-1, "%s: NULL array", who);
   if (n_seg > (int64_t)INT32_MAX * 4) return fail(-1, "n_segments %lld too large", (long long)n_seg);
   hipStream_t s = (hipStream_t)stream;
   // lanes per segment: about a tenth of the mean length, so that a lane has several
@@ -1614,16 +1638,32 @@ int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_se
   while (g < 64 && g * 12 <= mean) g *= 2;
   if (const char *env = getenv("APC_SEGMIN_GROUP")) g = atoi(env);
   switch (g) {
-    case 1: launch_segmented_min<1>(values, seg_ptr, n_seg, mins, args, s); break;
-    case 2: launch_segmented_min<2>(values, seg_ptr, n_seg, mins, args, s); break;
-    case 4: launch_segmented_min<4>(values, seg_ptr, n_seg, mins, args, s); break;
-    case 8: launch_segmented_min<8>(values, seg_ptr, n_seg, mins, args, s); break;
-    case 16: launch_segmented_min<16>(values, seg_ptr, n_seg, mins, args, s); break;
-    case 32: launch_segmented_min<32>(values, seg_ptr, n_seg, mins, args, s); break;
-    case 64: launch_segmented_min<64>(values, seg_ptr, n_seg, mins, args, s); break;
+    case 1: launch_segmented_min<1>(values, seg_ptr, n_seg, mins, args, copies, s); break;
+    case 2: launch_segmented_min<2>(values, seg_ptr, n_seg, mins, args, copies, s); break;
+    case 4: launch_segmented_min<4>(values, seg_ptr, n_seg, mins, args, copies, s); break;
+    case 8: launch_segmented_min<8>(values, seg_ptr, n_seg, mins, args, copies, s); break;
+    case 16: launch_segmented_min<16>(values, seg_ptr, n_seg, mins, args, copies, s); break;
+    case 32: launch_segmented_min<32>(values, seg_ptr, n_seg, mins, args, copies, s); break;
+    case 64: launch_segmented_min<64>(values, seg_ptr, n_seg, mins, args, copies, s); break;
     default: return fail(-1, "segment group width %d is not a power of two up to 64", g);
   }
-  return check_launch("apc_segmented_min");
+  return check_launch(who);
+}
+
+extern "C" {
+
+int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_seg, int64_t n_values, double *mins,
+                      int32_t *args, void *stream) {
+  return segmented_min_impl(values, seg_ptr, n_seg, n_values, mins, args, nullptr, "apc_segmented_min", stream);
+}
+
+int apc_segmented_min_copies(const double *values, const int64_t *seg_ptr, int64_t n_selected, const int64_t *selected,
+                             const int64_t *copy_ptr, const int64_t *copy_segments, int64_t n_values_selected,
+                             double *mins, int32_t *args, void *stream) {
+  if (n_selected > 0 && (!selected || !copy_ptr)) return fail(-1, "apc_segmented_min_copies: NULL selection");
+  const SegmentCopies copies{selected, copy_ptr, copy_segments};
+  return segmented_min_impl(values, seg_ptr, n_selected, n_values_selected, mins, args, &copies,
+                            "apc_segmented_min_copies", stream);
 }
 
 int apc_strategy_bounds(int64_t n_strategies, const int32_t *strat_node, const int64_t *node_strat_begin,

@@ -317,9 +317,17 @@ class DeviceCostTables:
             n_seg = row_ptr.numel() - 1
             assert n_seg == self.row_min.numel()
             self._step_keepalive.append(row_ptr)
-            a_min = (P(self.cost), P(row_ptr), ctypes.c_int64(n_seg), ctypes.c_int64(tb.n_entries), P(self.row_min),
-                     P(self.row_argmin), stream)
-            step["segmented_min"] = bind(lib.apc_segmented_min, a_min, "apc_segmented_min")
+            copies = self._row_copies()
+            if copies is not None:  # identical edges: every distinct row is read once, its minimum stored to all
+                selected, copy_ptr, copy_rows, n_read = copies
+                self._step_keepalive.append(copies)
+                a_min = (P(self.cost), P(row_ptr), ctypes.c_int64(selected.numel()), P(selected), P(copy_ptr),
+                         P(copy_rows), ctypes.c_int64(n_read), P(self.row_min), P(self.row_argmin), stream)
+                step["segmented_min"] = bind(lib.apc_segmented_min_copies, a_min, "apc_segmented_min_copies")
+            else:
+                a_min = (P(self.cost), P(row_ptr), ctypes.c_int64(n_seg), ctypes.c_int64(tb.n_entries), P(self.row_min),
+                         P(self.row_argmin), stream)
+                step["segmented_min"] = bind(lib.apc_segmented_min, a_min, "apc_segmented_min")
         return step
 
     @_guarded
@@ -357,6 +365,41 @@ class DeviceCostTables:
         return graph
 
     # ---- segmented min ---------------------------------------------------------------------
+    def _row_copies(self):
+        """Device arrays of ``CostTables.row_copies()`` when reading only the distinct rows saves
+        at least a quarter of the matrix bytes, else None."""
+        tb = self.tables
+        if tb.dup_entry_begin is None or len(tb.dup_entry_begin) == 0:
+            return None
+        selected, copy_ptr, copy_rows, n_read = tb.row_copies()
+        if n_read > 0.75 * tb.n_entries:
+            return None
+        return (_to_device(selected, self.device), _to_device(copy_ptr, self.device),
+                _to_device(copy_rows, self.device), n_read)
+
+    @_guarded
+    def row_minima(self):
+        """(min, first argmin) of every matrix row of ``cost``: what the table launch already took,
+        else a segmented minimum that reads every distinct row once."""
+        if self.row_min is not None:
+            return self.row_min, self.row_argmin
+        tb = self.tables
+        copies = self._row_copies()
+        row_ptr = _to_device(tb.row_ptr(), self.device)
+        if copies is None:
+            return self.segmented_min(self.cost, row_ptr, check=False)
+        selected, copy_ptr, copy_rows, n_read = copies
+        n_rows = row_ptr.numel() - 1
+        mins = self._empty((n_rows,), torch.float64)
+        args = self._empty((n_rows,), torch.int32)
+        with torch.cuda.device(self.device):
+            rc = self.lib.apc_segmented_min_copies(self._p(self.cost), self._p(row_ptr), ctypes.c_int64(selected.numel()),
+                                                   self._p(selected), self._p(copy_ptr), self._p(copy_rows),
+                                                   ctypes.c_int64(n_read), self._p(mins), self._p(args), self._stream())
+        _native.check(rc, "apc_segmented_min_copies")
+        torch.cuda.current_stream(self.device).synchronize()  # the index arrays die with this frame
+        return mins, args
+
     @_guarded
     def segmented_min(self, values: torch.Tensor, seg_ptr, check: bool = True):
         if not isinstance(seg_ptr, torch.Tensor):

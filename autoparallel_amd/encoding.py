@@ -460,6 +460,29 @@ class CostTables:
         te = self.tile_edge.astype(np.int64)
         return bool((self.tile_col_begin == 0).all() and (self.tile_col_count == ns[te]).all())
 
+    def row_copies(self):
+        """-> (selected, copy_ptr, copy_rows, n_values_selected): the matrix rows of the edges that
+        are tiled, and for each of them the rows of the identical edges that receive the same
+        values (rows numbered as in ``row_ptr()``).  A minimum taken over ``selected`` and
+        stored to the copies covers every row while reading each distinct row once."""
+        nt = self.edge_n_tgt.astype(np.int64)
+        ns = self.edge_n_src.astype(np.int64)
+        rb = self.edge_row_begin()
+        canon = np.nonzero(self.edge_canonical == np.arange(self.n_edges))[0]
+        ntc = nt[canon]
+        n_sel = int(ntc.sum())
+        first = np.cumsum(ntc) - ntc
+        r = np.arange(n_sel, dtype=np.int64) - np.repeat(first, ntc)  # consumer strategy of every selected row
+        selected = np.repeat(rb[canon], ntc) + r
+        per_row = np.repeat(self.edge_dup_count[canon].astype(np.int64), ntc)
+        copy_ptr = np.zeros(n_sel + 1, np.int64)
+        np.cumsum(per_row, out=copy_ptr[1:])
+        which = np.repeat(np.arange(n_sel, dtype=np.int64), per_row)
+        k = np.arange(int(copy_ptr[-1]), dtype=np.int64) - copy_ptr[which]
+        dup_first = np.repeat(self.edge_dup_begin[canon].astype(np.int64), ntc)
+        copy_rows = self.dup_row_begin[dup_first[which] + k] + r[which] if len(which) else _i64([])
+        return _i64(selected), _i64(copy_ptr), _i64(copy_rows), int((ns[canon] * ntc).sum())
+
     def row_ptr(self) -> np.ndarray:
         """CSR pointer of matrix rows over the entry array: one segment per
         (edge, consumer strategy), length = that edge's producer count."""

@@ -98,15 +98,15 @@ class DeviceBackend:
         from .device_tables import _real_tensors
 
         with _real_tensors():
-            if self._are_matrix_rows(row_ptr):  # the table launch already took them
-                return self.dev.row_min.cpu().numpy(), self.dev.row_argmin.cpu().numpy()
-            mins, args = self.dev.segmented_min(self.dev.cost, row_ptr)
+            if self._are_matrix_rows(row_ptr):  # taken by the table launch, or one read of every distinct row
+                mins, args = self.dev.row_minima()
+            else:
+                mins, args = self.dev.segmented_min(self.dev.cost, row_ptr)
             return mins.cpu().numpy(), args.cpu().numpy()
 
     def _are_matrix_rows(self, row_ptr) -> bool:
-        d = self.dev
-        return d.row_min is not None and len(row_ptr) == d.row_min.numel() + 1 and \
-            np.array_equal(row_ptr, d.tables.row_ptr())
+        tb = self.dev.tables
+        return len(row_ptr) == int(tb.edge_n_tgt.astype(np.int64).sum()) + 1 and np.array_equal(row_ptr, tb.row_ptr())
 
     def greedy(self, row_ptr):
         """-> (bound per strategy, min per node, argmin per node) from the row minima of the cost table"""
@@ -114,7 +114,7 @@ class DeviceBackend:
 
         with _real_tensors():
             if self._are_matrix_rows(row_ptr):
-                mins = self.dev.row_min
+                mins, _ = self.dev.row_minima()
             else:
                 mins, _ = self.dev.segmented_min(self.dev.cost, row_ptr)
             return tuple(x.cpu().numpy() for x in self.dev.greedy_strategies(mins))

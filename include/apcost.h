@@ -252,6 +252,17 @@ int apc_build_tables_row_min(const apc_params *params, int64_t n_tensors, const 
 int apc_segmented_min(const double *values, const int64_t *seg_ptr, int64_t n_segments, int64_t n_values,
                       double *seg_min, int32_t *seg_argmin, void *stream);
 
+/* apc_segmented_min over selected segments only, for value arrays in which whole segments
+ * repeat (the rows of identical edges, which the table kernels fill with the same values):
+ * segment selected[i] is reduced (seg_ptr indexed by segment id, as above) and its result is
+ * stored at seg_min / seg_argmin [selected[i]] and at [copy_segments[k]] for k in
+ * [copy_ptr[i], copy_ptr[i + 1]).  The caller vouches that those segments hold the same
+ * values; segments that are neither selected nor a copy are left unwritten.
+ * n_values_selected = total length of the selected segments.  No counterpart in the reference. */
+int apc_segmented_min_copies(const double *values, const int64_t *seg_ptr, int64_t n_selected, const int64_t *selected,
+                             const int64_t *copy_ptr, const int64_t *copy_segments, int64_t n_values_selected,
+                             double *seg_min, int32_t *seg_argmin, void *stream);
+
 /* Optimistic cost of every (node, strategy): bound[s] = sum, over the edges e of the node that
  * owns strategy s (edges_by_node[node_edge_begin[n] .. node_edge_begin[n + 1]), added in that
  * order), of row_min[edge_row_begin[e] + (s - node_strat_begin[n])], where row_min holds the

@@ -136,6 +136,37 @@ def test_deduplicated_tiles_write_every_entry_exactly_once():
     assert int((other.edge_canonical != np.arange(other.n_edges)).sum()) < n_dup
 
 
+def test_row_copies_cover_every_row_once_and_pair_identical_rows():
+    """``row_copies``: the rows of the tiled edges plus their copies are every matrix row exactly
+    once; a copy is the same consumer strategy of an identical edge; rows are numbered as in
+    ``row_ptr`` / ``edge_row_begin`` (what the row-minimum launches write to)."""
+    tb = twin_graph(stress_dag(seed=3, n_nodes=150, mesh_sizes=(4, 2), frac_nonspec_nodes=0.03))
+    tb.build_tiles(1024, dedupe=True, max_copies=8)
+    selected, copy_ptr, copy_rows, n_read = tb.row_copies()
+    n_rows = int(tb.edge_n_tgt.sum())
+    seen = np.zeros(n_rows, np.int64)
+    np.add.at(seen, selected, 1)
+    np.add.at(seen, copy_rows, 1)
+    assert (seen == 1).all() and len(copy_rows) > 0
+    row_edge = np.repeat(np.arange(tb.n_edges), tb.edge_n_tgt)
+    rb = tb.edge_row_begin()
+    assert np.array_equal(rb, np.cumsum(tb.edge_n_tgt.astype(np.int64)) - tb.edge_n_tgt)
+    which = np.repeat(np.arange(len(selected)), np.diff(copy_ptr))
+    assert np.array_equal(tb.edge_canonical[row_edge[copy_rows]], row_edge[selected[which]])
+    assert np.array_equal(copy_rows - rb[row_edge[copy_rows]], selected[which] - rb[row_edge[selected[which]]])
+    lens = np.diff(tb.row_ptr())
+    assert n_read == int(lens[selected].sum()) < tb.n_entries
+    # the rows the tiles' duplicate lists name are the same ones
+    for e in np.nonzero(tb.edge_dup_count)[0][:20]:
+        dups = tb.dup_row_begin[tb.edge_dup_begin[e]:tb.edge_dup_begin[e] + tb.edge_dup_count[e]]
+        assert np.array_equal(tb.edge_canonical[row_edge[dups]], np.full(len(dups), e))
+    # without identical edges: every row selected, no copies
+    plain = stress_dag(seed=3, n_nodes=50, mesh_sizes=(4, 2))
+    selected, copy_ptr, copy_rows, n_read = plain.row_copies()
+    assert np.array_equal(selected, np.arange(int(plain.edge_n_tgt.sum()))) and len(copy_rows) == 0
+    assert n_read == plain.n_entries and plain.rows_fit_tiles()
+
+
 def test_validator_rejects_bad_duplicate_offsets():
     tb = twin_graph(stress_dag(seed=8, n_nodes=60, mesh_sizes=(4, 2), max_strategies=10))
     tb.build_tiles(256, dedupe=True)

@@ -304,6 +304,26 @@ def test_row_min_of_cost_tables(gpu_device):
     assert d.row_min is None
 
 
+@pytest.mark.parametrize("copies", [2, 8])
+def test_row_minima_read_every_distinct_row_once(gpu_device, copies):
+    """apc_segmented_min_copies on a table with identical edges (and some empty rows): the same
+    minima and argmins as apc_segmented_min over every row and as the oracle, with a third of the
+    rows written through the copy lists."""
+    from test_abi_and_encoding import twin_graph
+
+    mesh = (8, 8, 8)
+    tb = twin_graph(stress_dag(seed=21, n_nodes=400, mesh_sizes=mesh, max_strategies=90, frac_nonspec_nodes=0.02))
+    tb.build_tiles(1024, dedupe=True, max_copies=copies)
+    assert not tb.rows_fit_tiles()  # producers with more than 64 strategies: the tiles cannot take the minima
+    d, want = _run_and_compare(tb, mesh, 2.2, gpu_device)
+    assert d.row_min is None and d._row_copies() is not None
+    mins, args = d.row_minima()
+    plain_min, plain_arg = d.segmented_min(d.cost, tb.row_ptr())
+    wm, wa = c_oracle.segmented_min(want["cost"], tb.row_ptr())
+    assert np.array_equal(mins.cpu().numpy(), wm) and np.array_equal(args.cpu().numpy(), wa)
+    assert torch.equal(mins, plain_min) and torch.equal(args, plain_arg)
+
+
 @pytest.mark.parametrize("mesh", [(32, 8), (16, 8, 4)])
 def test_strategy_bounds_and_greedy_strategies_match_oracle(gpu_device, mesh):
     """Per-strategy sums of row minima and the per-node (min, argmin): same bits as the oracle
