@@ -837,23 +837,65 @@ __device__ __forceinline__ void store_entry(const TileOut &o, int dup_count, con
   }
 }
 
+// A 32-bit value from the lane `N` further on within the lane's row of 16 (DPP row_shl:N); a
+// lane whose source lies outside its row keeps its own value.
+template <int N>
+__device__ __forceinline__ int from_lane_ahead(int x) {
+  return __builtin_amdgcn_update_dpp(x, x, 0x100 + N, 0xF, 0xF, false);
+}
+template <int N>
+__device__ __forceinline__ double from_lane_ahead(double x) {
+  const int lo = from_lane_ahead<N>(__double2loint(x)), hi = from_lane_ahead<N>(__double2hiint(x));
+  return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double value_of_lane(double x, int lane) {  // lane: a constant
+  const int lo = __builtin_amdgcn_readlane(__double2loint(x), lane), hi = __builtin_amdgcn_readlane(__double2hiint(x), lane);
+  return __hiloint2double(hi, lo);
+}
+
 // Row minima inside the tile kernel.  The 64 lanes of a wavefront hold 64 consecutive entries
-// of the tile (inactive lanes: +inf), row after row.  A segmented minimum by doubling leaves, in
-// the first lane of every run of one row, the minimum of the run and the first column that has
-// it; that lane writes the row's slot.  `c` is the lane's column, `cols` the row length.
+// of the tile (inactive lanes: +inf), row after row.  `c` is the lane's column, `cols` the row
+// length.  First a segmented minimum by doubling inside every 16 lanes (data-parallel
+// primitives: vector ALU only, the LDS pipe stays free for the entry loop's lookups): a lane
+// then holds the minimum, and the first column that has it, of its row's entries from itself to
+// the end of its 16 lanes.  Lanes 16, 32 and 48 hold such a part for a row that came in from the
+// lanes before them: their values are read as scalars and joined, in lane order, by the lanes
+// whose row reaches them.  The first lane of every run of one row writes the row's slot.
 __device__ __forceinline__ void row_min_chunk(double (&rmin)[2][APC_TILE_MAX_ROWS], int (&rarg)[2][APC_TILE_MAX_ROWS],
                                               bool active, double value, int r, int c, int cols, int lane) {
   double m = active ? value : __builtin_inf();
   int mc = c;
-  for (int off = 1; off < 64 && off < cols; off <<= 1) {  // (cols is wave-uniform)
-    const double om = __shfl_down(m, off, 64);
-    const int oc = __shfl_down(mc, off, 64);
-    // the lane `off` further on holds an entry of the same row (entries are consecutive)
-    if (lane + off < 64 && c + off < cols && om < m) {  // strict: ties keep the lower column
-      m = om;
-      mc = oc;
-    }
+  const int in_row16 = lane & 15;
+#define APC_ROW_MIN_STEP(N_)                                                            \
+  if (N_ < cols) { /* (cols is wave-uniform) */                                         \
+    const double om = from_lane_ahead<N_>(m);                                           \
+    const int oc = from_lane_ahead<N_>(mc);                                             \
+    /* that lane holds an entry of the same row; strict <: ties keep the lower column */ \
+    if (in_row16 + N_ < 16 && c + N_ < cols && om < m) {                                \
+      m = om;                                                                           \
+      mc = oc;                                                                          \
+    }                                                                                   \
   }
+  APC_ROW_MIN_STEP(1)
+  APC_ROW_MIN_STEP(2)
+  APC_ROW_MIN_STEP(4)
+  APC_ROW_MIN_STEP(8)
+#undef APC_ROW_MIN_STEP
+#define APC_ROW_MIN_JOIN(LANE_)                                              \
+  {                                                                          \
+    const double pm = value_of_lane(m, LANE_);                               \
+    const int pc = __builtin_amdgcn_readlane(mc, LANE_);                     \
+    if (LANE_ > lane && c + (LANE_ - lane) < cols && pm < m) {               \
+      m = pm;                                                                \
+      mc = pc;                                                               \
+    }                                                                        \
+  }
+  if (cols > 1) {
+    APC_ROW_MIN_JOIN(16)
+    APC_ROW_MIN_JOIN(32)
+    APC_ROW_MIN_JOIN(48)
+  }
+#undef APC_ROW_MIN_JOIN
   if (active && (c == 0 || lane == 0)) {
     const int slot = c == 0 ? 0 : 1;
     rmin[slot][r] = m;
@@ -1055,18 +1097,35 @@ __device__ __forceinline__ void tile_entries(const apc_params &p, const TableArg
 }
 
 template <int M, int kTileThreads, bool RM>
-__global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_params p, TableArgs a, int n_tiles,
-                                                                          int xcd_shift) {
-  __shared__ TileStage<M, RM> s_stage;
+__device__ __forceinline__ void redistribute_tile(const apc_params &p, const TableArgs &a, int n_tiles, int xcd_shift,
+                                                  TileStage<M, RM> &stage) {
   const int64_t tile_id = xcd_chunked_unit(xcd_shift);
   if (tile_id >= n_tiles) return;
   static_assert(kTileThreads == 64 || kTileThreads == 128 || kTileThreads == 256, "wavefronts per tile: 1, 2 or 4");
   static_assert(kTileThreads >= APC_TILE_MAX_COLS && kTileThreads >= APC_TILE_MAX_ROWS &&
                 2 * kTileThreads > APC_TILE_MAX_DUPS, "one staging round covers a tile");
   const apc_tile tile = a.tiles[tile_id];
-  stage_tile<M, false>(p, a, tile, s_stage, threadIdx.x, kTileThreads);
+  stage_tile<M, false>(p, a, tile, stage, threadIdx.x, kTileThreads);
   __syncthreads();
-  tile_entries<M, false>(p, a, s_stage, view_of(tile), threadIdx.x, kTileThreads);
+  tile_entries<M, false>(p, a, stage, view_of(tile), threadIdx.x, kTileThreads);
+}
+
+template <int M, int kTileThreads>
+__global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_params p, TableArgs a, int n_tiles,
+                                                                          int xcd_shift) {
+  __shared__ TileStage<M, false> s_stage;
+  redistribute_tile<M, kTileThreads, false>(p, a, n_tiles, xcd_shift, s_stage);
+}
+
+// The same with the row minima.  Occupancy is asked for explicitly: left alone, the compiler
+// sizes this kernel's register budget by the LDS it uses, 97 registers and 4 wavefronts per
+// SIMD on a 3-D mesh, where 67 registers do without spilling and 7 wavefronts fit (stress
+// table: 2.58 ms against 2.94 ms).
+template <int M, int kTileThreads>
+__global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(M <= 3 ? 7 : 4, 8)))
+void redistribute_tiles_row_min_kernel(apc_params p, TableArgs a, int n_tiles, int xcd_shift) {
+  __shared__ TileStage<M, true> s_stage;
+  redistribute_tile<M, kTileThreads, true>(p, a, n_tiles, xcd_shift, s_stage);
 }
 
 // Every table of a pass in one launch: workgroups [0, tile_blocks) take the tiles of the
@@ -1486,19 +1545,19 @@ static int redistribute_tables_impl(const apc_params *params, const int64_t *ten
   const int64_t per_tile = n_entries / n_tiles;
   int threads = per_tile >= 1536 ? 256 : per_tile >= 512 ? 128 : 64;
   if (const char *env = getenv("APC_TILE_THREADS")) threads = atoi(env);  // tuning override
-#define APC_LAUNCH_RM(M_, RM_)                                                                                  \
-  if (threads >= 256) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 256, RM_>), grid, dim3(256), 0, s, *params, a, nt, xs); \
-  else if (threads >= 128) hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 128, RM_>), grid, dim3(128), 0, s, *params, a, nt, xs); \
-  else hipLaunchKernelGGL((redistribute_tiles_kernel<M_, 64, RM_>), grid, dim3(64), 0, s, *params, a, nt, xs)
+#define APC_LAUNCH_K(KERNEL_, M_)                                                                               \
+  if (threads >= 256) hipLaunchKernelGGL((KERNEL_<M_, 256>), grid, dim3(256), 0, s, *params, a, nt, xs);            \
+  else if (threads >= 128) hipLaunchKernelGGL((KERNEL_<M_, 128>), grid, dim3(128), 0, s, *params, a, nt, xs);       \
+  else hipLaunchKernelGGL((KERNEL_<M_, 64>), grid, dim3(64), 0, s, *params, a, nt, xs)
 #define APC_LAUNCH(M_)                        \
-  if (rows) { APC_LAUNCH_RM(M_, true); } else { APC_LAUNCH_RM(M_, false); }
+  if (rows) { APC_LAUNCH_K(redistribute_tiles_row_min_kernel, M_); } else { APC_LAUNCH_K(redistribute_tiles_kernel, M_); }
   switch (params->mesh_ndim) {
     case 1: APC_LAUNCH(1); break;
     case 2: APC_LAUNCH(2); break;
     case 3: APC_LAUNCH(3); break;
     default: APC_LAUNCH(4); break;
   }
-#undef APC_LAUNCH_RM
+#undef APC_LAUNCH_K
 #undef APC_LAUNCH
   return check_launch("apc_redistribute_tables");
 }
