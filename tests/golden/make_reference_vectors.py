@@ -1,17 +1,26 @@
-"""Writes ``reference_compute_costs.json``: the compute cost of every (node, strategy) of
-four traced graphs as the reference's own ``estimate_strategy_runtime_cost``
-(autoparallel/compute_estimation.py:334-365) returns it.  That function runs each operator on
-fake tensors of the sharded argument shapes, so its result depends on what every operator's
-meta kernel and flop formula return: no closed form pins it for operators other than mm.
+"""Writes ``reference_strategies_and_costs.json``: for four traced graphs, what the reference itself
+produces for the two steps of the path that no closed form pins:
 
-Runs only where /root/reference exists (never on a GPU box, never from a test).  Only
-``autoparallel.compute_estimation`` is imported: it needs nothing but torch.  The reference's
-strategy enumeration (``autoparallel.utils`` / ``propagation_rules`` / ``dtensor_util``) does
-not import under the installed torch (``register_op_strategy`` has left
-``torch.distributed.tensor._ops.utils``), and no stand-in was written for it.  So the graphs
-and the strategy lists are this repository's own (capture + ``StrategyEnumerator``): they are
-the INPUT of the vectors, stored beside the costs so that a test can tell a changed input from
-a changed result.
+  * the strategy list of every node, content AND order: ``get_placement_options``
+    (autoparallel/utils.py:154-192) driven as ``ShardingOptimizer.build_sharding_metadata`` drives
+    it (optimize_sharding.py:156-209), ``_create_all_options`` (autoparallel/propagation_rules.py)
+    for placeholders;
+  * the compute cost of every (node, strategy): ``estimate_strategy_runtime_cost``
+    (autoparallel/compute_estimation.py:334-365), which runs each operator on fake tensors of the
+    sharded argument shapes, so its result depends on every operator's meta kernel and flop formula.
+
+Runs only where /root/reference exists (never on a GPU box, never from a test).  What is imported:
+``autoparallel.compute_estimation``, ``autoparallel.utils``, ``autoparallel.propagation_rules``
+(and through them ``autoparallel.dtensor_util``): torch-only modules.  Under the installed torch
+2.10 their import needs one name restored: ``register_op_strategy`` has moved from
+``torch.distributed.tensor._ops.utils`` to ``torch.distributed.tensor._ops.registration``; this
+script re-exports torch's own function under the old module path before importing (no reference
+or torch code is replaced or re-implemented).  ``autoparallel.optimize_sharding`` is not imported
+(its solver front-end ``pulp`` is not installed), so its node loop is driven from here.
+
+The graphs are this repository's own captures of the test models and of one decoder layer of
+the benchmark models: they are the INPUT of the vectors; every record stores its node's operator
+and argument shapes so that a test can tell a changed graph from a changed result.
 
 The environment is the one the reference's planner tests patch in
 (tests/test_optimize_placement.py:141-142): 8 devices per host, device name "H100".
@@ -101,15 +110,26 @@ def make_graph(kind, mesh):
 
 
 def reference_tables(gm, mesh):
+    from torch.utils._pytree import tree_map_only
+
     from autoparallel.compute_estimation import estimate_strategy_runtime_cost
+    from autoparallel.propagation_rules import _create_all_options
+    from autoparallel.utils import get_placement_options
 
-    from autoparallel_amd.graphs.strategies import enumerate_strategies
-
-    strats, _ = enumerate_strategies(gm, mesh)
-    records = []
+    strats, records = {}, []
     for node in gm.graph.nodes:
-        if node.op == "output":
+        if node.op == "placeholder":
+            strats[node] = _create_all_options(mesh, node.meta["val"].shape, tensor=node.meta["val"])
+        elif node.op == "call_function":
+            assert not node.meta.get("local_map_kwargs"), "local_map regions are not part of these vectors"
+            user_strats = tree_map_only(torch.fx.Node, lambda x: strats[x], node.args)
+            user_args = tree_map_only(torch.fx.Node, lambda x: x.meta["val"], node.args)
+            user_kwargs = tree_map_only(torch.fx.Node, lambda x: x.meta["val"], node.kwargs)
+            strats[node] = get_placement_options(mesh, node.target, user_strats, user_args, user_kwargs)
+        elif node.op == "output":
             continue
+        else:
+            raise ValueError(node.op)
         strategies = strats[node].strategies
         costs = [float(estimate_strategy_runtime_cost(node, s)) for s in strategies]
         records.append((node.name, node_signature(node), [strategy_code(s) for s in strategies],
@@ -140,9 +160,15 @@ def main():
 
     assert os.path.isdir(REFERENCE), "the reference is not present here: the committed vectors are used as they are"
     sys.path.insert(0, REFERENCE)
+    # torch 2.10 moved this function; the reference imports it from its old place
+    import torch.distributed.tensor._ops.registration as registration
+    import torch.distributed.tensor._ops.utils as ops_utils
+
+    if not hasattr(ops_utils, "register_op_strategy"):
+        ops_utils.register_op_strategy = registration.register_op_strategy
     dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=512)
     out = {"provenance": "written by tests/golden/make_reference_vectors.py from the reference's "
-                         "estimate_strategy_runtime_cost (autoparallel/compute_estimation.py:334-365), "
+                         "get_placement_options / _create_all_options (strategy lists) and estimate_strategy_runtime_cost (costs), "
                          f"torch {torch.__version__}",
            "environment": {"devices_per_host": 8, "device_name": "H100"},
            "cases": {}}
@@ -163,7 +189,7 @@ def main():
         print(name, len(records), "nodes,", sum(len(r[2]) for r in records), "strategies,",
               len(out["cases"][name]["strategy_lists"]), "distinct lists,",
               len(out["cases"][name]["cost_values_us"]), "distinct costs", flush=True)
-    path = os.path.join(HERE, "reference_compute_costs.json")
+    path = os.path.join(HERE, "reference_strategies_and_costs.json")
     with open(path, "w") as f:
         json.dump(out, f, separators=(",", ":"))
     print(path, os.path.getsize(path), "bytes")

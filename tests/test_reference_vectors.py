@@ -1,14 +1,17 @@
-"""Compute-cost parity against vectors written by the reference itself.
+"""Strategy-list and compute-cost parity against vectors written by the reference itself.
 
-``tests/golden/reference_compute_costs.json`` holds, for every (node, strategy) of four traced
-graphs (the reference tests' FFN and transformer block on (32, 8); one decoder layer of
-Llama-3-8B on (32, 8) and of Llama-3-70B on (8, 8, 8), at the benchmark shapes), what the
-reference's ``estimate_strategy_runtime_cost`` (autoparallel/compute_estimation.py:334-365)
-returned for it: the operator run on fake tensors of the sharded shapes under torch's flop
-counter.  Here the same number comes from the shard-shape table, one shape-function run per
-distinct key, and the compute-cost kernel (CPU test: the oracle's restatement of the tail);
-equality is exact.  The graphs and strategy lists are this repository's own; the fixture stores
-them as the vectors' inputs and the test first checks that they are unchanged."""
+``tests/golden/reference_strategies_and_costs.json`` holds, for every node of four traced graphs
+(the reference tests' FFN and transformer block on (32, 8); one decoder layer of Llama-3-8B on
+(32, 8) and of Llama-3-70B on (8, 8, 8), at the benchmark shapes):
+  * its strategy list, content and order, as the reference's ``get_placement_options`` /
+    ``_create_all_options`` produce it (autoparallel/utils.py:154-192, propagation_rules.py);
+  * for every strategy what the reference's ``estimate_strategy_runtime_cost``
+    (autoparallel/compute_estimation.py:334-365) returned: the operator run on fake tensors of the
+    sharded shapes under torch's flop counter.
+Here the lists come from ``StrategyEnumerator`` and the costs from the shard-shape table, one
+shape-function run per distinct key, and the compute-cost kernel (CPU test: the oracle's
+restatement of the tail); equality is exact.  The graphs are this repository's own captures; the
+fixture stores every node's operator and argument shapes and the test checks them first."""
 
 import json
 import os
@@ -28,7 +31,7 @@ from oracle_backend import OracleBackend
 sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
 from make_reference_vectors import node_signature, strategy_code  # noqa: E402  (pure helpers; imports no reference code)
 
-with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_compute_costs.json")) as f:
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_strategies_and_costs.json")) as f:
     FIXTURE = json.load(f)
 
 
@@ -71,12 +74,13 @@ def _check(planner_cls, name):
         assert len(nodes) == len(case["nodes"])
         n_checked = n_positive = 0
         for node, (want_name, sig_i, list_i, cost_is) in zip(nodes, case["nodes"]):
-            # the vectors' inputs: same node, operator, argument shapes and strategy list
+            # the vectors' inputs: same node, operator and argument shapes
             assert node.name == want_name
             assert _portable(node_signature(node)) == _portable(case["signatures"][sig_i]), node
+            # the vectors' outputs: the reference's strategy list (content and order) ...
             strategies = o.strats[node].strategies
             assert [strategy_code(s) for s in strategies] == case["strategy_lists"][list_i], node
-            # the vectors' outputs
+            # ... and its compute cost of every strategy
             begin = o.encoded.strat_begin[o.node_map[node]]
             got = o.compute_cost[begin:begin + len(strategies)]
             want = np.array([values[i] for i in cost_is])
@@ -91,11 +95,11 @@ def _check(planner_cls, name):
 
 
 @pytest.mark.parametrize("name", list(FIXTURE["cases"]))
-def test_oracle_compute_costs_equal_the_reference_vectors(fake_pg, name):
+def test_strategy_lists_and_oracle_compute_costs_equal_the_reference_vectors(fake_pg, name):
     assert _check(OraclePlanner, name) == "OracleBackend"
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", list(FIXTURE["cases"]))
-def test_device_compute_costs_equal_the_reference_vectors(gpu_device, fake_pg, name):
+def test_strategy_lists_and_device_compute_costs_equal_the_reference_vectors(gpu_device, fake_pg, name):
     assert _check(AutoParallelPlanner, name) == "DeviceBackend"
