@@ -30,6 +30,7 @@ The environment is the one the reference's planner tests patch in
 
 import json
 import os
+import re
 import sys
 import warnings
 from unittest.mock import patch
@@ -49,6 +50,7 @@ CASES = [
     ("block_32x8", "block", (32, 8)),
     ("llama3_8b_1layer_32x8", "llama3_8b", (32, 8)),
     ("llama3_70b_1layer_8x8x8", "llama3_70b", (8, 8, 8)),
+    ("local_map_block_8x8x4", "local_map_block", (8, 8, 4)),  # attention inside a local_map region
 ]
 
 
@@ -86,10 +88,11 @@ def node_signature(node) -> str:
             if isinstance(v, torch.Tensor):
                 return f"T{tuple(v.shape)}{tuple(v.stride())}{str(v.dtype).replace('torch.', '')}"
             return "V"
-        return repr(x)
+        return re.sub(r" at 0x[0-9a-f]+", "", repr(x))  # (functions and modules print their address)
 
     flat, _ = tree_flatten((node.args, node.kwargs))
-    return f"{node.target} " + " ".join(one(x) for x in flat)
+    target = node.target if isinstance(node.target, torch._ops.OpOverload) else getattr(node.target, "__name__", "?")
+    return f"{target} " + " ".join(one(x) for x in flat)
 
 
 def make_graph(kind, mesh):
@@ -106,7 +109,8 @@ def make_graph(kind, mesh):
     model_fn, input_fn = make_model_and_inputs(mesh, kind)
     with torch.device("meta"):
         model = model_fn()
-    return capture_joint_graph(model, input_fn, param_dtype=None, device="cpu", dynamo=False)
+    # a local_map region survives only a Dynamo capture of the forward (api.py:152-192)
+    return capture_joint_graph(model, input_fn, param_dtype=None, device="cpu", dynamo=kind == "local_map_block")
 
 
 def reference_tables(gm, mesh):
@@ -114,18 +118,23 @@ def reference_tables(gm, mesh):
 
     from autoparallel.compute_estimation import estimate_strategy_runtime_cost
     from autoparallel.propagation_rules import _create_all_options
-    from autoparallel.utils import get_placement_options
+    from autoparallel.utils import get_local_map_placement_option, get_placement_options
 
     strats, records = {}, []
     for node in gm.graph.nodes:
         if node.op == "placeholder":
             strats[node] = _create_all_options(mesh, node.meta["val"].shape, tensor=node.meta["val"])
         elif node.op == "call_function":
-            assert not node.meta.get("local_map_kwargs"), "local_map regions are not part of these vectors"
             user_strats = tree_map_only(torch.fx.Node, lambda x: strats[x], node.args)
             user_args = tree_map_only(torch.fx.Node, lambda x: x.meta["val"], node.args)
             user_kwargs = tree_map_only(torch.fx.Node, lambda x: x.meta["val"], node.kwargs)
-            strats[node] = get_placement_options(mesh, node.target, user_strats, user_args, user_kwargs)
+            if local_map_kwargs := node.meta.get("local_map_kwargs", {}):  # optimize_sharding.py:174-196
+                assert not user_kwargs
+                strats[node] = get_local_map_placement_option(
+                    mesh, user_strats, user_args, node, local_map_kwargs["in_placements"],
+                    local_map_kwargs["out_placements"])
+            else:
+                strats[node] = get_placement_options(mesh, node.target, user_strats, user_args, user_kwargs)
         elif node.op == "output":
             continue
         else:

@@ -2,7 +2,8 @@
 
 ``tests/golden/reference_strategies_and_costs.json`` holds, for every node of four traced graphs
 (the reference tests' FFN and transformer block on (32, 8); one decoder layer of Llama-3-8B on
-(32, 8) and of Llama-3-70B on (8, 8, 8), at the benchmark shapes):
+(32, 8) and of Llama-3-70B on (8, 8, 8), at the benchmark shapes; the transformer block with its attention inside a
+``local_map`` region on (8, 8, 4)):
   * its strategy list, content and order, as the reference's ``get_placement_options`` /
     ``_create_all_options`` produce it (autoparallel/utils.py:154-192, propagation_rules.py);
   * for every strategy what the reference's ``estimate_strategy_runtime_cost``
@@ -60,7 +61,8 @@ def _planner(planner_cls, case):
     model_fn, input_fn = make_model_and_inputs(mesh, kind)
     with torch.device("meta"):
         model = model_fn()
-    return planner_cls(model, input_fn, mesh)
+    # a local_map region survives only a Dynamo capture of the forward
+    return planner_cls(model, input_fn, mesh, dynamo=kind == "local_map_block")
 
 
 def _check(planner_cls, name):
