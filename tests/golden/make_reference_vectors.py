@@ -51,7 +51,14 @@ CASES = [
     ("llama3_8b_1layer_32x8", "llama3_8b", (32, 8)),
     ("llama3_70b_1layer_8x8x8", "llama3_70b", (8, 8, 8)),
     ("local_map_block_8x8x4", "local_map_block", (8, 8, 4)),  # attention inside a local_map region
+    ("dsv3_moe_tiny_64x4", "dsv3_moe_tiny", (64, 4)),  # one dense and one mixture-of-experts layer, widths divided down
 ]
+
+# the DeepSeek-V3 style configuration with every width divided down: same operators, same graph shape
+TINY_MOE = dict(dim=256, n_layers=2, n_dense_layers=1, n_heads=8, q_lora_rank=64, kv_lora_rank=32, qk_nope_head_dim=16,
+                qk_rope_head_dim=8, v_head_dim=16, inter_dim=512, moe_inter_dim=64, n_routed_experts=64, top_k=4,
+                vocab_size=1024, max_seq_len=512)
+TINY_MOE_BATCH, TINY_MOE_SEQ = 16, 512
 
 
 def placement_code(p) -> str:
@@ -104,6 +111,13 @@ def make_graph(kind, mesh):
 
         model, input_fn, _, _ = build_model(kind, mesh, n_layers=1)
         return capture_joint_graph(model, input_fn, param_dtype=torch.bfloat16, device="cpu", dynamo=False)
+    if kind == "dsv3_moe_tiny":
+        from autoparallel_amd.graphs.dsv3 import DeepSeekV3Config
+        from autoparallel_amd.graphs.workloads import build_model
+
+        model, input_fn, _, _ = build_model("dsv3_moe", mesh, batch=TINY_MOE_BATCH, seq=TINY_MOE_SEQ,
+                                            config=DeepSeekV3Config(**TINY_MOE))
+        return capture_joint_graph(model, input_fn, param_dtype=torch.bfloat16, device="cpu", dynamo=True)
     from models import make_model_and_inputs
 
     model_fn, input_fn = make_model_and_inputs(mesh, kind)

@@ -3,7 +3,8 @@
 ``tests/golden/reference_strategies_and_costs.json`` holds, for every node of four traced graphs
 (the reference tests' FFN and transformer block on (32, 8); one decoder layer of Llama-3-8B on
 (32, 8) and of Llama-3-70B on (8, 8, 8), at the benchmark shapes; the transformer block with its attention inside a
-``local_map`` region on (8, 8, 4)):
+``local_map`` region on (8, 8, 4); a DeepSeek-V3 style dense + mixture-of-experts layer pair,
+widths divided down, on (64, 4)):
   * its strategy list, content and order, as the reference's ``get_placement_options`` /
     ``_create_all_options`` produce it (autoparallel/utils.py:154-192, propagation_rules.py);
   * for every strategy what the reference's ``estimate_strategy_runtime_cost``
@@ -58,6 +59,13 @@ def _planner(planner_cls, case):
         model, input_fn, _, _ = workloads.build_model(kind, mesh, n_layers=1)
         # no reduce dtype: the gradient rescale does not touch compute costs
         return planner_cls(model, input_fn, mesh, param_dtype=torch.bfloat16)
+    if kind == "dsv3_moe_tiny":
+        from autoparallel_amd.graphs.dsv3 import DeepSeekV3Config
+        from make_reference_vectors import TINY_MOE, TINY_MOE_BATCH, TINY_MOE_SEQ
+
+        model, input_fn, _, _ = workloads.build_model("dsv3_moe", mesh, batch=TINY_MOE_BATCH, seq=TINY_MOE_SEQ,
+                                                      config=DeepSeekV3Config(**TINY_MOE))
+        return planner_cls(model, input_fn, mesh, param_dtype=torch.bfloat16, dynamo=True)
     model_fn, input_fn = make_model_and_inputs(mesh, kind)
     with torch.device("meta"):
         model = model_fn()
