@@ -18,7 +18,6 @@ from dataclasses import dataclass, field
 import numpy as np
 import torch
 from torch.distributed.tensor._dtensor_spec import DTensorSpec
-from torch.utils._pytree import tree_flatten
 
 from .._native import APC_MAX_RANK
 from ..encoding import (EDGE_GRAD_RESCALE, EDGE_NO_PRODUCER, PARTIAL_OPS, CostTables, pack_codes, partial_code,
@@ -54,8 +53,23 @@ class PlacementCoder:
 
 
 def all_input_nodes(node) -> list:
-    """node.all_input_nodes with duplicates kept, args only (optimize_sharding.py:382-387)."""
-    return [x for x in tree_flatten(node.args)[0] if isinstance(x, torch.fx.Node)]
+    """node.all_input_nodes with duplicates kept, args only (optimize_sharding.py:382-387):
+    the Nodes among the leaves of ``tree_flatten(node.args)``, in that order.  (Walked by hand:
+    the planner asks this several times per node, and a pytree flatten is ten times the work.)"""
+    out: list = []
+
+    def walk(x):
+        if isinstance(x, torch.fx.Node):
+            out.append(x)
+        elif isinstance(x, (tuple, list)):
+            for y in x:
+                walk(y)
+        elif isinstance(x, dict):
+            for y in x.values():
+                walk(y)
+
+    walk(node.args)
+    return out
 
 
 @dataclass
