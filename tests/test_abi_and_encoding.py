@@ -136,6 +136,34 @@ def test_deduplicated_tiles_write_every_entry_exactly_once():
     assert int((other.edge_canonical != np.arange(other.n_edges)).sum()) < n_dup
 
 
+def test_row_minimum_entry_points_reject_incomplete_arguments():
+    """Argument checks of apc_*_row_min run on the host before anything is launched: a NULL
+    descriptor, a descriptor without its arrays, and row minima without all three outputs."""
+    import ctypes
+
+    lib = _native.lib()
+    p = CostModelParams.from_mesh((4, 2)).to_c()
+    one = ctypes.c_void_p(8)  # a non-NULL placeholder: every call below fails before it is read
+    tables = (ctypes.byref(p), one, one, one, one, None, one, ctypes.c_int64(1), one, None, ctypes.c_int64(1))
+
+    def error_of(rc):
+        assert rc != 0
+        return lib.apc_last_error().decode()
+
+    assert "NULL rows" in error_of(lib.apc_redistribute_tables_row_min(*tables, one, one, one, None, None))
+    empty = _native.ApcRowMinima(None, None, None, None)
+    assert "NULL row-minimum array" in error_of(
+        lib.apc_redistribute_tables_row_min(*tables, one, one, one, ctypes.byref(empty), None))
+    rows = _native.ApcRowMinima(one, None, one, one)
+    assert "need comm_out, transition_out and cost_out" in error_of(
+        lib.apc_redistribute_tables_row_min(*tables, one, None, one, ctypes.byref(rows), None))
+    with_dups = tables[:9] + (one,) + tables[10:]
+    assert "dup_row_begin" in error_of(
+        lib.apc_redistribute_tables_row_min(*with_dups, one, one, one, ctypes.byref(rows), None))
+    assert "NULL selection" in error_of(lib.apc_segmented_min_copies(
+        one, one, ctypes.c_int64(3), None, None, None, ctypes.c_int64(9), one, one, None))
+
+
 def test_row_copies_cover_every_row_once_and_pair_identical_rows():
     """``row_copies``: the rows of the tiled edges plus their copies are every matrix row exactly
     once; a copy is the same consumer strategy of an identical edge; rows are numbered as in
