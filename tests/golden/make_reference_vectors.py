@@ -50,6 +50,7 @@ CASES = [
     ("block_32x8", "block", (32, 8)),
     ("llama3_8b_1layer_32x8", "llama3_8b", (32, 8)),
     ("llama3_70b_1layer_8x8x8", "llama3_70b", (8, 8, 8)),
+    ("block_1k_64", "block_1k", (64,)),  # the single transformer block of the CPU-runnable configuration
     ("local_map_block_8x8x4", "local_map_block", (8, 8, 4)),  # attention inside a local_map region
     ("dsv3_moe_tiny_64x4", "dsv3_moe_tiny", (64, 4)),  # one dense and one mixture-of-experts layer, widths divided down
 ]
@@ -105,11 +106,12 @@ def node_signature(node) -> str:
 def make_graph(kind, mesh):
     from autoparallel_amd.graphs.capture import capture_joint_graph
 
-    if kind.startswith("llama3"):
+    if kind.startswith("llama3") or kind == "block_1k":
         # one decoder layer of the benchmark model at its full shapes, bf16 parameter casts
+        # (block_1k: batch 64 instead of 8, so that it divides the 64 ranks)
         from autoparallel_amd.graphs.workloads import build_model
 
-        model, input_fn, _, _ = build_model(kind, mesh, n_layers=1)
+        model, input_fn, _, _ = build_model(kind, mesh, n_layers=1, batch=64 if kind == "block_1k" else None)
         return capture_joint_graph(model, input_fn, param_dtype=torch.bfloat16, device="cpu", dynamo=False)
     if kind == "dsv3_moe_tiny":
         from autoparallel_amd.graphs.dsv3 import DeepSeekV3Config

@@ -2,7 +2,8 @@
 
 ``tests/golden/reference_strategies_and_costs.json`` holds, for every node of four traced graphs
 (the reference tests' FFN and transformer block on (32, 8); one decoder layer of Llama-3-8B on
-(32, 8) and of Llama-3-70B on (8, 8, 8), at the benchmark shapes; the transformer block with its attention inside a
+(32, 8) and of Llama-3-70B on (8, 8, 8), at the benchmark shapes; the single block of the CPU-runnable configuration on
+(64,); the transformer block with its attention inside a
 ``local_map`` region on (8, 8, 4); a DeepSeek-V3 style dense + mixture-of-experts layer pair,
 widths divided down, on (64, 4)):
   * its strategy list, content and order, as the reference's ``get_placement_options`` /
@@ -55,8 +56,8 @@ class OraclePlanner(AutoParallelPlanner):
 def _planner(planner_cls, case):
     kind, mesh_sizes = case["kind"], tuple(case["mesh"])
     mesh = workloads.logical_mesh(mesh_sizes)
-    if kind.startswith("llama3"):
-        model, input_fn, _, _ = workloads.build_model(kind, mesh, n_layers=1)
+    if kind.startswith("llama3") or kind == "block_1k":
+        model, input_fn, _, _ = workloads.build_model(kind, mesh, n_layers=1, batch=64 if kind == "block_1k" else None)
         # no reduce dtype: the gradient rescale does not touch compute costs
         return planner_cls(model, input_fn, mesh, param_dtype=torch.bfloat16)
     if kind == "dsv3_moe_tiny":
