@@ -328,7 +328,7 @@ def main():
                      "avg_launch_us": t_kernel * 1e6,
                      "avg_launch_us_event_pair_per_launch": t_kernel_pair * 1e6,
                      "frac_event_pair_per_launch": alg_bytes / t_kernel_pair / 1e9 / HBM_PEAK_GBPS,
-                     "min_launch_us": kernel_ms_min[main] * 1e3,
+                     "min_launch_us_event_pair_per_launch": kernel_ms_min[main] * 1e3,
                      "timing": ("one HIP event pair on the launch stream around the K back-to-back launches of the timed "
                                 "region (the pass is this one kernel), / K" if single_kernel_pass else
                                 "HIP events around every launch of the kernel inside the timed region")},
