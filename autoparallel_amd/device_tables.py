@@ -372,11 +372,16 @@ class DeviceCostTables:
         tb = self.tables
         if tb.dup_entry_begin is None or len(tb.dup_entry_begin) == 0:
             return None
+        cached = getattr(self, "_row_copies_cache", None)
+        if cached is not None and cached[0] is tb.tile_records:  # (a new tiling packs new records)
+            return cached[1]
         selected, copy_ptr, copy_rows, n_read = tb.row_copies()
-        if n_read > 0.75 * tb.n_entries:
-            return None
-        return (_to_device(selected, self.device), _to_device(copy_ptr, self.device),
-                _to_device(copy_rows, self.device), n_read)
+        out = None
+        if n_read <= 0.75 * tb.n_entries:
+            out = (_to_device(selected, self.device), _to_device(copy_ptr, self.device),
+                   _to_device(copy_rows, self.device), n_read)
+        self._row_copies_cache = (tb.tile_records, out)
+        return out
 
     @_guarded
     def row_minima(self):
@@ -398,8 +403,7 @@ class DeviceCostTables:
                                                    self._p(selected), self._p(copy_ptr), self._p(copy_rows),
                                                    ctypes.c_int64(n_read), self._p(mins), self._p(args), self._stream())
         _native.check(rc, "apc_segmented_min_copies")
-        torch.cuda.current_stream(self.device).synchronize()  # the index arrays die with this frame
-        return mins, args
+        return mins, args  # (the index arrays stay cached with the tables)
 
     @_guarded
     def segmented_min(self, values: torch.Tensor, seg_ptr, check: bool = True):
