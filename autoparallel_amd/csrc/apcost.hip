@@ -1110,28 +1110,29 @@ __device__ __forceinline__ void redistribute_tile(const apc_params &p, const Tab
   tile_entries<M, false>(p, a, stage, view_of(tile), threadIdx.x, kTileThreads);
 }
 
-template <int M, int kTileThreads>
-__global__ __launch_bounds__(kTileThreads) void redistribute_tiles_kernel(apc_params p, TableArgs a, int n_tiles,
-                                                                          int xcd_shift) {
-  __shared__ TileStage<M, false> s_stage;
-  redistribute_tile<M, kTileThreads, false>(p, a, n_tiles, xcd_shift, s_stage);
-}
-
-// Wavefronts per SIMD the row-minimum tile kernel asks for: what its LDS use leaves room for
-// (one-wavefront workgroups and 4-D meshes hold more LDS per wavefront).
-constexpr int row_min_waves_per_simd(int mesh_ndim, int threads) {
+// Wavefronts per SIMD the tile kernels ask for: what the LDS of their larger, row-minimum
+// instantiation leaves room for (one-wavefront workgroups and 4-D meshes hold more LDS per
+// wavefront).  Asked for explicitly because the compiler sizes its register budget by the LDS
+// use otherwise: the row-minimum kernel got 97 registers and 4 wavefronts on a 3-D mesh where 67
+// registers do without spilling (stress table 2.94 -> 2.58 ms); the kernel without the minima
+// gains 1 - 2 % (same box: stress 1.93 -> 1.88 ms, Llama-3-70B 251 -> 248 us).
+constexpr int tile_waves_per_simd(int mesh_ndim, int threads) {
   if (mesh_ndim >= 4) return threads >= 256 ? 4 : threads >= 128 ? 3 : 2;
   if (threads < 128) return mesh_ndim <= 1 ? 7 : mesh_ndim == 2 ? 6 : 4;
   return 7;
 }
 
-// The same with the row minima.  Occupancy is asked for explicitly: left alone, the compiler
-// sizes this kernel's register budget by the LDS it uses, 97 registers and 4 wavefronts per
-// SIMD on a 3-D mesh, where 67 registers do without spilling and 7 wavefronts fit (stress
-// table: 2.58 ms against 2.94 ms).
+template <int M, int kTileThreads>
+__global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads), 8)))
+void redistribute_tiles_kernel(apc_params p, TableArgs a, int n_tiles, int xcd_shift) {
+  __shared__ TileStage<M, false> s_stage;
+  redistribute_tile<M, kTileThreads, false>(p, a, n_tiles, xcd_shift, s_stage);
+}
+
+// The same with the row minima.
 template <int M, int kTileThreads>
 __global__ __launch_bounds__(kTileThreads)
-__attribute__((amdgpu_waves_per_eu(row_min_waves_per_simd(M, kTileThreads), 8)))
+__attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads), 8)))
 void redistribute_tiles_row_min_kernel(apc_params p, TableArgs a, int n_tiles, int xcd_shift) {
   __shared__ TileStage<M, true> s_stage;
   redistribute_tile<M, kTileThreads, true>(p, a, n_tiles, xcd_shift, s_stage);
