@@ -37,6 +37,8 @@ MEASURED_TRAFFIC_BYTES = {
     (1_821_368, 1_616, 73_586_428): (3_142.9 * 2.000 + 68_599.2) * 1024,           # llama3_8b, mesh (32, 8), all tables and the row minima in one launch
     (1_821_368, 1_616, 71_794_420): (3_037.5 * 2.000 + 65_983.1) * 1024,           # the same, --row-min separate
     (1_821_368, 1_616, 32_348_914): (670.7 * 2.000 + 31_445.9) * 1024,             # the same, --table-launches 2
+    (1_073_460, 1_387, 47_179_580): (2_310.1 * 2.000 + 43_498.1) * 1024,            # dsv3_moe, mesh (64, 4)
+    (2_986, 129, 374_304): (249.0 * 2.000 + 317.4) * 1024,                          # block_1k, mesh (64,)
     (73_251_434, 40_727, 1_255_915_920): (12_322.6 * 2.000 + 1_221_016.0) * 1024,   # llama3_70b, mesh (8, 8, 8)
     (464_235_576, 426_918, 8_178_099_438): (165_040.2 * 2.000 + 7_953_223.0) * 1024,  # stress, mesh (16, 8, 4), row minima in the tiles
     (464_235_576, 426_918, 8_003_825_874): (159_776.0 * 2.000 + 7_760_473.5) * 1024,  # the same, --row-min separate
