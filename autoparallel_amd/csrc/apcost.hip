@@ -1146,8 +1146,13 @@ void redistribute_tiles_row_min_kernel(apc_params p, TableArgs a, int n_tiles, i
 // table workgroups use (TableArgs), so the values are the same bits.  One launch instead of
 // two spares a table of a few tens of MB one ramp-up and one drain of the chip, which at that
 // size are a third of each kernel.
+// (Wavefronts per SIMD are capped at 5 on 1-D and 2-D meshes: with more resident, the launch's
+// many store streams hinder each other a little.  Llama-3-8B table, each pair on one box:
+// 18.5 us against 18.9 us uncapped, 18.7 us against 18.8 us on another box; capped at 6 as
+// uncapped; 20.3 us capped at 3 or when asked for 8.  The mixture-of-experts table: no change.)
 template <int M, int kThreads, bool RM>
-__global__ __launch_bounds__(kThreads) void build_tables_kernel(apc_params p, TableArgs a, TensorTableArgs t,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(M <= 2 ? 5 : 1, M <= 2 ? 5 : 8)))
+void build_tables_kernel(apc_params p, TableArgs a, TensorTableArgs t,
                                                                 SpecTableArgs sp, ComputeCostArgs c, int n_tiles,
                                                                 int64_t tile_blocks, int64_t spec_blocks,
                                                                 int64_t tensor_blocks, int xcd_shift) {
