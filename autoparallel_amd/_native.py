@@ -77,6 +77,8 @@ EXPORTS = (
     "apc_segmented_min",
     "apc_segmented_min_copies",
     "apc_strategy_bounds",
+    "apc_cost_objective",
+    "apc_validate_row_minima_host",
 )
 
 _lib = None

@@ -820,20 +820,28 @@ struct TileOut {
   int64_t entry_begin;  // first entry of the tile's edge (an identical edge's values sit at its own first entry)
 };
 
-// Stores one entry's values to its edge and to every identical edge.  ALL: every output
-// array is present (no per-store checks).
-template <bool ALL>
+// Which of the three per-entry output arrays a launch writes, as a compile-time choice of the
+// kernel (no per-store checks, and the registers of streams that are not written are free):
+// the planner's table build wants the assembled cost alone (what the ILP objective is summed
+// from, optimize_sharding.py:650-655; comm and transition are fetched by a later launch only
+// if a report asks for them), a caller that wants every array gets all three, any other subset
+// is checked per store.
+enum : int { kOutAny = 0, kOutAll = 1, kOutCost = 2 };
+
+// Stores one entry's values to its edge and to every identical edge.
+template <int OUT>
 __device__ __forceinline__ void store_entry(const TileOut &o, int dup_count, const int64_t *s_dup, uint32_t local,
                                             double comm, double total, int trans) {
+  constexpr bool ALL = OUT == kOutAll, COST = OUT == kOutCost;
   const uint32_t off8 = local * 8u;
-  if (ALL || o.comm) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.comm) + off8) = comm;
-  if (ALL || o.trans) o.trans[local] = (uint8_t)trans;
-  if (ALL || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost) + off8) = total;
+  if (ALL || (!COST && o.comm)) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.comm) + off8) = comm;
+  if (ALL || (!COST && o.trans)) o.trans[local] = (uint8_t)trans;
+  if (ALL || COST || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost) + off8) = total;
   for (int d = 0; d < dup_count; ++d) {
     const int64_t delta = uniform_i64(s_dup[d]) - o.entry_begin;
-    if (ALL || o.comm) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.comm + delta) + off8) = comm;
-    if (ALL || o.trans) (o.trans + delta)[local] = (uint8_t)trans;
-    if (ALL || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost + delta) + off8) = total;
+    if (ALL || (!COST && o.comm)) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.comm + delta) + off8) = comm;
+    if (ALL || (!COST && o.trans)) (o.trans + delta)[local] = (uint8_t)trans;
+    if (ALL || COST || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost + delta) + off8) = total;
   }
 }
 
@@ -931,7 +939,7 @@ __device__ __forceinline__ void row_min_finish(const TableArgs &a, TileStage<M, 
 // uniform_tile_entries, except that every lane of a wavefront makes the same number of
 // passes (a lane in front of the tile's first entry idles in the first pass instead of
 // wrapping round), so that the lanes of one pass hold consecutive entries.
-template <int M, bool CONT, bool RESCALE>
+template <int M, bool CONT, bool RESCALE, int OUT>
 __device__ __forceinline__ void uniform_tile_entries_row_min(const apc_params &p, const TableArgs &a, TileStage<M, true> &st,
                                                              const TileView &v, int tid, int nthreads) {
   const int n = v.rows * v.cols;
@@ -942,15 +950,16 @@ __device__ __forceinline__ void uniform_tile_entries_row_min(const apc_params &p
   int idx = tid - shift;
   const int first = idx < 0 ? idx + nthreads : idx;
   int r = first / v.cols, c = first - r * v.cols;
-  const TileOut out{a.comm_out + tile_base, a.trans_out + tile_base, a.cost_out + tile_base, v.entry_begin};
+  const TileOut out{a.comm_out ? a.comm_out + tile_base : nullptr, a.trans_out ? a.trans_out + tile_base : nullptr,
+                    a.cost_out ? a.cost_out + tile_base : nullptr, v.entry_begin};
   for (int wave_first = tid - lane - shift; wave_first < n; wave_first += nthreads, idx += nthreads) {
     const bool active = idx >= 0 && idx < n;
     double comm, total = 0.0;
     int trans;
     if (active) {
       uniform_entry<M, CONT, RESCALE>(p, st, r, c, comm, total, trans);
-      store_entry<true>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
-                        trans);
+      store_entry<OUT>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
+                       trans);
     }
     row_min_chunk(st.rmin, st.rarg, active, total, r, c, v.cols, lane);
     if (active) {
@@ -967,7 +976,7 @@ __device__ __forceinline__ void uniform_tile_entries_row_min(const apc_params &p
 
 // The per-entry loop of such a tile for `nthreads` threads (this one is `tid`): a flattened
 // (row, column) walk, so a wavefront writes 64 consecutive entries.
-template <int M, bool CONT, bool RESCALE, bool ALL, bool RM>
+template <int M, bool CONT, bool RESCALE, int OUT, bool RM>
 __device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M, RM> &st,
                                                      const TileView &v, int tid, int nthreads) {
   const int n = v.rows * v.cols;
@@ -985,7 +994,7 @@ __device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const 
     double comm, total;
     int trans;
     uniform_entry<M, CONT, RESCALE>(p, st, r, c, comm, total, trans);
-    store_entry<ALL>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
+    store_entry<OUT>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
                      trans);
     c += dc;
     r += dr;
@@ -1059,13 +1068,12 @@ __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const 
 
 // All entries of a staged tile.  Row minima are taken when the caller wants them and the tile
 // holds whole rows (which the host arranges for every tile of a table before asking).
-template <int M, bool DERIVE, bool RM>
+template <int M, bool DERIVE, bool RM, int OUT>
 __device__ __forceinline__ void tile_entries(const apc_params &p, const TableArgs &a, TileStage<M, RM> &st,
                                              const TileView &v, int tid, int nthreads) {
   int mixed = st.mixed[0];
   for (int w = 1; w < nthreads / 64; ++w) mixed |= st.mixed[w];
-  const bool all = a.comm_out && a.trans_out && a.cost_out;
-  const bool row_minima = RM && all && v.cols == v.n_src;
+  const bool row_minima = RM && v.cols == v.n_src;
   if (uniform_i32(mixed)) {
     if constexpr (RM) {
       if (row_minima) {
@@ -1081,12 +1089,11 @@ __device__ __forceinline__ void tile_entries(const apc_params &p, const TableArg
   do {                                                                                            \
     if constexpr (RM) {                                                                           \
       if (row_minima) {                                                                           \
-        uniform_tile_entries_row_min<M, CONT_, RESCALE_>(p, a, st, v, tid, nthreads);             \
+        uniform_tile_entries_row_min<M, CONT_, RESCALE_, OUT>(p, a, st, v, tid, nthreads);        \
         break;                                                                                    \
       }                                                                                           \
     }                                                                                             \
-    if (all) uniform_tile_entries<M, CONT_, RESCALE_, true>(p, a, st, v, tid, nthreads);          \
-    else uniform_tile_entries<M, CONT_, RESCALE_, false>(p, a, st, v, tid, nthreads);             \
+    uniform_tile_entries<M, CONT_, RESCALE_, OUT>(p, a, st, v, tid, nthreads);                    \
   } while (0)
   if (uniform_i32(st.cont)) {
     if (rescale) { APC_TILE_LOOP(true, true); } else { APC_TILE_LOOP(true, false); }
@@ -1096,7 +1103,7 @@ __device__ __forceinline__ void tile_entries(const apc_params &p, const TableArg
 #undef APC_TILE_LOOP
 }
 
-template <int M, int kTileThreads, bool RM>
+template <int M, int kTileThreads, bool RM, int OUT>
 __device__ __forceinline__ void redistribute_tile(const apc_params &p, const TableArgs &a, int n_tiles, int xcd_shift,
                                                   TileStage<M, RM> &stage) {
   const int64_t tile_id = xcd_chunked_unit(xcd_shift);
@@ -1105,9 +1112,9 @@ __device__ __forceinline__ void redistribute_tile(const apc_params &p, const Tab
   static_assert(kTileThreads >= APC_TILE_MAX_COLS && kTileThreads >= APC_TILE_MAX_ROWS &&
                 2 * kTileThreads > APC_TILE_MAX_DUPS, "one staging round covers a tile");
   const apc_tile tile = a.tiles[tile_id];
-  stage_tile<M, false>(p, a, tile, stage, threadIdx.x, kTileThreads);
+  stage_tile<M, false, RM>(p, a, tile, stage, threadIdx.x, kTileThreads);
   __syncthreads();
-  tile_entries<M, false>(p, a, stage, view_of(tile), threadIdx.x, kTileThreads);
+  tile_entries<M, false, RM, OUT>(p, a, stage, view_of(tile), threadIdx.x, kTileThreads);
 }
 
 // Wavefronts per SIMD the tile kernels ask for: what the LDS of their larger, row-minimum
@@ -1122,20 +1129,20 @@ constexpr int tile_waves_per_simd(int mesh_ndim, int threads) {
   return 7;
 }
 
-template <int M, int kTileThreads>
+template <int M, int kTileThreads, int OUT>
 __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads), 8)))
 void redistribute_tiles_kernel(apc_params p, TableArgs a, int n_tiles, int xcd_shift) {
   __shared__ TileStage<M, false> s_stage;
-  redistribute_tile<M, kTileThreads, false>(p, a, n_tiles, xcd_shift, s_stage);
+  redistribute_tile<M, kTileThreads, false, OUT>(p, a, n_tiles, xcd_shift, s_stage);
 }
 
 // The same with the row minima.
-template <int M, int kTileThreads>
+template <int M, int kTileThreads, int OUT>
 __global__ __launch_bounds__(kTileThreads)
 __attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads), 8)))
 void redistribute_tiles_row_min_kernel(apc_params p, TableArgs a, int n_tiles, int xcd_shift) {
   __shared__ TileStage<M, true> s_stage;
-  redistribute_tile<M, kTileThreads, true>(p, a, n_tiles, xcd_shift, s_stage);
+  redistribute_tile<M, kTileThreads, true, OUT>(p, a, n_tiles, xcd_shift, s_stage);
 }
 
 // Every table of a pass in one launch: workgroups [0, tile_blocks) take the tiles of the
@@ -1150,7 +1157,7 @@ void redistribute_tiles_row_min_kernel(apc_params p, TableArgs a, int n_tiles, i
 // many store streams hinder each other a little.  Llama-3-8B table, each pair on one box:
 // 18.5 us against 18.9 us uncapped, 18.7 us against 18.8 us on another box; capped at 6 as
 // uncapped; 20.3 us capped at 3 or when asked for 8.  The mixture-of-experts table: no change.)
-template <int M, int kThreads, bool RM>
+template <int M, int kThreads, bool RM, int OUT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(M <= 2 ? 5 : 1, M <= 2 ? 5 : 8)))
 void build_tables_kernel(apc_params p, TableArgs a, TensorTableArgs t,
                                                                 SpecTableArgs sp, ComputeCostArgs c, int n_tiles,
@@ -1167,9 +1174,9 @@ void build_tables_kernel(apc_params p, TableArgs a, TensorTableArgs t,
     if (tile_id >= n_tiles) return;
     TileStage<M, RM> &stage = *reinterpret_cast<TileStage<M, RM> *>(s_raw);
     const apc_tile tile = a.tiles[tile_id];
-    stage_tile<M, true>(p, a, tile, stage, threadIdx.x, kThreads);
+    stage_tile<M, true, RM>(p, a, tile, stage, threadIdx.x, kThreads);
     __syncthreads();
-    tile_entries<M, true>(p, a, stage, view_of(tile), threadIdx.x, kThreads);
+    tile_entries<M, true, RM, OUT>(p, a, stage, view_of(tile), threadIdx.x, kThreads);
     return;
   }
   const int64_t tb = b - tile_blocks;
@@ -1303,6 +1310,46 @@ __global__ __launch_bounds__(kBlock) void strategy_bounds_kernel(int64_t n_strat
   double sum = 0.0;
   for (int64_t j = node_edge_begin[n]; j < node_edge_begin[n + 1]; ++j) sum += row_min[edge_row_begin[edges_by_node[j]] + k];
   bound[s] = sum;
+}
+
+// ------------------------------------------------------------------------------------------
+// The ILP objective, summed on the device.  Entries of linked nodes share an ILP variable
+// (optimize_sharding.py:211-231) and the objective coefficient of a variable is the sum of the
+// costs of its entries, added one by one in entry order starting from 0
+// (optimize_sharding.py:650-655: opt_target[va] += cost over ds.values()); a cost that is not
+// finite counts as inf_replacement and forces the variable to 0 (:522-536).  Variables are
+// numbered group by group: a group is a set of edges with matrices of the same shape whose
+// entries share variables position by position (one edge when nothing is linked); variable
+// group_var_begin[g] + k sums entry k of every member edge, members in ascending entry order.
+// One thread per variable: neighbouring lanes read neighbouring entries of each member.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void cost_objective_kernel(int64_t n_vars, int64_t n_groups,
+                                                                const int64_t *__restrict__ group_var_begin,
+                                                                const int64_t *__restrict__ group_member_begin,
+                                                                const int64_t *__restrict__ member_entry_begin,
+                                                                const double *__restrict__ cost, double inf_replacement,
+                                                                double *__restrict__ objective,
+                                                                uint8_t *__restrict__ forced_zero) {
+  const int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (v >= n_vars) return;
+  int64_t lo = 0, hi = n_groups;  // last group whose first variable is <= v
+  while (hi - lo > 1) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (group_var_begin[mid] <= v) lo = mid; else hi = mid;
+  }
+  const int64_t k = v - group_var_begin[lo];
+  double sum = 0.0;
+  bool forced = false;
+  for (int64_t m = group_member_begin[lo], end = group_member_begin[lo + 1]; m < end; ++m) {
+    double c = cost[member_entry_begin[m] + k];
+    if (!(__builtin_fabs(c) < __builtin_inf())) {  // inf or nan: math.isfinite is false
+      c = inf_replacement;
+      forced = true;
+    }
+    sum += c;
+  }
+  objective[v] = sum;
+  forced_zero[v] = forced ? 1 : 0;
 }
 
 inline unsigned blocks_for(int64_t n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
@@ -1496,16 +1543,20 @@ int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t 
                      const int8_t *dtype, const uint8_t *zero_cost, const int32_t *num_args, double *compute,
                      double *per_arg, int32_t *error_flag, void *stream) {
   if (int rc = check_params(params)) return rc;
-  if (int rc = check_width(shape_width)) return rc;
   if (n_tensors < 0 || n_specs < 0 || n_strategies < 0) return fail(-1, "apc_input_tables: negative count");
   if (n_tensors > 0 && (!rank || !itemsize || !shape || !stride || !tensor_bytes || !tensor_contiguous))
     return fail(-1, "apc_input_tables: NULL tensor array");
-  if (n_specs > 0 && (!spec_codes || !spec_tensor || !rank || !itemsize || !shape || !stride || !num_shards ||
-                      !local_shape || !local_stride || !local_numel || !local_bytes))
-    return fail(-1, "apc_input_tables: NULL spec array");
+  // the five spec-table outputs may all be NULL: the spec table is then skipped
+  const bool spec_table = num_shards || local_shape || local_stride || local_numel || local_bytes;
+  if (spec_table)
+    if (int rc = check_width(shape_width)) return rc;
+  if (spec_table && n_specs > 0 && (!spec_codes || !spec_tensor || !rank || !itemsize || !shape || !stride ||
+                                    !num_shards || !local_shape || !local_stride || !local_numel || !local_bytes))
+    return fail(-1, "apc_input_tables: the spec table needs all five of its outputs");
   if (n_strategies > 0 && (!flops || !rw_bytes || !dtype || !zero_cost || !num_args))
     return fail(-1, "apc_input_tables: NULL strategy array");
-  const int64_t sb = blocks_for(n_specs, kBlock), tb = blocks_for(n_tensors, kBlock), cb = blocks_for(n_strategies, kBlock);
+  const int64_t sb = spec_table ? blocks_for(n_specs, kBlock) : 0, tb = blocks_for(n_tensors, kBlock),
+                cb = blocks_for(n_strategies, kBlock);
   if (sb + tb + cb == 0) return 0;
   if (sb + tb + cb > INT32_MAX) return fail(-1, "apc_input_tables: too many rows for one launch");
   hipLaunchKernelGGL(input_tables_kernel, dim3((unsigned)(sb + tb + cb)), dim3(kBlock), 0, (hipStream_t)stream, *params,
@@ -1520,14 +1571,21 @@ int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t 
 
 }  // extern "C"
 
-// Row minima need all three outputs and, when some tile serves identical edges, their rows.
-static int check_row_minima(const apc_row_minima *rows, const double *comm_out, const uint8_t *trans_out,
-                            const double *cost_out, const int64_t *dup_entry_begin, const char *who) {
+// Row minima need their index arrays and, when some tile serves identical edges, those edges' rows.
+static int check_row_minima(const apc_row_minima *rows, const int64_t *dup_entry_begin, const char *who) {
   if (!rows) return 0;
   if (!rows->edge_row_begin || !rows->row_min || !rows->row_argmin) return fail(-1, "%s: NULL row-minimum array", who);
   if (dup_entry_begin && !rows->dup_row_begin) return fail(-1, "%s: identical edges need dup_row_begin", who);
-  if (!comm_out || !trans_out || !cost_out) return fail(-1, "%s: row minima need comm_out, transition_out and cost_out", who);
   return 0;
+}
+
+// The compile-time output mode of a launch (kOut*).  The specialised modes exist for 2-D and
+// 3-D meshes (the planned graphs); other mesh ranks check their output pointers per store.
+static int out_mode(int mesh_ndim, const double *comm_out, const uint8_t *trans_out, const double *cost_out) {
+  if (mesh_ndim != 2 && mesh_ndim != 3) return kOutAny;
+  if (comm_out && trans_out && cost_out) return kOutAll;
+  if (cost_out && !comm_out && !trans_out) return kOutCost;
+  return kOutAny;
 }
 
 static int redistribute_tables_impl(const apc_params *params, const int64_t *tensor_bytes,
@@ -1539,8 +1597,7 @@ static int redistribute_tables_impl(const apc_params *params, const int64_t *ten
   if (int rc = check_params(params)) return rc;
   if (n_tiles < 0 || n_tiles > (1 << 30)) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tiles == 0) return 0;
-  if (int rc = check_row_minima(rows, comm_out, trans_out, cost_out, dup_entry_begin, "apc_redistribute_tables_row_min"))
-    return rc;
+  if (int rc = check_row_minima(rows, dup_entry_begin, "apc_redistribute_tables_row_min")) return rc;
   if (n_entries < 0) return fail(-1, "n_entries < 0");
   if (!tensor_bytes || !tensor_contiguous || !spec_codes || !spec_tensor || !tiles)
     return fail(-1, "apc_redistribute_tables: NULL table");
@@ -1560,20 +1617,34 @@ static int redistribute_tables_impl(const apc_params *params, const int64_t *ten
   const int64_t per_tile = n_entries / n_tiles;
   int threads = per_tile >= 1536 ? 256 : per_tile >= 512 ? 128 : 64;
   if (const char *env = getenv("APC_TILE_THREADS")) threads = atoi(env);  // tuning override
-#define APC_LAUNCH_K(KERNEL_, M_)                                                                               \
-  if (threads >= 256) hipLaunchKernelGGL((KERNEL_<M_, 256>), grid, dim3(256), 0, s, *params, a, nt, xs);            \
-  else if (threads >= 128) hipLaunchKernelGGL((KERNEL_<M_, 128>), grid, dim3(128), 0, s, *params, a, nt, xs);       \
-  else hipLaunchKernelGGL((KERNEL_<M_, 64>), grid, dim3(64), 0, s, *params, a, nt, xs)
-#define APC_LAUNCH(M_)                        \
-  if (rows) { APC_LAUNCH_K(redistribute_tiles_row_min_kernel, M_); } else { APC_LAUNCH_K(redistribute_tiles_kernel, M_); }
-  switch (params->mesh_ndim) {
-    case 1: APC_LAUNCH(1); break;
-    case 2: APC_LAUNCH(2); break;
-    case 3: APC_LAUNCH(3); break;
-    default: APC_LAUNCH(4); break;
+  const int om = out_mode(params->mesh_ndim, comm_out, trans_out, cost_out);
+#define APC_LAUNCH_T(KERNEL_, M_, OUT_)                                                                              \
+  if (threads >= 256) hipLaunchKernelGGL((KERNEL_<M_, 256, OUT_>), grid, dim3(256), 0, s, *params, a, nt, xs);       \
+  else if (threads >= 128) hipLaunchKernelGGL((KERNEL_<M_, 128, OUT_>), grid, dim3(128), 0, s, *params, a, nt, xs);  \
+  else hipLaunchKernelGGL((KERNEL_<M_, 64, OUT_>), grid, dim3(64), 0, s, *params, a, nt, xs)
+#define APC_LAUNCH_K(KERNEL_, M_)                                   \
+  if (om == kOutAll) { APC_LAUNCH_T(KERNEL_, M_, kOutAll); }        \
+  else if (om == kOutCost) { APC_LAUNCH_T(KERNEL_, M_, kOutCost); } \
+  else { APC_LAUNCH_T(KERNEL_, M_, kOutAny); }
+#define APC_LAUNCH_ANY(KERNEL_, M_) APC_LAUNCH_T(KERNEL_, M_, kOutAny)
+  if (rows) {
+    switch (params->mesh_ndim) {
+      case 1: APC_LAUNCH_ANY(redistribute_tiles_row_min_kernel, 1); break;
+      case 2: APC_LAUNCH_K(redistribute_tiles_row_min_kernel, 2); break;
+      case 3: APC_LAUNCH_K(redistribute_tiles_row_min_kernel, 3); break;
+      default: APC_LAUNCH_ANY(redistribute_tiles_row_min_kernel, 4); break;
+    }
+  } else {
+    switch (params->mesh_ndim) {
+      case 1: APC_LAUNCH_ANY(redistribute_tiles_kernel, 1); break;
+      case 2: APC_LAUNCH_K(redistribute_tiles_kernel, 2); break;
+      case 3: APC_LAUNCH_K(redistribute_tiles_kernel, 3); break;
+      default: APC_LAUNCH_ANY(redistribute_tiles_kernel, 4); break;
+    }
   }
+#undef APC_LAUNCH_T
 #undef APC_LAUNCH_K
-#undef APC_LAUNCH
+#undef APC_LAUNCH_ANY
   return check_launch("apc_redistribute_tables");
 }
 
@@ -1588,7 +1659,7 @@ static int build_tables_impl(const apc_params *params, int64_t n_tensors, const 
                      double *cost_out, const apc_row_minima *rows, void *stream) {
   if (int rc = check_params(params)) return rc;
   if (n_tiles > 0)
-    if (int rc = check_row_minima(rows, comm_out, trans_out, cost_out, dup_entry_begin, "apc_build_tables_row_min")) return rc;
+    if (int rc = check_row_minima(rows, dup_entry_begin, "apc_build_tables_row_min")) return rc;
   if (n_tensors < 0 || n_specs < 0 || n_strategies < 0 || n_entries < 0) return fail(-1, "apc_build_tables: negative count");
   if (n_tiles < 0 || n_tiles > (1 << 30)) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
   if (n_tensors > 0 && (!rank || !itemsize || !shape || !stride || !tensor_bytes || !tensor_contiguous))
@@ -1629,20 +1700,29 @@ static int build_tables_impl(const apc_params *params, int64_t n_tensors, const 
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)blocks);
   const int nt = (int)n_tiles;
-#define APC_LAUNCH_ALL_RM(M_, RM_)                                                                                      \
-  if (threads == 256) hipLaunchKernelGGL((build_tables_kernel<M_, 256, RM_>), grid, dim3(256), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
-  else if (threads == 128) hipLaunchKernelGGL((build_tables_kernel<M_, 128, RM_>), grid, dim3(128), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
-  else hipLaunchKernelGGL((build_tables_kernel<M_, 64, RM_>), grid, dim3(64), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs)
+  const int om = out_mode(params->mesh_ndim, comm_out, trans_out, cost_out);
+#define APC_LAUNCH_ALL_T(M_, RM_, OUT_)                                                                                 \
+  if (threads == 256) hipLaunchKernelGGL((build_tables_kernel<M_, 256, RM_, OUT_>), grid, dim3(256), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
+  else if (threads == 128) hipLaunchKernelGGL((build_tables_kernel<M_, 128, RM_, OUT_>), grid, dim3(128), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
+  else hipLaunchKernelGGL((build_tables_kernel<M_, 64, RM_, OUT_>), grid, dim3(64), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs)
+#define APC_LAUNCH_ALL_RM(M_, RM_)                                   \
+  if (om == kOutAll) { APC_LAUNCH_ALL_T(M_, RM_, kOutAll); }         \
+  else if (om == kOutCost) { APC_LAUNCH_ALL_T(M_, RM_, kOutCost); }  \
+  else { APC_LAUNCH_ALL_T(M_, RM_, kOutAny); }
 #define APC_LAUNCH_ALL(M_)                    \
   if (rows) { APC_LAUNCH_ALL_RM(M_, true); } else { APC_LAUNCH_ALL_RM(M_, false); }
+#define APC_LAUNCH_ALL_ANY(M_)                \
+  if (rows) { APC_LAUNCH_ALL_T(M_, true, kOutAny); } else { APC_LAUNCH_ALL_T(M_, false, kOutAny); }
   switch (params->mesh_ndim) {
-    case 1: APC_LAUNCH_ALL(1); break;
+    case 1: APC_LAUNCH_ALL_ANY(1); break;
     case 2: APC_LAUNCH_ALL(2); break;
     case 3: APC_LAUNCH_ALL(3); break;
-    default: APC_LAUNCH_ALL(4); break;
+    default: APC_LAUNCH_ALL_ANY(4); break;
   }
+#undef APC_LAUNCH_ALL_T
 #undef APC_LAUNCH_ALL_RM
 #undef APC_LAUNCH_ALL
+#undef APC_LAUNCH_ALL_ANY
   return check_launch("apc_build_tables");
 }
 
@@ -1752,6 +1832,40 @@ int apc_strategy_bounds(int64_t n_strategies, const int32_t *strat_node, const i
                      n_strategies, strat_node, node_strat_begin, node_edge_begin, edges_by_node, edge_row_begin, row_min,
                      bound);
   return check_launch("apc_strategy_bounds");
+}
+
+int apc_cost_objective(int64_t n_vars, int64_t n_groups, const int64_t *group_var_begin, const int64_t *group_member_begin,
+                       const int64_t *member_entry_begin, const double *cost, double inf_replacement, double *objective,
+                       uint8_t *forced_zero, void *stream) {
+  if (n_vars < 0 || n_groups < 0) return fail(-1, "apc_cost_objective: negative count");
+  if (n_vars == 0) return 0;
+  if (n_groups == 0) return fail(-1, "apc_cost_objective: %lld variables and no group", (long long)n_vars);
+  if (!group_var_begin || !group_member_begin || !member_entry_begin || !cost || !objective || !forced_zero)
+    return fail(-1, "apc_cost_objective: NULL array");
+  if ((n_vars + kBlock - 1) / kBlock > INT32_MAX) return fail(-1, "n_vars %lld too large", (long long)n_vars);
+  hipLaunchKernelGGL(cost_objective_kernel, dim3(blocks_for(n_vars, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, n_vars,
+                     n_groups, group_var_begin, group_member_begin, member_entry_begin, cost, inf_replacement, objective,
+                     forced_zero);
+  return check_launch("apc_cost_objective");
+}
+
+int apc_validate_row_minima_host(int64_t n_edges, const int32_t *edge_n_src, const int32_t *edge_n_tgt, int64_t n_tiles,
+                                 const apc_tile *tiles) {
+  if (n_edges < 0 || n_tiles < 0) return fail(-1, "apc_validate_row_minima_host: negative count");
+  if ((n_edges > 0 && (!edge_n_src || !edge_n_tgt)) || (n_tiles > 0 && !tiles))
+    return fail(-1, "apc_validate_row_minima_host: NULL array");
+  for (int64_t e = 0; e < n_edges; ++e)
+    if (edge_n_tgt[e] > 0 && (edge_n_src[e] < 1 || edge_n_src[e] > APC_TILE_MAX_COLS))
+      return fail(-2, "edge %lld: %d producer strategies; row minima inside the table launch need 1 .. %d", (long long)e,
+                  edge_n_src[e], APC_TILE_MAX_COLS);
+  for (int64_t t = 0; t < n_tiles; ++t) {
+    const apc_tile &tl = tiles[t];
+    if (tl.edge < 0 || tl.edge >= n_edges) return fail(-2, "tile %lld: edge %d out of range", (long long)t, tl.edge);
+    if (tl.col_begin != 0 || (tl.counts >> 16) != edge_n_src[tl.edge])
+      return fail(-2, "tile %lld: columns [%d, +%d) are not the whole rows of edge %d (%d columns)", (long long)t,
+                  tl.col_begin, tl.counts >> 16, tl.edge, edge_n_src[tl.edge]);
+  }
+  return 0;
 }
 
 }  // extern "C"

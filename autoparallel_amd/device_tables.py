@@ -192,10 +192,12 @@ class DeviceCostTables:
             self.run_compute_costs()
         self.alloc_outputs(comm, transition, cost)
         if row_min is None:
-            row_min = bool(comm and transition and cost) and self.row_min_in_tiles_pays()
+            row_min = self.row_min_in_tiles_pays()
+        if row_min:
+            self.tables.validate_row_minima()  # raises when some matrix row is spread over tiles
         self.row_min = self.row_argmin = None
         if row_min:
-            n_rows = int(self.tables.edge_n_tgt.astype(np.int64).sum())
+            n_rows = self.tables.n_rows
             self.row_min = self._empty((n_rows,), torch.float64)
             self.row_argmin = self._empty((n_rows,), torch.int32)
         self.launch_redistribute_tables(row_min=bool(row_min))
@@ -230,8 +232,39 @@ class DeviceCostTables:
         computed = int((tb.tile_row_count.astype(np.int64) * tb.tile_col_count.astype(np.int64)).sum())
         return 0.5e-3 * tb.n_tiles + 1.0e-6 * computed < 4.0 + 8.0 * tb.n_entries / 4.5e6
 
+    def _alloc_input_tables(self, spec_table: bool):
+        """Allocates (does not fill) the outputs of the tensor, compute-cost and, when wanted,
+        spec tables."""
+        tb = self.tables
+        self.tensor_bytes = self._empty((tb.n_tensors,), torch.int64)
+        self.tensor_contiguous = self._empty((tb.n_tensors,), torch.uint8)
+        self.compute_cost = self._empty((tb.n_strategies,), torch.float64)
+        self.compute_cost_per_arg = self._empty((tb.n_strategies,), torch.float64)
+        if not spec_table:
+            return None
+        n, width = tb.n_specs, tb.shape_width()
+        self.spec_out = {
+            "num_shards": self._empty((n,), torch.int64),
+            "local_shape": self._empty((n, width), torch.int64),
+            "local_stride": self._empty((n, width), torch.int64),
+            "local_numel": self._empty((n,), torch.int64),
+            "local_bytes": self._empty((n,), torch.int64),
+        }
+        return self.spec_out
+
+    def pass_bytes(self, outputs=("comm", "transition", "cost"), spec_table=True, row_min_in_tiles=False) -> int:
+        """Bytes a pass with these outputs must move at minimum (what its launches write, plus
+        the spec lists and edge headers the tiles read)."""
+        tb = self.tables
+        total = tb.algorithmic_bytes(comm="comm" in outputs, transition="transition" in outputs, cost="cost" in outputs)
+        total += tb.algorithmic_bytes_input_tables(spec_table=spec_table)
+        if row_min_in_tiles:
+            total += 12 * tb.n_rows
+        return total
+
     @_guarded
-    def prepare_step(self, row_min=True, fused_inputs=False, one_launch=None, row_min_in_tiles=None):
+    def prepare_step(self, row_min=True, fused_inputs=False, one_launch=None, row_min_in_tiles=None,
+                     outputs=("comm", "transition", "cost"), spec_table=True):
         """Allocates every output once and returns ``{kernel name: zero-argument launcher}``
         in launch order.  A launcher only enqueues (no allocation, no synchronisation), so a
         timed loop measures the kernels and not Python argument marshalling.  With
@@ -241,31 +274,42 @@ class DeviceCostTables:
         ``ONE_LAUNCH_MAX_BYTES`` when ``fused_inputs`` is set.  ``row_min_in_tiles``: the launch
         that writes the cost matrices takes the row minima too (no ``segmented_min`` launch, no
         second read of the matrices); it needs every row inside one tile
-        (``CostTables.rows_fit_tiles``), and ``None`` takes it when ``row_min_in_tiles_pays``."""
+        (``CostTables.rows_fit_tiles``), and ``None`` takes it when ``row_min_in_tiles_pays``.
+        ``outputs``: which of the per-entry arrays the pass writes; ``spec_table=False`` leaves
+        the local shard shapes out (a planner has computed them before it could fill in the
+        flop / byte counts this pass reads)."""
+        outputs = tuple(outputs)
+        if not outputs or any(o not in ("comm", "transition", "cost") for o in outputs):
+            raise ValueError(f"outputs must name some of comm, transition, cost: {outputs}")
+        if not spec_table and not fused_inputs:
+            raise ValueError("a pass without the spec table is built with fused_inputs")
         fits = self.tables.rows_fit_tiles()
-        total = self.tables.algorithmic_bytes() + self.tables.algorithmic_bytes_input_tables()
         if row_min_in_tiles is None:
             row_min_in_tiles = self.row_min_in_tiles_pays()
         row_min_in_tiles = bool(row_min_in_tiles) and bool(row_min)
         if row_min_in_tiles and not fits:
             raise ValueError("row minima inside the table launch need every matrix row inside one tile")
+        if row_min and not row_min_in_tiles and "cost" not in outputs:
+            raise ValueError("a segmented_min launch over the rows reads the cost array: ask for it")
+        total = self.pass_bytes(outputs, spec_table, row_min_in_tiles)
         if one_launch is None:
             one_launch = bool(fused_inputs) and total <= self.ONE_LAUNCH_MAX_BYTES
-        self.run_tensor_tables()
-        spec = self.run_spec_tables()
-        self.run_compute_costs()
-        self.alloc_outputs(True, True, True)
+        spec = self._alloc_input_tables(spec_table)
+        self.alloc_outputs("comm" in outputs, "transition" in outputs, "cost" in outputs)
+        self.row_min = self.row_argmin = None
         lib, P, cp = self.lib, self._p, ctypes.byref(self.c_params)
         stream = self._stream()
         tb = self.tables
         err = torch.zeros((1,), dtype=torch.int32, device=self.device)
         self._step_keepalive = [err, spec]
+        null = vp(0)
         a_tensor = (ctypes.c_int64(tb.n_tensors), P("tensor_rank"), P("tensor_itemsize"), P("tensor_shape"),
                     P("tensor_stride"), P(self.tensor_bytes), P(self.tensor_contiguous), stream)
+        spec_outs = (P(spec["num_shards"]), P(spec["local_shape"]), P(spec["local_stride"]),
+                     ctypes.c_int32(spec["local_shape"].shape[1]), P(spec["local_numel"]), P(spec["local_bytes"])) \
+            if spec_table else (null, null, null, ctypes.c_int32(tb.shape_width()), null, null)
         a_spec = (cp, ctypes.c_int64(tb.n_specs), P("spec_codes"), P("spec_tensor"), P("tensor_rank"),
-                  P("tensor_itemsize"), P("tensor_shape"), P("tensor_stride"), P(spec["num_shards"]),
-                  P(spec["local_shape"]), P(spec["local_stride"]), ctypes.c_int32(spec["local_shape"].shape[1]),
-                  P(spec["local_numel"]), P(spec["local_bytes"]), stream)
+                  P("tensor_itemsize"), P("tensor_shape"), P("tensor_stride")) + spec_outs + (stream,)
         a_compute = (cp, ctypes.c_int64(tb.n_strategies), P("strat_flops"), P("strat_rw_bytes"), P("strat_dtype"),
                      P("strat_zero_cost"), P("strat_num_args"), P(self.compute_cost), P(self.compute_cost_per_arg),
                      P(err), stream)
@@ -284,9 +328,8 @@ class DeviceCostTables:
 
         rows_arg = ()
         if row_min:
-            n_rows = int(tb.edge_n_tgt.astype(np.int64).sum())
-            self.row_min = self._empty((n_rows,), torch.float64)
-            self.row_argmin = self._empty((n_rows,), torch.int32)
+            self.row_min = self._empty((tb.n_rows,), torch.float64)
+            self.row_argmin = self._empty((tb.n_rows,), torch.int32)
         if row_min_in_tiles:
             edge_row_begin = _to_device(tb.edge_row_begin(), self.device)
             self._step_keepalive.append(edge_row_begin)
@@ -329,7 +372,80 @@ class DeviceCostTables:
                 a_min = (P(self.cost), P(row_ptr), ctypes.c_int64(n_seg), ctypes.c_int64(tb.n_entries), P(self.row_min),
                          P(self.row_argmin), stream)
                 step["segmented_min"] = bind(lib.apc_segmented_min, a_min, "apc_segmented_min")
+        self._step_error_flag = err
         return step
+
+    # ---- the planner's table build -------------------------------------------------------------
+    PLANNER_OUTPUTS = ("cost",)
+
+    def planner_pass(self):
+        """The launches ``ShardingOptimizer.build_ds`` issues once the flop / byte counts are in
+        the strategy table (optimize_sharding.py:270-380 in one pass): the tensor and
+        compute-cost tables and the assembled cost of every entry, the array the ILP objective
+        is summed from, in one launch for tables up to ``ONE_LAUNCH_MAX_BYTES`` (else the input
+        tables, then the matrices); the launch also takes the row minima when that is cheaper
+        than reading the matrices back (``row_min_in_tiles_pays``), otherwise they are taken
+        when asked for.  The spec table is not part of it (the planner needed the local shard
+        shapes before it could count flops); ``comm`` and ``transition`` are written only when a
+        report asks (``fetch``)."""
+        return self.prepare_step(row_min=self.row_min_in_tiles_pays(), fused_inputs=True,
+                                 outputs=self.PLANNER_OUTPUTS, spec_table=False)
+
+    def check_error_flag(self):
+        """After a synchronisation: raises if a strategy with flops had an unsupported dtype."""
+        err = getattr(self, "_step_error_flag", None)
+        if err is not None and int(err.item()) != 0:
+            # compute_estimation.py:198-201
+            raise ValueError(f"a strategy with non-zero flops uses a dtype not supported on {self.params.device_name}")
+
+    @_guarded
+    def fetch(self, name: str) -> torch.Tensor:
+        """The device array ``comm`` / ``transition`` / ``cost``; one that the pass did not write
+        is computed now by a launch of the table kernel with that output alone (same values:
+        the kernel evaluates an entry the same way whichever arrays it stores)."""
+        have = {"comm": self.comm, "transition": self.transition, "cost": self.cost}
+        if name not in have:
+            raise KeyError(name)
+        if have[name] is not None:
+            return have[name]
+        if self.tensor_bytes is None or self.compute_cost_per_arg is None:
+            raise RuntimeError("no table pass has run yet")
+        n = self.tables.n_entries
+        out = self._empty((n,), torch.uint8 if name == "transition" else torch.float64)
+        ptrs = {k: self._p(out) if k == name else vp(0) for k in have}
+        with torch.cuda.device(self.device):
+            rc = self.lib.apc_redistribute_tables(
+                ctypes.byref(self.c_params), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
+                self._p("spec_codes"), self._p("spec_tensor"), self._p("pt_values"), self._p(self.compute_cost_per_arg),
+                ctypes.c_int64(self.tables.n_tiles), self._p("tile_records"), self._p("dup_entry_begin"),
+                ctypes.c_int64(n), ptrs["comm"], ptrs["transition"], ptrs["cost"], self._stream())
+        _native.check(rc, "apc_redistribute_tables")
+        setattr(self, name, out)
+        return out
+
+    @_guarded
+    def cost_objective(self, n_vars: int, group_var_begin, group_member_begin, member_entry_begin):
+        """-> (objective f64[n_vars], forced_zero u8[n_vars]) on the device: the ILP objective
+        summed from ``cost`` (``apc_cost_objective``).  The index arrays are host arrays."""
+        gv = _to_device(np.ascontiguousarray(group_var_begin, np.int64), self.device)
+        gm = _to_device(np.ascontiguousarray(group_member_begin, np.int64), self.device)
+        me = _to_device(np.ascontiguousarray(member_entry_begin, np.int64), self.device)
+        n_groups = len(group_var_begin) - 1
+        if n_groups < 0 or len(group_member_begin) != n_groups + 1:
+            raise ValueError("group_var_begin and group_member_begin must have n_groups + 1 rows")
+        if n_groups and (int(group_var_begin[0]) != 0 or int(group_var_begin[-1]) != n_vars
+                         or int(group_member_begin[-1]) != len(member_entry_begin)):
+            raise ValueError("group pointers do not span the variables / members")
+        cost = self.fetch("cost")
+        obj = self._empty((n_vars,), torch.float64)
+        forced = self._empty((n_vars,), torch.uint8)
+        with torch.cuda.device(self.device):
+            rc = self.lib.apc_cost_objective(ctypes.c_int64(n_vars), ctypes.c_int64(n_groups), self._p(gv), self._p(gm),
+                                             self._p(me), self._p(cost), ctypes.c_double(self.params.inf_replacement_cost),
+                                             self._p(obj), self._p(forced), self._stream())
+        _native.check(rc, "apc_cost_objective")
+        self._objective_keepalive = (gv, gm, me)
+        return obj, forced
 
     @_guarded
     def capture_step_graph(self, step):
@@ -393,14 +509,14 @@ class DeviceCostTables:
         copies = self._row_copies()
         row_ptr = _to_device(tb.row_ptr(), self.device)
         if copies is None:
-            return self.segmented_min(self.cost, row_ptr, check=False)
+            return self.segmented_min(self.fetch("cost"), row_ptr, check=False)
         selected, copy_ptr, copy_rows, n_read = copies
         n_rows = row_ptr.numel() - 1
         mins = self._empty((n_rows,), torch.float64)
         args = self._empty((n_rows,), torch.int32)
         with torch.cuda.device(self.device):
-            rc = self.lib.apc_segmented_min_copies(self._p(self.cost), self._p(row_ptr), ctypes.c_int64(selected.numel()),
-                                                   self._p(selected), self._p(copy_ptr), self._p(copy_rows),
+            rc = self.lib.apc_segmented_min_copies(self._p(self.fetch("cost")), self._p(row_ptr),
+                                                   ctypes.c_int64(selected.numel()), self._p(selected), self._p(copy_ptr), self._p(copy_rows),
                                                    ctypes.c_int64(n_read), self._p(mins), self._p(args), self._stream())
         _native.check(rc, "apc_segmented_min_copies")
         return mins, args  # (the index arrays stay cached with the tables)
@@ -436,7 +552,7 @@ class DeviceCostTables:
         t = self.tables
         if row_min.dtype != torch.float64 or not row_min.is_contiguous():
             raise TypeError("strategy_bounds takes a contiguous float64 array of row minima")
-        if row_min.numel() != int(t.edge_n_tgt.astype(np.int64).sum()):
+        if row_min.numel() != t.n_rows:
             raise ValueError("row_min must hold one value per matrix row")
         if getattr(self, "_bound_index", None) is None:
             self._bound_index = {k: _to_device(v, self.device) for k, v in t.strategy_bound_index().items()}

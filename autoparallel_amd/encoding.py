@@ -219,12 +219,37 @@ class CostTables:
         top = int(self.tensor_rank.max()) if self.n_tensors else 0
         return max(2, top + (top & 1))
 
-    def algorithmic_bytes_input_tables(self) -> int:
+    def algorithmic_bytes_input_tables(self, spec_table: bool = True) -> int:
         """Bytes the tensor, spec and compute-cost tables must move at minimum: per tensor 136 B
         read (rank, itemsize, shape, stride) and 9 B written; per spec 8 B read and 24 B + two
         rows of ``shape_width()`` values written (shard count, local element and byte counts,
         local shape and stride); per strategy 22 B read and 16 B written."""
-        return 145 * self.n_tensors + (32 + 16 * self.shape_width()) * self.n_specs + 38 * self.n_strategies
+        spec = (32 + 16 * self.shape_width()) * self.n_specs if spec_table else 0
+        return 145 * self.n_tensors + spec + 38 * self.n_strategies
+
+    def algorithmic_bytes_priced_per_unit(self, row_minima: bool = True) -> int:
+        """The same pass priced by fixed per-unit figures, whatever arrays a launch happens to
+        write: 8 B (one fp64 cost) + 1 B (transition flag) per entry; per edge its two spec lists
+        (one byte per mesh dim and spec) and a 64-byte header; 8 B written + 17 B read per
+        (node, strategy) compute cost; 12 B written per row minimum."""
+        m = len(self.mesh_sizes)
+        per_edge = (self.edge_n_src.astype(np.int64) + self.edge_n_tgt.astype(np.int64)) * m + 64
+        return 9 * self.n_entries + int(per_edge.sum()) + 25 * self.n_strategies + (12 * self.n_rows if row_minima else 0)
+
+    @property
+    def n_rows(self) -> int:
+        """Matrix rows over all edges: one per (edge, consumer strategy)."""
+        return int(self.edge_n_tgt.astype(np.int64).sum())
+
+    def validate_row_minima(self) -> None:
+        """Raises unless every matrix row lies inside one tile (the precondition of the
+        ``apc_*_row_min`` entry points), through the library's host-side check."""
+        def p(a):
+            return a.ctypes.data_as(ctypes.c_void_p)
+
+        rc = _native.lib().apc_validate_row_minima_host(ctypes.c_int64(self.n_edges), p(self.edge_n_src), p(self.edge_n_tgt),
+                                                        ctypes.c_int64(self.n_tiles), p(self.tile_records))
+        _native.check(rc, "apc_validate_row_minima_host")
 
     # ---- tiles -------------------------------------------------------------------------
     def edge_signatures(self) -> list:

@@ -47,13 +47,19 @@ logger = logging.getLogger(__name__)
 
 
 class DeviceBackend:
-    """Runs the table kernels on the GPU (the only backend of the product)."""
+    """Runs the table kernels on the GPU (the only backend of the product).
+
+    The table pass is enqueued and left running while the host numbers the ILP variables;
+    what comes back afterwards is one objective coefficient and one forced-to-zero flag per
+    variable plus the per-strategy compute costs.  The per-entry arrays stay in HBM and are
+    copied (``comm`` and ``transition`` are even computed) only when a report asks for them."""
 
     def __init__(self, tables, params: CostModelParams, device="cuda:0"):
         from .device_tables import DeviceCostTables
 
         self.dev = DeviceCostTables(tables, params, device=device)
         self.timings = {}
+        self.launches = ()
 
     def local_shapes(self):
         from .device_tables import _real_tensors
@@ -69,30 +75,60 @@ class DeviceBackend:
         self.dev.refresh("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "tile_records",
                          "dup_entry_begin", "dup_row_begin")
 
-    def build(self):
+    def launch_tables(self):
+        """Enqueues the planner's table pass (``DeviceCostTables.planner_pass``) and returns."""
         from .device_tables import _real_tensors
 
         with _real_tensors():
-            return self._build()
+            d = self.dev
+            step = d.planner_pass()
+            self.launches = tuple(step)
+            self._events = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            with torch.cuda.device(d.device):
+                self._events[0].record()
+                for launch in step.values():
+                    launch()
+                self._events[1].record()
 
-    def _build(self):
-        d = self.dev
-        t0 = time.perf_counter()
-        d.build_all()
-        torch.cuda.synchronize(d.device)
-        self.timings["kernels_s"] = time.perf_counter() - t0
-        logger.info("%s %.3f s", "kernels_s", self.timings["kernels_s"])
-        t0 = time.perf_counter()
-        out = {
-            "comm": d.comm.cpu().numpy(),
-            "transition": d.transition.cpu().numpy(),
-            "cost": d.cost.cpu().numpy(),
-            "compute": d.compute_cost.cpu().numpy(),
-            "compute_per_arg": d.compute_cost_per_arg.cpu().numpy(),
-        }
-        self.timings["copy_back_s"] = time.perf_counter() - t0
-        logger.info("%s %.3f s", "copy_back_s", self.timings["copy_back_s"])
+    def finish(self, n_vars, group_var_begin, group_member_begin, member_entry_begin):
+        """Sums the ILP objective on the device and copies back what the planner needs:
+        -> {"objective", "forced_zero", "compute", "compute_per_arg"} (host arrays)."""
+        from .device_tables import _real_tensors
+
+        with _real_tensors():
+            d = self.dev
+            with torch.cuda.device(d.device):
+                obj, forced = d.cost_objective(n_vars, group_var_begin, group_member_begin, member_entry_begin)
+                torch.cuda.synchronize(d.device)
+            d.check_error_flag()
+            self.timings["kernels_s"] = self._events[0].elapsed_time(self._events[1]) * 1e-3
+            t0 = time.perf_counter()
+            out = {
+                "objective": obj.cpu().numpy(),
+                "forced_zero": forced.cpu().numpy().astype(bool),
+                "compute": d.compute_cost.cpu().numpy(),
+                "compute_per_arg": d.compute_cost_per_arg.cpu().numpy(),
+            }
+            self.timings["copy_back_s"] = time.perf_counter() - t0
+        for k in ("kernels_s", "copy_back_s"):
+            logger.info("%s %.6f s", k, self.timings[k])
         return out
+
+    def host_array(self, name):
+        """``comm`` / ``transition`` / ``cost`` of every entry, copied (computed first, if the
+        table pass did not write it) now."""
+        from .device_tables import _real_tensors
+
+        with _real_tensors():
+            return self.dev.fetch(name).cpu().numpy()
+
+    def gather(self, name, entries):
+        """The values of a few entries of ``comm`` / ``transition`` / ``cost``."""
+        from .device_tables import _real_tensors
+
+        with _real_tensors():
+            idx = torch.from_numpy(np.ascontiguousarray(entries, np.int64)).to(self.dev.device)
+            return self.dev.fetch(name)[idx].cpu().numpy()
 
     def row_min(self, row_ptr):
         from .device_tables import _real_tensors
@@ -101,12 +137,12 @@ class DeviceBackend:
             if self._are_matrix_rows(row_ptr):  # taken by the table launch, or one read of every distinct row
                 mins, args = self.dev.row_minima()
             else:
-                mins, args = self.dev.segmented_min(self.dev.cost, row_ptr)
+                mins, args = self.dev.segmented_min(self.dev.fetch("cost"), row_ptr)
             return mins.cpu().numpy(), args.cpu().numpy()
 
     def _are_matrix_rows(self, row_ptr) -> bool:
         tb = self.dev.tables
-        return len(row_ptr) == int(tb.edge_n_tgt.astype(np.int64).sum()) + 1 and np.array_equal(row_ptr, tb.row_ptr())
+        return len(row_ptr) == tb.n_rows + 1 and np.array_equal(row_ptr, tb.row_ptr())
 
     def greedy(self, row_ptr):
         """-> (bound per strategy, min per node, argmin per node) from the row minima of the cost table"""
@@ -116,7 +152,7 @@ class DeviceBackend:
             if self._are_matrix_rows(row_ptr):
                 mins, _ = self.dev.row_minima()
             else:
-                mins, _ = self.dev.segmented_min(self.dev.cost, row_ptr)
+                mins, _ = self.dev.segmented_min(self.dev.fetch("cost"), row_ptr)
             return tuple(x.cpu().numpy() for x in self.dev.greedy_strategies(mins))
 
 
@@ -174,12 +210,17 @@ class CostRecords(Mapping):
                     yield (s_i, argi, ss, ii)
 
     def key_of_entry(self, idx: int):
+        return self.keys_of_entries(np.asarray([idx], np.int64))[0]
+
+    def keys_of_entries(self, entries) -> list:
         tb = self._o.encoded.tables
-        e = int(np.searchsorted(tb.edge_entry_begin, idx, side="right")) - 1
-        s_i, argi = self._o.encoded.edge_keys[e]
-        ns = int(tb.edge_n_src[e])
-        local = idx - int(tb.edge_entry_begin[e])
-        return (s_i, argi, local // ns, local % ns)
+        entries = np.asarray(entries, np.int64)
+        # the last edge that starts at or before the entry and is not empty
+        e = np.searchsorted(tb.edge_entry_begin, entries, side="right") - 1
+        ns = tb.edge_n_src[e].astype(np.int64)
+        local = entries - tb.edge_entry_begin[e]
+        keys = self._o.encoded.edge_keys
+        return [(*keys[ee], int(r), int(c)) for ee, r, c in zip(e.tolist(), (local // ns).tolist(), (local % ns).tolist())]
 
 
 class ClusterLinks(Mapping):
@@ -243,6 +284,9 @@ class ShardingOptimizer:
     # variable.  Same feasible plans and optimum, far fewer branching variables for the solver.
     node_choice_variables = True
     compact_constraints = True  # with choice variables: the structural constraints written through them
+    # copy ``comm`` back and write it into every OpSpec.redistribute_cost at construction
+    # (optimize_sharding.py:361-363); off: ``materialize_redistribute_costs()`` does it on request
+    write_back_redistribute_cost = False
 
     def __init__(self, gm, mesh, rescale_grad_comm_cost_for_mp=1.0, repeated_subgraphs=False):
         # Construction allocates millions of small long-lived objects (strategies, cost rows)
@@ -283,6 +327,7 @@ class ShardingOptimizer:
         self.validate()
         self.cluster_links = ClusterLinks(self)
         self.create_cluster_links()
+        self._finish_tables()
         self.prob = BinaryProgram(self.n_variables + self.n_choice_variables, "AutoParallel")
         self.res = None
         self.add_default_constraints()
@@ -326,24 +371,83 @@ class ShardingOptimizer:
         self.backend.upload_strategy_inputs(tb, self.tile_entries, self.dedupe, self.max_copies)
         self.timings["flops_bytes_s"] = time.perf_counter() - t0
         logger.info("%s %.3f s", "flops_bytes_s", self.timings["flops_bytes_s"])
+        # the table pass runs on the device while the host numbers the ILP variables;
+        # _finish_tables() collects what the planner needs of it
         t0 = time.perf_counter()
-        out = self.backend.build()
-        self.timings["tables_s"] = time.perf_counter() - t0
-        logger.info("%s %.3f s", "tables_s", self.timings["tables_s"])
-        self.timings.update({f"backend_{k}": v for k, v in getattr(self.backend, "timings", {}).items()})
-        self.comm_cost = out["comm"]
-        self.transition_cost = out["transition"]
-        self.cost = out["cost"].copy()
+        self.backend.launch_tables()
+        self.timings["launch_tables_s"] = time.perf_counter() - t0
+        self._host_arrays = {}
+        self._inf_entries = None
+        self.var_of_entry = np.arange(tb.n_entries, dtype=np.int64)
+        if self.write_back_redistribute_cost:
+            self.materialize_redistribute_costs()
+        return CostRecords(self), self.encoded.num_inp_out, self.encoded.num_args
+
+    def _finish_tables(self):
+        """Objective coefficients, forced-to-zero flags and compute costs from the backend: one
+        number per ILP variable instead of three arrays per entry (optimize_sharding.py:522-536,
+        650-655, evaluated where the costs are)."""
+        t0 = time.perf_counter()
+        tb = self.encoded.tables
+        begin = tb.edge_entry_begin.astype(np.int64)
+        sizes = begin[1:] - begin[:-1]
+        live = sizes > 0
+        roots = np.nonzero(self.edge_is_representative & live)[0]
+        members = np.nonzero(live)[0]
+        members = members[np.argsort(self.edge_rep[members], kind="stable")]  # grouped by root, ascending inside
+        group_var_begin = np.concatenate([self.edge_var_base[roots], [self.n_variables]]).astype(np.int64)
+        counts = np.bincount(np.searchsorted(roots, self.edge_rep[members]), minlength=len(roots))
+        group_member_begin = np.zeros(len(roots) + 1, np.int64)
+        np.cumsum(counts, out=group_member_begin[1:])
+        self.objective_groups = (self.n_variables, group_var_begin, group_member_begin, begin[:-1][members])
+        out = self.backend.finish(*self.objective_groups)
+        self.objective_vector = out["objective"]
+        self.forced_zero_vars = out["forced_zero"]
         self.compute_cost = out["compute"]  # per (node, strategy), before the division by num_args
         self.compute_cost_per_arg = out["compute_per_arg"]
-        self.var_of_entry = np.arange(tb.n_entries, dtype=np.int64)
-        # the recomputed costs are written back into OpSpec.redistribute_cost, which
-        # print_costs_for_node reads (optimize_sharding.py:361-363)
-        t0 = time.perf_counter()
-        self._write_back_redistribute_cost()
-        self.timings["write_back_s"] = time.perf_counter() - t0
-        logger.info("%s %.3f s", "write_back_s", self.timings["write_back_s"])
-        return CostRecords(self), self.encoded.num_inp_out, self.encoded.num_args
+        self.timings["tables_s"] = self.timings.pop("launch_tables_s") + time.perf_counter() - t0
+        logger.info("%s %.3f s", "tables_s", self.timings["tables_s"])
+        self.timings.update({f"backend_{k}": v for k, v in getattr(self.backend, "timings", {}).items()})
+
+    # ---- per-entry arrays: they stay with the backend until somebody reads them --------------------
+    def _host_array(self, name):
+        a = self._host_arrays.get(name)
+        if a is None:
+            a = self.backend.host_array(name)
+            if name == "cost":
+                # optimize_sharding.py:531-533: a cost that is not finite reads 10000.0 afterwards
+                bad = ~np.isfinite(a)
+                self._inf_entries = np.nonzero(bad)[0]
+                a = np.where(bad, self.params.inf_replacement_cost, a)
+            self._host_arrays[name] = a
+        return a
+
+    @property
+    def comm_cost(self):
+        return self._host_array("comm")
+
+    @property
+    def transition_cost(self):
+        return self._host_array("transition")
+
+    @property
+    def cost(self):
+        return self._host_array("cost")
+
+    @property
+    def inf_entries(self):
+        self._host_array("cost")
+        return self._inf_entries
+
+    def _values(self, name, entries):
+        """A few entries of a per-entry array, without copying the whole array to the host."""
+        entries = np.asarray(entries, np.int64)
+        if name in self._host_arrays:
+            return self._host_arrays[name][entries]
+        v = self.backend.gather(name, entries)
+        if name == "cost":
+            v = np.where(np.isfinite(v), v, self.params.inf_replacement_cost)
+        return v
 
     def create_cluster_links(self):
         """Entries of a linked node share the ILP variables of its representative's entries
@@ -370,6 +474,7 @@ class ShardingOptimizer:
         base = np.zeros(n_edges, np.int64)
         base[is_root] = np.cumsum(sizes[is_root]) - sizes[is_root]
         self.edge_var_base = base[edge_rep]
+        self.edge_rep = edge_rep
         self.edge_is_representative = is_root
         self.var_of_entry = np.repeat(self.edge_var_base - begin[:-1], sizes) + np.arange(tb.n_entries, dtype=np.int64)
         self.n_variables = int(sizes[is_root].sum())
@@ -397,7 +502,11 @@ class ShardingOptimizer:
             self.choice_var_of_strategy = choice
             self.n_choice_variables = next_free - self.n_variables
 
-    def _write_back_redistribute_cost(self):
+    def materialize_redistribute_costs(self):
+        """Writes the recomputed communication costs into ``OpSpec.redistribute_cost`` of every
+        strategy (optimize_sharding.py:361-363).  Nothing in the planner reads them there
+        (``print_costs_for_node`` takes the flat array), so this copy of the whole ``comm`` array
+        is made only on request, or at construction with ``write_back_redistribute_cost = True``."""
         tb = self.encoded.tables
         comm = self.comm_cost
         for e, (s_i, argi) in enumerate(self.encoded.edge_keys):
@@ -494,11 +603,9 @@ class ShardingOptimizer:
                                "output_input_consistent")
 
     def add_inf_cost_constraint(self):
-        """Non-finite costs become 10000 and their variable is forced to 0."""
-        bad = np.nonzero(~np.isfinite(self.cost))[0]
-        self.cost[bad] = self.params.inf_replacement_cost
-        self.prob.force_zero(self.var_of_entry[bad])
-        self.inf_entries = bad
+        """Non-finite costs become 10000 and their variable is forced to 0 (the flags come with
+        the objective vector: one per variable, set where any entry of the variable is not finite)."""
+        self.prob.force_zero(np.nonzero(self.forced_zero_vars)[0])
 
     def add_choice_link_constraint(self):
         """choice[node, strategy] = sum of the entry variables of that strategy's row of the
@@ -595,36 +702,35 @@ class ShardingOptimizer:
 
     # ---- solve (optimize_sharding.py:648-701) ------------------------------------------------
     def get_solution(self, verbose=False):
-        # linked entries share a variable: their costs add up
-        obj = np.bincount(self.var_of_entry, weights=self.cost, minlength=self.prob.n_vars).astype(np.float64)
+        # linked entries share a variable: their costs add up (summed where the costs are)
+        obj = np.zeros(self.prob.n_vars, np.float64)
+        obj[:self.n_variables] = self.objective_vector
         self.prob.objective = obj
         status = self.prob.solve(verbose=verbose, time_limit=self.solver_time_limit, mip_rel_gap=self.solver_rel_gap)
         if status == -1:
             print(self.get_violated_constraints_log())
             raise RuntimeError("Unsolvable problem")
         chosen = np.nonzero(self.prob.x[self.var_of_entry] == 1)[0]
-        self.res = [self.ds.key_of_entry(int(i)) for i in chosen]
+        self.res = self.ds.keys_of_entries(chosen)
         self.res_entries = chosen
 
-        opt = {}
+        # one strategy pair per (node, argument), one strategy per node (optimize_sharding.py:676-696)
         nodes = self.nodes
-        for key in self.res:
-            opt.setdefault(nodes[key[0]], []).append(self.ds[key])
         seen = set()
-        for r in self.res:
-            key = (r[0], r[1])
-            if key in seen:
-                raise RuntimeError(
-                    f"Multiple solutions for {nodes[key[0]]}, key={key}, "
-                    f"solutions: {[str(x['full_strat']) for x in opt[nodes[key[0]]]]}")
-            seen.add(key)
-        for k in opt.values():
-            assert all(k[0]["full_strat"] == kk["full_strat"] for kk in k), \
-                f"{[kk['va'] for kk in k]}: {[str(kk['full_strat']) for kk in k]}"
-        return {k: v[0]["full_strat"] for k, v in opt.items()}
+        chosen_strategy = {}
+        for s_i, argi, ss, _ in self.res:
+            node = nodes[s_i]
+            if (s_i, argi) in seen:
+                raise RuntimeError(f"Multiple solutions for {node}, key={(s_i, argi)}, solutions: "
+                                   f"{[str(self.strats[node].strategies[k[2]]) for k in self.res if k[0] == s_i]}")
+            seen.add((s_i, argi))
+            first = chosen_strategy.setdefault(node, ss)
+            assert first == ss or self.strats[node].strategies[first] == self.strats[node].strategies[ss], \
+                f"{node}: arguments chose different strategies {first} and {ss}"
+        return {node: self.strats[node].strategies[ss] for node, ss in chosen_strategy.items()}
 
     def objective_value(self) -> float:
-        return float(self.cost[self.res_entries].sum())
+        return float(self._values("cost", self.res_entries).sum())
 
     def get_violated_constraints_log(self):
         names = self.prob.violated_constraints()
@@ -774,10 +880,10 @@ class ShardingOptimizer:
         code = "\n".join(code)
         idx = self.res_entries
         strat_rows = np.asarray([self.encoded.strat_begin[k[0]] + k[2] for k in self.res], np.int64)
-        code += f"\ntotal_cost: {self.cost[idx].sum():.2f}"
-        code += f"\n  comm_cost: {self.comm_cost[idx].sum():.2f}"
+        code += f"\ntotal_cost: {self._values('cost', idx).sum():.2f}"
+        code += f"\n  comm_cost: {self._values('comm', idx).sum():.2f}"
         code += f"\n  compute_cost: {self.compute_cost_per_arg[strat_rows].sum():.2f}"
-        code += f"\n  transition_cost: {self.transition_cost[idx].astype(np.float64).sum():.2f}"
+        code += f"\n  transition_cost: {self._values('transition', idx).astype(np.float64).sum():.2f}"
         code += "\n" + self.get_violated_constraints_log()
         return code
 

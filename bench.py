@@ -1,17 +1,22 @@
 """Benchmark of the sharding-cost table build on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3_8b|llama3_70b|block_1k|stress]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3_8b|llama3_70b|dsv3_moe|block_1k|stress]
 
-A step is one complete device-side pass of the hot path over the workload's flattened
-tables, already resident in HBM: tensor byte/contiguity table, local shard shapes,
-per-strategy compute costs, the redistribution-cost matrices with assembled ILP costs, and
-the row minima.  The default workload is the Llama-3-8B joint forward+backward graph
-planned on a (32, 8) logical mesh; ``stress`` is the seeded 200k-node synthetic DAG on a
-(16, 8, 4) mesh.
+A step is the device pass ``ShardingOptimizer.build_ds`` issues once the flop / byte counts
+are in the strategy table (``DeviceCostTables.planner_pass``): the tensor byte / contiguity
+table, the per-strategy compute costs and the assembled cost of every entry of every
+redistribution-cost matrix, with the row minima where taking them there is cheaper than
+reading the matrices back; tables already resident in HBM.  On the default workload, the
+Llama-3-8B joint forward+backward graph planned on a (32, 8) logical mesh, that is ONE launch.
+``stress`` is the seeded 200k-node synthetic DAG on a (16, 8, 4) mesh.
 
-One JSON line is printed: whole-pass throughput in cost entries/s (``value``), the
-redistribution-cost kernel against the HBM roofline (``roofline``), and the CPU oracle
-timed on a bounded sample of the same tables (``cpu_baseline``).
+One JSON line is printed: whole-pass throughput in cost entries/s (``value``), the launch that
+writes the cost matrices against the HBM roofline (``roofline``), the CPU oracle timed on a
+bounded sample of the same tables (``cpu_baseline``), the plan wall-time by stage, and under
+``extra`` the same roofline figures on the two tables large enough to be bandwidth-bound
+(Llama-3-70B on (8, 8, 8) and the stress DAG).  Outside the timed region the pass's outputs are
+compared with the launch-by-launch build of all arrays and with the C oracle; a mismatch fails
+the run.
 """
 
 from __future__ import annotations
@@ -27,22 +32,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+ORACLE_CHECK_MAX_ENTRIES = 60_000_000  # larger tables are checked against the C oracle on a prefix of their edges
 
-# HBM bytes per launch of the kernel that writes the cost matrices, measured with rocprofv3 --pmc
-# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, KiB per dispatch; the factors come from the same
-# counters read on a plain 1 GiB copy, --calibrate-copy).  A hardware counter cannot be read
-# from inside this process, so the figure is the one of the profiled run of the same command
-# and only reported for exactly that table: (entries, tiles, algorithmic bytes) must match.
-MEASURED_TRAFFIC_BYTES = {
-    (1_821_368, 1_616, 73_586_428): (3_184.3 * 2.000 + 68_345.1) * 1024,           # llama3_8b, mesh (32, 8), all tables and the row minima in one launch
-    (1_821_368, 1_616, 71_794_420): (3_037.5 * 2.000 + 65_983.1) * 1024,           # the same, --row-min separate
-    (1_821_368, 1_616, 32_348_914): (670.7 * 2.000 + 31_445.9) * 1024,             # the same, --table-launches 2
-    (1_073_460, 1_387, 47_179_580): (2_310.1 * 2.000 + 43_498.1) * 1024,            # dsv3_moe, mesh (64, 4)
-    (2_986, 129, 374_304): (249.0 * 2.000 + 317.4) * 1024,                          # block_1k, mesh (64,)
-    (73_251_434, 40_727, 1_255_915_920): (12_322.6 * 2.000 + 1_221_016.0) * 1024,   # llama3_70b, mesh (8, 8, 8)
-    (464_235_576, 426_918, 8_178_099_438): (165_040.2 * 2.000 + 7_953_223.0) * 1024,  # stress, mesh (16, 8, 4), row minima in the tiles
-    (464_235_576, 426_918, 8_003_825_874): (159_776.0 * 2.000 + 7_760_473.5) * 1024,  # the same, --row-min separate
-}
+WORKLOADS = ["llama3_8b", "llama3_70b", "dsv3_moe", "block_1k", "stress"]
 
 
 def parse_args():
@@ -50,7 +42,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="llama3_8b", choices=["llama3_8b", "llama3_70b", "dsv3_moe", "block_1k", "stress"])
+    ap.add_argument("--workload", default="llama3_8b", choices=WORKLOADS)
     ap.add_argument("--layers", type=int, default=None, help="override the number of decoder layers")
     ap.add_argument("--stress-nodes", type=int, default=200_000)
     ap.add_argument("--tile-entries", type=int, default=None, help="entries per tile (default: chosen from the table)")
@@ -60,25 +52,24 @@ def parse_args():
     ap.add_argument("--no-clustering", action="store_true", help="one ILP variable per entry (no variable sharing)")
     ap.add_argument("--no-dedupe", action="store_true", help="tile every edge even if an identical one exists")
     ap.add_argument("--max-copies", type=int, default=8, help="identical edges served by one tiled edge")
-    ap.add_argument("--table-launches", type=int, default=None, choices=[1, 2, 4],
-                    help="launches that build the tables of a pass: 1 = everything in one (apc_build_tables), "
-                         "2 = input tables, then cost matrices, 4 = tensor, spec and compute-cost tables on their own "
-                         "(default: 1 for tables up to 128 MiB, else 2)")
-    ap.add_argument("--row-min", choices=["auto", "tiles", "separate"], default="auto",
-                    help="where the row minima of a pass are taken: by the launch that writes the cost matrices "
-                         "(tiles), by a segmented_min launch that reads them back (separate); auto = tiles whenever "
-                         "every matrix row lies inside one tile")
+    ap.add_argument("--pass", dest="pass_kind", choices=["planner", "all"], default="planner",
+                    help="planner: the pass build_ds issues (assembled cost, no spec table); all: every table and all "
+                         "three per-entry arrays (the composite of the earlier benchmark, labelled as such)")
+    ap.add_argument("--extra", default="llama3_70b,stress",
+                    help="comma-separated workloads measured after the main one and reported under 'extra' "
+                         "(fewer steps, no CPU baseline, no solve); '' for none")
+    ap.add_argument("--no-verify", action="store_true", help="skip the comparison of the pass's outputs (timing runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy three times (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
     return ap.parse_args()
 
 
-def build_workload(args):
+def build_workload(name, args):
     """-> (tables, params, description, device tables or None, planner or None, host timings)"""
     from autoparallel_amd import CostModelParams
 
-    if args.workload == "stress":
+    if name == "stress":
         from autoparallel_amd.synthetic import stress_dag
 
         mesh = (16, 8, 4)
@@ -90,16 +81,16 @@ def build_workload(args):
         return tables, CostModelParams.from_mesh(mesh, rescale=2.2), desc, None, None, timings
 
     # traced workloads go through the product path: capture -> ShardingOptimizer (which
-    # enumerates, clusters, encodes, builds the device tables and copies them back)
+    # enumerates, clusters, encodes, runs the table pass and takes the objective vector back)
     import torch
 
     from autoparallel_amd.api import AutoParallelPlanner
     from autoparallel_amd.graphs import workloads
     from autoparallel_amd.optimize_sharding import ShardingOptimizer
 
-    mesh_sizes = workloads.WORKLOADS[args.workload][1]
+    mesh_sizes = workloads.WORKLOADS[name][1]
     mesh = workloads.logical_mesh(mesh_sizes)
-    model, input_fn, workload_desc, needs_dynamo = workloads.build_model(args.workload, mesh, n_layers=args.layers)
+    model, input_fn, workload_desc, needs_dynamo = workloads.build_model(name, mesh, n_layers=args.layers)
 
     class Optimizer(ShardingOptimizer):
         tile_entries = args.tile_entries
@@ -114,11 +105,11 @@ def build_workload(args):
     planner.__enter__()
     opt = planner.sharding_optimizer
     desc = {"workload": workload_desc, "mesh": list(mesh_sizes), "graph_nodes": len(opt.nodes), "ilp_variables": opt.n_variables,
-            "clustered_nodes": len(opt.node_representative)}
+            "clustered_nodes": len(opt.node_representative), "planner_launches": list(opt.backend.launches)}
     return opt.encoded.tables, opt.params, desc, opt.backend.dev, planner, dict(planner.timings)
 
 
-def solve_plan(planner, args):
+def solve_plan(planner, workload):
     """The ILP leg of the plan (input / output constraints of the reference's Llama example:
     examples/example_llama3.py:205-218)."""
     from torch.distributed.tensor.placement_types import Replicate, Shard
@@ -127,8 +118,8 @@ def solve_plan(planner, args):
     planner.add_parameter_memory_constraint(low=None, high=None)
     nd = planner.mesh.ndim
     x_sharding = (Shard(0),) + (Replicate(),) * (nd - 1)
-    out_sharding = (Shard(0), Shard(2)) if (nd == 2 and args.workload != "block_1k") else x_sharding
-    if args.workload in ("block_1k", "dsv3_moe"):
+    out_sharding = (Shard(0), Shard(2)) if (nd == 2 and workload != "block_1k") else x_sharding
+    if workload in ("block_1k", "dsv3_moe"):
         # the batch (8 / 16) does not divide the mesh's first dim, so no batch-sharded placement
         # exists (the default constraint would raise, as the reference's does): pin the sequence
         x_sharding = out_sharding = (Shard(1),) + (Replicate(),) * (nd - 1)
@@ -137,12 +128,11 @@ def solve_plan(planner, args):
     constraints_s = time.perf_counter() - t0
     planner.optimize_placement()
     opt = planner.sharding_optimizer
-    t0 = time.perf_counter()
-    _, lower_bound = opt.greedy_strategies()  # row minima -> per-strategy bounds -> per-node minima, on the device
-    bound_s = time.perf_counter() - t0
-    return {"constraints_s": constraints_s, "solve_s": planner.timings["solve_s"],
-            "objective": opt.objective_value(), "ilp_rows": getattr(opt.prob, "rows_after_dedupe", None),
-            "ilp_variables": opt.n_variables, "lower_bound_from_row_minima": lower_bound, "lower_bound_s": bound_s}
+    out = {"constraints_s": constraints_s, "solve_s": planner.timings["solve_s"],
+           "objective": opt.objective_value(), "ilp_rows": getattr(opt.prob, "rows_after_dedupe", None),
+           "ilp_variables": opt.n_variables}
+    out.update(getattr(opt, "solve_stats", {}))
+    return out
 
 
 def cpu_baseline(tables, params, target_seconds):
@@ -170,16 +160,255 @@ def cpu_baseline(tables, params, target_seconds):
     out = po.build_tables(enc, op, edge_range=(0, hi))
     dt = time.perf_counter() - t0
     n = len(out["comm"])
-    # the plain-C restatement on the whole workload, for scale
-    t0 = time.perf_counter()
-    c_oracle.build_tables(enc, op)
-    c_dt = time.perf_counter() - t0
+    # the plain-C restatement on the whole workload, for scale (second of two runs: the first
+    # one pays for the page faults of its fresh output arrays)
+    c_dt = float("inf")
+    for _ in range(2):
+        t0 = time.perf_counter()
+        c_oracle.build_tables(enc, op)
+        c_dt = min(c_dt, time.perf_counter() - t0)
     return {
         "value": n / dt, "unit": "entries/s", "cores": 1, "kind": "port",
         "sample": f"scalar Python oracle over the first {hi} of {tables.n_edges} edges ({n} entries, {dt:.1f} s), "
                   f"compute costs + redistribution costs + assembly",
         "c_port_entries_per_s": tables.n_entries / c_dt, "host_cpu_count": os.cpu_count(),
     }
+
+
+def prepare(dev, pass_kind):
+    if pass_kind == "planner":
+        return dev.planner_pass()
+    return dev.prepare_step(row_min=True, fused_inputs=True)
+
+
+def time_pass(dev, step, steps, warmup):
+    """Warm-up, then exactly ``steps`` passes twice: once with a HIP event pair around every
+    launch (per-kernel durations), once plain with one event pair around the whole region (the
+    pass rate; when a pass is one kernel, region / steps is that kernel's back-to-back duration
+    without the 1 - 2 us an event pair adds to a launch)."""
+    import numpy as np
+    import torch
+
+    names = list(step)
+    launchers = [step[k] for k in names]
+    for _ in range(warmup):
+        for launch in launchers:
+            launch()
+    torch.cuda.synchronize()
+    ev = {k: [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+          for k in names}
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        for k, launch in zip(names, launchers):
+            a, b = ev[k][i]
+            a.record()
+            launch()
+            b.record()
+    torch.cuda.synchronize()
+    wall_events = time.perf_counter() - t0
+    kernel_ms = {k: float(np.mean([a.elapsed_time(b) for a, b in ev[k]])) for k in names}
+    kernel_ms_min = {k: float(np.min([a.elapsed_time(b) for a, b in ev[k]])) for k in names}
+    region = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    region[0].record()
+    for i in range(steps):
+        for launch in launchers:
+            launch()
+    region[1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return {"names": names, "wall_s": wall, "wall_events_s": wall_events, "region_ms": region[0].elapsed_time(region[1]),
+            "kernel_ms": kernel_ms, "kernel_ms_min": kernel_ms_min}
+
+
+def verify_pass(dev, tables, params, log):
+    """Outside the timed region: what the timed launches left in HBM against (1) the
+    launch-by-launch build of every array on a second set of buffers and (2) the C oracle
+    (whole table up to ORACLE_CHECK_MAX_ENTRIES, else a prefix of the edges)."""
+    import numpy as np
+    import torch
+
+    from autoparallel_amd.device_tables import DeviceCostTables
+    from oracle import c_oracle
+    from oracle import cost_oracle as po
+
+    torch.cuda.synchronize()
+    dev.check_error_flag()
+    ref = DeviceCostTables(tables, params, device=dev.device, validate=False)
+    ref.build_all()
+    torch.cuda.synchronize()
+    checked = []
+
+    def same(name, a, b):
+        if a is None:
+            return
+        if not torch.equal(a, b):
+            raise SystemExit(f"bench.py: PARITY FAILURE: {name} of the timed pass differs from the launch-by-launch build")
+        checked.append(name)
+
+    same("cost", dev.cost, ref.cost)
+    same("comm", dev.comm, ref.comm)
+    same("transition", dev.transition, ref.transition)
+    same("compute_cost", dev.compute_cost, ref.compute_cost)
+    same("compute_cost_per_arg", dev.compute_cost_per_arg, ref.compute_cost_per_arg)
+    same("tensor_bytes", dev.tensor_bytes, ref.tensor_bytes)
+    ref_min, ref_arg = ref.row_minima()
+    if dev.row_min is not None:
+        same("row_min", dev.row_min, ref_min)
+        same("row_argmin", dev.row_argmin, ref_arg)
+    # the C oracle
+    op = po.make_params(params.mesh_sizes, device_name=params.device_name, rescale=params.rescale)
+    enc = tables.as_dict()
+    eb = tables.edge_entry_begin
+    hi = tables.n_edges
+    if tables.n_entries > ORACLE_CHECK_MAX_ENTRIES:
+        hi = max(1, int(np.searchsorted(eb, ORACLE_CHECK_MAX_ENTRIES, side="right")) - 1)
+    n = int(eb[hi])
+    want_cc, want_pa = c_oracle.compute_costs(enc, op)
+    want = c_oracle.build_tables(enc, op, edge_range=(0, hi), per_arg=want_pa)
+    if not np.array_equal(dev.cost[:n].cpu().numpy(), want["cost"]):
+        raise SystemExit("bench.py: PARITY FAILURE: cost of the timed pass differs from the C oracle")
+    if not np.array_equal(dev.compute_cost.cpu().numpy(), want_cc):
+        raise SystemExit("bench.py: PARITY FAILURE: compute costs of the timed pass differ from the C oracle")
+    if not np.array_equal(ref.comm[:n].cpu().numpy(), want["comm"]) or \
+            not np.array_equal(ref.transition[:n].cpu().numpy(), want["transition"]):
+        raise SystemExit("bench.py: PARITY FAILURE: comm / transition differ from the C oracle")
+    n_rows = int(tables.edge_n_tgt[:hi].astype(np.int64).sum())
+    wm, wa = c_oracle.segmented_min(want["cost"], tables.row_ptr()[:n_rows + 1])
+    if not (np.array_equal(ref_min[:n_rows].cpu().numpy(), wm) and np.array_equal(ref_arg[:n_rows].cpu().numpy(), wa)):
+        raise SystemExit("bench.py: PARITY FAILURE: row minima differ from the C oracle")
+    del ref
+    torch.cuda.empty_cache()
+    log.info("verified: %s equal to the launch-by-launch build; %d of %d entries equal to the C oracle",
+             ", ".join(checked), n, tables.n_entries)
+    return {"timed_pass_equals_launch_by_launch_build": checked, "entries_equal_to_c_oracle": n,
+            "entries": tables.n_entries, "bit_exact": True}
+
+
+def roofline_of(dev, tables, timing, steps, pass_kind):
+    """The launch that writes the cost matrices against the HBM peak, two ways: over the bytes
+    that launch must move (``frac``) and over fixed per-unit prices (``frac_survey_8d``: 9 B per
+    entry, the spec lists and a 64-byte header per edge, 25 B per strategy when the launch also
+    builds the compute costs, 12 B per row minimum it takes)."""
+    import numpy as np
+
+    names = timing["names"]
+    one_launch = "build_tables" in names
+    main = "build_tables" if one_launch else "redistribute_tables"
+    in_tiles = dev.row_min is not None and "segmented_min" not in names
+    outputs = tuple(k for k in ("comm", "transition", "cost") if getattr(dev, k) is not None)
+    spec_table = pass_kind == "all"
+    m = len(tables.mesh_sizes)
+    per_edge = int(((tables.edge_n_src.astype(np.int64) + tables.edge_n_tgt.astype(np.int64)) * m + 64).sum())
+    per_entry = 8 * ("comm" in outputs) + 1 * ("transition" in outputs) + 8 * ("cost" in outputs)
+    launch_bytes = per_entry * tables.n_entries + per_edge + (12 * tables.n_rows if in_tiles else 0)
+    priced = 9 * tables.n_entries + per_edge + (12 * tables.n_rows if in_tiles else 0)
+    if one_launch:
+        launch_bytes += tables.algorithmic_bytes_input_tables(spec_table=spec_table)
+        priced += 25 * tables.n_strategies
+    t_pair = timing["kernel_ms"][main] * 1e-3
+    single = len(names) == 1
+    t_kernel = timing["region_ms"] * 1e-3 / steps if single else t_pair
+    return {
+        "bound": "hbm",
+        "kernel": ("build_tables_kernel" if one_launch else
+                   "redistribute_tiles_row_min_kernel" if in_tiles else "redistribute_tiles_kernel"),
+        "launch": main + (" (the one launch of the pass)" if single else ""),
+        "arrays_written_per_entry": list(outputs),
+        "row_minima_taken_by_this_launch": bool(in_tiles),
+        "achieved": launch_bytes / t_kernel / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": launch_bytes / t_kernel / 1e9 / HBM_PEAK_GBPS,
+        "frac_survey_8d": priced / t_kernel / 1e9 / HBM_PEAK_GBPS,
+        "traffic": None,
+        "bytes_per_launch": launch_bytes, "bytes_per_launch_survey_8d": priced,
+        "avg_launch_us": t_kernel * 1e6,
+        "avg_launch_us_event_pair_per_launch": t_pair * 1e6,
+        "min_launch_us_event_pair_per_launch": timing["kernel_ms_min"][main] * 1e3,
+        "timing": ("one HIP event pair on the launch stream around the K back-to-back launches of the timed "
+                   "region (the pass is this one kernel), / K" if single else
+                   "HIP events around every launch of the kernel inside the timed region"),
+        "traffic_note": "hardware counters cannot be read from inside the process: FETCH_SIZE / WRITE_SIZE per dispatch "
+                        "of this kernel are in profiles/ (rocprofv3 --pmc runs of this command)",
+    }
+
+
+def measure(name, args, log, steps, warmup, main_run):
+    """Builds one workload, times its pass, verifies it; -> (result dict, planner or None, ...)."""
+    import numpy as np
+    import torch
+
+    from autoparallel_amd.device_tables import DeviceCostTables, _real_tensors
+
+    t_setup = time.perf_counter()
+    tables, params, desc, dev, planner, host_timings = build_workload(name, args)
+    # a traced workload keeps its capture context (a fake-tensor mode) open until the plan is
+    # solved; the measurements below work on real device buffers
+    guard = _real_tensors()
+    guard.__enter__()
+    try:
+        t0 = time.perf_counter()
+        if dev is None:
+            if args.tile_entries:
+                tables.build_tiles(args.tile_entries)
+            dev = DeviceCostTables(tables, params, device="cuda:0")
+        log.info("%s: tables resident: %d entries, %d tiles", name, tables.n_entries, tables.n_tiles)
+        step = prepare(dev, args.pass_kind)
+        torch.cuda.synchronize()
+        host_timings["upload_and_prepare_s"] = time.perf_counter() - t0
+        host_timings["setup_total_s"] = time.perf_counter() - t_setup
+        timing = time_pass(dev, step, steps, warmup)
+        ms_per_step = timing["wall_s"] / steps * 1e3
+        log.info("%s: timed region done: %.4f ms/step", name, ms_per_step)
+        parity = None if args.no_verify else verify_pass(dev, tables, params, log)
+        roof = roofline_of(dev, tables, timing, steps, args.pass_kind)
+        # the planner's follow-up launch: the ILP objective summed on the device from the cost
+        # array (its own kernel, after the host has numbered the variables; not part of the table
+        # pass); without a planner every entry is its own variable
+        objective_us = None
+        if dev.cost is not None:
+            if planner is not None:
+                groups = planner.sharding_optimizer.objective_groups
+            else:
+                eb = tables.edge_entry_begin.astype(np.int64)
+                live = np.nonzero(np.diff(eb) > 0)[0]
+                groups = (tables.n_entries, np.concatenate([eb[:-1][live], [tables.n_entries]]),
+                          np.arange(len(live) + 1, dtype=np.int64), eb[:-1][live])
+            pair = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            dev.cost_objective(*groups)
+            torch.cuda.synchronize()
+            pair[0].record()
+            dev.cost_objective(*groups)
+            pair[1].record()
+            torch.cuda.synchronize()
+            objective_us = pair[0].elapsed_time(pair[1]) * 1e3
+        E = tables.n_entries
+        out = {
+            "value": E * steps / timing["wall_s"], "ms_per_step": ms_per_step,
+            "config": {**desc, "edges": tables.n_edges, "strategies": tables.n_strategies, "specs": tables.n_specs,
+                       "entries": E, "tiles": tables.n_tiles, "tiling": tables.tiling, "matrix_rows": tables.n_rows,
+                       "edges_deduplicated": int((tables.edge_canonical != np.arange(tables.n_edges)).sum()),
+                       "device_row": params.device_name, "devices_per_host": 8,
+                       "step": " + ".join(timing["names"]) + (
+                           ": DeviceCostTables.planner_pass, the launches ShardingOptimizer.build_ds issues "
+                           "(tensor + compute-cost tables and the assembled cost of every entry"
+                           + (", row minima taken by the same launch" if roof["row_minima_taken_by_this_launch"] else "")
+                           + "; the spec table was built before, comm / transition are written only on request)"
+                           if args.pass_kind == "planner" else
+                           ": every table and all three per-entry arrays (composite pass, not what the planner issues)")},
+            "roofline": roof,
+            "kernel_us": {k: v * 1e3 for k, v in timing["kernel_ms"].items()},
+            "objective_reduction_us_including_index_upload": objective_us,
+            "ms_per_step_with_events": timing["wall_events_s"] / steps * 1e3,
+            "host_timings_s": {k: round(v, 6) for k, v in host_timings.items()},
+            "parity": parity,
+        }
+        if main_run and not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_baseline(tables, params, args.cpu_seconds)
+    finally:
+        guard.__exit__(None, None, None)
+    return out, planner, tables, host_timings
 
 
 def main():
@@ -193,7 +422,6 @@ def main():
         print("bench.py: this build runs on one GPU; cost tables shard by edge range without any exchange step, "
               "but no multi-GPU path is part of it. Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
-    import numpy as np
     import torch
 
     if not torch.cuda.is_available():
@@ -209,156 +437,69 @@ def main():
         print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 8, "calibrate_copy_bytes_written": src.numel() * 8,
                           "copies": 3}))
         return
-    from autoparallel_amd.device_tables import DeviceCostTables
 
-    t_setup = time.perf_counter()
-    tables, params, desc, dev, planner, host_timings = build_workload(args)
-    # a traced workload keeps its capture context (a fake-tensor mode) open until the plan is
-    # solved; the measurements below work on real device buffers
-    from autoparallel_amd.device_tables import _real_tensors
-
-    guard = _real_tensors()
-    guard.__enter__()
-    t0 = time.perf_counter()
-    if dev is None:
-        if args.tile_entries:
-            tables.build_tiles(args.tile_entries)
-        dev = DeviceCostTables(tables, params, device="cuda:0")
-    log.info("tables resident: %d entries, %d tiles", tables.n_entries, tables.n_tiles)
-    step = dev.prepare_step(row_min=True, fused_inputs=args.table_launches != 4,
-                            one_launch=None if args.table_launches is None else args.table_launches == 1,
-                            row_min_in_tiles={"auto": None, "tiles": True, "separate": False}[args.row_min])
-    row_min_in_tiles = "segmented_min" not in step
-    args.table_launches = 1 if "build_tables" in step else 2 if "input_tables" in step else 4
-    torch.cuda.synchronize()
-    host_timings["upload_and_prepare_s"] = time.perf_counter() - t0
-    host_timings["setup_total_s"] = time.perf_counter() - t_setup
-
-    names = list(step)
-    launchers = [step[k] for k in names]
-    for _ in range(args.warmup):
-        for launch in launchers:
-            launch()
-    torch.cuda.synchronize()
-
-    # ---- timed region: exactly K steps -------------------------------------------------------
     K = args.steps
-    ev = {k: [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
-          for k in names}
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(K):
-        for k, launch in zip(names, launchers):
-            a, b = ev[k][i]
-            a.record()
-            launch()
-            b.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    kernel_ms = {k: float(np.mean([a.elapsed_time(b) for a, b in ev[k]])) for k in names}
-    kernel_ms_min = {k: float(np.min([a.elapsed_time(b) for a, b in ev[k]])) for k in names}
-
-    # the same K steps without per-kernel events: the whole-pass rate.  One event pair brackets
-    # the region on the launch stream: when a pass is a single kernel, region / K is that kernel's
-    # average duration back to back, without the 1 - 2 us an event pair adds to every launch.
-    region = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    region[0].record()
-    for i in range(K):
-        for launch in launchers:
-            launch()
-    region[1].record()
-    torch.cuda.synchronize()
-    wall_plain = time.perf_counter() - t0
-    region_ms = region[0].elapsed_time(region[1])
-
-    # copy-back of the results, for the PCIe-inclusive figure
-    t0 = time.perf_counter()
-    host_out = [x.cpu() for x in (dev.comm, dev.transition, dev.cost) if x is not None]
-    copy_back_s = time.perf_counter() - t0
-    del host_out
-
-    log.info("timed region done: %.3f ms/step", wall_plain / K * 1e3)
-    E = tables.n_entries
-    # the launch that writes the cost matrices; in one-launch mode it also writes the input tables
-    main = "build_tables" if args.table_launches == 1 else "redistribute_tables"
-    alg_bytes = tables.algorithmic_bytes(comm=True, transition=True, cost=True)
-    if args.table_launches == 1:
-        alg_bytes += tables.algorithmic_bytes_input_tables()
-    n_rows = int(tables.edge_n_tgt.astype(np.int64).sum())
-    if row_min_in_tiles:
-        alg_bytes += 12 * n_rows  # minimum f64 + argmin i32 per matrix row, written by the same launch
-    t_kernel_pair = kernel_ms[main] * 1e-3  # an event pair around every launch
-    single_kernel_pass = len(names) == 1
-    t_kernel = region_ms * 1e-3 / K if single_kernel_pass else t_kernel_pair
-    achieved = alg_bytes / t_kernel / 1e9
-    ms_per_step = wall_plain / K * 1e3
+    out, planner, tables, host_timings = measure(args.workload, args, log, K, args.warmup, main_run=True)
     result = {
         "metric": "redistribution_cost_entries_per_s",
-        "value": E * K / wall_plain,
+        "value": out["value"],
         "unit": "entries/s",
         "n_gpus": 1,
         "steps": K,
         "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
+        "ms_per_step": out["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f64",
         "data": "synthetic",
-        "config": {**desc, "edges": tables.n_edges, "strategies": tables.n_strategies, "specs": tables.n_specs,
-                   "entries": E, "tiles": tables.n_tiles, "tiling": tables.tiling,
-                   "edges_deduplicated": int((tables.edge_canonical != np.arange(tables.n_edges)).sum()), "device_row": params.device_name,
-                   "devices_per_host": 8,
-                   "step": {1: "build_tables(tensor, spec and compute-cost tables + comm, transition, cost: one launch)",
-                            2: "input_tables(tensor + spec + compute-cost tables, one launch) + "
-                               "redistribute_tables(comm, transition, cost)",
-                            4: "tensor_tables + spec_tables + compute_costs + redistribute_tables(comm, transition, cost)"
-                            }[args.table_launches] +
-                           (", row minima taken by that launch" if row_min_in_tiles else " + segmented_min(rows)"),
-                   "matrix_rows": n_rows},
-        "roofline": {"bound": "hbm", "kernel": "build_tables_kernel" if args.table_launches == 1 else
-                     "redistribute_tiles_row_min_kernel" if row_min_in_tiles else "redistribute_tiles_kernel",
-                     "achieved": achieved,
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((E, tables.n_tiles, alg_bytes)),
-                     "algorithmic_bytes_input_tables": tables.algorithmic_bytes_input_tables() if args.table_launches == 1 else 0,
-                     "algorithmic_bytes_per_launch": alg_bytes,
-                     "bytes_written_per_entry": {"comm_f64": 8, "transition_u8": 1, "cost_f64": 8},
-                     "bytes_written_per_matrix_row": 12 if row_min_in_tiles else 0,
-                     "avg_launch_us": t_kernel * 1e6,
-                     "avg_launch_us_event_pair_per_launch": t_kernel_pair * 1e6,
-                     "frac_event_pair_per_launch": alg_bytes / t_kernel_pair / 1e9 / HBM_PEAK_GBPS,
-                     "min_launch_us_event_pair_per_launch": kernel_ms_min[main] * 1e3,
-                     "timing": ("one HIP event pair on the launch stream around the K back-to-back launches of the timed "
-                                "region (the pass is this one kernel), / K" if single_kernel_pass else
-                                "HIP events around every launch of the kernel inside the timed region")},
-        "kernel_us": {k: v * 1e3 for k, v in kernel_ms.items()},
-        "ms_per_step_with_events": wall / K * 1e3,
-        "host_timings_s": {k: round(v, 4) for k, v in host_timings.items()},
-        "copy_back_s": copy_back_s,
-        "entries_per_s_including_copy_back": E / (ms_per_step * 1e-3 + copy_back_s),
+        "config": out["config"],
+        "roofline": out["roofline"],
+        "kernel_us": out["kernel_us"],
+        "objective_reduction_us_including_index_upload": out["objective_reduction_us_including_index_upload"],
+        "ms_per_step_with_events": out["ms_per_step_with_events"],
+        "host_timings_s": out["host_timings_s"],
+        "parity": out["parity"],
     }
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(tables, params, args.cpu_seconds)
-    guard.__exit__(None, None, None)
+    if "cpu_baseline" in out:
+        result["cpu_baseline"] = out["cpu_baseline"]
     if planner is not None:
-        plan = {"stages_s": {k: round(v, 4) for k, v in host_timings.items()}}
+        plan = {"stages_s": {k: round(v, 6) for k, v in host_timings.items()}}
         if not args.no_solve:
             log.info("solving the ILP: %d variables", planner.sharding_optimizer.n_variables)
-            plan.update(solve_plan(planner, args))
+            plan.update(solve_plan(planner, args.workload))
         table_stage = host_timings.get("optimizer_tables_s", 0.0)
         other = host_timings.get("capture_s", 0.0) + host_timings.get("optimizer_s", 0.0) - table_stage \
             + plan.get("constraints_s", 0.0) + plan.get("solve_s", 0.0)
         plan["total_with_gpu_tables_s"] = other + table_stage
         if "cpu_baseline" in result:
             # the same plan with the tables built by the CPU port: only the table stage differs
-            cpu_tables = E / result["cpu_baseline"]["value"]
+            cpu_tables = tables.n_entries / result["cpu_baseline"]["value"]
             plan["cpu_table_stage_s"] = cpu_tables
             plan["total_with_cpu_tables_s"] = other + cpu_tables
         result["plan_wall_time"] = plan
         planner.__exit__(None, None, None)
+    del planner, tables
+    # ---- the bandwidth-bound tables, beside the headline ---------------------------------------
+    extra = {}
+    for name in [x for x in args.extra.split(",") if x and x != args.workload]:
+        if name not in WORKLOADS:
+            raise SystemExit(f"bench.py: unknown extra workload {name}")
+        import gc
+
+        gc.collect()
+        torch.cuda.empty_cache()
+        k = max(5, min(K, 20))
+        o, pl, _, _ = measure(name, args, log, k, min(args.warmup, 5), main_run=False)
+        if pl is not None:
+            pl.__exit__(None, None, None)
+        extra[name] = {"workload": o["config"]["workload"], "entries": o["config"]["entries"], "steps": k,
+                       "ms_per_step": o["ms_per_step"], "entries_per_s": o["value"], "step": o["config"]["step"],
+                       "tiles": o["config"]["tiles"], "roofline": o["roofline"], "kernel_us": o["kernel_us"],
+                       "parity": o["parity"], "host_timings_s": o["host_timings_s"]}
+        del o, pl
+    if extra:
+        result["extra"] = extra
     print(json.dumps(result))
 
 

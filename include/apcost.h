@@ -16,6 +16,9 @@
  *     enqueue work and return; they never synchronise and never allocate.
  *   - Return value 0 = success; negative = error, text via apc_last_error().
  *   - The library owns no memory.  Outputs are caller-allocated.
+ *   - Device arrays come from hipMalloc (or an allocator built on it): a byte array may be
+ *     read as aligned 4-byte words, i.e. up to its end rounded up to a multiple of 4, which
+ *     such allocations always cover (tensor_contiguous is read this way).
  *   - No CPU fallback exists: without a HIP device every launch entry fails.
  *
  * Flattened graph tables ("encoding")
@@ -158,7 +161,8 @@ int apc_compute_costs(const apc_params *params, int64_t n_strategies, const int6
  * reads another's output): same arguments, same results, two launches fewer.  For a caller that
  * already holds the per-strategy flop / byte counts, e.g. when the tables of a graph are
  * rebuilt under another cost model.  (A planner that still has to infer those counts from the
- * local shard shapes, compute_estimation.py:244-300, calls the three entry points in turn.) */
+ * local shard shapes, compute_estimation.py:244-300, calls apc_spec_tables first and alone.)
+ * The five spec-table outputs may all be NULL: the spec table is then skipped. */
 int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
                      const int32_t *tensor_itemsize, const int64_t *tensor_shape, const int64_t *tensor_stride,
                      int64_t *tensor_bytes, uint8_t *tensor_contiguous, int64_t n_specs, const uint32_t *spec_codes,
@@ -175,7 +179,10 @@ int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t 
  * torch allgather_cost / allreduce_cost / reduce_scatter_cost
  * (distributed/tensor/_collective_utils.py:281-313), the transition tie-break
  * (:345-351), the grad rescale (:358-359) and cost assembly (:368-372).
- * comm_out / transition_out / cost_out are [n_entries]; any may be NULL. */
+ * comm_out / transition_out / cost_out are [n_entries]; any may be NULL (an array that is not
+ * wanted costs nothing: "all three" and "cost_out alone", the array the ILP objective is summed
+ * from, are separate instantiations of the kernel on 2-D and 3-D meshes).
+ * tensor_contiguous: see "Device arrays" above. */
 int apc_redistribute_tables(const apc_params *params, const int64_t *tensor_bytes,
                             const uint8_t *tensor_contiguous, const uint32_t *spec_codes,
                             const int32_t *spec_tensor, const double *pt_values,
@@ -211,9 +218,10 @@ int apc_build_tables(const apc_params *params, int64_t n_tensors, const int32_t 
  * Rows are numbered edge by edge: row = edge_row_begin[edge] + consumer strategy.
  * dup_row_begin[k] is the first row of the identical edge whose first entry is
  * dup_entry_begin[k] (NULL when dup_entry_begin is).
- * Precondition, for the caller to check: every edge with rows has between 1 and
- * APC_TILE_MAX_COLS producer strategies and every tile holds whole rows (col_begin = 0,
+ * Precondition (apc_validate_row_minima_host checks it): every edge with rows has between 1
+ * and APC_TILE_MAX_COLS producer strategies and every tile holds whole rows (col_begin = 0,
  * col_count = n_src); rows of tiles that do not are left unwritten.
+ * The minima are those of the assembled cost whether or not cost_out is written.
  * No counterpart in the reference (see apc_segmented_min). */
 typedef struct apc_row_minima {
   const int64_t *edge_row_begin; /* [n_edges] */
@@ -222,7 +230,12 @@ typedef struct apc_row_minima {
   int32_t *row_argmin;           /* [n_rows] */
 } apc_row_minima;
 
-/* apc_redistribute_tables with the row minima; all three outputs are required. */
+/* Host-side check of the precondition above (HOST pointers); 0 when the row minima can be
+ * taken by the table launch. */
+int apc_validate_row_minima_host(int64_t n_edges, const int32_t *edge_n_src_host, const int32_t *edge_n_tgt_host,
+                                 int64_t n_tiles, const apc_tile *tiles_host);
+
+/* apc_redistribute_tables with the row minima; any of the three outputs may be NULL. */
 int apc_redistribute_tables_row_min(const apc_params *params, const int64_t *tensor_bytes,
                                     const uint8_t *tensor_contiguous, const uint32_t *spec_codes,
                                     const int32_t *spec_tensor, const double *pt_values,
@@ -231,7 +244,7 @@ int apc_redistribute_tables_row_min(const apc_params *params, const int64_t *ten
                                     uint8_t *transition_out, double *cost_out, const apc_row_minima *rows,
                                     void *stream);
 
-/* apc_build_tables with the row minima; all three outputs are required. */
+/* apc_build_tables with the row minima; any of the three outputs may be NULL. */
 int apc_build_tables_row_min(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
                              const int32_t *tensor_itemsize, const int64_t *tensor_shape,
                              const int64_t *tensor_stride, int64_t *tensor_bytes, uint8_t *tensor_contiguous,
@@ -275,6 +288,22 @@ int apc_segmented_min_copies(const double *values, const int64_t *seg_ptr, int64
 int apc_strategy_bounds(int64_t n_strategies, const int32_t *strat_node, const int64_t *node_strat_begin,
                         const int64_t *node_edge_begin, const int32_t *edges_by_node, const int64_t *edge_row_begin,
                         const double *row_min, double *bound, void *stream);
+
+/* The ILP objective vector, summed on the device so that only one number per variable (not
+ * three arrays per entry) has to leave it.
+ * Replaces the accumulation at optimize_sharding.py:650-655 (opt_target[va] += cost over
+ * ds.values(): entries that share a variable, optimize_sharding.py:211-231, add up in entry
+ * order starting from 0) and the substitution of add_inf_cost_constraint (:522-536: a cost
+ * that is not finite counts as inf_replacement, 10000.0 in the reference, and its variable is
+ * forced to 0).
+ * Variables are numbered group by group.  Group g owns variables [group_var_begin[g],
+ * group_var_begin[g + 1]) and has members [group_member_begin[g], group_member_begin[g + 1]):
+ * edges whose matrices have group_var_begin[g + 1] - group_var_begin[g] entries each and share
+ * variables position by position; member_entry_begin[m] is the member's first entry, members
+ * of a group in ascending order.  objective[v] / forced_zero[v] are [n_vars]. */
+int apc_cost_objective(int64_t n_vars, int64_t n_groups, const int64_t *group_var_begin,
+                       const int64_t *group_member_begin, const int64_t *member_entry_begin, const double *cost,
+                       double inf_replacement, double *objective, uint8_t *forced_zero, void *stream);
 
 #ifdef __cplusplus
 }

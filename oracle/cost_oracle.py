@@ -472,6 +472,24 @@ def segmented_min(values, seg_ptr):
     return mins, args
 
 
+def cost_objective(cost, var_of_entry, n_vars: int, inf_replacement: float = 10000.0):
+    """Objective coefficient and forced-to-zero flag of every ILP variable.
+    ref: autoparallel/optimize_sharding.py:650-655 (``opt_target = defaultdict(int)``;
+    ``opt_target[x["va"]] += x["cost"]`` over ``ds.values()``: entries that share a variable
+    add up one by one, in entry order, starting from the int 0) after :522-536 (a cost that is
+    not finite has been replaced by 10000.0 and its variable forced to 0).
+    Pinned by ``numpy.bincount`` (a sequential accumulation in input order) and by hand cases."""
+    obj = [0] * n_vars
+    forced = [False] * n_vars
+    for c, v in zip(cost, var_of_entry):
+        c, v = float(c), int(v)
+        if not math.isfinite(c):
+            c = inf_replacement
+            forced[v] = True
+        obj[v] += c
+    return [float(x) for x in obj], forced
+
+
 def strategy_bounds(enc: dict, row_min):
     """Optimistic cost of every (node, strategy): the sum, over the node's edges in edge
     order, of that consumer strategy's row minimum (``row_min`` ordered by edge, then consumer

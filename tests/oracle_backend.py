@@ -24,14 +24,38 @@ class OracleBackend:
         tables.build_tiles(tile_entries, dedupe=dedupe, max_copies=max_copies)
         tables.validate(self.product_params)
 
-    def build(self):
+    def launch_tables(self):
         enc = self.tables.as_dict()
         compute, per_arg = c_oracle.compute_costs(enc, self.params)
-        out = c_oracle.build_tables(enc, self.params, per_arg=per_arg)
-        out["compute"] = compute
-        out["compute_per_arg"] = per_arg
-        self.cost = out["cost"]
-        return out
+        self.out = c_oracle.build_tables(enc, self.params, per_arg=per_arg)
+        self.out["compute"] = compute
+        self.out["compute_per_arg"] = per_arg
+        self.cost = self.out["cost"]
+        self.launches = ("oracle",)
+
+    def finish(self, n_vars, group_var_begin, group_member_begin, member_entry_begin):
+        import numpy as np
+
+        # variable of every entry from the group arrays, then the reference's accumulation
+        # (numpy.bincount adds the weights one by one in input order, like the oracle's loop)
+        sizes = np.diff(group_var_begin)
+        var = np.full(len(self.cost), -1, np.int64)
+        for g in range(len(sizes)):
+            for m in range(int(group_member_begin[g]), int(group_member_begin[g + 1])):
+                b = int(member_entry_begin[m])
+                var[b:b + sizes[g]] = group_var_begin[g] + np.arange(sizes[g])
+        assert (var >= 0).all()
+        bad = ~np.isfinite(self.cost)
+        obj = np.bincount(var, weights=np.where(bad, 10000.0, self.cost), minlength=n_vars)
+        forced = np.bincount(var, weights=bad, minlength=n_vars) > 0
+        return {"objective": obj, "forced_zero": forced, "compute": self.out["compute"],
+                "compute_per_arg": self.out["compute_per_arg"]}
+
+    def host_array(self, name):
+        return self.out[name]
+
+    def gather(self, name, entries):
+        return self.out[name][entries]
 
     def row_min(self, row_ptr):
         return c_oracle.segmented_min(self.cost, row_ptr)

@@ -138,7 +138,8 @@ def test_deduplicated_tiles_write_every_entry_exactly_once():
 
 def test_row_minimum_entry_points_reject_incomplete_arguments():
     """Argument checks of apc_*_row_min run on the host before anything is launched: a NULL
-    descriptor, a descriptor without its arrays, and row minima without all three outputs."""
+    descriptor, a descriptor without its arrays, identical edges without their rows; the host
+    check of the whole-row precondition; the objective's argument checks."""
     import ctypes
 
     lib = _native.lib()
@@ -155,13 +156,38 @@ def test_row_minimum_entry_points_reject_incomplete_arguments():
     assert "NULL row-minimum array" in error_of(
         lib.apc_redistribute_tables_row_min(*tables, one, one, one, ctypes.byref(empty), None))
     rows = _native.ApcRowMinima(one, None, one, one)
-    assert "need comm_out, transition_out and cost_out" in error_of(
-        lib.apc_redistribute_tables_row_min(*tables, one, None, one, ctypes.byref(rows), None))
     with_dups = tables[:9] + (one,) + tables[10:]
     assert "dup_row_begin" in error_of(
         lib.apc_redistribute_tables_row_min(*with_dups, one, one, one, ctypes.byref(rows), None))
     assert "NULL selection" in error_of(lib.apc_segmented_min_copies(
         one, one, ctypes.c_int64(3), None, None, None, ctypes.c_int64(9), one, one, None))
+    assert "no group" in error_of(lib.apc_cost_objective(
+        ctypes.c_int64(4), ctypes.c_int64(0), one, one, one, one, ctypes.c_double(10000.0), one, one, None))
+    assert "NULL array" in error_of(lib.apc_cost_objective(
+        ctypes.c_int64(4), ctypes.c_int64(1), one, one, one, None, ctypes.c_double(10000.0), one, one, None))
+
+
+def test_row_minimum_precondition_is_checked_on_the_host():
+    """apc_validate_row_minima_host: tiles of whole rows pass; an edge with more producer
+    strategies than a tile holds, or a tile cut by columns, is named."""
+    tb = stress_dag(seed=5, n_nodes=60, mesh_sizes=(4, 2))
+    tb.build_tiles(4096)
+    assert tb.rows_fit_tiles()
+    tb.validate_row_minima()
+    wide = stress_dag(seed=5, n_nodes=60, mesh_sizes=(4, 2), max_strategies=100)
+    wide.build_tiles(4096)
+    assert not wide.rows_fit_tiles()
+    with pytest.raises(RuntimeError, match="producer strategies"):
+        wide.validate_row_minima()
+    # cut one tile by columns: same edge, half the columns
+    rec = tb.tile_records.copy()
+    t = int(np.argmax((rec["counts"] >> 16) >= 2))
+    rc, cc = int(rec["counts"][t]) & 0xFFFF, int(rec["counts"][t]) >> 16
+    assert cc >= 2
+    rec["counts"][t] = rc | ((cc // 2) << 16)
+    tb.tile_records = rec
+    with pytest.raises(RuntimeError, match="not the whole rows"):
+        tb.validate_row_minima()
 
 
 def test_row_copies_cover_every_row_once_and_pair_identical_rows():

@@ -561,7 +561,12 @@ def test_randomized_configurations(gpu_device, monkeypatch):
         d = DeviceCostTables(tb, CostModelParams.from_mesh(mesh, rescale=rescale), device=gpu_device)
         in_tiles = tb.rows_fit_tiles() and bool(rng.random() < 0.7)  # row minima taken by the table launch
         assert tb.rows_fit_tiles() or maxs > 64
-        step = d.prepare_step(row_min=True, fused_inputs=True, one_launch=one_launch, row_min_in_tiles=in_tiles)
+        # which per-entry arrays the pass writes: all three, the assembled cost alone (the planner's
+        # pass; both are compile-time modes of the kernels on 2-D and 3-D meshes) or another subset
+        outputs = [("comm", "transition", "cost"), ("cost",), ("comm", "cost"), ("transition", "cost")][int(rng.integers(0, 4))]
+        spec_table = bool(rng.random() < 0.5)
+        step = d.prepare_step(row_min=True, fused_inputs=True, one_launch=one_launch, row_min_in_tiles=in_tiles,
+                              outputs=outputs, spec_table=spec_table)
         assert ("segmented_min" in step) != in_tiles
         d.row_min.fill_(-1.0)
         d.row_argmin.fill_(-7)
@@ -572,10 +577,17 @@ def test_randomized_configurations(gpu_device, monkeypatch):
         want_cc, want_pa = c_oracle.compute_costs(enc, op)
         want = c_oracle.build_tables(enc, op, per_arg=want_pa)
         want_min, want_arg = c_oracle.segmented_min(want["cost"], tb.row_ptr())
-        what = f"case {it}: mesh {mesh}, {maxs} strategies, {copies} copies, threads {threads or 'auto'}, one launch {one_launch}, row minima in tiles {in_tiles}"
-        _assert_costs(d.comm.cpu().numpy(), want["comm"], what + " comm")
+        what = (f"case {it}: mesh {mesh}, {maxs} strategies, {copies} copies, threads {threads or 'auto'}, one launch "
+                f"{one_launch}, row minima in tiles {in_tiles}, outputs {outputs}, spec table {spec_table}")
+        assert (d.comm is None) == ("comm" not in outputs) and (d.transition is None) == ("transition" not in outputs)
+        if d.comm is not None:
+            _assert_costs(d.comm.cpu().numpy(), want["comm"], what + " comm")
         _assert_costs(d.cost.cpu().numpy(), want["cost"], what + " cost")
-        assert np.array_equal(d.transition.cpu().numpy(), want["transition"]), what
+        if d.transition is not None:
+            assert np.array_equal(d.transition.cpu().numpy(), want["transition"]), what
+        # an array the pass left out is computed on request, by a launch that writes it alone
+        _assert_costs(d.fetch("comm").cpu().numpy(), want["comm"], what + " fetched comm")
+        assert np.array_equal(d.fetch("transition").cpu().numpy(), want["transition"]), what + " fetched transition"
         _assert_costs(d.compute_cost.cpu().numpy(), want_cc, what + " compute_cost")
         assert np.array_equal(d.row_min.cpu().numpy(), want_min) and np.array_equal(d.row_argmin.cpu().numpy(), want_arg), what
 

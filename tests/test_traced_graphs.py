@@ -36,6 +36,7 @@ TINY_MOE = DeepSeekV3Config(dim=256, n_layers=3, n_dense_layers=1, n_heads=8, q_
 CASES = {
     # name: (config, mesh, batch, seq)
     "block_1k_mesh64": (BLOCK_1K, (64,), 8 * 8, 2048),  # batch x8 so that it divides the 64-rank mesh
+    "block_1k_batch8_mesh64": (BLOCK_1K, (64,), 8, 2048),  # the configuration as stated: no batch-sharded placement exists
     "llama3_8b_1layer_mesh32x8": (dataclasses.replace(LLAMA3_8B, n_layers=1), (32, 8), 32, 8192),
     "llama3_70b_1layer_mesh8x8x8": (dataclasses.replace(LLAMA3_70B, n_layers=1), (8, 8, 8), 64, 8192),
     "dsv3_moe_tiny_mesh64x4": (TINY_MOE, (64, 4), 16, 512),  # batch 16 < 64 ranks: tokens shard along the sequence
@@ -148,6 +149,9 @@ def test_device_tables_match_oracle_on_benchmark_configurations(gpu_device, fake
             out = {name: getattr(tb, name).copy() for name in ("strat_flops", "strat_rw_bytes", "strat_dtype",
                                                                "strat_zero_cost", "spec_codes", "spec_tensor",
                                                                "edge_flags")}
+            # what the planner takes from the backend: one objective coefficient and one flag per variable
+            out.update(objective=o.objective_vector.copy(), forced=o.forced_zero_vars.copy())
+            assert not o._host_arrays, "no per-entry array has left the backend so far"
             out.update(comm=o.comm_cost.copy(), transition=o.transition_cost.copy(), cost=o.cost.copy(),
                        per_arg=o.compute_cost_per_arg.copy(), n_entries=tb.n_entries,
                        backend=type(o.backend).__name__)
@@ -163,6 +167,48 @@ def test_device_tables_match_oracle_on_benchmark_configurations(gpu_device, fake
             assert np.array_equal(d[name], o[name]), name
     # something was actually costed: finite positive comm and compute costs exist
     assert (d["comm"][np.isfinite(d["comm"])] > 0).any() and (d["per_arg"] > 0).any()
+
+
+def _solve_llama(autop):
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    # examples/example_llama3.py:205-218
+    autop.add_parameter_memory_constraint(low=None, high=None)
+    autop.add_input_constraints([(Shard(0), Replicate())])
+    autop.add_output_constraints([(Shard(0), Shard(2))])
+    return autop.optimize_placement()
+
+
+@pytest.mark.gpu
+def test_full_depth_llama3_8b_on_mesh_32x8(gpu_device, fake_pg):
+    """The headline configuration at full size: Llama-3-8B, 32 layers, batch 32 x 8192 tokens,
+    mesh (32, 8), linked layers (examples/example_llama3.py:56-68, 205-218).  Every one of the
+    1.8 M comm / transition / cost entries, the compute costs, the row minima and the objective
+    vector against the C oracle, then the same plan and objective from device and oracle tables."""
+    results = {}
+    for name, planner_cls in (("device", AutoParallelPlanner), ("oracle", OraclePlanner)):
+        with _planner(planner_cls, LLAMA3_8B, (32, 8), 32, 8192, repeated_subgraphs=True) as autop:
+            o = autop.sharding_optimizer
+            tb = o.encoded.tables
+            assert type(o.backend).__name__ == ("DeviceBackend" if name == "device" else "OracleBackend")
+            if name == "device":
+                assert o.backend.launches == ("build_tables",), "the planner's table build is one launch"
+                assert o.backend.dev.comm is None and o.backend.dev.transition is None
+            plan = _solve_llama(autop)
+            out = {"objective_vector": o.objective_vector.copy(), "forced": o.forced_zero_vars.copy(),
+                   "plan": {n.name: str(s) for n, s in plan.items()}, "objective": o.objective_value(),
+                   "res": list(o.res), "n_entries": tb.n_entries, "n_variables": o.n_variables,
+                   "per_arg": o.compute_cost_per_arg.copy(), "compute": o.compute_cost.copy()}
+            assert not o._host_arrays, "planning copies no per-entry array to the host"
+            out["row_min"], out["row_argmin"] = o.row_minima()
+            out.update(comm=o.comm_cost.copy(), transition=o.transition_cost.copy(), cost=o.cost.copy())
+            results[name] = out
+    d, o = results["device"], results["oracle"]
+    assert d["n_entries"] == o["n_entries"] == 1_821_368 and d["n_variables"] == o["n_variables"] < 100_000
+    for key in ("comm", "transition", "cost", "compute", "per_arg", "row_min", "row_argmin", "objective_vector", "forced"):
+        assert np.array_equal(d[key], o[key]), key
+    assert d["res"] == o["res"] and d["plan"] == o["plan"]
+    assert d["objective"] == o["objective"] > 0
 
 
 def test_split_tensor_rule(fake_pg):
