@@ -220,17 +220,18 @@ class DeviceCostTables:
     def row_min_in_tiles_pays(self) -> bool:
         """Whether the launch that writes the cost matrices should take the row minima itself.
         Inside the tiles the minima cost about 0.5 ns per tile (a barrier and the stores of the
-        row results) plus 1 ps per entry a tile computes (identical edges are computed, and
+        row results) plus 1.6 ps per entry a tile computes (identical edges are computed, and
         reduced, once for all their copies); a ``segmented_min`` launch costs about 4 us plus
-        reading every stored entry back at about 4.5 TB/s.  Measured per pass, in tiles /
-        separate: Llama-3-8B on (32, 8) 18.8 / 23.9 us (34.2 / 31.5 us when every identical edge
-        is computed on its own: 12 497 tiles of 146 entries), the mixture of experts 15.8 /
-        17.7 us, the 464 M-entry stress table 3.16 / 3.32 ms."""
+        reading every stored entry back at about 4.5 TB/s.  Measured, in tiles / separate:
+        Llama-3-8B on (32, 8), whose tiles compute an eighth of the entries they store, 18.8 /
+        23.9 us per pass with all three arrays written; the 464 M-entry stress table, where every
+        entry is computed, 2.42 ms for the launch that writes the cost alone with the minima
+        against 1.45 ms without them plus 0.87 ms for the separate launch."""
         tb = self.tables
         if tb.n_tiles == 0 or not tb.rows_fit_tiles():
             return False
         computed = int((tb.tile_row_count.astype(np.int64) * tb.tile_col_count.astype(np.int64)).sum())
-        return 0.5e-3 * tb.n_tiles + 1.0e-6 * computed < 4.0 + 8.0 * tb.n_entries / 4.5e6
+        return 0.5e-3 * tb.n_tiles + 1.6e-6 * computed < 4.0 + 8.0 * tb.n_entries / 4.5e6
 
     def _alloc_input_tables(self, spec_table: bool):
         """Allocates (does not fill) the outputs of the tensor, compute-cost and, when wanted,
