@@ -79,6 +79,7 @@ EXPORTS = (
     "apc_strategy_bounds",
     "apc_cost_objective",
     "apc_validate_row_minima_host",
+    "apc_diffusion_sweeps",
 )
 
 _lib = None

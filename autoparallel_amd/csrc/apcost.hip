@@ -1352,6 +1352,123 @@ __global__ __launch_bounds__(kBlock) void cost_objective_kernel(int64_t n_vars, 
   forced_zero[v] = forced ? 1 : 0;
 }
 
+// ------------------------------------------------------------------------------------------
+// a14 put to work: min-sum diffusion over the planning program's labelling form.  A class
+// (linked nodes) has a unary cost vector; an edge between two classes has a cost matrix
+// (rows = labels of class edge_i, columns = labels of class edge_j, +inf = forbidden pair).
+// A node update takes, for every incident matrix, the minima of the rows (or columns) the
+// class labels out of the matrix and into the class, then hands their sum back to the
+// incident matrices in equal shares.  Every update leaves the cost of every labelling unchanged
+// and never lowers  sum_classes min unary + sum_edges min matrix,  a lower bound of the
+// program's optimum; min-marginals read off the reparametrised costs prune the program.
+// One workgroup per class of one colour (classes of a colour share no edge, so they update
+// together); the sweep is the sequence of colours.  Arithmetic in a fixed order (the sum over
+// incident edges in incidence order, one division, one subtraction and one addition per
+// matrix element): the same bits as the CPU restatement.
+// ------------------------------------------------------------------------------------------
+constexpr int kDiffusionMaxLabels = 2048;
+
+struct DiffusionArgs {
+  const int32_t *nodes;  // the classes of this launch
+  const int64_t *label_begin, *inc_begin;
+  const int32_t *inc_edge;
+  const uint8_t *inc_side;
+  const int64_t *edge_begin;
+  const int32_t *edge_i, *edge_j;
+  double *theta, *unary;
+};
+
+__device__ __forceinline__ double wave_min(double v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const double o = __shfl_xor(v, off, 64);
+    v = o < v ? o : v;
+  }
+  return v;
+}
+
+__global__ __launch_bounds__(kBlock) void diffusion_node_update_kernel(DiffusionArgs a) {
+  __shared__ double s_tot[kDiffusionMaxLabels];
+  const int c = a.nodes[blockIdx.x];
+  const int64_t l0 = a.label_begin[c];
+  const int n_labels = (int)(a.label_begin[c + 1] - l0);
+  const int64_t t0 = a.inc_begin[c], t1 = a.inc_begin[c + 1];
+  if (t1 == t0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int kWaves = kBlock / 64;
+  const double inf = __builtin_inf();
+  for (int x = tid; x < n_labels; x += kBlock) s_tot[x] = a.unary[l0 + x];
+  __syncthreads();
+  // pull: the minimum of every row / column of the class out of each incident matrix
+  for (int64_t t = t0; t < t1; ++t) {
+    const int k = a.inc_edge[t];
+    double *m = a.theta + a.edge_begin[k];
+    const int ej = a.edge_j[k];
+    const int nj = (int)(a.label_begin[ej + 1] - a.label_begin[ej]);
+    if (a.inc_side[t] == 0) {  // the class labels the rows: one wavefront per row
+      for (int x = wave; x < n_labels; x += kWaves) {
+        double *row = m + (int64_t)x * nj;
+        double d = inf;
+        for (int y = lane; y < nj; y += 64) {
+          const double v = row[y];
+          d = v < d ? v : d;
+        }
+        d = wave_min(d);
+        if (d < inf)
+          for (int y = lane; y < nj; y += 64) row[y] -= d;
+        if (lane == 0) s_tot[x] += d;
+      }
+    } else {  // the class labels the columns: one thread per column
+      const int ei = a.edge_i[k];
+      const int ni = (int)(a.label_begin[ei + 1] - a.label_begin[ei]);
+      for (int y = tid; y < n_labels; y += kBlock) {
+        double d = inf;
+        for (int x = 0; x < ni; ++x) {
+          const double v = m[(int64_t)x * n_labels + y];
+          d = v < d ? v : d;
+        }
+        if (d < inf)
+          for (int x = 0; x < ni; ++x) m[(int64_t)x * n_labels + y] -= d;
+        s_tot[y] += d;
+      }
+    }
+    __syncthreads();
+  }
+  // share: an equal part of the total for every incident matrix; a label without a finite
+  // pair on some edge can never be taken: +inf everywhere
+  const double degree = (double)(t1 - t0);
+  for (int x = tid; x < n_labels; x += kBlock) {
+    const double tot = s_tot[x];
+    const bool finite = tot < inf;
+    s_tot[x] = finite ? tot / degree : inf;
+    a.unary[l0 + x] = finite ? 0.0 : inf;
+  }
+  __syncthreads();
+  for (int64_t t = t0; t < t1; ++t) {
+    const int k = a.inc_edge[t];
+    double *m = a.theta + a.edge_begin[k];
+    if (a.inc_side[t] == 0) {
+      const int ej = a.edge_j[k];
+      const int nj = (int)(a.label_begin[ej + 1] - a.label_begin[ej]);
+      for (int x = wave; x < n_labels; x += kWaves) {
+        double *row = m + (int64_t)x * nj;
+        const double share = s_tot[x];
+        for (int y = lane; y < nj; y += 64) row[y] = share < inf ? row[y] + share : inf;
+      }
+    } else {
+      const int ei = a.edge_i[k];
+      const int ni = (int)(a.label_begin[ei + 1] - a.label_begin[ei]);
+      for (int y = tid; y < n_labels; y += kBlock) {
+        const double share = s_tot[y];
+        for (int x = 0; x < ni; ++x) {
+          double *p = m + (int64_t)x * n_labels + y;
+          *p = share < inf ? *p + share : inf;
+        }
+      }
+    }
+  }
+}
+
 inline unsigned blocks_for(int64_t n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
 
 template <int G>
@@ -1864,6 +1981,32 @@ int apc_validate_row_minima_host(int64_t n_edges, const int32_t *edge_n_src, con
     if (tl.col_begin != 0 || (tl.counts >> 16) != edge_n_src[tl.edge])
       return fail(-2, "tile %lld: columns [%d, +%d) are not the whole rows of edge %d (%d columns)", (long long)t,
                   tl.col_begin, tl.counts >> 16, tl.edge, edge_n_src[tl.edge]);
+  }
+  return 0;
+}
+
+int apc_diffusion_sweeps(int32_t n_sweeps, int32_t n_colors, const int64_t *color_begin_host, const int32_t *color_nodes,
+                         int64_t n_classes, const int64_t *label_begin, const int64_t *inc_begin, const int32_t *inc_edge,
+                         const uint8_t *inc_side, const int64_t *edge_begin, const int32_t *edge_i, const int32_t *edge_j,
+                         int32_t max_labels, double *theta, double *unary, void *stream) {
+  if (n_sweeps < 0 || n_colors < 0 || n_classes < 0) return fail(-1, "apc_diffusion_sweeps: negative count");
+  if (n_sweeps == 0 || n_colors == 0 || n_classes == 0) return 0;
+  if (max_labels > kDiffusionMaxLabels)
+    return fail(-1, "apc_diffusion_sweeps: a class has %d labels, at most %d are staged", max_labels, kDiffusionMaxLabels);
+  if (!color_begin_host || !color_nodes || !label_begin || !inc_begin || !edge_begin || !theta || !unary)
+    return fail(-1, "apc_diffusion_sweeps: NULL array");
+  if (color_begin_host[0] != 0 || color_begin_host[n_colors] != n_classes)
+    return fail(-1, "apc_diffusion_sweeps: the colours must partition the classes");
+  for (int32_t s = 0; s < n_sweeps; ++s) {
+    for (int32_t c = 0; c < n_colors; ++c) {
+      const int64_t n = color_begin_host[c + 1] - color_begin_host[c];
+      if (n < 0 || n > INT32_MAX) return fail(-1, "apc_diffusion_sweeps: colour %d has %lld classes", c, (long long)n);
+      if (n == 0) continue;
+      hipLaunchKernelGGL(diffusion_node_update_kernel, dim3((unsigned)n), dim3(kBlock), 0, (hipStream_t)stream,
+                         DiffusionArgs{color_nodes + color_begin_host[c], label_begin, inc_begin, inc_edge, inc_side,
+                                       edge_begin, edge_i, edge_j, theta, unary});
+    }
+    if (int rc = check_launch("apc_diffusion_sweeps")) return rc;
   }
   return 0;
 }

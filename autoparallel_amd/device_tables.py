@@ -547,6 +547,32 @@ class DeviceCostTables:
         _native.check(rc, "apc_segmented_min")
         return mins, args
 
+    # ---- dual ascent over the planning program's labelling form ---------------------------------
+    @_guarded
+    def diffusion_sweeps(self, graph, theta: np.ndarray, unary: np.ndarray, n_sweeps: int):
+        """``n_sweeps`` sweeps of min-sum diffusion (``apc_diffusion_sweeps``) over ``graph``
+        (``pruning.LabelGraph``) starting from the host arrays ``theta`` / ``unary``; returns the
+        updated pair as new host arrays.  The graph's index arrays are uploaded once."""
+        cached = getattr(self, "_diffusion_graph", None)
+        if cached is None or cached[0] is not graph:
+            names = ("color_nodes", "label_begin", "inc_begin", "inc_edge", "inc_side", "edge_begin", "edge_i", "edge_j")
+            cached = (graph, {k: _to_device(np.ascontiguousarray(getattr(graph, k)), self.device) for k in names})
+            self._diffusion_graph = cached
+        d = cached[1]
+        th = torch.from_numpy(np.ascontiguousarray(theta, np.float64)).to(self.device)
+        un = torch.from_numpy(np.ascontiguousarray(unary, np.float64)).to(self.device)
+        color_begin = np.ascontiguousarray(graph.color_begin, np.int64)
+        max_labels = int(np.diff(graph.label_begin).max()) if graph.n_classes else 0
+        with torch.cuda.device(self.device):
+            rc = self.lib.apc_diffusion_sweeps(
+                ctypes.c_int32(int(n_sweeps)), ctypes.c_int32(len(color_begin) - 1),
+                color_begin.ctypes.data_as(ctypes.c_void_p), self._p(d["color_nodes"]), ctypes.c_int64(graph.n_classes),
+                self._p(d["label_begin"]), self._p(d["inc_begin"]), self._p(d["inc_edge"]), self._p(d["inc_side"]),
+                self._p(d["edge_begin"]), self._p(d["edge_i"]), self._p(d["edge_j"]), ctypes.c_int32(max_labels),
+                self._p(th), self._p(un), self._stream())
+        _native.check(rc, "apc_diffusion_sweeps")
+        return th.cpu().numpy(), un.cpu().numpy()
+
     def strategy_bounds(self, row_min: torch.Tensor) -> torch.Tensor:
         """Per-(node, strategy) sum of the row minima of the node's edges (``row_min`` in the
         order of ``CostTables.row_ptr()``)."""

@@ -130,6 +130,10 @@ class DeviceBackend:
             idx = torch.from_numpy(np.ascontiguousarray(entries, np.int64)).to(self.dev.device)
             return self.dev.fetch(name)[idx].cpu().numpy()
 
+    def diffusion_sweeps(self, graph, theta, unary, n_sweeps):
+        """Sweeps of the dual ascent that prunes the program (pruning.py), on the device."""
+        return self.dev.diffusion_sweeps(graph, theta, unary, n_sweeps)
+
     def row_min(self, row_ptr):
         from .device_tables import _real_tensors
 
@@ -284,6 +288,14 @@ class ShardingOptimizer:
     # variable.  Same feasible plans and optimum, far fewer branching variables for the solver.
     node_choice_variables = True
     compact_constraints = True  # with choice variables: the structural constraints written through them
+    # Before the solver runs: a dual ascent over the program's labelling form (row / column minima
+    # of the reparametrised cost matrices, on the device), an incumbent rounded from it, and every
+    # strategy and strategy pair whose bound exceeds the incumbent fixed to zero (pruning.py).
+    # Sweeps are run in these chunks; after each the bound and the incumbent are re-evaluated and
+    # the ascent stops once they agree to ``prune_gap``.
+    prune_before_solve = True
+    prune_sweep_chunks = (40, 40, 80, 80, 160)
+    prune_gap = 2e-4
     # copy ``comm`` back and write it into every OpSpec.redistribute_cost at construction
     # (optimize_sharding.py:361-363); off: ``materialize_redistribute_costs()`` does it on request
     write_back_redistribute_cost = False
@@ -330,6 +342,11 @@ class ShardingOptimizer:
         self._finish_tables()
         self.prob = BinaryProgram(self.n_variables + self.n_choice_variables, "AutoParallel")
         self.res = None
+        # what the user constraints mean on the labelling form (read by _label_graph)
+        self._label_masks = {}  # s_i -> allowed strategies
+        self._pair_ties = []  # (s_i, s_j, [(strategy of i, strategy of j) that go together])
+        self._linear_rows = []  # ([(s_i, coefficient per strategy)], lower, upper)
+        self.solve_stats = {}
         self.add_default_constraints()
 
     # ------------------------------------------------------------------------------------
@@ -706,7 +723,13 @@ class ShardingOptimizer:
         obj = np.zeros(self.prob.n_vars, np.float64)
         obj[:self.n_variables] = self.objective_vector
         self.prob.objective = obj
+        self.solve_stats = {"columns": int((self.prob.upper > 0).sum())}
+        if self.prune_before_solve and self.node_choice_variables:
+            self.prune()
+        t0 = time.perf_counter()
         status = self.prob.solve(verbose=verbose, time_limit=self.solver_time_limit, mip_rel_gap=self.solver_rel_gap)
+        self.solve_stats.update(solver_s=time.perf_counter() - t0, solved_by=self.prob.solved_by,
+                                columns_solved=getattr(self.prob, "cols_after_fixing", None))
         if status == -1:
             print(self.get_violated_constraints_log())
             raise RuntimeError("Unsolvable problem")
@@ -729,6 +752,153 @@ class ShardingOptimizer:
                 f"{node}: arguments chose different strategies {first} and {ss}"
         return {node: self.strats[node].strategies[ss] for node, ss in chosen_strategy.items()}
 
+    # ---- pruning before the solve (no counterpart in the reference, see pruning.py) ----------------
+    def _label_graph(self):
+        """The program as a pairwise labelling problem over classes of nodes that must take the
+        same strategy (linked nodes, and nodes tied through a shared variable block)."""
+        from . import pruning
+
+        parent = {}
+
+        def find(x):
+            parent.setdefault(x, x)
+            while parent[x] != x:
+                parent[x] = parent[parent[x]]
+                x = parent[x]
+            return x
+
+        raw = {}  # var base -> [nt, ns, row choice bases, column choice bases]
+        for s_i, node in enumerate(self.nodes):
+            if node.op == "output":
+                continue
+            cb = self.node_choice_base[s_i]
+            find(cb)
+            for argi in range(self.num_args[s_i]):
+                b, nt, ns = self._edge_vars(s_i, argi)
+                raw.setdefault(b, [nt, ns, [], []])[2].append(cb)
+            for user in node.users:
+                if user.op == "output":
+                    continue
+                s_j = self.node_map[user]
+                argj = [i for i, x in enumerate(user.all_input_nodes) if x == node]
+                bc, ntc, nsc = self._edge_vars(s_j, argj[0])
+                raw.setdefault(bc, [ntc, nsc, [], []])[3].append(cb)
+        for nt, ns, rows, cols in raw.values():
+            for side in (rows, cols):
+                for cb in side[1:]:
+                    parent[find(cb)] = find(side[0])
+        class_id, class_sizes, members = {}, [], []
+        for s_i, node in enumerate(self.nodes):
+            if node.op == "output":
+                continue
+            root = find(self.node_choice_base[s_i])
+            if root not in class_id:
+                class_id[root] = len(class_sizes)
+                class_sizes.append(len(self.strats[node].strategies))
+                members.append(set())
+            members[class_id[root]].add(self.node_choice_base[s_i])
+            assert class_sizes[class_id[root]] == len(self.strats[node].strategies)
+        cls = lambda cb: class_id[find(cb)]  # noqa: E731
+        blocks = [pruning.Block(b, nt, ns, cls(rows[0]), cls(cols[0]) if cols else -1)
+                  for b, (nt, ns, rows, cols) in raw.items()]
+        forbidden = self.forced_zero_vars | (self.prob.upper[:self.n_variables] == 0)
+
+        def block_costs(b):
+            sl = slice(b.var_begin, b.var_begin + b.nt * b.ns)
+            return np.where(forbidden[sl], np.inf, self.objective_vector[sl]).reshape(b.nt, b.ns)
+
+        masks = {}
+        for s_i, allowed in self._label_masks.items():
+            c = cls(self.node_choice_base[s_i])
+            masks[c] = masks.get(c, True) & allowed
+        # a linear row over the strategies of several nodes: a strategy whose coefficient cannot be
+        # made up for by the best choices of all other nodes is infeasible
+        for per_node, lo, hi in self._linear_rows:
+            least = math.fsum(min(r) for _, r in per_node)
+            most = math.fsum(max(r) for _, r in per_node)
+            for s_i, ratios in per_node:
+                r = np.asarray(ratios)
+                ok = (r - r.min() <= (hi - least) + 1e-9) & (r.max() - r <= (most - lo) + 1e-9)
+                c = cls(self.node_choice_base[s_i])
+                masks[c] = masks.get(c, True) & ok
+        ties = []
+        for s_i, s_j, pairs in self._pair_ties:
+            ci, cj = cls(self.node_choice_base[s_i]), cls(self.node_choice_base[s_j])
+            m = np.zeros((class_sizes[ci], class_sizes[cj]))
+            for a, b in pairs:  # strategy a of the parameter goes with strategy b of its gradient, and only with it
+                m[a, :] = np.inf
+            for a, b in pairs:
+                col = np.full(class_sizes[ci], np.inf)
+                col[[x for x, y in pairs if y == b]] = 0.0
+                m[:, b] = col
+            ties.append((ci, cj, m))
+        graph = pruning.build_label_graph(blocks, class_sizes, block_costs, masks, ties)
+        graph.members = members
+        return graph
+
+    def _plan_vector(self, graph, labels):
+        """The 0/1 vector of the program for a labelling of the classes."""
+        x = np.zeros(self.prob.n_vars, np.float64)
+        for c, bases in enumerate(graph.members):
+            for cb in bases:
+                x[cb + labels[c]] = 1.0
+        forbidden = self.forced_zero_vars | (self.prob.upper[:self.n_variables] == 0)
+        for b in graph.blocks:
+            r = int(labels[b.row_class])
+            if b.col_class >= 0:
+                col = int(labels[b.col_class])
+            else:
+                row = slice(b.var_begin + r * b.ns, b.var_begin + (r + 1) * b.ns)
+                col = int(np.argmin(np.where(forbidden[row], np.inf, self.objective_vector[row])))
+            x[b.var_begin + r * b.ns + col] = 1.0
+        return x
+
+    def prune(self):
+        """Fixes to zero the variables that the bound proves to be in no optimal plan."""
+        from . import pruning
+
+        t0 = time.perf_counter()
+        stats = self.solve_stats
+        graph = self._label_graph()
+        if graph.n_classes == 0 or int(np.diff(graph.label_begin).max()) > pruning.MAX_LABELS:
+            stats["pruning"] = "skipped"
+            return
+        theta, unary = graph.theta.copy(), graph.unary.copy()
+        best_ub, best_x, sweeps, bound = math.inf, None, 0, -math.inf
+        for chunk in self.prune_sweep_chunks:
+            theta, unary = self.backend.diffusion_sweeps(graph, theta, unary, chunk)
+            sweeps += chunk
+            bound = pruning.lower_bound(graph, theta, unary)[0]
+            labels = pruning.decode(graph, theta, unary)
+            x = self._plan_vector(graph, labels)
+            if (x <= self.prob.upper).all() and not self.prob.violated_constraints(x):
+                ub = float(self.prob.objective @ x)
+                if ub < best_ub:
+                    best_ub, best_x = ub, x
+            if best_ub - bound <= self.prune_gap * abs(best_ub):
+                break
+        stats.update(prune_sweeps=sweeps, lower_bound=bound, incumbent=best_ub if best_x is not None else None,
+                     label_classes=graph.n_classes, label_edges=graph.n_edges)
+        if best_x is not None:
+            dead_label, dead_pair = pruning.prune_masks(graph, theta, unary, best_ub)
+            lb = graph.label_begin
+            off = []
+            for c, bases in enumerate(graph.members):
+                d = np.nonzero(dead_label[lb[c]:lb[c + 1]])[0]
+                off.extend(cb + d for cb in bases)
+            for b in graph.blocks:
+                dead = dead_label[lb[b.row_class]:lb[b.row_class + 1]][:, None] & np.ones((1, b.ns), bool)
+                if b.col_class >= 0:
+                    pair = graph.matrix(dead_pair, b.edge)
+                    dead = dead | (pair.T if b.transposed else pair)
+                off.append(b.var_begin + np.nonzero(dead.ravel())[0])
+            off = np.concatenate(off) if off else np.zeros(0, np.int64)
+            assert not best_x[off].any(), "the incumbent uses a variable the bound rules out"
+            self.prob.force_zero(off)
+            self.incumbent = best_x
+        stats["columns_after_pruning"] = int((self.prob.upper > 0).sum())
+        stats["prune_s"] = time.perf_counter() - t0
+
     def objective_value(self) -> float:
         return float(self._values("cost", self.res_entries).sum())
 
@@ -742,6 +912,9 @@ class ShardingOptimizer:
             constraint_name = "user_constraint"
         s_i = self.node_map[node]
         rows = np.asarray(sorted(output_constraint_indices), np.int64)
+        allowed = np.zeros(len(self.strats[node].strategies), bool)
+        allowed[rows] = True
+        self._label_masks[s_i] = self._label_masks.get(s_i, True) & allowed
         for argi in range(self.num_args[s_i]):
             b, nt, ns = self._edge(s_i, argi)
             idx = (b + rows[:, None] * ns + np.arange(ns)[None, :]).ravel()
@@ -762,6 +935,7 @@ class ShardingOptimizer:
             strat_gp = [str(s.output_specs) for s in self.strats[grad].strategies]
             bp, _, nsp = self._edge(s_i, 0)
             bg, _, nsg = self._edge(s_j, 0)
+            self._pair_ties.append((s_i, s_j, [(oi, strat_gp.index(sp)) for oi, sp in enumerate(strat_p) if sp in strat_gp]))
             for oi in range(num_out):
                 sp = strat_p[oi]
                 if sp not in strat_gp:
@@ -779,12 +953,14 @@ class ShardingOptimizer:
         world_size = math.prod(self.mesh.shape)
         cols, vals = [], []
         considered = 0
+        per_node = []
         for node in get_param_nodes(self.graph):
             s_i = self.node_map[node]
             if node.meta["val"].numel() < world_size:
                 continue
             considered += 1
             b, nt, ns = self._edge(s_i, 0)
+            ratios = []
             for oi in range(self.num_inp_out[(s_i, 0)]["num_output_strat"]):
                 spec: DTensorSpec = self.strats[node].strategies[oi].input_specs[0]
                 shape = list(spec.tensor_meta.shape)
@@ -793,10 +969,14 @@ class ShardingOptimizer:
                     if p.is_shard():
                         shape[p.dim] = (shape[p.dim] + n - 1) // n
                 cols.append(b + oi * ns)
-                vals.append(math.prod(shape) / old)
+                ratios.append(math.prod(shape) / old)
+            vals.extend(ratios)
+            per_node.append((s_i, ratios) if ns == 1 else None)
         cols = self.var_of_entry[np.asarray(cols, np.int64)]
         self.prob.add_row(cols, vals, -np.inf, memory_factor_high * considered, "memory_constraint_high")
         self.prob.add_row(cols, vals, memory_factor_low * considered, np.inf, "memory_constraint_low")
+        if all(x is not None for x in per_node):  # (a parameter's only column is its own strategy)
+            self._linear_rows.append((per_node, memory_factor_low * considered, memory_factor_high * considered))
 
     def add_node_constraint(self, node, placement=None, constraint_name=None):
         assert node in self.strats, (node, self.strats.keys())

@@ -109,7 +109,7 @@ def build_workload(name, args):
     return opt.encoded.tables, opt.params, desc, opt.backend.dev, planner, dict(planner.timings)
 
 
-def solve_plan(planner, workload):
+def solve_plan(planner, workload, compare_full=True):
     """The ILP leg of the plan (input / output constraints of the reference's Llama example:
     examples/example_llama3.py:205-218)."""
     from torch.distributed.tensor.placement_types import Replicate, Shard
@@ -126,12 +126,23 @@ def solve_plan(planner, workload):
     planner.add_input_constraints([x_sharding])
     planner.add_output_constraints([out_sharding])
     constraints_s = time.perf_counter() - t0
-    planner.optimize_placement()
     opt = planner.sharding_optimizer
+    upper = opt.prob.upper.copy()
+    planner.optimize_placement()
     out = {"constraints_s": constraints_s, "solve_s": planner.timings["solve_s"],
            "objective": opt.objective_value(), "ilp_rows": getattr(opt.prob, "rows_after_dedupe", None),
            "ilp_variables": opt.n_variables}
-    out.update(getattr(opt, "solve_stats", {}))
+    out.update({k: v for k, v in getattr(opt, "solve_stats", {}).items()})
+    if compare_full and "columns_after_pruning" in out:
+        # the same program without the pruning in front of the solver, for scale
+        x = opt.prob.x.copy()
+        opt.prob.upper = upper
+        t0 = time.perf_counter()
+        opt.prob.solve(time_limit=opt.solver_time_limit, mip_rel_gap=opt.solver_rel_gap)
+        out["solve_s_without_pruning"] = time.perf_counter() - t0
+        out["objective_without_pruning"] = float(opt.prob.objective @ opt.prob.x)
+        out["objective_of_pruned_plan_in_full_program"] = float(opt.prob.objective @ x)
+        opt.prob.x = x
     return out
 
 

@@ -305,6 +305,28 @@ int apc_cost_objective(int64_t n_vars, int64_t n_groups, const int64_t *group_va
                        const int64_t *group_member_begin, const int64_t *member_entry_begin, const double *cost,
                        double inf_replacement, double *objective, uint8_t *forced_zero, void *stream);
 
+/* Min-sum diffusion sweeps over the planning program written as a pairwise labelling problem
+ * (no counterpart in the reference, which hands the whole program to the solver,
+ * optimize_sharding.py:648-659): the row / column minima of the (reparametrised) cost matrices
+ * are moved into the classes and handed back in equal shares, which raises the lower bound
+ * sum_classes min unary + sum_edges min matrix  without changing the cost of any labelling.
+ * The planner rounds an incumbent from the result and fixes to zero every variable whose bound
+ * exceeds it (ILP pruning and warm start).
+ *   class c        labels [label_begin[c], label_begin[c + 1]) of unary (f64, +inf = not allowed)
+ *   edge k         matrix theta[edge_begin[k] ..], rows = labels of class edge_i[k], columns =
+ *                  labels of class edge_j[k], row-major, +inf = forbidden pair
+ *   incidence      edges of class c: inc_edge / inc_side [inc_begin[c], inc_begin[c + 1]),
+ *                  side 0 = c labels the rows, 1 = the columns
+ *   colours        color_nodes holds the classes grouped by colour, color_begin_host (HOST array,
+ *                  n_colors + 1) the groups; two classes of one colour share no edge.
+ * One sweep = one launch per colour, in order; theta and unary are updated in place.
+ * max_labels = the largest label count of a class (at most 2048). */
+int apc_diffusion_sweeps(int32_t n_sweeps, int32_t n_colors, const int64_t *color_begin_host,
+                         const int32_t *color_nodes, int64_t n_classes, const int64_t *label_begin,
+                         const int64_t *inc_begin, const int32_t *inc_edge, const uint8_t *inc_side,
+                         const int64_t *edge_begin, const int32_t *edge_i, const int32_t *edge_j, int32_t max_labels,
+                         double *theta, double *unary, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -490,6 +490,53 @@ def cost_objective(cost, var_of_entry, n_vars: int, inf_replacement: float = 100
     return [float(x) for x in obj], forced
 
 
+def diffusion_sweeps(n_sweeps, label_begin, inc_begin, inc_edge, inc_side, edge_begin, edge_i, edge_j, color_begin,
+                     color_nodes, theta, unary):
+    """Min-sum diffusion over a pairwise labelling problem, in place on ``theta`` / ``unary``
+    (numpy fp64 arrays).  No reference counterpart (the reference does no pruning,
+    ref: autoparallel/optimize_sharding.py:648-659); defined by this build and pinned by its
+    invariants: every update leaves the cost of every labelling unchanged (brute force on tiny
+    problems), the bound never decreases and never exceeds the brute-force optimum.
+    One sweep updates the classes colour by colour, in ``color_nodes`` order.  A node update:
+      tot = unary of the class; for every incident edge, in incidence order: d = row minima
+      (the class labels the rows) or column minima of the edge matrix; rows / columns with a
+      finite minimum have it subtracted; tot += d.  Then share = tot / degree; labels with a
+      finite share get unary 0 and share added back to their row / column of every incident
+      matrix; the others (no finite pair left on some edge) get unary +inf and +inf rows."""
+    import numpy as np
+
+    def mat(k):
+        ni = int(label_begin[edge_i[k] + 1] - label_begin[edge_i[k]])
+        nj = int(label_begin[edge_j[k] + 1] - label_begin[edge_j[k]])
+        return theta[int(edge_begin[k]):int(edge_begin[k + 1])].reshape(ni, nj)
+
+    for _ in range(int(n_sweeps)):
+        for c in color_nodes:
+            c = int(c)
+            lo, hi = int(inc_begin[c]), int(inc_begin[c + 1])
+            if hi == lo:
+                continue
+            u = unary[int(label_begin[c]):int(label_begin[c + 1])]
+            tot = u.copy()
+            for t in range(lo, hi):
+                m = mat(int(inc_edge[t]))
+                if inc_side[t] == 1:
+                    m = m.T
+                d = m.min(axis=1)
+                fin = np.isfinite(d)
+                m[fin, :] -= d[fin, None]
+                tot = tot + d
+            share = tot / float(hi - lo)
+            fin = np.isfinite(tot)
+            for t in range(lo, hi):
+                m = mat(int(inc_edge[t]))
+                if inc_side[t] == 1:
+                    m = m.T
+                m[fin, :] += share[fin, None]
+                m[~fin, :] = np.inf
+            u[:] = np.where(fin, 0.0, np.inf)
+
+
 def strategy_bounds(enc: dict, row_min):
     """Optimistic cost of every (node, strategy): the sum, over the node's edges in edge
     order, of that consumer strategy's row minimum (``row_min`` ordered by edge, then consumer

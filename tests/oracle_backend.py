@@ -51,6 +51,13 @@ class OracleBackend:
         return {"objective": obj, "forced_zero": forced, "compute": self.out["compute"],
                 "compute_per_arg": self.out["compute_per_arg"]}
 
+    def diffusion_sweeps(self, graph, theta, unary, n_sweeps):
+        theta, unary = theta.copy(), unary.copy()
+        po.diffusion_sweeps(n_sweeps, graph.label_begin, graph.inc_begin, graph.inc_edge, graph.inc_side,
+                            graph.edge_begin, graph.edge_i, graph.edge_j, graph.color_begin, graph.color_nodes,
+                            theta, unary)
+        return theta, unary
+
     def host_array(self, name):
         return self.out[name]
 

@@ -245,6 +245,44 @@ def test_device_tables_give_identical_tables_plan_and_objective(gpu_device, mesh
     assert dlb <= d.objective_value() * (1 + 1e-12)
 
 
+@pytest.mark.parametrize("kind,mesh_key,high_mem", [("ffn", "2d", None), ("block", "2d", None), ("block", "1d", None),
+                                                    ("block", "1d", 1.0)])
+def test_pruning_before_the_solve_changes_neither_plan_nor_objective(meshes, kind, mesh_key, high_mem):
+    """The dual ascent + incumbent + bound-based fixing in front of the solver (pruning.py): on the
+    reference's test models the solver receives a fraction of the columns and returns the
+    objective of the full program with a plan that is optimal in the full program
+    (where several plans tie, e.g. a backward permute that may stay Partial or not at equal cost,
+    the two solves may return different ones); the reference's expected placements hold for both."""
+
+    class FullOptimizer(OracleOptimizer):
+        prune_before_solve = False
+
+    class FullPlanner(AutoParallelPlanner):
+        optimizer_cls = FullOptimizer
+
+    a, plan_a = _plan(OraclePlanner, meshes[mesh_key], kind, high_mem)
+    b, plan_b = _plan(FullPlanner, meshes[mesh_key], kind, high_mem)
+    oa, ob = a.sharding_optimizer, b.sharding_optimizer
+    sa, sb = oa.solve_stats, ob.solve_stats
+    assert "columns_after_pruning" in sa and "columns_after_pruning" not in sb
+    assert sa["incumbent"] is not None and sa["lower_bound"] <= sa["incumbent"] * (1 + 1e-9)
+    assert sa["columns_after_pruning"] < 0.5 * sa["columns"] and sb["columns_solved"] == sb["columns"]
+    # (tied plans sum different entries: equal to the last bits, not always bit for bit)
+    assert math.isclose(oa.objective_value(), ob.objective_value(), rel_tol=1e-13)
+    # the pruned program's plan is a feasible plan of the full program with the full optimum as its cost
+    assert not ob.prob.violated_constraints(oa.prob.x)
+    assert math.isclose(float(ob.prob.objective @ oa.prob.x), ob.prob.objective_value, rel_tol=1e-12)
+    # so is the incumbent the pruning worked with (feasible; no better than the optimum)
+    assert not ob.prob.violated_constraints(oa.incumbent)
+    assert float(ob.prob.objective @ oa.incumbent) >= ob.prob.objective_value * (1 - 1e-12)
+    # no variable of the full program's optimum was fixed to zero unless another optimum was kept
+    for autop, plan in ((a, plan_a), (b, plan_b)):
+        if mesh_key == "2d":
+            _check_2d(autop, plan, kind)
+        else:
+            _check_1d(autop, plan, kind, high_mem)
+
+
 @pytest.mark.parametrize("kind,mesh_key", [("ffn", "2d"), ("block", "1d")])
 def test_node_choice_variables_do_not_change_the_optimum(meshes, kind, mesh_key):
     """Declaring only the per-(node, strategy) variables integral is a reformulation: the

@@ -5,6 +5,7 @@ CPU: strategy enumeration / encoding / clustering invariants with oracle-built t
 GPU: device-built tables bit-identical to oracle-built ones on every configuration."""
 
 import dataclasses
+import math
 
 import numpy as np
 import pytest
@@ -184,9 +185,19 @@ def test_full_depth_llama3_8b_on_mesh_32x8(gpu_device, fake_pg):
     """The headline configuration at full size: Llama-3-8B, 32 layers, batch 32 x 8192 tokens,
     mesh (32, 8), linked layers (examples/example_llama3.py:56-68, 205-218).  Every one of the
     1.8 M comm / transition / cost entries, the compute costs, the row minima and the objective
-    vector against the C oracle, then the same plan and objective from device and oracle tables."""
+    vector against the C oracle, then the same plan and objective from device and oracle tables.
+    Both legs prune the program before the solve (the dual ascent of pruning.py, on the device and
+    by its CPU restatement): same bound, same incumbent, same pruned program, same plan; a third
+    leg solves the full program: its optimum is the pruned programs' optimum."""
+
+    class FullOptimizer(OracleOptimizer):
+        prune_before_solve = False
+
+    class FullOraclePlanner(AutoParallelPlanner):
+        optimizer_cls = FullOptimizer
+
     results = {}
-    for name, planner_cls in (("device", AutoParallelPlanner), ("oracle", OraclePlanner)):
+    for name, planner_cls in (("device", AutoParallelPlanner), ("oracle", OraclePlanner), ("full", FullOraclePlanner)):
         with _planner(planner_cls, LLAMA3_8B, (32, 8), 32, 8192, repeated_subgraphs=True) as autop:
             o = autop.sharding_optimizer
             tb = o.encoded.tables
@@ -195,6 +206,14 @@ def test_full_depth_llama3_8b_on_mesh_32x8(gpu_device, fake_pg):
                 assert o.backend.launches == ("build_tables",), "the planner's table build is one launch"
                 assert o.backend.dev.comm is None and o.backend.dev.transition is None
             plan = _solve_llama(autop)
+            stats = o.solve_stats
+            if name == "full":
+                assert stats["columns_solved"] == stats["columns"], stats
+                results[name] = {"objective": o.objective_value()}
+                continue
+            assert stats["incumbent"] is not None and stats["columns_after_pruning"] < 0.1 * stats["columns"], stats
+            assert stats["lower_bound"] <= stats["incumbent"] * (1 + 1e-9)
+            results[name + "_stats"] = dict(stats)
             out = {"objective_vector": o.objective_vector.copy(), "forced": o.forced_zero_vars.copy(),
                    "plan": {n.name: str(s) for n, s in plan.items()}, "objective": o.objective_value(),
                    "res": list(o.res), "n_entries": tb.n_entries, "n_variables": o.n_variables,
@@ -209,6 +228,10 @@ def test_full_depth_llama3_8b_on_mesh_32x8(gpu_device, fake_pg):
         assert np.array_equal(d[key], o[key]), key
     assert d["res"] == o["res"] and d["plan"] == o["plan"]
     assert d["objective"] == o["objective"] > 0
+    assert math.isclose(d["objective"], results["full"]["objective"], rel_tol=1e-13)  # (tied plans may differ in the last bit)
+    # the dual ascent itself: device and CPU restatement reach the same bound, incumbent and pruning
+    for key in ("lower_bound", "incumbent", "prune_sweeps", "columns_after_pruning"):
+        assert results["device_stats"][key] == results["oracle_stats"][key], key
 
 
 def test_split_tensor_rule(fake_pg):
