@@ -143,12 +143,13 @@ def dynamo_capture(model: nn.Module, inputs: tuple) -> torch.fx.GraphModule:
 
 @contextlib.contextmanager
 def capture_joint_graph(model: nn.Module, input_fn, param_dtype: torch.dtype | None = None, device="cpu",
-                        add_aliases: bool = True, dynamo: bool = False):
+                        add_aliases: bool = True, dynamo: bool = False, prepare: bool = True):
     """Context manager yielding ``(gm, joint_with_descriptors)`` for ``model`` (built on
     the meta device) and ``input_fn`` (called under the fake mode; returns a tensor or a
     tuple of tensors).  The fake mode stays usable inside the ``with`` block.  ``dynamo``
     captures the forward with Dynamo first (needed for models with ``local_map`` regions,
-    which plain AOT tracing would inline)."""
+    which plain AOT tracing would inline).  ``prepare=False`` yields the exported graph as it
+    is, before dead-code / no-op removal and alias insertion."""
     from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
 
     fake_mode = FakeTensorMode()
@@ -172,7 +173,8 @@ def capture_joint_graph(model: nn.Module, input_fn, param_dtype: torch.dtype | N
             if node.op == "call_function" and getattr(node.target, "namespace", "") == "_c10d_functional":
                 raise RuntimeError(f"the model already contains a collective ({node.target}); "
                                    "planning needs a single-device graph")
-        cleanup_graph(gm)
-        if add_aliases:
-            add_alias_nodes(gm)
+        if prepare:
+            cleanup_graph(gm)
+            if add_aliases:
+                add_alias_nodes(gm)
         yield gm, joint

@@ -79,19 +79,23 @@ class BinaryProgram:
 
         if not self._names:
             return csr_matrix((0, self.n_vars))
+        cached = getattr(self, "_matrix_cache", None)
+        if cached is not None and cached[0] == len(self._names):  # rows are only ever appended
+            return cached[1]
         indptr = np.zeros(len(self._row_len) + 1, np.int64)
         np.cumsum(self._row_len, out=indptr[1:])
         cols = np.concatenate(self._cols) if self._cols else np.zeros(0, np.int64)
         vals = np.concatenate(self._vals) if self._vals else np.zeros(0, np.float64)
         m = csr_matrix((vals, cols, indptr), shape=(len(self._row_len), self.n_vars))
         m.sum_duplicates()
+        self._matrix_cache = (len(self._names), m)
         return m
 
     def deduplicated(self):
         """(matrix, lb, ub) with repeated rows removed.  Variable sharing makes many
         constraints of linked nodes literally identical; rows are compared through two
         independent 64-bit hashes of their (column, coefficient) pairs."""
-        a = self.matrix()
+        a = self.matrix().copy()
         lb, ub = np.asarray(self._lb), np.asarray(self._ub)
         if a.shape[0] == 0:
             return a, lb, ub

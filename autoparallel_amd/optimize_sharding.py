@@ -286,6 +286,11 @@ class ShardingOptimizer:
     # declared integral: with a node's and its producers' choices fixed to unit vectors the
     # row / column sum constraints leave exactly one feasible (integral) value for every entry
     # variable.  Same feasible plans and optimum, far fewer branching variables for the solver.
+    # how repeated subgraphs are found when the constructor is asked for them: "neighbourhood" (this
+    # package's refinement of node keys by their surroundings) or "regions" (the reference's region
+    # growing, graph_clustering.py:101-206, which under torch 2.10 fails its own sanity check on
+    # Llama-shaped graphs)
+    clustering = "neighbourhood"
     node_choice_variables = True
     compact_constraints = True  # with choice variables: the structural constraints written through them
     # Before the solver runs: a dual ascent over the program's labelling form (row / column minima
@@ -329,10 +334,11 @@ class ShardingOptimizer:
 
         self.node_representative = {}
         if repeated_subgraphs:
-            from .graphs.clustering import cluster_nodes
+            from .graphs import clustering
 
             t0 = time.perf_counter()
-            self.node_representative = cluster_nodes(self.graph, self.strats)
+            find = {"neighbourhood": clustering.cluster_nodes, "regions": clustering.cluster_regions}[self.clustering]
+            self.node_representative = find(self.graph, self.strats)
             self.timings["cluster_s"] = time.perf_counter() - t0
             logger.info("%s %.3f s", "cluster_s", self.timings["cluster_s"])
         self.ds, self.num_inp_out, self.num_args = self.build_ds()
@@ -665,6 +671,9 @@ class ShardingOptimizer:
         seen = set()
         one_cols, one_lens = [], []
         cols, vals, lens = [], [], []
+        # which class of nodes labels the rows / the columns of which block of entry variables
+        # (read again by the pruning in front of the solver)
+        self._block_sides = sides = {}
         for s_i, node in enumerate(self.nodes):
             if node.op == "output":
                 continue
@@ -680,6 +689,7 @@ class ShardingOptimizer:
                 if ("row", b, cb) in seen:
                     continue
                 seen.add(("row", b, cb))
+                sides.setdefault(b, [nt, ns, [], []])[2].append(cb)
                 entries = b + np.arange(nt)[:, None] * ns + np.arange(ns)[None, :]
                 cols.append(np.concatenate([entries, (cb + np.arange(nt))[:, None]], axis=1).ravel())
                 vals.append(np.tile(np.concatenate([np.ones(ns), [-1.0]]), nt))
@@ -695,6 +705,7 @@ class ShardingOptimizer:
                 if ("col", bc, cb) in seen:
                     continue
                 seen.add(("col", bc, cb))
+                sides.setdefault(bc, [ntc, nsc, [], []])[3].append(cb)
                 entries = bc + np.arange(ntc)[None, :] * nsc + np.arange(nsc)[:, None]  # column o of the consumer
                 cols.append(np.concatenate([entries, (cb + np.arange(nsc))[:, None]], axis=1).ravel())
                 vals.append(np.tile(np.concatenate([np.ones(ntc), [-1.0]]), nsc))
@@ -767,37 +778,42 @@ class ShardingOptimizer:
                 x = parent[x]
             return x
 
-        raw = {}  # var base -> [nt, ns, row choice bases, column choice bases]
-        for s_i, node in enumerate(self.nodes):
-            if node.op == "output":
-                continue
-            cb = self.node_choice_base[s_i]
-            find(cb)
-            for argi in range(self.num_args[s_i]):
-                b, nt, ns = self._edge_vars(s_i, argi)
-                raw.setdefault(b, [nt, ns, [], []])[2].append(cb)
-            for user in node.users:
-                if user.op == "output":
+        raw = getattr(self, "_block_sides", None)  # var base -> [nt, ns, row choice bases, column choice bases]
+        if raw is None:
+            raw = {}
+            for s_i, node in enumerate(self.nodes):
+                if node.op == "output":
                     continue
-                s_j = self.node_map[user]
-                argj = [i for i, x in enumerate(user.all_input_nodes) if x == node]
-                bc, ntc, nsc = self._edge_vars(s_j, argj[0])
-                raw.setdefault(bc, [ntc, nsc, [], []])[3].append(cb)
+                cb = self.node_choice_base[s_i]
+                for argi in range(self.num_args[s_i]):
+                    b, nt, ns = self._edge_vars(s_i, argi)
+                    raw.setdefault(b, [nt, ns, [], []])[2].append(cb)
+                for user in node.users:
+                    if user.op == "output":
+                        continue
+                    s_j = self.node_map[user]
+                    argj = [i for i, x in enumerate(user.all_input_nodes) if x == node]
+                    bc, ntc, nsc = self._edge_vars(s_j, argj[0])
+                    raw.setdefault(bc, [ntc, nsc, [], []])[3].append(cb)
         for nt, ns, rows, cols in raw.values():
             for side in (rows, cols):
                 for cb in side[1:]:
                     parent[find(cb)] = find(side[0])
         class_id, class_sizes, members = {}, [], []
-        for s_i, node in enumerate(self.nodes):
-            if node.op == "output":
-                continue
-            root = find(self.node_choice_base[s_i])
+        size_of = {}  # choice base -> number of strategies
+        for nt, ns, rows, cols in raw.values():
+            for cb in rows:
+                size_of[cb] = nt
+            for cb in cols:
+                size_of[cb] = ns
+        for cb in sorted(size_of):
+            root = find(cb)
             if root not in class_id:
                 class_id[root] = len(class_sizes)
-                class_sizes.append(len(self.strats[node].strategies))
+                class_sizes.append(size_of[cb])
                 members.append(set())
-            members[class_id[root]].add(self.node_choice_base[s_i])
-            assert class_sizes[class_id[root]] == len(self.strats[node].strategies)
+            members[class_id[root]].add(cb)
+            assert class_sizes[class_id[root]] == size_of[cb], "nodes tied through a block have the same strategies"
         cls = lambda cb: class_id[find(cb)]  # noqa: E731
         blocks = [pruning.Block(b, nt, ns, cls(rows[0]), cls(cols[0]) if cols else -1)
                   for b, (nt, ns, rows, cols) in raw.items()]
@@ -860,13 +876,18 @@ class ShardingOptimizer:
         t0 = time.perf_counter()
         stats = self.solve_stats
         graph = self._label_graph()
+        stats["prune_graph_s"] = time.perf_counter() - t0
+        t_sweeps = t_round = 0.0
         if graph.n_classes == 0 or int(np.diff(graph.label_begin).max()) > pruning.MAX_LABELS:
             stats["pruning"] = "skipped"
             return
         theta, unary = graph.theta.copy(), graph.unary.copy()
         best_ub, best_x, sweeps, bound = math.inf, None, 0, -math.inf
         for chunk in self.prune_sweep_chunks:
+            t1 = time.perf_counter()
             theta, unary = self.backend.diffusion_sweeps(graph, theta, unary, chunk)
+            t_sweeps += time.perf_counter() - t1
+            t1 = time.perf_counter()
             sweeps += chunk
             bound = pruning.lower_bound(graph, theta, unary)[0]
             labels = pruning.decode(graph, theta, unary)
@@ -875,8 +896,10 @@ class ShardingOptimizer:
                 ub = float(self.prob.objective @ x)
                 if ub < best_ub:
                     best_ub, best_x = ub, x
+            t_round += time.perf_counter() - t1
             if best_ub - bound <= self.prune_gap * abs(best_ub):
                 break
+        stats.update(prune_sweeps_s=t_sweeps, prune_rounding_s=t_round)
         stats.update(prune_sweeps=sweeps, lower_bound=bound, incumbent=best_ub if best_x is not None else None,
                      label_classes=graph.n_classes, label_edges=graph.n_edges)
         if best_x is not None:

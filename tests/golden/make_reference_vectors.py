@@ -53,7 +53,13 @@ CASES = [
     ("block_1k_64", "block_1k", (64,)),  # the single transformer block of the CPU-runnable configuration
     ("local_map_block_8x8x4", "local_map_block", (8, 8, 4)),  # attention inside a local_map region
     ("dsv3_moe_tiny_64x4", "dsv3_moe_tiny", (64, 4)),  # one dense and one mixture-of-experts layer, widths divided down
+    ("llama_tiny_3layers_32x8", "llama_tiny", (32, 8)),  # three identical decoder layers: repeated subgraphs to link
 ]
+
+# a Llama-shaped decoder small enough to keep three layers in the fixture
+TINY_LLAMA = dict(dim=512, n_layers=3, n_heads=8, n_kv_heads=4, vocab_size=2048, ffn_dim_multiplier=1.0, multiple_of=256,
+                  max_seq_len=256)
+TINY_LLAMA_BATCH, TINY_LLAMA_SEQ = 64, 256
 
 # the DeepSeek-V3 style configuration with every width divided down: same operators, same graph shape
 TINY_MOE = dict(dim=256, n_layers=2, n_dense_layers=1, n_heads=8, q_lora_rank=64, kv_lora_rank=32, qk_nope_head_dim=16,
@@ -103,9 +109,21 @@ def node_signature(node) -> str:
     return f"{target} " + " ".join(one(x) for x in flat)
 
 
-def make_graph(kind, mesh):
-    from autoparallel_amd.graphs.capture import capture_joint_graph
+def make_graph(kind, mesh, prepare=True):
+    """``prepare=False``: the joint export before dead-code / no-op removal and alias insertion."""
+    import functools
 
+    from autoparallel_amd.graphs import capture
+
+    capture_joint_graph = functools.partial(capture.capture_joint_graph, prepare=prepare)
+    if kind == "llama_tiny":
+        from autoparallel_amd.graphs.llama3 import Llama, LlamaConfig
+
+        cfg = LlamaConfig(**TINY_LLAMA)
+        with torch.device("meta"):
+            model = Llama(cfg)
+        return capture_joint_graph(model, lambda: torch.randint(0, cfg.vocab_size, (TINY_LLAMA_BATCH, TINY_LLAMA_SEQ)),
+                                   param_dtype=torch.bfloat16, device="cpu", dynamo=False)
     if kind.startswith("llama3") or kind == "block_1k":
         # one decoder layer of the benchmark model at its full shapes, bf16 parameter casts
         # (block_1k: batch 64 instead of 8, so that it divides the 64 ranks)
@@ -159,7 +177,52 @@ def reference_tables(gm, mesh):
         costs = [float(estimate_strategy_runtime_cost(node, s)) for s in strategies]
         records.append((node.name, node_signature(node), [strategy_code(s) for s in strategies],
                         [c.hex() for c in costs]))  # float.hex keeps every bit
-    return records
+    return records, strats
+
+
+def reference_cluster_links(gm, strats):
+    """node name -> name of the node whose ILP variables it shares: the reference's
+    ``get_identical_regions`` (autoparallel/graph_clustering.py:101-206) with the pairing of
+    ``ShardingOptimizer.create_cluster_links`` (optimize_sharding.py:211-231: the regions of a
+    group are zipped against its first region)."""
+    from autoparallel.graph_clustering import get_identical_regions
+
+    strats = dict(strats)
+    for node in gm.graph.nodes:  # the reference's build_sharding_metadata gives the output node its producers' strategies
+        if node.op == "output":
+            strats[node] = [strats[x] for x in node.all_input_nodes]
+    links = {}
+    for group in get_identical_regions(gm.graph, strats):
+        first = group[0]
+        for region in group[1:]:
+            assert len(region) == len(first)
+            for n0, ni in zip(first, region):
+                links[ni.name] = n0.name
+    return links
+
+
+def graph_listing(gm):
+    """[name, op, target, [argument node names]] per node: what graph preparation decides."""
+    def target(n):
+        return str(n.target) if n.op == "call_function" else n.op
+
+    return [[n.name, n.op, target(n), [a.name for a in n.all_input_nodes]] for n in gm.graph.nodes]
+
+
+def reference_prepared_graph(kind, mesh):
+    """The joint export of this repository's capture put through the reference's own graph
+    preparation: ``cleanup_graph`` and ``_add_alias(gm, "v2")`` (autoparallel/graph_utils.py:17-39,
+    76-150), as ``AutoParallel.build_model_graph`` applies them (api.py:367-373)."""
+    from autoparallel.graph_utils import _add_alias, cleanup_graph
+
+    ctx = make_graph(kind, mesh, prepare=False)
+    gm, _ = ctx.__enter__()
+    try:
+        cleanup_graph(gm)
+        _add_alias(gm, version="v2")
+        return graph_listing(gm)
+    finally:
+        ctx.__exit__(None, None, None)
 
 
 def pack(records):
@@ -176,6 +239,17 @@ def pack(records):
                       [intern(values, c) for c in costs]])
     return {"signatures": list(signatures), "strategy_lists": [list(x) for x in lists],
             "cost_values_us": list(values), "nodes": nodes}
+
+
+def pack_listing(listing):
+    """Targets repeat: stored once and named by index.  node = [name, op, target index, [argument names]]."""
+    targets = {}
+    nodes = [[name, op, targets.setdefault(target, len(targets)), args] for name, op, target, args in listing]
+    return {"targets": list(targets), "nodes": nodes}
+
+
+def unpack_listing(packed):
+    return [[name, op, packed["targets"][t], args] for name, op, t, args in packed["nodes"]]
 
 
 def main():
@@ -207,13 +281,21 @@ def main():
             with patch("torch.cuda.device_count", lambda: 8), \
                     patch("torch.cuda.get_device_name", lambda device=None: "H100"), \
                     patch.object(type(_mesh_resources), "num_devices_per_host", lambda self, device_type: 8):
-                records = reference_tables(gm, mesh)
+                records, strats = reference_tables(gm, mesh)
+                try:
+                    links, links_error = reference_cluster_links(gm, strats), None
+                except RuntimeError as e:  # the reference's own sanity check (graph_clustering.py:197-205)
+                    links, links_error = {}, f"{type(e).__name__}: {e}"
         finally:
             ctx.__exit__(None, None, None)
-        out["cases"][name] = {"kind": kind, "mesh": list(mesh_sizes), **pack(records)}
+        prepared = reference_prepared_graph(kind, mesh)
+        out["cases"][name] = {"kind": kind, "mesh": list(mesh_sizes), **pack(records), "cluster_links": links,
+                              "cluster_links_error": links_error, "prepared_graph": pack_listing(prepared)}
         print(name, len(records), "nodes,", sum(len(r[2]) for r in records), "strategies,",
               len(out["cases"][name]["strategy_lists"]), "distinct lists,",
-              len(out["cases"][name]["cost_values_us"]), "distinct costs", flush=True)
+              len(out["cases"][name]["cost_values_us"]), "distinct costs,",
+              f"{len(links)} linked nodes," if links_error is None else f"clustering raised {links_error},",
+              len(prepared), "nodes after the reference's preparation", flush=True)
     path = os.path.join(HERE, "reference_strategies_and_costs.json")
     with open(path, "w") as f:
         json.dump(out, f, separators=(",", ":"))

@@ -32,7 +32,8 @@ from models import make_model_and_inputs
 from oracle_backend import OracleBackend
 
 sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
-from make_reference_vectors import node_signature, strategy_code  # noqa: E402  (pure helpers; imports no reference code)
+from make_reference_vectors import (graph_listing, node_signature, strategy_code,  # noqa: E402  (pure helpers;
+                                    unpack_listing)  # they import no reference code)
 
 with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_strategies_and_costs.json")) as f:
     FIXTURE = json.load(f)
@@ -56,6 +57,15 @@ class OraclePlanner(AutoParallelPlanner):
 def _planner(planner_cls, case):
     kind, mesh_sizes = case["kind"], tuple(case["mesh"])
     mesh = workloads.logical_mesh(mesh_sizes)
+    if kind == "llama_tiny":
+        from autoparallel_amd.graphs.llama3 import Llama, LlamaConfig
+        from make_reference_vectors import TINY_LLAMA, TINY_LLAMA_BATCH, TINY_LLAMA_SEQ
+
+        cfg = LlamaConfig(**TINY_LLAMA)
+        with torch.device("meta"):
+            model = Llama(cfg)
+        return planner_cls(model, lambda: torch.randint(0, cfg.vocab_size, (TINY_LLAMA_BATCH, TINY_LLAMA_SEQ)), mesh,
+                           param_dtype=torch.bfloat16)
     if kind.startswith("llama3") or kind == "block_1k":
         model, input_fn, _, _ = workloads.build_model(kind, mesh, n_layers=1, batch=64 if kind == "block_1k" else None)
         # no reduce dtype: the gradient rescale does not touch compute costs
@@ -114,3 +124,37 @@ def test_strategy_lists_and_oracle_compute_costs_equal_the_reference_vectors(fak
 @pytest.mark.parametrize("name", list(FIXTURE["cases"]))
 def test_strategy_lists_and_device_compute_costs_equal_the_reference_vectors(gpu_device, fake_pg, name):
     assert _check(AutoParallelPlanner, name) == "DeviceBackend"
+
+
+def _without_addresses(listing):
+    return [[name, op, re.sub(r" at 0x[0-9a-f]+", "", target), args] for name, op, target, args in listing]
+
+
+@pytest.mark.parametrize("name", list(FIXTURE["cases"]))
+def test_graph_preparation_and_region_clustering_equal_the_reference(fake_pg, name):
+    """What the reference's own functions made of the same joint export, held by the fixture:
+      * graph preparation: ``cleanup_graph`` and ``_add_alias(gm, "v2")`` (autoparallel/graph_utils.py:17-39,
+        76-150) applied to the export: node names, operators and argument lists, in order, equal to
+        what ``graphs/capture.py`` produces (this decides which nodes and edges the tables are built over);
+      * repeated subgraphs: the links of ``get_identical_regions`` + ``create_cluster_links``
+        (graph_clustering.py:101-206, optimize_sharding.py:211-231) equal to ``cluster_regions``'s, node
+        for node; where the reference's function ended in its own "Duplicate node" check (every Llama-shaped
+        graph, under the installed torch), ``cluster_regions`` raises the same error."""
+    from autoparallel_amd.graphs.clustering import cluster_nodes, cluster_regions
+
+    case = FIXTURE["cases"][name]
+    with _planner(OraclePlanner, case) as p:
+        o = p.sharding_optimizer
+        assert _without_addresses(graph_listing(p.gm)) == _without_addresses(unpack_listing(case["prepared_graph"]))
+        if case["cluster_links_error"] is None:
+            links = {n.name: r.name for n, r in cluster_regions(o.graph, o.strats).items()}
+            assert links == case["cluster_links"]
+        else:
+            with pytest.raises(RuntimeError, match="Duplicate node"):
+                cluster_regions(o.graph, o.strats)
+        # the planner's default algorithm links nodes on every graph; a linked node has its
+        # representative's operator, strategies (as text) and argument count
+        rep = cluster_nodes(o.graph, o.strats)
+        for node, r in rep.items():
+            assert node.target == r.target and str(o.strats[node]) == str(o.strats[r])
+            assert o.num_args[o.node_map[node]] == o.num_args[o.node_map[r]]

@@ -100,9 +100,11 @@ def test_tiny_llama_tables_and_clustering(fake_pg):
         autop.add_input_constraints([(Shard(0), Replicate())])
         autop.add_output_constraints([(Shard(0), Shard(2))])
         plan = autop.optimize_placement()
-        # sharing variables restricts the search: never better than the free optimum, and close to it
+        # sharing variables restricts the search (every layer takes the strategies of the first, although
+        # the first and the last layer border different neighbours): never better than the free optimum,
+        # and here 0.3 % above it
         assert opt.objective_value() >= free_objective - 1e-6
-        assert opt.objective_value() <= free_objective * 1.10
+        assert opt.objective_value() <= free_objective * 1.01
         # linked nodes chose the same strategy as their representative
         for node, rep in opt.node_representative.items():
             assert str(plan[node]) == str(plan[rep])
