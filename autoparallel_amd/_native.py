@@ -80,6 +80,7 @@ EXPORTS = (
     "apc_cost_objective",
     "apc_validate_row_minima_host",
     "apc_diffusion_sweeps",
+    "apc_redistribute_tables_static",
 )
 
 _lib = None

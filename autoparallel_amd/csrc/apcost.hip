@@ -2012,3 +2012,73 @@ int apc_diffusion_sweeps(int32_t n_sweeps, int32_t n_colors, const int64_t *colo
 }
 
 }  // extern "C"
+
+// ------------------------------------------------------------------------------------------
+// An entry point that allocates nothing and needs no caller-provided staging: the cost
+// matrices straight from the tensor and strategy tables.  The staging tables the tile kernel
+// reads (bytes and contiguity per tensor, compute cost / num_args per strategy; what
+// apc_input_tables writes into caller arrays for apc_redistribute_tables) live in a file-scope
+// device array of fixed size.  Every device holds its own copy of the array at its own address,
+// looked up once per device; calls on one device share it, so calls that overlap on a device race.
+// ------------------------------------------------------------------------------------------
+constexpr int64_t kStaticMaxTensors = 1 << 16;     // 8 B + 1 B each
+constexpr int64_t kStaticMaxStrategies = 1 << 21;  // 8 B each (compute cost / num_args)
+constexpr size_t kStaticBytesOff = 0;
+constexpr size_t kStaticPerArgOff = kStaticBytesOff + (size_t)kStaticMaxTensors * sizeof(int64_t);
+constexpr size_t kStaticContigOff = kStaticPerArgOff + (size_t)kStaticMaxStrategies * sizeof(double);
+constexpr size_t kStaticScratchBytes = kStaticContigOff + (size_t)kStaticMaxTensors;  // 17.1 MB
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void *g_scratch_of_device[kMaxDevices];  // the array's device address, per device (0 = not looked up yet)
+
+// The address of this device's copy of `scratch` (the array's name is only a host-side handle).
+static int scratch_of_current_device(unsigned char **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(-3, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(-1, "device %d outside [0, %d)", dev, kMaxDevices);
+  void *p = __atomic_load_n(&g_scratch_of_device[dev], __ATOMIC_ACQUIRE);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return fail(-3, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    __atomic_store_n(&g_scratch_of_device[dev], p, __ATOMIC_RELEASE);  // (every thread finds the same address)
+  }
+  *out = static_cast<unsigned char *>(p);
+  return 0;
+}
+
+extern "C" {
+
+int apc_redistribute_tables_static(const apc_params *params, int64_t n_tensors, const int32_t *rank, const int32_t *itemsize,
+                                   const int64_t *shape, const int64_t *stride, int64_t n_strategies, const int64_t *flops,
+                                   const int64_t *rw_bytes, const int8_t *dtype, const uint8_t *zero_cost,
+                                   const int32_t *num_args, const uint32_t *spec_codes, const int32_t *spec_tensor,
+                                   const double *pt_values, int64_t n_tiles, const apc_tile *tiles,
+                                   const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out, uint8_t *trans_out,
+                                   double *cost_out, void *stream) {
+  if (n_tensors < 0 || n_strategies < 0) return fail(-1, "apc_redistribute_tables_static: negative count");
+  if (n_tensors > kStaticMaxTensors)
+    return fail(-1, "apc_redistribute_tables_static: %lld tensors, the static staging holds %lld (use apc_input_tables + "
+                "apc_redistribute_tables with caller-allocated staging)", (long long)n_tensors, (long long)kStaticMaxTensors);
+  if (n_strategies > kStaticMaxStrategies)
+    return fail(-1, "apc_redistribute_tables_static: %lld strategies, the static staging holds %lld (use apc_input_tables + "
+                "apc_redistribute_tables with caller-allocated staging)", (long long)n_strategies,
+                (long long)kStaticMaxStrategies);
+  unsigned char *base = nullptr;
+  if (int rc = scratch_of_current_device(&base)) return rc;
+  int64_t *tensor_bytes = reinterpret_cast<int64_t *>(base + kStaticBytesOff);
+  double *per_arg = reinterpret_cast<double *>(base + kStaticPerArgOff);
+  uint8_t *tensor_contiguous = base + kStaticContigOff;
+  // staging tables into the static array (no spec table, no per-strategy compute cost, no error
+  // flag: a strategy with flops and an unsupported dtype shows as NaN costs), then the tiles;
+  // both launches on the caller's stream, so the second sees what the first wrote
+  if (int rc = apc_input_tables(params, n_tensors, rank, itemsize, shape, stride, tensor_bytes, tensor_contiguous, 0, nullptr,
+                                nullptr, nullptr, nullptr, nullptr, 2, nullptr, nullptr, n_strategies, flops, rw_bytes, dtype,
+                                zero_cost, num_args, nullptr, per_arg, nullptr, stream))
+    return rc;
+  return redistribute_tables_impl(params, tensor_bytes, tensor_contiguous, spec_codes, spec_tensor, pt_values, per_arg, n_tiles,
+                                  tiles, dup_entry_begin, n_entries, comm_out, trans_out, cost_out, nullptr, stream);
+}
+
+}  // extern "C"

@@ -327,6 +327,26 @@ int apc_diffusion_sweeps(int32_t n_sweeps, int32_t n_colors, const int64_t *colo
                          const int64_t *edge_begin, const int32_t *edge_i, const int32_t *edge_j, int32_t max_labels,
                          double *theta, double *unary, void *stream);
 
+/* apc_redistribute_tables for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  It takes the tensor and strategy tables themselves instead of the staging tables
+ * apc_input_tables would write from them (tensor_bytes, tensor_contiguous,
+ * compute_cost_per_arg): those are staged in a fixed device array inside the library (17.1 MB
+ * that every GPU the library runs on holds until the process ends), at most 65 536 tensors and
+ * 2 097 152 strategies; larger tables are rejected with an error.  Two launches on `stream`
+ * (staging, then the tiles); no hipMalloc / hipFree, no synchronisation.  Results equal those of
+ * apc_input_tables followed by apc_redistribute_tables.  All calls on one GPU share the array:
+ * calls that overlap on a GPU (two streams, two threads) race.  A strategy with flops whose
+ * dtype has no throughput on the device row yields NaN costs (there is no error flag). */
+int apc_redistribute_tables_static(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
+                                   const int32_t *tensor_itemsize, const int64_t *tensor_shape,
+                                   const int64_t *tensor_stride, int64_t n_strategies, const int64_t *flops,
+                                   const int64_t *rw_bytes, const int8_t *dtype_code, const uint8_t *zero_cost,
+                                   const int32_t *num_args, const uint32_t *spec_codes, const int32_t *spec_tensor,
+                                   const double *pt_values, int64_t n_tiles, const apc_tile *tiles,
+                                   const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out,
+                                   uint8_t *transition_out, double *cost_out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

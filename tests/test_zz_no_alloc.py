@@ -1,0 +1,63 @@
+"""The entry point that allocates nothing (apc_redistribute_tables_static: staging tables in a
+device array inside the library) against apc_input_tables + apc_redistribute_tables with
+caller-allocated staging, through the C ABI: bit-identical outputs on two calls in a row, the
+second on a smaller table (the array keeps the first call's contents)."""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from autoparallel_amd import CostModelParams, _native
+from autoparallel_amd.device_tables import DeviceCostTables
+from autoparallel_amd.synthetic import stress_dag
+
+pytestmark = pytest.mark.gpu
+
+
+def _static_call(d, outputs):
+    tb = d.tables
+    n = tb.n_entries
+    out = {"comm": torch.full((n,), -1.0, dtype=torch.float64, device=d.device) if "comm" in outputs else None,
+           "transition": torch.full((n,), 9, dtype=torch.uint8, device=d.device) if "transition" in outputs else None,
+           "cost": torch.full((n,), -1.0, dtype=torch.float64, device=d.device) if "cost" in outputs else None}
+    P = d._p
+    with torch.cuda.device(d.device):
+        rc = d.lib.apc_redistribute_tables_static(
+            ctypes.byref(d.c_params), ctypes.c_int64(tb.n_tensors), P("tensor_rank"), P("tensor_itemsize"),
+            P("tensor_shape"), P("tensor_stride"), ctypes.c_int64(tb.n_strategies), P("strat_flops"), P("strat_rw_bytes"),
+            P("strat_dtype"), P("strat_zero_cost"), P("strat_num_args"), P("spec_codes"), P("spec_tensor"), P("pt_values"),
+            ctypes.c_int64(tb.n_tiles), P("tile_records"), P("dup_entry_begin"), ctypes.c_int64(n), P(out["comm"]),
+            P(out["transition"]), P(out["cost"]), d._stream())
+    _native.check(rc, "apc_redistribute_tables_static")
+    return out
+
+
+def test_static_staging_matches_caller_allocated_staging(gpu_device):
+    mesh = (16, 8, 4)
+    p = CostModelParams.from_mesh(mesh, rescale=2.2)
+    cases = [(stress_dag(seed=11, n_nodes=3000, mesh_sizes=mesh, frac_nonspec_nodes=0.03, frac_noncontiguous=0.2),
+              ("comm", "transition", "cost")),
+             (stress_dag(seed=12, n_nodes=400, mesh_sizes=mesh, frac_nonspec_nodes=0.03, frac_noncontiguous=0.3), ("cost",))]
+    assert cases[1][0].n_strategies < cases[0][0].n_strategies and cases[1][0].n_tensors < cases[0][0].n_tensors
+    allocated_before = None
+    for tb, outputs in cases:  # two calls in a row on the same device, the second on a smaller table
+        d = DeviceCostTables(tb, p, device=gpu_device)
+        step = d.prepare_step(row_min=False, fused_inputs=True, one_launch=False, outputs=outputs, spec_table=False)
+        assert list(step) == ["input_tables", "redistribute_tables"]
+        for launch in step.values():
+            launch()
+        torch.cuda.synchronize()
+        want = {k: getattr(d, k) for k in outputs}
+        allocated_before = torch.cuda.memory_allocated(gpu_device)
+        got = _static_call(d, outputs)
+        torch.cuda.synchronize()
+        for k in outputs:
+            assert torch.equal(got[k], want[k]), k
+        assert (want["cost"] > 0).any()
+    # tables beyond the static staging are refused with a clear error, before anything is launched
+    rc = d.lib.apc_redistribute_tables_static(
+        ctypes.byref(d.c_params), ctypes.c_int64(1 << 17), *([None] * 4), ctypes.c_int64(10), *([None] * 5), None, None, None,
+        ctypes.c_int64(0), None, None, ctypes.c_int64(0), None, None, None, None)
+    assert rc != 0 and "static staging holds" in d.lib.apc_last_error().decode()
