@@ -502,29 +502,41 @@ __device__ __forceinline__ int placement_class(uint32_t code) {
   return k == 2 ? 2 + (dim_of(code) != 0 ? 1 : 0) : k;
 }
 
-constexpr int kLdsTermArrays = 6;  // zeros, all-gather, reduce-scatter, all-reduce, all-to-all, read+write
+// Term arrays staged per tile, one value per running-bytes state: [0] zeros, [1] all-gather,
+// [2] reduce-scatter, [3] all-reduce, [4] all-to-all (= reduce-scatter shaped term x a2a_scale,
+// :22-32), [5] one read+write, [6] two read+writes (2.0 x [5]: the same bits as (double)2 * rw).
+constexpr int kLdsTermArrays = 7;
+constexpr int kRw1Array = 5;
 
-// Words of the staged action rows per producer spec: one row per mesh dim, padded to a power
-// of two so that a spec's rows are one aligned LDS read.
-template <int M>
-struct ActionRows {
-  static constexpr int kWords = M == 1 ? 1 : M == 2 ? 2 : 4;
-  __device__ static __forceinline__ void load(const uint32_t *s_act, int c, uint32_t (&act)[M]) {
-    if constexpr (M == 1) {
-      act[0] = s_act[c];
-    } else if constexpr (M == 2) {
-      const uint2 v = reinterpret_cast<const uint2 *>(s_act)[c];
-      act[0] = v.x;
-      act[1] = v.y;
-    } else {
-      const uint4 v = reinterpret_cast<const uint4 *>(s_act)[c];
-      act[0] = v.x;
-      act[1] = v.y;
-      act[2] = v.z;
-      if constexpr (M == 4) act[3] = v.w;
-    }
-  }
-};
+// Lookup words.  What a mesh dim adds to an entry depends on the producer spec (its class at
+// that dim and which dims it shards), on the consumer's class at that dim and on the history of
+// the earlier dims; everything but the history is known per (producer spec, dim, consumer
+// class) when the tile is staged.  One 32-bit word per such triple holds, as byte offsets into
+// the term arrays for history 0 (the entry adds history x 8):
+//   bits  0-14  offset of the collective's term   (array of pair_action's term, state of the
+//               bytes the collective moves: after the update for an all-gather, before it else)
+//   bits 15-29  offset of the read+write term     (array 0 / 5 / 6 for 0 / 1 / 2 reshuffles,
+//               same state)
+//   bit  30     the running bytes change after this dim (history bit)
+//   bit  31     banned transition: the entry costs inf
+// Slot 4 of a (spec, dim) is the word of "same placement": 0 (the zero array, no update); slot
+// 5 is the offset of one read+write at the state BEFORE the dim, charged once to a
+// non-contiguous tensor.
+constexpr int kWordsPerDim = 6;
+// The part of a lookup word that does not depend on the state: array offsets for state 0 and the
+// two flags, by (producer class, consumer class); the state's offset (x 8, in both fields) is
+// added when a tile is staged.  NS = number of states of the mesh rank.
+__host__ __device__ constexpr uint32_t pair_word_base(int c, int t, int ns);
+constexpr uint32_t kWordOffsetMask = 0x7FFFu, kWordUpdate = 1u << 30, kWordBan = 1u << 31;
+static_assert(kLdsTermArrays * States<APC_MAX_MESH>::kCount * 8 <= 0x7FFF + 1, "term offsets fit their 15 bits");
+
+__host__ __device__ constexpr uint32_t pair_word_base(int c, int t, int ns) {
+  const uint32_t e = pair_action(c, t);
+  const uint32_t sel = e & 7u, copies = (e >> 3) & 3u;
+  const uint32_t rw_array = copies == 0u ? 0u : (uint32_t)kRw1Array + copies - 1u;
+  return (sel * (uint32_t)ns * 8u) | ((rw_array * (uint32_t)ns * 8u) << 15) | ((e & 64u) ? (1u << 30) : 0u) |
+         ((e & 32u) ? (1u << 31) : 0u);
+}
 
 // Everything the entry loops need about one tile, in LDS.
 // What a tile that also takes its row minima keeps in LDS beside the rest (a launch that does
@@ -542,11 +554,10 @@ struct NoRowMinStage {};
 
 template <int M, bool RM>
 struct TileStage : std::conditional_t<RM, RowMinStage, NoRowMinStage> {
-  // term arrays: [0] zeros, [1] all-gather, [2] reduce-scatter, [3] all-reduce,
-  // [4] all-to-all (= reduce-scatter shaped term x a2a_scale, :22-32), [5] read+write
   double terms[kLdsTermArrays * States<M>::kCount];
   uint2 colh[APC_TILE_MAX_COLS];  // producer specs: x = codes, y = info
-  alignas(16) uint32_t act[APC_TILE_MAX_COLS * ActionRows<M>::kWords];  // one action row per mesh dim
+  uint32_t words[APC_TILE_MAX_COLS * M * kWordsPerDim];  // lookup words per (producer spec, dim, consumer class)
+  alignas(16) uint32_t pair_base[16];  // pair_word_base by producer class x 4 + consumer class
   uint2 row[APC_TILE_MAX_ROWS];   // consumer specs: x = codes, y = info
   double cpa[APC_TILE_MAX_ROWS];  // compute cost / num_args of the consumer strategies
   int64_t dup[APC_TILE_MAX_DUPS];  // first entries of the identical edges
@@ -593,12 +604,13 @@ template <int M, bool DERIVE, bool RM>
 __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs &a, const apc_tile &tile,
                                            TileStage<M, RM> &st, int tid, int nthreads) {
   constexpr int NS = States<M>::kCount;
-  constexpr int AW = ActionRows<M>::kWords;
   const int rows = tile.counts & 0xFFFF, cols = tile.counts >> 16;
   const int t0 = tile.tensor;  // spec_tensor of the tile's first producer spec (checked by the host)
   const bool no_producer = (tile.flags & APC_EDGE_NO_PRODUCER) != 0;
   const bool terms_wanted = t0 >= 0 && !no_producer;
   bool mixed = !terms_wanted;
+  // (written and read by the first wavefront only, which stages the producer specs: in order)
+  if (tid < 16) st.pair_base[tid] = pair_word_base(tid >> 2, tid & 3, NS);
   // ---- the round of vector loads ------------------------------------------------------------
   // producer spec tid, consumer spec nthreads - 1 - tid (taken from the far end: with two
   // wavefronts one loads the producer specs while the other loads the consumer specs).
@@ -688,7 +700,9 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
       st.terms[2 * NS + k] = rs;
       st.terms[3 * NS + k] = ar;
       st.terms[4 * NS + k] = a2a;
-      st.terms[5 * NS + k] = rw_time_r(gb * 2 * 1073741824.0, p);
+      const double rw = rw_time_r(gb * 2 * 1073741824.0, p);
+      st.terms[5 * NS + k] = rw;
+      st.terms[6 * NS + k] = 2.0 * rw;
     }
     if (tid == 0) st.gb_unsharded = fbytes / 1024 / 1024 / 1024;
   } else if (tid == 0) {
@@ -707,24 +721,39 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   if (has_col) {
     // info: bit0 valid spec, bit1 fully replicated, bits 4.. mask of sharded mesh dims
     uint32_t info = (col_tensor >= 0 ? 1u : 0u) | (col_codes == 0u ? 2u : 0u);
+    uint32_t mask = 0;
+#pragma unroll
+    for (int i = 0; i < M; ++i) mask |= (kind_of((col_codes >> (8 * i)) & 0xFF) == 2 ? 1u : 0u) << i;
+    info |= mask << 4;
+    st.colh[jc] = make_uint2(col_codes, info);
 #pragma unroll
     for (int i = 0; i < M; ++i) {
-      const uint32_t c = (col_codes >> (8 * i)) & 0xFF;
-      const int cls = placement_class(c);
-      info |= (cls >= 2 ? 1u : 0u) << (4 + i);
-      st.act[jc * AW + i] = cls == 0 ? pair_row(0) : cls == 1 ? pair_row(1) : cls == 2 ? pair_row(2) : pair_row(3);
+      const int cls = placement_class((col_codes >> (8 * i)) & 0xFF);
+      const uint4 base = reinterpret_cast<const uint4 *>(st.pair_base)[cls];
+      // states of this dim for history 0: before the dim, and after an update at it
+      const uint32_t k = (uint32_t)States<M>::index(i, 0, 0) + (mask << i);
+      const uint32_t k2 = (uint32_t)States<M>::index(i + 1, 0, 0) + (mask << (i + 1)) + (1u << i);
+      // the all-gather (a sharding producer, a replicating consumer: class 0) is charged on the
+      // gathered bytes; the state's offset goes into both fields of the word
+      const uint32_t kk0 = cls >= 2 ? k2 : k;
+      uint32_t *w = st.words + (jc * M + i) * kWordsPerDim;
+      w[0] = base.x + kk0 * 0x40008u;
+      w[1] = base.y + k * 0x40008u;
+      w[2] = base.z + k * 0x40008u;
+      w[3] = base.w + k * 0x40008u;
+      w[4] = 0u;
+      w[5] = ((uint32_t)kRw1Array * NS + k) * 8u;
     }
-    st.colh[jc] = make_uint2(col_codes, info);
     if (col_tensor != t0 || col_tensor < 0) mixed = true;
   }
   if (has_row) {
-    // info: bit0 valid spec, bits 1 + 5i .. : 8 x class of mesh dim i, bit 30 every dim is a Shard
+    // info: bit0 valid spec, bits 1 + 5i .. : class of mesh dim i, bit 30 every dim is a Shard
     uint32_t info = row_tensor >= 0 ? 1u : 0u;
     bool all_shard = true;
 #pragma unroll
     for (int i = 0; i < M; ++i) {
       const uint32_t t = (row_codes >> (8 * i)) & 0xFF;
-      info |= (uint32_t)(placement_class(t) * 8) << (1 + 5 * i);
+      info |= (uint32_t)placement_class(t) << (1 + 5 * i);
       all_shard &= kind_of(t) == 2;
     }
     if (all_shard) info |= 1u << 30;
@@ -747,44 +776,36 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
 template <int M, bool CONT, bool RESCALE, bool RM>
 __device__ __forceinline__ void uniform_entry(const apc_params &p, const TileStage<M, RM> &st, int r, int c,
                                               double &comm_o, double &total_o, int &trans_o) {
-  constexpr int NS = States<M>::kCount;
   const uint2 colv = st.colh[c];
   const uint32_t src = colv.x, cinfo = colv.y;
-  uint32_t act[M];
-  ActionRows<M>::load(st.act, c, act);
   const uint2 rowv = st.row[r];
   const uint32_t tgt = rowv.x, tinfo = rowv.y;
   const double cpa = st.cpa[r];
   const uint32_t x = src ^ tgt;
-  const uint32_t mask = (cinfo >> 4) & 0xF;
-  // ---- integer part: which term of which state each mesh dim adds ------------------------
-  uint32_t hist = 0, seen = 0;
-  uint32_t term_at[M], rw_at[M], nc_at[M], copies[M];
+  const uint32_t *words = st.words + c * (M * kWordsPerDim);
+  const char *terms = reinterpret_cast<const char *>(st.terms);
+  // ---- integer part: which term of which state each mesh dim adds --------------------------
+  uint32_t hist8 = 0, seen = 0;  // hist8 = 8 x history of the earlier dims
+  uint32_t term_at[M], rw_at[M], nc_at[M];
   bool neq[M];
 #pragma unroll
   for (int i = 0; i < M; ++i) {
     neq[i] = ((x >> (8 * i)) & 0xFF) != 0;
-    const uint32_t tsh = (tinfo >> (1 + 5 * i)) & 0x1F;
-    uint32_t e = (act[i] >> tsh) & 0x7F;
-    e = neq[i] ? e : 0u;
-    const uint32_t sel = e & 7u;
-    const uint32_t k = (uint32_t)States<M>::index(i, 0, 0) + (mask << i) + hist;
-    hist |= ((e >> 6) & 1u) << i;
-    const uint32_t k2 = (uint32_t)States<M>::index(i + 1, 0, 0) + (mask << (i + 1)) + hist;
-    const uint32_t kk = sel == 1u ? k2 : k;  // the all-gather is charged on the gathered bytes
-    term_at[i] = sel * NS + kk;
-    rw_at[i] = 5 * NS + kk;
-    nc_at[i] = 5 * NS + k;
-    copies[i] = (e >> 3) & 3u;
-    seen |= e;
+    const uint32_t cls = neq[i] ? (tinfo >> (1 + 5 * i)) & 7u : 4u;  // slot 4: same placement, nothing to add
+    const uint32_t w = words[i * kWordsPerDim + cls];
+    term_at[i] = (w & kWordOffsetMask) + hist8;
+    rw_at[i] = ((w >> 15) & kWordOffsetMask) + hist8;
+    if (!CONT) nc_at[i] = words[i * kWordsPerDim + 5] + hist8;
+    hist8 += ((w >> 30) & 1u) << (3 + i);
+    seen |= w;
   }
   // ---- lookups ------------------------------------------------------------------------------
   double term[M], rw[M], nc[M];
 #pragma unroll
   for (int i = 0; i < M; ++i) {
-    term[i] = st.terms[term_at[i]];
-    rw[i] = st.terms[rw_at[i]];
-    if (!CONT) nc[i] = st.terms[nc_at[i]];
+    term[i] = *reinterpret_cast<const double *>(terms + term_at[i]);
+    rw[i] = *reinterpret_cast<const double *>(terms + rw_at[i]);
+    if (!CONT) nc[i] = *reinterpret_cast<const double *>(terms + nc_at[i]);
   }
   // ---- additions in the reference's order (0.0 + t == t for these non-negative terms) ------------
   double cost = 0.0;
@@ -798,9 +819,9 @@ __device__ __forceinline__ void uniform_entry(const apc_params &p, const TileSta
     }
     if (CONT && i == 0) cost = term[0];
     else cost += term[i];
-    cost += (double)copies[i] * rw[i];
+    cost += rw[i];  // 0, 1 or 2 read+writes: (double)copies * rw, picked from the staged multiples
   }
-  double comm = (seen & 32u) ? INFINITY : cost;
+  double comm = (seen & kWordBan) ? INFINITY : cost;
   const int trans = x != 0u ? p.transition_scale : 0;  // optimize_sharding.py:345-351
   if (M == 2 && src == 0x4040u && (tinfo >> 30)) {  // (Partial, Partial) -> all Shard walks dim 1 first
     comm = entry_cost<M>(src, tgt, st.gb_unsharded, CONT, p);
