@@ -1351,13 +1351,23 @@ __global__ __launch_bounds__(kBlock) void cost_objective_kernel(int64_t n_vars, 
                                                                 const double *__restrict__ cost, double inf_replacement,
                                                                 double *__restrict__ objective,
                                                                 uint8_t *__restrict__ forced_zero) {
-  const int64_t v = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (v >= n_vars) return;
-  int64_t lo = 0, hi = n_groups;  // last group whose first variable is <= v
-  while (hi - lo > 1) {
-    const int64_t mid = (lo + hi) >> 1;
-    if (group_var_begin[mid] <= v) lo = mid; else hi = mid;
+  // the group of the workgroup's first variable by bisection, once; every thread then walks on
+  // from there (a workgroup's 256 variables span few groups)
+  __shared__ int64_t s_first_group;
+  const int64_t v0 = (int64_t)blockIdx.x * kBlock;
+  if (threadIdx.x == 0) {
+    int64_t lo = 0, hi = n_groups;  // last group whose first variable is <= v0
+    while (hi - lo > 1) {
+      const int64_t mid = (lo + hi) >> 1;
+      if (group_var_begin[mid] <= v0) lo = mid; else hi = mid;
+    }
+    s_first_group = lo;
   }
+  __syncthreads();
+  const int64_t v = v0 + threadIdx.x;
+  if (v >= n_vars) return;
+  int64_t lo = s_first_group;
+  while (lo + 1 < n_groups && group_var_begin[lo + 1] <= v) ++lo;
   const int64_t k = v - group_var_begin[lo];
   double sum = 0.0;
   bool forced = false;

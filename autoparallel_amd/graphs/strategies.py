@@ -30,6 +30,7 @@ import itertools
 import logging
 import math
 import operator
+import threading
 
 import torch
 from torch.distributed.tensor._dtensor_spec import DTensorSpec, TensorMeta
@@ -55,23 +56,31 @@ def _registry():
     return DTensor._op_dispatcher.sharding_propagator
 
 
+_COST_STUB_LOCK = threading.RLock()
+
+
 @contextlib.contextmanager
 def _cheap_placeholder_costs(enabled: bool):
     """torch's strategy functions fill ``redistribute_cost`` rows by calling its own
     redistribute_cost for every (producer strategy, input spec) pair.  The planner
-    recomputes every such entry with its own model, so during enumeration the call can be
-    a constant."""
+    recomputes every such entry with its own model (and keeps a rule-provided value only where
+    a side is not a DTensorSpec, which torch's function never sees), so during enumeration the
+    call can be a constant.  The name is a module attribute of torch, so the stub is process-wide
+    while it is in: one enumeration at a time holds it (a lock), and it is taken out again on
+    any exit.  ``StrategyEnumerator(cheap_costs=False)`` leaves torch's function alone; the
+    tables are the same either way (tests/test_traced_graphs.py)."""
     if not enabled:
         yield
         return
     import torch.distributed.tensor._ops.utils as ops_utils
 
-    saved = ops_utils.redistribute_cost
-    ops_utils.redistribute_cost = lambda current_spec, target_spec: 0.0
-    try:
-        yield
-    finally:
-        ops_utils.redistribute_cost = saved
+    with _COST_STUB_LOCK:
+        saved = ops_utils.redistribute_cost
+        ops_utils.redistribute_cost = lambda current_spec, target_spec: 0.0
+        try:
+            yield
+        finally:
+            ops_utils.redistribute_cost = saved
 
 
 def _tensor_meta(t) -> TensorMeta:

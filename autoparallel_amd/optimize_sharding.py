@@ -68,7 +68,7 @@ class DeviceBackend:
             out = self.dev.run_spec_tables()
             return out["local_shape"].cpu().numpy(), out["local_stride"].cpu().numpy()
 
-    def upload_strategy_inputs(self, tables, tile_entries=None, dedupe=True, max_copies=8):
+    def upload_strategy_inputs(self, tables, tile_entries=None, dedupe=True, max_copies=16):
         """The strategy table is final: tile the edges (identical edges once) and send both."""
         tables.build_tiles(tile_entries, dedupe=dedupe, max_copies=max_copies)
         tables.validate(self.dev.params)
@@ -280,7 +280,7 @@ class ShardingOptimizer:
     # edge may serve at most
     tile_entries = None
     dedupe = True
-    max_copies = 8
+    max_copies = 16
     # ILP formulation: besides the reference's one binary per cost entry, one binary per (node,
     # strategy) tied to the entry variables of that strategy's row.  Only these need to be
     # declared integral: with a node's and its producers' choices fixed to unit vectors the
@@ -291,6 +291,9 @@ class ShardingOptimizer:
     # growing, graph_clustering.py:101-206, which under torch 2.10 fails its own sanity check on
     # Llama-shaped graphs)
     clustering = "neighbourhood"
+    # during enumeration torch's own redistribute_cost (whose values the table build replaces) is
+    # stubbed by a constant; False leaves it alone (same tables, slower enumeration)
+    cheap_enumeration_costs = True
     node_choice_variables = True
     compact_constraints = True  # with choice variables: the structural constraints written through them
     # Before the solver runs: a dual ascent over the program's labelling form (row / column minima
@@ -357,7 +360,7 @@ class ShardingOptimizer:
 
     # ------------------------------------------------------------------------------------
     def build_sharding_metadata(self):
-        self.enumerator = StrategyEnumerator(self.mesh)
+        self.enumerator = StrategyEnumerator(self.mesh, cheap_costs=self.cheap_enumeration_costs)
         return self.enumerator.enumerate(self.graph)
 
     def _grad_param_nodes(self):

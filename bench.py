@@ -51,7 +51,7 @@ def parse_args():
     ap.add_argument("--no-solve", action="store_true", help="skip the ILP leg of the plan wall-time")
     ap.add_argument("--no-clustering", action="store_true", help="one ILP variable per entry (no variable sharing)")
     ap.add_argument("--no-dedupe", action="store_true", help="tile every edge even if an identical one exists")
-    ap.add_argument("--max-copies", type=int, default=8, help="identical edges served by one tiled edge")
+    ap.add_argument("--max-copies", type=int, default=16, help="identical edges served by one tiled edge")
     ap.add_argument("--pass", dest="pass_kind", choices=["planner", "all"], default="planner",
                     help="planner: the pass build_ds issues (assembled cost, no spec table); all: every table and all "
                          "three per-entry arrays (the composite of the earlier benchmark, labelled as such)")

@@ -19,7 +19,7 @@ class OracleBackend:
         _, lshape, lstride, _, _ = c_oracle.spec_tables(self.tables.as_dict(), self.tables.mesh_sizes)
         return lshape, lstride
 
-    def upload_strategy_inputs(self, tables, tile_entries=None, dedupe=True, max_copies=8):
+    def upload_strategy_inputs(self, tables, tile_entries=None, dedupe=True, max_copies=16):
         # host-side tiling / de-duplication runs as in the product (the oracle ignores the tiles)
         tables.build_tiles(tile_entries, dedupe=dedupe, max_copies=max_copies)
         tables.validate(self.product_params)

@@ -111,6 +111,41 @@ def test_tiny_llama_tables_and_clustering(fake_pg):
         assert not opt.prob.violated_constraints()
 
 
+def test_enumeration_cost_stub_is_scoped_and_changes_no_table(fake_pg):
+    """While strategies are enumerated torch's own ``redistribute_cost`` is replaced by a constant
+    (the table build recomputes every entry it produced): the replacement is taken out again on an
+    exception, and the encoded tables, pass-through values included, are the same without it."""
+    import torch.distributed.tensor._ops.utils as ops_utils
+
+    from autoparallel_amd.graphs.strategies import _cheap_placeholder_costs
+
+    original = ops_utils.redistribute_cost
+    with pytest.raises(ZeroDivisionError):
+        with _cheap_placeholder_costs(True):
+            assert ops_utils.redistribute_cost is not original
+            1 / 0
+    assert ops_utils.redistribute_cost is original
+
+    class UnstubbedOptimizer(OracleOptimizer):
+        cheap_enumeration_costs = False
+
+    class UnstubbedPlanner(AutoParallelPlanner):
+        optimizer_cls = UnstubbedOptimizer
+
+    tables = []
+    for planner_cls in (OraclePlanner, UnstubbedPlanner):
+        for cfg, mesh in ((TINY, (32, 8)), (TINY_MOE, (8, 4))):
+            batch, seq = (64, 256) if cfg is TINY else (16, 64)
+            with _planner(planner_cls, cfg, mesh, batch, seq) as autop:
+                tb = autop.sharding_optimizer.encoded.tables
+                assert ops_utils.redistribute_cost is original
+                tables.append({k: v for k, v in tb.as_dict().items() if isinstance(v, np.ndarray)})
+    for a, b in zip(tables[:2], tables[2:]):
+        assert a.keys() == b.keys() and len(a["pt_values"]) > 0
+        for k in a:
+            assert np.array_equal(a[k], b[k]), k
+
+
 def test_tiny_moe_regions_and_plan(fake_pg):
     """The mixture-of-experts decoder: every routed-expert region is one forward and one
     backward node with the single strategy its author declared; the graph plans."""
