@@ -62,7 +62,128 @@ def parse_args():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy three times (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
+    ap.add_argument("--no-traffic", action="store_true",
+                    help="skip the HBM-traffic reading (four short child runs of this script under rocprofv3 --pmc)")
+    ap.add_argument("--replay-tables", default=None,
+                    help="(child of the traffic reading) load the encoded tables from this .npz, run the pass three "
+                         "times and exit")
     return ap.parse_args()
+
+
+# ---- HBM traffic of the dominant launch, read from the hardware counters --------------------------
+# A counter cannot be read from inside the process, so the pass is replayed in child processes
+# under ``rocprofv3 --pmc`` (one counter per run: FETCH_SIZE, then WRITE_SIZE, KiB per dispatch),
+# each scaled by what the same counter reads for a plain 1 GiB device-to-device copy.  The
+# children load the parent's encoded tables from a temporary file, so they take seconds.
+TABLE_FIELDS_SKIP = ("mesh_sizes", "tiling")
+
+
+def save_tables(tables, params, pass_kind, path):
+    import numpy as np
+
+    arrays = {k: v for k, v in tables.as_dict().items() if isinstance(v, np.ndarray)}
+    np.savez(path, **arrays, _mesh=np.asarray(tables.mesh_sizes), _rescale=np.asarray([params.rescale]),
+             _pass=np.asarray([pass_kind]))
+
+
+def replay_tables(path):
+    """Child process: the pass over tables loaded from ``path``, three times."""
+    import numpy as np
+    import torch
+
+    from autoparallel_amd import CostModelParams
+    from autoparallel_amd.device_tables import DeviceCostTables
+    from autoparallel_amd.encoding import CostTables
+
+    z = np.load(path)
+    mesh = tuple(int(x) for x in z["_mesh"])
+    fields = {k: z[k] for k in z.files if not k.startswith("_")}
+    tables = CostTables(mesh_sizes=mesh, **fields)
+    dev = DeviceCostTables(tables, CostModelParams.from_mesh(mesh, rescale=float(z["_rescale"][0])), device="cuda:0",
+                           validate=False)
+    step = prepare(dev, str(z["_pass"][0]))
+    for _ in range(3):
+        for launch in step.values():
+            launch()
+    torch.cuda.synchronize()
+    print(json.dumps({"replayed": list(step), "entries": tables.n_entries}))
+
+
+def read_counter(counter, child_args, kernel_substring, log, timeout_s=120):
+    """Average ``counter`` per dispatch of the kernels whose name contains ``kernel_substring`` in a
+    child run of this script under rocprofv3; None (and a log line) if anything goes wrong."""
+    import csv
+    import glob
+    import shutil
+    import signal
+    import subprocess
+    import tempfile
+
+    rocprof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    if not os.path.exists(rocprof):
+        log.info("traffic: rocprofv3 not found")
+        return None
+    out_dir = tempfile.mkdtemp(prefix="apc_pmc_", dir="/tmp")
+    cmd = [rocprof, "--pmc", counter, "-d", out_dir, "-o", "pmc", "--output-format", "csv", "--",
+           sys.executable, os.path.abspath(__file__), *child_args]
+    try:
+        proc = subprocess.Popen(cmd, cwd="/tmp", env={**os.environ, "TMPDIR": "/tmp"}, stdout=subprocess.DEVNULL,
+                                stderr=subprocess.DEVNULL, start_new_session=True)
+        try:
+            rc = proc.wait(timeout=timeout_s)
+        except subprocess.TimeoutExpired:
+            os.killpg(proc.pid, signal.SIGKILL)  # the child's own process group, nothing else
+            proc.wait()
+            log.info("traffic: %s run timed out", counter)
+            return None
+        if rc != 0:
+            log.info("traffic: %s run exited with %d", counter, rc)
+            return None
+        files = glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True)
+        values = []
+        for f in files:
+            with open(f) as fh:
+                for row in csv.DictReader(fh):
+                    if kernel_substring in row["Kernel_Name"] and row["Counter_Name"] == counter:
+                        values.append(float(row["Counter_Value"]))
+        return sum(values) / len(values) if values else None
+    except OSError as e:
+        log.info("traffic: %s", e)
+        return None
+    finally:
+        shutil.rmtree(out_dir, ignore_errors=True)
+
+
+def measure_traffic(tables, params, pass_kind, kernel, log, factor=None):
+    """-> dict for ``roofline`` (traffic in bytes per launch and how it was read) or None.
+    ``factor``: the copy-kernel scale factors of an earlier reading in this run (not read again)."""
+    import tempfile
+
+    gib_kib = float(1 << 20)  # a 1 GiB copy reads and writes 2^20 KiB
+    path = os.path.join(tempfile.mkdtemp(prefix="apc_tables_", dir="/tmp"), "tables.npz")
+    try:
+        save_tables(tables, params, pass_kind, path)
+        reading, factor = {}, dict(factor or {})
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            if counter not in factor:
+                copy = read_counter(counter, ["--calibrate-copy"], "copyBuffer", log)
+                if not copy:
+                    return None
+                factor[counter] = gib_kib / copy
+            value = read_counter(counter, ["--replay-tables", path], kernel, log, timeout_s=240)
+            if value is None:
+                return None
+            reading[counter] = value
+        traffic = (reading["FETCH_SIZE"] * factor["FETCH_SIZE"] + reading["WRITE_SIZE"] * factor["WRITE_SIZE"]) * 1024.0
+        return {"traffic": traffic,
+                "traffic_reading": {"kib_per_dispatch": reading, "scale_from_1gib_copy": factor,
+                                    "how": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (one run each) over a replay of this "
+                                           "pass on the same tables in a child process; each scaled by the same "
+                                           "counter's reading of a plain 1 GiB device-to-device copy"}}
+    finally:
+        import shutil
+
+        shutil.rmtree(os.path.dirname(path), ignore_errors=True)
 
 
 def build_workload(name, args):
@@ -332,7 +453,7 @@ def roofline_of(dev, tables, timing, steps, pass_kind):
         "achieved": launch_bytes / t_kernel / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": launch_bytes / t_kernel / 1e9 / HBM_PEAK_GBPS,
         "frac_survey_8d": priced / t_kernel / 1e9 / HBM_PEAK_GBPS,
-        "traffic": None,
+        "traffic": None,  # filled in by measure_traffic for the main workload
         "bytes_per_launch": launch_bytes, "bytes_per_launch_survey_8d": priced,
         "avg_launch_us": t_kernel * 1e6,
         "avg_launch_us_event_pair_per_launch": t_pair * 1e6,
@@ -340,8 +461,6 @@ def roofline_of(dev, tables, timing, steps, pass_kind):
         "timing": ("one HIP event pair on the launch stream around the K back-to-back launches of the timed "
                    "region (the pass is this one kernel), / K" if single else
                    "HIP events around every launch of the kernel inside the timed region"),
-        "traffic_note": "hardware counters cannot be read from inside the process: FETCH_SIZE / WRITE_SIZE per dispatch "
-                        "of this kernel are in profiles/ (rocprofv3 --pmc runs of this command)",
     }
 
 
@@ -414,6 +533,7 @@ def measure(name, args, log, steps, warmup, main_run):
             "ms_per_step_with_events": timing["wall_events_s"] / steps * 1e3,
             "host_timings_s": {k: round(v, 6) for k, v in host_timings.items()},
             "parity": parity,
+            "params": params,
         }
         if main_run and not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline(tables, params, args.cpu_seconds)
@@ -439,6 +559,9 @@ def main():
         print("bench.py needs a HIP device (there is no CPU path for the product)", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if args.replay_tables:
+        replay_tables(args.replay_tables)
+        return
     if args.calibrate_copy:
         src = torch.ones(1 << 27, dtype=torch.float64, device="cuda:0")  # 1 GiB
         dst = torch.empty_like(src)
@@ -450,6 +573,7 @@ def main():
         return
 
     K = args.steps
+    copy_factor = None
     out, planner, tables, host_timings = measure(args.workload, args, log, K, args.warmup, main_run=True)
     result = {
         "metric": "redistribution_cost_entries_per_s",
@@ -474,6 +598,17 @@ def main():
     }
     if "cpu_baseline" in out:
         result["cpu_baseline"] = out["cpu_baseline"]
+    if not args.no_traffic:
+        from autoparallel_amd.device_tables import _real_tensors
+
+        with _real_tensors():
+            t0 = time.perf_counter()
+            read = measure_traffic(tables, out["params"], args.pass_kind, out["roofline"]["kernel"], log)
+            log.info("traffic reading: %.1f s", time.perf_counter() - t0)
+        if read is not None:
+            result["roofline"].update(read)
+            result["roofline"]["traffic_over_bytes_per_launch"] = read["traffic"] / result["roofline"]["bytes_per_launch"]
+            copy_factor = read["traffic_reading"]["scale_from_1gib_copy"]
     if planner is not None:
         plan = {"stages_s": {k: round(v, 6) for k, v in host_timings.items()}}
         if not args.no_solve:
@@ -501,9 +636,15 @@ def main():
         gc.collect()
         torch.cuda.empty_cache()
         k = max(5, min(K, 20))
-        o, pl, _, _ = measure(name, args, log, k, min(args.warmup, 5), main_run=False)
+        o, pl, tb, _ = measure(name, args, log, k, min(args.warmup, 5), main_run=False)
         if pl is not None:
             pl.__exit__(None, None, None)
+        if not args.no_traffic and copy_factor is not None:
+            read = measure_traffic(tb, o["params"], args.pass_kind, o["roofline"]["kernel"], log, factor=copy_factor)
+            if read is not None:
+                o["roofline"].update(read)
+                o["roofline"]["traffic_over_bytes_per_launch"] = read["traffic"] / o["roofline"]["bytes_per_launch"]
+        del tb
         extra[name] = {"workload": o["config"]["workload"], "entries": o["config"]["entries"], "steps": k,
                        "ms_per_step": o["ms_per_step"], "entries_per_s": o["value"], "step": o["config"]["step"],
                        "tiles": o["config"]["tiles"], "roofline": o["roofline"], "kernel_us": o["kernel_us"],
