@@ -433,6 +433,20 @@ __global__ __launch_bounds__(kBlock) void input_tables_kernel(apc_params p, Tens
 // staging below: fewer, longer-lived workgroups keep fewer stores in flight.)
 // ------------------------------------------------------------------------------------------
 
+// What is the same for every tile of a launch (see "Term arrays" and "Lookup words" below):
+// the layout of the term arrays and the part of the lookup words that does not depend on the
+// producer spec (by dim x 16 + producer class x 4 +
+// consumer class; the producer spec's state or exponent index is added, to both fields, when
+// a tile is staged).
+struct TermLayout {
+  uint32_t pair[APC_MAX_MESH * 16];
+  int32_t exponents;          // 0: general layout; else E, the number of exponents
+  int32_t lg[APC_MAX_MESH];   // log2 of the mesh sizes (power-of-two layout)
+  int32_t lg_total;           // L
+  uint32_t rw1_base;          // first entry of the one-read+write array
+  uint32_t exponent_magic;    // ceil(65536 / E): t / E = (t * magic) >> 16 for t < 512
+};
+
 struct TableArgs {
   const int64_t *tensor_bytes;
   const uint8_t *tensor_contiguous;
@@ -461,6 +475,7 @@ struct TableArgs {
   const int64_t *dup_row_begin;
   double *row_min_out;
   int32_t *row_arg_out;
+  TermLayout lay;  // the launch's term-array layout and lookup-word bases
 };
 
 // Bytes and contiguity of tensor t: read from the tensor table, or (DERIVE) derived from its
@@ -502,40 +517,100 @@ __device__ __forceinline__ int placement_class(uint32_t code) {
   return k == 2 ? 2 + (dim_of(code) != 0 ? 1 : 0) : k;
 }
 
-// Term arrays staged per tile, one value per running-bytes state: [0] zeros, [1] all-gather,
+// Term arrays staged per tile.  Two layouts, chosen per launch by the host (TermLayout):
+//
+// General (any mesh): one value per running-bytes state, arrays [0] zeros, [1] all-gather,
 // [2] reduce-scatter, [3] all-reduce, [4] all-to-all (= reduce-scatter shaped term x a2a_scale,
-// :22-32), [5] one read+write, [6] two read+writes (2.0 x [5]: the same bits as (double)2 * rw).
-constexpr int kLdsTermArrays = 7;
-constexpr int kRw1Array = 5;
+// :22-32), [5] one read+write, [6] two read+writes (2.0 x [5]: the same bits as (double)2 * rw),
+// [7] +inf (banned transitions).  An entry's running index is the history of the earlier dims.
+//
+// Power-of-two meshes (every mesh size a power of two, world size below 2^31): the running
+// bytes are the tensor's bytes times a power of two, bytes x 2^e with e in [-30 - L, -30],
+// L = log2(world size): dividing by the shards, x n after an all-gather and / n after a
+// reduce-scatter are exact.  Every term is then a rounding-free rescaling of ONE chain of
+// operations on the tensor's bytes: RN(2^e x) = 2^e RN(x) for the multiplications and divisions
+// of the ring and read+write formulas (no underflow: bytes < 2^53, e >= -61), so
+//   ring term of dim d at exponent e = latency_d + ldexp(B_d, e - log2 n_d),
+//       B_d = RN(RN(RN(bytes x hops_d) / bw_d) x 1e6)      (two hops per step: B doubles)
+//   read+write at exponent e = max(ldexp(R, e + 31), launch floor),
+//       R = RN(RN(RN(bytes / hbm_bw) x 1e6) / rw_eff)
+// and one value per (array, exponent) replaces one per (array, state): arrays [0] zeros, [1]
+// +inf, then per mesh dim d [2 + 3d] one-hop ring (all-gather and reduce-scatter), [3 + 3d]
+// two-hop ring (all-reduce), [4 + 3d] all-to-all, then one read+write, two read+writes; E =
+// L + 1 values each.  An entry's running index is e + 30 + L.  (3-D mesh of 512 devices: 110
+// computed values, each a handful of operations, against 120 states x 6 terms of two
+// divisions each.)
+constexpr int kMaxExponents = 32;
+template <int M>
+struct TermTable {
+  static constexpr int kGeneral = 8 * States<M>::kCount;
+  static constexpr int kPow2 = (4 + 3 * M) * kMaxExponents;
+  static constexpr int kEntries = kGeneral > kPow2 ? kGeneral : kPow2;
+};
 
 // Lookup words.  What a mesh dim adds to an entry depends on the producer spec (its class at
-// that dim and which dims it shards), on the consumer's class at that dim and on the history of
-// the earlier dims; everything but the history is known per (producer spec, dim, consumer
-// class) when the tile is staged.  One 32-bit word per such triple holds, as byte offsets into
-// the term arrays for history 0 (the entry adds history x 8):
-//   bits  0-14  offset of the collective's term   (array of pair_action's term, state of the
-//               bytes the collective moves: after the update for an all-gather, before it else)
-//   bits 15-29  offset of the read+write term     (array 0 / 5 / 6 for 0 / 1 / 2 reshuffles,
-//               same state)
-//   bit  30     the running bytes change after this dim (history bit)
-//   bit  31     banned transition: the entry costs inf
-// Slot 4 of a (spec, dim) is the word of "same placement": 0 (the zero array, no update); slot
-// 5 is the offset of one read+write at the state BEFORE the dim, charged once to a
-// non-contiguous tensor.
+// that dim and which dims it shards), on the consumer's class at that dim and on the running
+// index left by the earlier dims; everything but the running index is known per (producer
+// spec, dim, consumer class) when the tile is staged.  One 32-bit word per such triple holds,
+// as indices into the term arrays for running index 0 (the entry adds its running index):
+//   bits  0-11  the collective's term  (general: array of pair_action's term, state of the
+//               bytes the collective moves: after the update for an all-gather, before it else;
+//               the +inf array for a banned transition)
+//   bits 12-23  the read+write term    (zeros / one / two reshuffles, same state)
+//   bits 24-31  signed step of the running index after this dim (general: the dim's history
+//               bit; power-of-two meshes: + log2 n after an all-gather, - log2 n after a
+//               reduce-scatter)
+// Slot 4 of a (spec, dim) is the word of "same placement": zeros, no step; slot 5 is the index
+// of one read+write at the state BEFORE the dim, charged once to a non-contiguous tensor.
 constexpr int kWordsPerDim = 6;
-// The part of a lookup word that does not depend on the state: array offsets for state 0 and the
-// two flags, by (producer class, consumer class); the state's offset (x 8, in both fields) is
-// added when a tile is staged.  NS = number of states of the mesh rank.
-__host__ __device__ constexpr uint32_t pair_word_base(int c, int t, int ns);
-constexpr uint32_t kWordOffsetMask = 0x7FFFu, kWordUpdate = 1u << 30, kWordBan = 1u << 31;
-static_assert(kLdsTermArrays * States<APC_MAX_MESH>::kCount * 8 <= 0x7FFF + 1, "term offsets fit their 15 bits");
+constexpr uint32_t kWordFieldMask = 0xFFFu, kWordBothFields = 0x1001u;
+static_assert(TermTable<APC_MAX_MESH>::kEntries <= 0xFFF + 1, "term indices fit their 12 bits");
 
-__host__ __device__ constexpr uint32_t pair_word_base(int c, int t, int ns) {
-  const uint32_t e = pair_action(c, t);
-  const uint32_t sel = e & 7u, copies = (e >> 3) & 3u;
-  const uint32_t rw_array = copies == 0u ? 0u : (uint32_t)kRw1Array + copies - 1u;
-  return (sel * (uint32_t)ns * 8u) | ((rw_array * (uint32_t)ns * 8u) << 15) | ((e & 64u) ? (1u << 30) : 0u) |
-         ((e & 32u) ? (1u << 31) : 0u);
+static TermLayout term_layout(const apc_params &p) {
+  TermLayout lay{};
+  const int M = p.mesh_ndim;
+  const int ns = (1 << M) * ((1 << (M + 1)) - 1);
+  bool pow2 = getenv("APC_GENERAL_TERMS") == nullptr;  // (testing override: the general layout on any mesh)
+  int total = 0;
+  for (int i = 0; i < M; ++i) {
+    const int n = p.mesh_size[i];
+    if (n < 1 || (n & (n - 1)) != 0) {
+      pow2 = false;
+      break;
+    }
+    int lg = 0;
+    while ((1 << lg) < n) ++lg;
+    lay.lg[i] = lg;
+    total += lg;
+  }
+  if (total + 1 > kMaxExponents) pow2 = false;
+  const int E = pow2 ? total + 1 : 0;
+  lay.exponents = E;
+  lay.lg_total = pow2 ? total : 0;
+  lay.rw1_base = pow2 ? (uint32_t)((2 + 3 * M) * E) : (uint32_t)(5 * ns);
+  lay.exponent_magic = pow2 ? (uint32_t)((65536 + E - 1) / E) : 0u;
+  for (int i = 0; i < M; ++i)
+    for (int c = 0; c < 4; ++c)
+      for (int t = 0; t < 4; ++t) {
+        const uint32_t e = pair_action(c, t);
+        const uint32_t sel = e & 7u, copies = (e >> 3) & 3u;
+        const bool ban = (e & 32u) != 0, upd = (e & 64u) != 0;
+        uint32_t term, rw;
+        int step;
+        if (!pow2) {
+          term = (ban ? 7u : sel) * (uint32_t)ns;
+          rw = (copies == 0u ? 0u : 5u + copies - 1u) * (uint32_t)ns;
+          step = upd ? (1 << i) : 0;
+        } else {
+          const uint32_t shift = sel == 1u ? (uint32_t)lay.lg[i] : 0u;  // an all-gather is charged on the gathered bytes
+          const uint32_t array = ban ? 1u : sel == 0u ? 0u : sel <= 2u ? 2u + 3u * i : sel == 3u ? 3u + 3u * i : 4u + 3u * i;
+          term = array * (uint32_t)E + shift;
+          rw = (copies == 0u ? 0u : (uint32_t)(2 + 3 * M) + copies - 1u) * (uint32_t)E + shift;
+          step = !upd ? 0 : sel == 1u ? lay.lg[i] : -lay.lg[i];
+        }
+        lay.pair[i * 16 + c * 4 + t] = term | (rw << 12) | ((uint32_t)(step & 0xFF) << 24);
+      }
+  return lay;
 }
 
 // Everything the entry loops need about one tile, in LDS.
@@ -554,17 +629,26 @@ struct NoRowMinStage {};
 
 template <int M, bool RM>
 struct TileStage : std::conditional_t<RM, RowMinStage, NoRowMinStage> {
-  double terms[kLdsTermArrays * States<M>::kCount];
   uint2 colh[APC_TILE_MAX_COLS];  // producer specs: x = codes, y = info
   uint32_t words[APC_TILE_MAX_COLS * M * kWordsPerDim];  // lookup words per (producer spec, dim, consumer class)
-  alignas(16) uint32_t pair_base[16];  // pair_word_base by producer class x 4 + consumer class
+  alignas(16) uint32_t pair_base[M * 16];  // TermLayout::pair of the launch
   uint2 row[APC_TILE_MAX_ROWS];   // consumer specs: x = codes, y = info
   double cpa[APC_TILE_MAX_ROWS];  // compute cost / num_args of the consumer strategies
   int64_t dup[APC_TILE_MAX_DUPS];  // first entries of the identical edges
   double gb_unsharded;  // bytes / 1024^3 of the tile's tensor
   int mixed[4];         // per staging wavefront: some spec is not a DTensorSpec on the tile's tensor (generic loop)
   int cont;             // the tile's tensor is contiguous
+  // Last: the tile kernels size their LDS per launch for the entries the layout in use needs
+  // (stage_lds_bytes), so that the small power-of-two layout leaves room for more workgroups.
+  alignas(16) double terms[TermTable<M>::kEntries];
 };
+
+// LDS bytes of a tile stage whose term arrays hold what the launch's layout needs.
+template <int M, bool RM>
+static size_t stage_lds_bytes(const TermLayout &lay) {
+  const size_t entries = lay.exponents ? (size_t)(4 + 3 * M) * lay.exponents : (size_t)TermTable<M>::kGeneral;
+  return sizeof(TileStage<M, RM>) - sizeof(double) * TermTable<M>::kEntries + sizeof(double) * entries;
+}
 
 // The fields of a tile record the entry loops use.
 struct TileView {
@@ -609,8 +693,12 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   const bool no_producer = (tile.flags & APC_EDGE_NO_PRODUCER) != 0;
   const bool terms_wanted = t0 >= 0 && !no_producer;
   bool mixed = !terms_wanted;
-  // (written and read by the first wavefront only, which stages the producer specs: in order)
-  if (tid < 16) st.pair_base[tid] = pair_word_base(tid >> 2, tid & 3, NS);
+  const TermLayout &lay = a.lay;
+  const int E = lay.exponents;  // wave-uniform; 0: general layout
+  // (written and read by the first wavefront only, which stages the producer specs: in order.
+  // A kernel argument indexed by the lane: one vector load, part of the round below.)
+  uint32_t pair_word = 0;
+  if (tid < 16 * M) pair_word = lay.pair[tid];
   // ---- the round of vector loads ------------------------------------------------------------
   // producer spec tid, consumer spec nthreads - 1 - tid (taken from the far end: with two
   // wavefronts one loads the producer specs while the other loads the consumer specs).
@@ -665,8 +753,37 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
       contiguous = ok ? 1u : 0u;
     }
   }
-  // ---- state terms (scalar operands only) ---------------------------------------------------
-  if (terms_wanted) {
+  // ---- term arrays (scalar operands only) ---------------------------------------------------
+  if (terms_wanted && E != 0) {
+    // power-of-two mesh: one value per (array, exponent), arrays 2 .. 3 + 3M
+    const double fbytes = (double)tensor_nbytes;
+    const int n_values = (3 * M + 2) * E;
+    for (int t = tid; t < n_values; t += nthreads) {
+      const int arr = (int)(((uint32_t)t * lay.exponent_magic) >> 16);
+      const int e = (t - arr * E) - lay.lg_total - 30;  // the running bytes are bytes x 2^e
+      double v;
+      if (arr < 3 * M) {  // a ring term (torch _collective_utils.py:281-313) of dim d
+        int d = 0;
+#pragma unroll
+        for (int i = 1; i < M; ++i) d += arr >= 3 * i ? 1 : 0;
+        const int typ = arr - 3 * d;  // 0 one hop per step, 1 two (all-reduce), 2 all-to-all
+        const double h = (double)(pick<M>(p.mesh_size, d) - 1);
+        const double b = div_by(fbytes * h, pick<M>(p.bw, d), pick<M>(p.inv_bw, d)) * 1e6;
+        const double hops = typ == 1 ? 2.0 * h : h;
+        const double latency = p.base_latency + hops * pick<M>(p.lat, d);
+        v = latency + __builtin_ldexp(b, e - pick<M>(lay.lg, d) + (typ == 1 ? 1 : 0));
+        if (typ == 2) v *= p.a2a_scale;  // collective_runtime_estimation.py:22-32
+      } else {  // read+write of the running bytes (compute_estimation.py:302-314)
+        const double r = div_by(div_by(fbytes, p.hbm_bw, p.inv_hbm_bw) * 1e6, p.rw_eff, p.inv_rw_eff);
+        const double tt = __builtin_ldexp(r, e + 31);
+        v = tt > p.launch_floor ? tt : p.launch_floor;
+        if (arr == 3 * M + 1) v = 2.0 * v;
+      }
+      st.terms[2 * E + t] = v;
+    }
+    if (tid < 2 * E) st.terms[tid] = tid < E ? 0.0 : __builtin_inf();
+    if (tid == 0) st.gb_unsharded = fbytes / 1024 / 1024 / 1024;
+  } else if (terms_wanted) {
     // every collective / read-write term the tile can need, once per running-bytes state, in
     // the reference's operation order (collective_runtime_estimation.py:66-68, :86, :128;
     // torch _collective_utils.py:281-313; compute_estimation.py:302-314)
@@ -703,6 +820,7 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
       const double rw = rw_time_r(gb * 2 * 1073741824.0, p);
       st.terms[5 * NS + k] = rw;
       st.terms[6 * NS + k] = 2.0 * rw;
+      st.terms[7 * NS + k] = __builtin_inf();
     }
     if (tid == 0) st.gb_unsharded = fbytes / 1024 / 1024 / 1024;
   } else if (tid == 0) {
@@ -710,6 +828,7 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   }
   // ---- what the loads brought, to LDS ---------------------------------------------------------
   if (tid == 0) st.cont = contiguous != 0;
+  if (tid < 16 * M) st.pair_base[tid] = pair_word;
   if (has_dup0) st.dup[tid] = dup0;
   if (has_dup1) st.dup[tid + nthreads] = dup1;
   if constexpr (RM) {
@@ -726,23 +845,27 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
     for (int i = 0; i < M; ++i) mask |= (kind_of((col_codes >> (8 * i)) & 0xFF) == 2 ? 1u : 0u) << i;
     info |= mask << 4;
     st.colh[jc] = make_uint2(col_codes, info);
+    // power-of-two mesh: the producer spec's exponent index, L - log2(its shards)
+    uint32_t j0 = (uint32_t)lay.lg_total;
+#pragma unroll
+    for (int i = 0; i < M; ++i) j0 -= ((mask >> i) & 1u) ? (uint32_t)lay.lg[i] : 0u;
 #pragma unroll
     for (int i = 0; i < M; ++i) {
       const int cls = placement_class((col_codes >> (8 * i)) & 0xFF);
-      const uint4 base = reinterpret_cast<const uint4 *>(st.pair_base)[cls];
-      // states of this dim for history 0: before the dim, and after an update at it
+      const uint4 base = reinterpret_cast<const uint4 *>(st.pair_base)[i * 4 + cls];
+      // general layout: states of this dim for history 0, before the dim and after an update at
+      // it; the all-gather (a sharding producer, a replicating consumer: class 0) is charged on
+      // the gathered bytes.  (Power-of-two layout: that shift is part of the word's base.)
       const uint32_t k = (uint32_t)States<M>::index(i, 0, 0) + (mask << i);
       const uint32_t k2 = (uint32_t)States<M>::index(i + 1, 0, 0) + (mask << (i + 1)) + (1u << i);
-      // the all-gather (a sharding producer, a replicating consumer: class 0) is charged on the
-      // gathered bytes; the state's offset goes into both fields of the word
-      const uint32_t kk0 = cls >= 2 ? k2 : k;
+      const uint32_t at = E != 0 ? j0 : k, at0 = E != 0 ? j0 : cls >= 2 ? k2 : k;
       uint32_t *w = st.words + (jc * M + i) * kWordsPerDim;
-      w[0] = base.x + kk0 * 0x40008u;
-      w[1] = base.y + k * 0x40008u;
-      w[2] = base.z + k * 0x40008u;
-      w[3] = base.w + k * 0x40008u;
-      w[4] = 0u;
-      w[5] = ((uint32_t)kRw1Array * NS + k) * 8u;
+      w[0] = base.x + at0 * kWordBothFields;
+      w[1] = base.y + at * kWordBothFields;
+      w[2] = base.z + at * kWordBothFields;
+      w[3] = base.w + at * kWordBothFields;
+      w[4] = at * kWordBothFields;
+      w[5] = lay.rw1_base + at;
     }
     if (col_tensor != t0 || col_tensor < 0) mixed = true;
   }
@@ -784,8 +907,8 @@ __device__ __forceinline__ void uniform_entry(const apc_params &p, const TileSta
   const uint32_t x = src ^ tgt;
   const uint32_t *words = st.words + c * (M * kWordsPerDim);
   const char *terms = reinterpret_cast<const char *>(st.terms);
-  // ---- integer part: which term of which state each mesh dim adds --------------------------
-  uint32_t hist8 = 0, seen = 0;  // hist8 = 8 x history of the earlier dims
+  // ---- integer part: which term at which running index each mesh dim adds -------------------
+  uint32_t at8 = 0;  // 8 x running index (history of the earlier dims / exponent steps), mod 2^32
   uint32_t term_at[M], rw_at[M], nc_at[M];
   bool neq[M];
 #pragma unroll
@@ -793,11 +916,10 @@ __device__ __forceinline__ void uniform_entry(const apc_params &p, const TileSta
     neq[i] = ((x >> (8 * i)) & 0xFF) != 0;
     const uint32_t cls = neq[i] ? (tinfo >> (1 + 5 * i)) & 7u : 4u;  // slot 4: same placement, nothing to add
     const uint32_t w = words[i * kWordsPerDim + cls];
-    term_at[i] = (w & kWordOffsetMask) + hist8;
-    rw_at[i] = ((w >> 15) & kWordOffsetMask) + hist8;
-    if (!CONT) nc_at[i] = words[i * kWordsPerDim + 5] + hist8;
-    hist8 += ((w >> 30) & 1u) << (3 + i);
-    seen |= w;
+    term_at[i] = ((w & kWordFieldMask) << 3) + at8;
+    rw_at[i] = (((w >> 12) & kWordFieldMask) << 3) + at8;
+    if (!CONT) nc_at[i] = (words[i * kWordsPerDim + 5] << 3) + at8;
+    at8 += (uint32_t)(((int32_t)w >> 24) << 3);
   }
   // ---- lookups ------------------------------------------------------------------------------
   double term[M], rw[M], nc[M];
@@ -821,7 +943,7 @@ __device__ __forceinline__ void uniform_entry(const apc_params &p, const TileSta
     else cost += term[i];
     cost += rw[i];  // 0, 1 or 2 read+writes: (double)copies * rw, picked from the staged multiples
   }
-  double comm = (seen & kWordBan) ? INFINITY : cost;
+  double comm = cost;  // (a banned transition added the +inf term)
   const int trans = x != 0u ? p.transition_scale : 0;  // optimize_sharding.py:345-351
   if (M == 2 && src == 0x4040u && (tinfo >> 30)) {  // (Partial, Partial) -> all Shard walks dim 1 first
     comm = entry_cost<M>(src, tgt, st.gb_unsharded, CONT, p);
@@ -1153,8 +1275,9 @@ constexpr int tile_waves_per_simd(int mesh_ndim, int threads) {
 template <int M, int kTileThreads, int OUT>
 __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads), 8)))
 void redistribute_tiles_kernel(apc_params p, TableArgs a, int n_tiles, int xcd_shift) {
-  __shared__ TileStage<M, false> s_stage;
-  redistribute_tile<M, kTileThreads, false, OUT>(p, a, n_tiles, xcd_shift, s_stage);
+  extern __shared__ __align__(16) unsigned char s_stage_bytes[];  // stage_lds_bytes<M, false>
+  redistribute_tile<M, kTileThreads, false, OUT>(p, a, n_tiles, xcd_shift,
+                                                 *reinterpret_cast<TileStage<M, false> *>(s_stage_bytes));
 }
 
 // The same with the row minima.
@@ -1162,8 +1285,9 @@ template <int M, int kTileThreads, int OUT>
 __global__ __launch_bounds__(kTileThreads)
 __attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads), 8)))
 void redistribute_tiles_row_min_kernel(apc_params p, TableArgs a, int n_tiles, int xcd_shift) {
-  __shared__ TileStage<M, true> s_stage;
-  redistribute_tile<M, kTileThreads, true, OUT>(p, a, n_tiles, xcd_shift, s_stage);
+  extern __shared__ __align__(16) unsigned char s_stage_bytes[];  // stage_lds_bytes<M, true>
+  redistribute_tile<M, kTileThreads, true, OUT>(p, a, n_tiles, xcd_shift,
+                                                *reinterpret_cast<TileStage<M, true> *>(s_stage_bytes));
 }
 
 // Every table of a pass in one launch: workgroups [0, tile_blocks) take the tiles of the
@@ -1754,7 +1878,7 @@ static int redistribute_tables_impl(const apc_params *params, const int64_t *ten
               tiles,        dup_entry_begin,   comm_out,   trans_out,   cost_out,
               nullptr,      nullptr,           nullptr,    nullptr,     nullptr, nullptr, nullptr, nullptr, nullptr,
               rows ? rows->edge_row_begin : nullptr, rows ? rows->dup_row_begin : nullptr,
-              rows ? rows->row_min : nullptr, rows ? rows->row_argmin : nullptr};
+              rows ? rows->row_min : nullptr, rows ? rows->row_argmin : nullptr, term_layout(*params)};
   const int nt = (int)n_tiles, xs = xcd_shift();
   hipStream_t s = (hipStream_t)stream;
   // Wavefronts per tile by the mean number of values a tile stores (n_entries counts the
@@ -1766,15 +1890,16 @@ static int redistribute_tables_impl(const apc_params *params, const int64_t *ten
   int threads = per_tile >= 1536 ? 256 : per_tile >= 512 ? 128 : 64;
   if (const char *env = getenv("APC_TILE_THREADS")) threads = atoi(env);  // tuning override
   const int om = out_mode(params->mesh_ndim, comm_out, trans_out, cost_out);
-#define APC_LAUNCH_T(KERNEL_, M_, OUT_)                                                                              \
-  if (threads >= 256) hipLaunchKernelGGL((KERNEL_<M_, 256, OUT_>), grid, dim3(256), 0, s, *params, a, nt, xs);       \
-  else if (threads >= 128) hipLaunchKernelGGL((KERNEL_<M_, 128, OUT_>), grid, dim3(128), 0, s, *params, a, nt, xs);  \
-  else hipLaunchKernelGGL((KERNEL_<M_, 64, OUT_>), grid, dim3(64), 0, s, *params, a, nt, xs)
+#define APC_LAUNCH_T(KERNEL_, M_, OUT_)                                                                               \
+  const size_t lds = rows ? stage_lds_bytes<M_, true>(a.lay) : stage_lds_bytes<M_, false>(a.lay);                      \
+  if (threads >= 256) hipLaunchKernelGGL((KERNEL_<M_, 256, OUT_>), grid, dim3(256), lds, s, *params, a, nt, xs);      \
+  else if (threads >= 128) hipLaunchKernelGGL((KERNEL_<M_, 128, OUT_>), grid, dim3(128), lds, s, *params, a, nt, xs); \
+  else hipLaunchKernelGGL((KERNEL_<M_, 64, OUT_>), grid, dim3(64), lds, s, *params, a, nt, xs)
 #define APC_LAUNCH_K(KERNEL_, M_)                                   \
   if (om == kOutAll) { APC_LAUNCH_T(KERNEL_, M_, kOutAll); }        \
   else if (om == kOutCost) { APC_LAUNCH_T(KERNEL_, M_, kOutCost); } \
   else { APC_LAUNCH_T(KERNEL_, M_, kOutAny); }
-#define APC_LAUNCH_ANY(KERNEL_, M_) APC_LAUNCH_T(KERNEL_, M_, kOutAny)
+#define APC_LAUNCH_ANY(KERNEL_, M_) { APC_LAUNCH_T(KERNEL_, M_, kOutAny); }
   if (rows) {
     switch (params->mesh_ndim) {
       case 1: APC_LAUNCH_ANY(redistribute_tiles_row_min_kernel, 1); break;
@@ -1840,7 +1965,7 @@ static int build_tables_impl(const apc_params *params, int64_t n_tensors, const 
   TableArgs a{nullptr, nullptr, spec_codes, spec_tensor, pt_values, nullptr, tiles, dup_entry_begin,
               comm_out, trans_out, cost_out, rank, itemsize, shape, stride, flops, rw_bytes, dtype, zero_cost, num_args,
               rows ? rows->edge_row_begin : nullptr, rows ? rows->dup_row_begin : nullptr,
-              rows ? rows->row_min : nullptr, rows ? rows->row_argmin : nullptr};
+              rows ? rows->row_min : nullptr, rows ? rows->row_argmin : nullptr, term_layout(*params)};
   const TensorTableArgs ta{n_tensors, rank, itemsize, shape, stride, tensor_bytes, tensor_contiguous};
   const SpecTableArgs sa{n_specs, spec_codes, spec_tensor, rank, itemsize, shape, stride, num_shards,
                          local_shape, local_stride, local_numel, local_bytes, shape_width};

@@ -58,8 +58,11 @@ def _run_and_compare(tb: CostTables, mesh, rescale, device):
     return d, want
 
 
-@pytest.mark.parametrize("mesh", [(64,), (32, 8), (8, 8, 8), (64, 4), (16, 8, 4), (6, 3), (5, 3, 2), (2, 3, 2, 2)])
+@pytest.mark.parametrize("mesh", [(64,), (32, 8), (8, 8, 8), (64, 4), (16, 8, 4), (6, 3), (5, 3, 2), (2, 3, 2, 2),
+                                  (2, 4, 2, 2), (4, 1, 2), (1,), (2048, 1024, 1024), (65536, 65536)])
 def test_tables_match_oracle_on_seeded_dags(gpu_device, mesh):
+    # (power-of-two meshes take the kernels' per-exponent term arrays: up to 32 exponents, which
+    # the mesh of 2^31 devices needs; the others, and the last one with 33, the per-state arrays)
     tb = stress_dag(seed=11, n_nodes=1500, mesh_sizes=mesh, frac_nonspec_nodes=0.02, frac_noncontiguous=0.2)
     d, want = _run_and_compare(tb, mesh, 2.2, gpu_device)
     # integer tables: bit-exact
@@ -72,6 +75,15 @@ def test_tables_match_oracle_on_seeded_dags(gpu_device, mesh):
                       c_oracle.spec_tables(enc, mesh)):
         assert _same_rows(got[key].cpu().numpy(), w), key
     assert got["local_shape"].shape[1] == tb.shape_width() <= 8
+
+
+@pytest.mark.parametrize("mesh", [(32, 8), (16, 8, 4), (2, 4, 2, 2)])
+def test_per_state_term_arrays_on_power_of_two_meshes(gpu_device, mesh, monkeypatch):
+    """The term arrays every mesh can use give the same bits on the meshes that normally take
+    the per-exponent arrays (the library reads APC_GENERAL_TERMS at every launch)."""
+    monkeypatch.setenv("APC_GENERAL_TERMS", "1")
+    tb = stress_dag(seed=12, n_nodes=800, mesh_sizes=mesh, frac_nonspec_nodes=0.02, frac_noncontiguous=0.2)
+    _run_and_compare(tb, mesh, 2.2, gpu_device)
 
 
 def test_python_oracle_agrees_on_a_small_case(gpu_device):
