@@ -434,17 +434,30 @@ __global__ __launch_bounds__(kBlock) void input_tables_kernel(apc_params p, Tens
 // ------------------------------------------------------------------------------------------
 
 // What is the same for every tile of a launch (see "Term arrays" and "Lookup words" below):
-// the layout of the term arrays and the part of the lookup words that does not depend on the
-// producer spec (by dim x 16 + producer class x 4 +
-// consumer class; the producer spec's state or exponent index is added, to both fields, when
-// a tile is staged).
+// the layout of the term arrays, the part of the lookup words that does not depend on the
+// producer spec (by dim x 16 + producer class x 4 + consumer class; the producer spec's state
+// or exponent index is added when a tile is staged) and, for the power-of-two layout, the
+// constants of every computed array.
+constexpr int kMaxTermArrays = 16;
+struct TermArrayConstants {  // value at exponent index j = max(lat + ldexp(B, j + shift), floor) x scale,
+  double hops;               // B = RN(RN(RN(RN(bytes x hops) / div1) x 1e6) / div2)
+  double div1, inv_div1;
+  double div2, inv_div2;
+  double lat;
+  double floor;
+  double scale;
+  int32_t shift;
+  int32_t pad_;
+};
 struct TermLayout {
   uint32_t pair[APC_MAX_MESH * 16];
-  int32_t exponents;          // 0: general layout; else E, the number of exponents
-  int32_t lg[APC_MAX_MESH];   // log2 of the mesh sizes (power-of-two layout)
-  int32_t lg_total;           // L
-  uint32_t rw1_base;          // first entry of the one-read+write array
-  uint32_t exponent_magic;    // ceil(65536 / E): t / E = (t * magic) >> 16 for t < 512
+  int32_t exponents;         // 0: general layout; else E, the number of exponents
+  int32_t lg[APC_MAX_MESH];  // log2 of the mesh sizes (power-of-two layout)
+  int32_t lg_total;          // L
+  int32_t state_stride;      // bytes between the entries of two consecutive states / exponents
+  uint32_t exponent_magic;   // ceil(65536 / E): t / E = (t * magic) >> 16 for t < 512
+  double inv_rescale;        // 1.0 / params.rescale
+  TermArrayConstants arrays[kMaxTermArrays - 2];  // of arrays 2 .. (power-of-two layout)
 };
 
 struct TableArgs {
@@ -517,14 +530,18 @@ __device__ __forceinline__ int placement_class(uint32_t code) {
   return k == 2 ? 2 + (dim_of(code) != 0 ? 1 : 0) : k;
 }
 
-// Term arrays staged per tile.  Two layouts, chosen per launch by the host (TermLayout):
+// Term arrays staged per tile, interleaved: the entry of (state s, array a) sits at byte
+// s x state_stride + 8 a, state_stride = 8 x (arrays + 1): an odd number of doubles, so that
+// lanes reading one array at different states hit different LDS banks.  Two layouts, chosen per
+// launch by the host (TermLayout):
 //
-// General (any mesh): one value per running-bytes state, arrays [0] zeros, [1] all-gather,
-// [2] reduce-scatter, [3] all-reduce, [4] all-to-all (= reduce-scatter shaped term x a2a_scale,
-// :22-32), [5] one read+write, [6] two read+writes (2.0 x [5]: the same bits as (double)2 * rw),
-// [7] +inf (banned transitions).  An entry's running index is the history of the earlier dims.
+// General (any mesh): one value per running-bytes state, 8 arrays: [0] zeros, [1] +inf (banned
+// transitions), [2] one read+write, [3] two read+writes (2.0 x [2]: the same bits as
+// (double)2 * rw), [4] all-gather, [5] reduce-scatter, [6] all-reduce, [7] all-to-all (=
+// reduce-scatter shaped term x a2a_scale, :22-32).  An entry's running index is the history of
+// the earlier dims.
 //
-// Power-of-two meshes (every mesh size a power of two, world size below 2^31): the running
+// Power-of-two meshes (every mesh size a power of two, world size at most 2^31): the running
 // bytes are the tensor's bytes times a power of two, bytes x 2^e with e in [-30 - L, -30],
 // L = log2(world size): dividing by the shards, x n after an all-gather and / n after a
 // reduce-scatter are exact.  Every term is then a rounding-free rescaling of ONE chain of
@@ -534,42 +551,47 @@ __device__ __forceinline__ int placement_class(uint32_t code) {
 //       B_d = RN(RN(RN(bytes x hops_d) / bw_d) x 1e6)      (two hops per step: B doubles)
 //   read+write at exponent e = max(ldexp(R, e + 31), launch floor),
 //       R = RN(RN(RN(bytes / hbm_bw) x 1e6) / rw_eff)
-// and one value per (array, exponent) replaces one per (array, state): arrays [0] zeros, [1]
-// +inf, then per mesh dim d [2 + 3d] one-hop ring (all-gather and reduce-scatter), [3 + 3d]
-// two-hop ring (all-reduce), [4 + 3d] all-to-all, then one read+write, two read+writes; E =
-// L + 1 values each.  An entry's running index is e + 30 + L.  (3-D mesh of 512 devices: 110
-// computed values, each a handful of operations, against 120 states x 6 terms of two
-// divisions each.)
+// and one value per (array, exponent) replaces one per (array, state); 16 arrays: [0] zeros,
+// [1] +inf, [2] one read+write, [3] two, then per mesh dim d [4 + 3d] one-hop ring (all-gather
+// and reduce-scatter), [5 + 3d] two-hop ring (all-reduce), [6 + 3d] all-to-all; E = L + 1
+// exponents.  An entry's running index is e + 30 + L.  Every computed array is one formula,
+// max(lat + ldexp(B, j + shift), floor) x scale with B from one chain bytes x hops / div1 x 1e6
+// / div2 (division by 1.0, x 1.0, 0.0 + x and max(x, -inf) return x), with constants the host
+// works out per launch (TermArrayConstants): a lane per array takes B, then a lane per (array,
+// exponent) the value.  (3-D mesh of 512 devices: 11 chains and 110 values of five operations,
+// against 120 states x 6 terms of two divisions each.)
 constexpr int kMaxExponents = 32;
+constexpr int kGeneralStride = 8 * (8 + 1), kPow2Stride = 8 * (kMaxTermArrays + 1);  // bytes per state / exponent
 template <int M>
 struct TermTable {
-  static constexpr int kGeneral = 8 * States<M>::kCount;
-  static constexpr int kPow2 = (4 + 3 * M) * kMaxExponents;
+  static constexpr int kGeneral = kGeneralStride / 8 * States<M>::kCount;
+  static constexpr int kPow2 = kPow2Stride / 8 * kMaxExponents;
   static constexpr int kEntries = kGeneral > kPow2 ? kGeneral : kPow2;
 };
+static_assert(4 + 3 * APC_MAX_MESH <= kMaxTermArrays, "arrays of the power-of-two layout");
 
 // Lookup words.  What a mesh dim adds to an entry depends on the producer spec (its class at
 // that dim and which dims it shards), on the consumer's class at that dim and on the running
 // index left by the earlier dims; everything but the running index is known per (producer
-// spec, dim, consumer class) when the tile is staged.  One 32-bit word per such triple holds,
-// as indices into the term arrays for running index 0 (the entry adds its running index):
-//   bits  0-11  the collective's term  (general: array of pair_action's term, state of the
-//               bytes the collective moves: after the update for an all-gather, before it else;
-//               the +inf array for a banned transition)
-//   bits 12-23  the read+write term    (zeros / one / two reshuffles, same state)
+// spec, dim, consumer class) when the tile is staged.  One 32-bit word per such triple, in
+// fields an instruction can take as a half or a byte of a register:
+//   bits  0-15  byte offset of the collective's term for running index 0 (general: array of
+//               pair_action's term, state of the bytes the collective moves: after the update
+//               for an all-gather, before it else; the +inf array for a banned transition)
+//   bits 16-23  signed: bytes from there to the read+write term of the same state (zeros / one
+//               / two reshuffles)
 //   bits 24-31  signed step of the running index after this dim (general: the dim's history
 //               bit; power-of-two meshes: + log2 n after an all-gather, - log2 n after a
 //               reduce-scatter)
-// Slot 4 of a (spec, dim) is the word of "same placement": zeros, no step; slot 5 is the index
-// of one read+write at the state BEFORE the dim, charged once to a non-contiguous tensor.
+// Slot 4 of a (spec, dim) is the word of "same placement": zeros, no step; slot 5 is the byte
+// offset of one read+write at the state BEFORE the dim, charged once to a non-contiguous tensor.
 constexpr int kWordsPerDim = 6;
-constexpr uint32_t kWordFieldMask = 0xFFFu, kWordBothFields = 0x1001u;
-static_assert(TermTable<APC_MAX_MESH>::kEntries <= 0xFFF + 1, "term indices fit their 12 bits");
+constexpr uint32_t kZerosArray = 0, kInfArray = 1, kRw1Array = 2;
+static_assert(TermTable<APC_MAX_MESH>::kEntries * 8 <= 0xFFFF + 1, "term offsets fit their 16 bits");
 
 static TermLayout term_layout(const apc_params &p) {
   TermLayout lay{};
   const int M = p.mesh_ndim;
-  const int ns = (1 << M) * ((1 << (M + 1)) - 1);
   bool pow2 = getenv("APC_GENERAL_TERMS") == nullptr;  // (testing override: the general layout on any mesh)
   int total = 0;
   for (int i = 0; i < M; ++i) {
@@ -587,29 +609,46 @@ static TermLayout term_layout(const apc_params &p) {
   const int E = pow2 ? total + 1 : 0;
   lay.exponents = E;
   lay.lg_total = pow2 ? total : 0;
-  lay.rw1_base = pow2 ? (uint32_t)((2 + 3 * M) * E) : (uint32_t)(5 * ns);
+  lay.state_stride = pow2 ? kPow2Stride : kGeneralStride;
   lay.exponent_magic = pow2 ? (uint32_t)((65536 + E - 1) / E) : 0u;
+  lay.inv_rescale = 1.0 / p.rescale;
   for (int i = 0; i < M; ++i)
     for (int c = 0; c < 4; ++c)
       for (int t = 0; t < 4; ++t) {
         const uint32_t e = pair_action(c, t);
         const uint32_t sel = e & 7u, copies = (e >> 3) & 3u;
         const bool ban = (e & 32u) != 0, upd = (e & 64u) != 0;
-        uint32_t term, rw;
+        const uint32_t rw_array = copies == 0u ? kZerosArray : kRw1Array + copies - 1u;
+        uint32_t term_array, state = 0;
         int step;
         if (!pow2) {
-          term = (ban ? 7u : sel) * (uint32_t)ns;
-          rw = (copies == 0u ? 0u : 5u + copies - 1u) * (uint32_t)ns;
+          term_array = ban ? kInfArray : sel == 0u ? kZerosArray : 3u + sel;
           step = upd ? (1 << i) : 0;
         } else {
-          const uint32_t shift = sel == 1u ? (uint32_t)lay.lg[i] : 0u;  // an all-gather is charged on the gathered bytes
-          const uint32_t array = ban ? 1u : sel == 0u ? 0u : sel <= 2u ? 2u + 3u * i : sel == 3u ? 3u + 3u * i : 4u + 3u * i;
-          term = array * (uint32_t)E + shift;
-          rw = (copies == 0u ? 0u : (uint32_t)(2 + 3 * M) + copies - 1u) * (uint32_t)E + shift;
+          if (sel == 1u) state = (uint32_t)lay.lg[i];  // an all-gather is charged on the gathered bytes
+          term_array = ban ? kInfArray : sel == 0u ? kZerosArray : sel <= 2u ? 4u + 3u * i : sel == 3u ? 5u + 3u * i : 6u + 3u * i;
           step = !upd ? 0 : sel == 1u ? lay.lg[i] : -lay.lg[i];
         }
-        lay.pair[i * 16 + c * 4 + t] = term | (rw << 12) | ((uint32_t)(step & 0xFF) << 24);
+        const int to_rw = ((int)rw_array - (int)term_array) * 8;
+        lay.pair[i * 16 + c * 4 + t] = (state * (uint32_t)lay.state_stride + term_array * 8u) | ((uint32_t)(to_rw & 0xFF) << 16) |
+                                       ((uint32_t)(step & 0xFF) << 24);
       }
+  if (pow2) {
+    const double ninf = -INFINITY;
+    // one read+write, two (compute_estimation.py:302-314 on bytes x 2^(e + 31))
+    lay.arrays[0] = {1.0, p.hbm_bw, p.inv_hbm_bw, p.rw_eff, p.inv_rw_eff, 0.0, p.launch_floor, 1.0, -total - 30 + 31, 0};
+    lay.arrays[1] = lay.arrays[0];
+    lay.arrays[1].scale = 2.0;
+    for (int d = 0; d < M; ++d) {  // torch _collective_utils.py:281-313 on bytes x 2^e
+      const double h = (double)(p.mesh_size[d] - 1);
+      const double lat1 = p.base_latency + h * p.lat[d];
+      const double lat2 = p.base_latency + (2.0 * h) * p.lat[d];
+      const int shift = -total - 30 - lay.lg[d];
+      lay.arrays[2 + 3 * d] = {h, p.bw[d], p.inv_bw[d], 1.0, 1.0, lat1, ninf, 1.0, shift, 0};
+      lay.arrays[3 + 3 * d] = {h, p.bw[d], p.inv_bw[d], 1.0, 1.0, lat2, ninf, 1.0, shift + 1, 0};
+      lay.arrays[4 + 3 * d] = {h, p.bw[d], p.inv_bw[d], 1.0, 1.0, lat1, ninf, p.a2a_scale, shift, 0};
+    }
+  }
   return lay;
 }
 
@@ -627,13 +666,34 @@ struct RowMinStage {
 };
 struct NoRowMinStage {};
 
+// A consumer spec of a tile: its placement codes; per mesh dim i, in byte i of `slots`, the
+// byte offset of its class's lookup word within a producer spec's words ((6 i + class) x 4;
+// byte 0 = 0xFF: not a DTensorSpec; on a 2-D mesh bit 24 = every dim is a Shard); the compute
+// cost / num_args of its strategy.  One 16-byte LDS read per entry.
+struct alignas(16) RowRecord {
+  uint32_t codes, slots;
+  double cpa;
+};
+constexpr uint32_t kRowNotASpec = 0xFFu, kRowAllShard = 1u << 24;
+
+// The part of TermArrayConstants a value needs after its array's chain.
+struct alignas(16) TermValueConstants {
+  double lat, floor, scale;
+  int32_t shift, pad_;
+};
+
 template <int M, bool RM>
 struct TileStage : std::conditional_t<RM, RowMinStage, NoRowMinStage> {
+  RowRecord row[APC_TILE_MAX_ROWS];  // consumer specs
   uint2 colh[APC_TILE_MAX_COLS];  // producer specs: x = codes, y = info
-  uint32_t words[APC_TILE_MAX_COLS * M * kWordsPerDim];  // lookup words per (producer spec, dim, consumer class)
+  uint32_t col_codes[APC_TILE_MAX_COLS];  // their codes again, packed (one LDS bank per lane)
+  // lookup words per (producer spec, dim, consumer class); an odd number of words per spec, so
+  // that the lanes of consecutive producer specs hit different banks
+  uint32_t words[APC_TILE_MAX_COLS * (M * kWordsPerDim + 1)];
   alignas(16) uint32_t pair_base[M * 16];  // TermLayout::pair of the launch
-  uint2 row[APC_TILE_MAX_ROWS];   // consumer specs: x = codes, y = info
-  double cpa[APC_TILE_MAX_ROWS];  // compute cost / num_args of the consumer strategies
+  // per staging wavefront (power-of-two layout): B and the value constants of every computed array
+  double chain[4][kMaxTermArrays];
+  TermValueConstants value_of[4][kMaxTermArrays];
   int64_t dup[APC_TILE_MAX_DUPS];  // first entries of the identical edges
   double gb_unsharded;  // bytes / 1024^3 of the tile's tensor
   int mixed[4];         // per staging wavefront: some spec is not a DTensorSpec on the tile's tensor (generic loop)
@@ -646,7 +706,7 @@ struct TileStage : std::conditional_t<RM, RowMinStage, NoRowMinStage> {
 // LDS bytes of a tile stage whose term arrays hold what the launch's layout needs.
 template <int M, bool RM>
 static size_t stage_lds_bytes(const TermLayout &lay) {
-  const size_t entries = lay.exponents ? (size_t)(4 + 3 * M) * lay.exponents : (size_t)TermTable<M>::kGeneral;
+  const size_t entries = lay.exponents ? (size_t)(kPow2Stride / 8) * lay.exponents : (size_t)TermTable<M>::kGeneral;
   return sizeof(TileStage<M, RM>) - sizeof(double) * TermTable<M>::kEntries + sizeof(double) * entries;
 }
 
@@ -699,6 +759,12 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   // A kernel argument indexed by the lane: one vector load, part of the round below.)
   uint32_t pair_word = 0;
   if (tid < 16 * M) pair_word = lay.pair[tid];
+  // power-of-two layout: the constants of array 2 + lane (whose chain this lane computes) and of
+  // the array of the first value this thread computes, also read by lane
+  constexpr int kComputed = 3 * M + 2;
+  const int lane = tid & 63, wave = tid >> 6;
+  TermArrayConstants chain_of{};
+  if (E != 0 && lane < kComputed) chain_of = lay.arrays[lane];
   // ---- the round of vector loads ------------------------------------------------------------
   // producer spec tid, consumer spec nthreads - 1 - tid (taken from the far end: with two
   // wavefronts one loads the producer specs while the other loads the consumer specs).
@@ -743,9 +809,9 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   if (terms_wanted) {
     if (!DERIVE) {
       const uint8_t *flag = a.tensor_contiguous + t0;
-      const uint32_t lane = (uint32_t)(reinterpret_cast<uintptr_t>(flag) & 3);
-      const uint32_t word = *reinterpret_cast<const uint32_t *>(flag - lane);
-      contiguous = (word >> (8 * lane)) & 0xFFu;
+      const uint32_t byte = (uint32_t)(reinterpret_cast<uintptr_t>(flag) & 3);
+      const uint32_t word = *reinterpret_cast<const uint32_t *>(flag - byte);
+      contiguous = (word >> (8 * byte)) & 0xFFu;
       tensor_nbytes = a.tensor_bytes[t0];
     } else {  // (t0 is wave-uniform: scalar loads and scalar arithmetic)
       bool ok;
@@ -755,33 +821,33 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   }
   // ---- term arrays (scalar operands only) ---------------------------------------------------
   if (terms_wanted && E != 0) {
-    // power-of-two mesh: one value per (array, exponent), arrays 2 .. 3 + 3M
+    // power-of-two mesh.  A lane per computed array takes the array's chain on the tensor's
+    // bytes (every wavefront its own copy: no barrier), then a lane per (array, exponent) the
+    // value.
     const double fbytes = (double)tensor_nbytes;
-    const int n_values = (3 * M + 2) * E;
-    for (int t = tid; t < n_values; t += nthreads) {
-      const int arr = (int)(((uint32_t)t * lay.exponent_magic) >> 16);
-      const int e = (t - arr * E) - lay.lg_total - 30;  // the running bytes are bytes x 2^e
-      double v;
-      if (arr < 3 * M) {  // a ring term (torch _collective_utils.py:281-313) of dim d
-        int d = 0;
-#pragma unroll
-        for (int i = 1; i < M; ++i) d += arr >= 3 * i ? 1 : 0;
-        const int typ = arr - 3 * d;  // 0 one hop per step, 1 two (all-reduce), 2 all-to-all
-        const double h = (double)(pick<M>(p.mesh_size, d) - 1);
-        const double b = div_by(fbytes * h, pick<M>(p.bw, d), pick<M>(p.inv_bw, d)) * 1e6;
-        const double hops = typ == 1 ? 2.0 * h : h;
-        const double latency = p.base_latency + hops * pick<M>(p.lat, d);
-        v = latency + __builtin_ldexp(b, e - pick<M>(lay.lg, d) + (typ == 1 ? 1 : 0));
-        if (typ == 2) v *= p.a2a_scale;  // collective_runtime_estimation.py:22-32
-      } else {  // read+write of the running bytes (compute_estimation.py:302-314)
-        const double r = div_by(div_by(fbytes, p.hbm_bw, p.inv_hbm_bw) * 1e6, p.rw_eff, p.inv_rw_eff);
-        const double tt = __builtin_ldexp(r, e + 31);
-        v = tt > p.launch_floor ? tt : p.launch_floor;
-        if (arr == 3 * M + 1) v = 2.0 * v;
-      }
-      st.terms[2 * E + t] = v;
+    if (lane < kComputed) {
+      st.chain[wave][lane] = div_by(div_by(fbytes * chain_of.hops, chain_of.div1, chain_of.inv_div1) * 1e6,
+                                    chain_of.div2, chain_of.inv_div2);
+      st.value_of[wave][lane] = TermValueConstants{chain_of.lat, chain_of.floor, chain_of.scale, chain_of.shift, 0};
     }
-    if (tid < 2 * E) st.terms[tid] = tid < E ? 0.0 : __builtin_inf();
+    __builtin_amdgcn_wave_barrier();  // (LDS operations of one wavefront complete in order)
+    // (The value constants go through LDS as well.  Read from the kernel arguments by a per-lane
+    // index inside the loop below, `lat + ldexp(..)` was compiled to `x + x` in the 4-D
+    // instantiations by hipcc 7.2: the placement-pair tests on 4-D power-of-two meshes show it.)
+    char *terms = reinterpret_cast<char *>(st.terms);
+    for (int t = tid; t < kComputed * E; t += nthreads) {
+      const int arr = (int)(((uint32_t)t * lay.exponent_magic) >> 16);  // t / E
+      const int j = t - arr * E;  // the running bytes are bytes x 2^(j - L - 30)
+      const TermValueConstants k = st.value_of[wave][arr];
+      double v = k.lat + __builtin_ldexp(st.chain[wave][arr], j + k.shift);
+      v = v > k.floor ? v : k.floor;
+      v = v * k.scale;
+      *reinterpret_cast<double *>(terms + j * kPow2Stride + (arr + 2) * 8) = v;
+    }
+    if (tid < 2 * E) {
+      const int j = tid < E ? tid : tid - E;
+      *reinterpret_cast<double *>(terms + j * kPow2Stride + (tid < E ? 0 : 8)) = tid < E ? 0.0 : __builtin_inf();
+    }
     if (tid == 0) st.gb_unsharded = fbytes / 1024 / 1024 / 1024;
   } else if (terms_wanted) {
     // every collective / read-write term the tile can need, once per running-bytes state, in
@@ -812,15 +878,16 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
       }
       double a2a = rs;
       a2a *= p.a2a_scale;
-      st.terms[k] = 0.0;
-      st.terms[NS + k] = ag;
-      st.terms[2 * NS + k] = rs;
-      st.terms[3 * NS + k] = ar;
-      st.terms[4 * NS + k] = a2a;
       const double rw = rw_time_r(gb * 2 * 1073741824.0, p);
-      st.terms[5 * NS + k] = rw;
-      st.terms[6 * NS + k] = 2.0 * rw;
-      st.terms[7 * NS + k] = __builtin_inf();
+      double *e = st.terms + k * (kGeneralStride / 8);
+      e[kZerosArray] = 0.0;
+      e[kInfArray] = __builtin_inf();
+      e[kRw1Array] = rw;
+      e[kRw1Array + 1] = 2.0 * rw;
+      e[4] = ag;
+      e[5] = rs;
+      e[6] = ar;
+      e[7] = a2a;
     }
     if (tid == 0) st.gb_unsharded = fbytes / 1024 / 1024 / 1024;
   } else if (tid == 0) {
@@ -845,6 +912,7 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
     for (int i = 0; i < M; ++i) mask |= (kind_of((col_codes >> (8 * i)) & 0xFF) == 2 ? 1u : 0u) << i;
     info |= mask << 4;
     st.colh[jc] = make_uint2(col_codes, info);
+    st.col_codes[jc] = col_codes;
     // power-of-two mesh: the producer spec's exponent index, L - log2(its shards)
     uint32_t j0 = (uint32_t)lay.lg_total;
 #pragma unroll
@@ -858,35 +926,37 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
       // the gathered bytes.  (Power-of-two layout: that shift is part of the word's base.)
       const uint32_t k = (uint32_t)States<M>::index(i, 0, 0) + (mask << i);
       const uint32_t k2 = (uint32_t)States<M>::index(i + 1, 0, 0) + (mask << (i + 1)) + (1u << i);
-      const uint32_t at = E != 0 ? j0 : k, at0 = E != 0 ? j0 : cls >= 2 ? k2 : k;
-      uint32_t *w = st.words + (jc * M + i) * kWordsPerDim;
-      w[0] = base.x + at0 * kWordBothFields;
-      w[1] = base.y + at * kWordBothFields;
-      w[2] = base.z + at * kWordBothFields;
-      w[3] = base.w + at * kWordBothFields;
-      w[4] = at * kWordBothFields;
-      w[5] = lay.rw1_base + at;
+      const uint32_t at = (E != 0 ? j0 : k) * (uint32_t)lay.state_stride;
+      const uint32_t at0 = (E != 0 ? j0 : cls >= 2 ? k2 : k) * (uint32_t)lay.state_stride;
+      uint32_t *w = st.words + jc * (M * kWordsPerDim + 1) + i * kWordsPerDim;
+      w[0] = base.x + at0;
+      w[1] = base.y + at;
+      w[2] = base.z + at;
+      w[3] = base.w + at;
+      w[4] = at;  // the zeros array, no read+write, no step
+      w[5] = at + kRw1Array * 8u;
     }
     if (col_tensor != t0 || col_tensor < 0) mixed = true;
   }
   if (has_row) {
-    // info: bit0 valid spec, bits 1 + 5i .. : class of mesh dim i, bit 30 every dim is a Shard
-    uint32_t info = row_tensor >= 0 ? 1u : 0u;
+    uint32_t slots = 0;
     bool all_shard = true;
 #pragma unroll
     for (int i = 0; i < M; ++i) {
       const uint32_t t = (row_codes >> (8 * i)) & 0xFF;
-      info |= (uint32_t)placement_class(t) << (1 + 5 * i);
+      slots |= (uint32_t)((kWordsPerDim * i + placement_class(t)) * 4) << (8 * i);
       all_shard &= kind_of(t) == 2;
     }
-    if (all_shard) info |= 1u << 30;
-    if (!(info & 1u)) mixed = true;  // a consumer spec that is not a DTensorSpec
-    st.row[jr] = make_uint2(row_codes, info);
+    if (M == 2 && all_shard) slots |= kRowAllShard;
+    if (row_tensor < 0) {  // a consumer spec that is not a DTensorSpec
+      slots |= kRowNotASpec;
+      mixed = true;
+    }
     if (DERIVE) {  // the value compute_costs_block writes for this strategy
       bool unsupported;
       row_cpa = compute_cost_of(p, row_zero != 0, row_rw, row_flops, row_dtype, unsupported) / (double)row_args;
     }
-    st.cpa[jr] = row_cpa;
+    st.row[jr] = RowRecord{row_codes, slots, row_cpa};
   }
   // one flag per wavefront, written unconditionally: nothing to clear beforehand
   const bool wave_mixed = __ballot(mixed) != 0;
@@ -897,29 +967,28 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
 // Straight-line code: all lookups of an entry are independent of its fp additions, so they
 // are issued together; no vector memory loads.
 template <int M, bool CONT, bool RESCALE, bool RM>
-__device__ __forceinline__ void uniform_entry(const apc_params &p, const TileStage<M, RM> &st, int r, int c,
-                                              double &comm_o, double &total_o, int &trans_o) {
-  const uint2 colv = st.colh[c];
-  const uint32_t src = colv.x, cinfo = colv.y;
-  const uint2 rowv = st.row[r];
-  const uint32_t tgt = rowv.x, tinfo = rowv.y;
-  const double cpa = st.cpa[r];
+__device__ __forceinline__ void uniform_entry(const apc_params &p, const TermLayout &lay, const TileStage<M, RM> &st,
+                                              int r, int c, double &comm_o, double &total_o, int &trans_o) {
+  const uint32_t src = st.col_codes[c];
+  const RowRecord row = st.row[r];
+  const uint32_t tgt = row.codes;
   const uint32_t x = src ^ tgt;
-  const uint32_t *words = st.words + c * (M * kWordsPerDim);
+  const char *words = reinterpret_cast<const char *>(st.words) + c * ((M * kWordsPerDim + 1) * 4);
   const char *terms = reinterpret_cast<const char *>(st.terms);
   // ---- integer part: which term at which running index each mesh dim adds -------------------
-  uint32_t at8 = 0;  // 8 x running index (history of the earlier dims / exponent steps), mod 2^32
+  uint32_t at = 0;  // byte offset of the running index (history of the earlier dims / exponent steps), mod 2^32
   uint32_t term_at[M], rw_at[M], nc_at[M];
   bool neq[M];
 #pragma unroll
   for (int i = 0; i < M; ++i) {
     neq[i] = ((x >> (8 * i)) & 0xFF) != 0;
-    const uint32_t cls = neq[i] ? (tinfo >> (1 + 5 * i)) & 7u : 4u;  // slot 4: same placement, nothing to add
-    const uint32_t w = words[i * kWordsPerDim + cls];
-    term_at[i] = ((w & kWordFieldMask) << 3) + at8;
-    rw_at[i] = (((w >> 12) & kWordFieldMask) << 3) + at8;
-    if (!CONT) nc_at[i] = (words[i * kWordsPerDim + 5] << 3) + at8;
-    at8 += (uint32_t)(((int32_t)w >> 24) << 3);
+    // (slot 4: same placement, nothing to add)
+    const uint32_t slot = neq[i] ? (row.slots >> (8 * i)) & 0xFFu : (uint32_t)((kWordsPerDim * i + 4) * 4);
+    const uint32_t w = *reinterpret_cast<const uint32_t *>(words + slot);
+    term_at[i] = (w & 0xFFFFu) + at;
+    rw_at[i] = term_at[i] + (uint32_t)(int32_t)(int8_t)(w >> 16);
+    if (!CONT) nc_at[i] = *reinterpret_cast<const uint32_t *>(words + (kWordsPerDim * i + 5) * 4) + at;
+    at += (uint32_t)(((int32_t)w >> 24) * lay.state_stride);
   }
   // ---- lookups ------------------------------------------------------------------------------
   double term[M], rw[M], nc[M];
@@ -932,7 +1001,7 @@ __device__ __forceinline__ void uniform_entry(const apc_params &p, const TileSta
   // ---- additions in the reference's order (0.0 + t == t for these non-negative terms) ------------
   double cost = 0.0;
   // a fully replicated producer returns before the non-contiguity term (:56-62)
-  bool cont = CONT || (cinfo & 2u);
+  bool cont = CONT || src == 0u;
 #pragma unroll
   for (int i = 0; i < M; ++i) {
     if (!CONT) {
@@ -945,12 +1014,13 @@ __device__ __forceinline__ void uniform_entry(const apc_params &p, const TileSta
   }
   double comm = cost;  // (a banned transition added the +inf term)
   const int trans = x != 0u ? p.transition_scale : 0;  // optimize_sharding.py:345-351
-  if (M == 2 && src == 0x4040u && (tinfo >> 30)) {  // (Partial, Partial) -> all Shard walks dim 1 first
+  if (M == 2 && src == 0x4040u && (row.slots & kRowAllShard)) {  // (Partial, Partial) -> all Shard walks dim 1 first
     comm = entry_cost<M>(src, tgt, st.gb_unsharded, CONT, p);
   }
-  if (RESCALE) comm = comm / p.rescale;  // :358-359
+  // :358-359; the quotient through the reciprocal is the division's (div_by), +inf stays +inf
+  if (RESCALE) comm = comm < __builtin_inf() ? div_by(comm, p.rescale, lay.inv_rescale) : comm;
   comm_o = comm;
-  total_o = comm + cpa + (double)trans;  // :368-372
+  total_o = comm + row.cpa + (double)trans;  // :368-372
   trans_o = trans;
 }
 
@@ -1100,7 +1170,7 @@ __device__ __forceinline__ void uniform_tile_entries_row_min(const apc_params &p
     double comm, total = 0.0;
     int trans;
     if (active) {
-      uniform_entry<M, CONT, RESCALE>(p, st, r, c, comm, total, trans);
+      uniform_entry<M, CONT, RESCALE>(p, a.lay, st, r, c, comm, total, trans);
       store_entry<OUT>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
                        trans);
     }
@@ -1136,7 +1206,7 @@ __device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const 
   for (int idx = first; idx < n; idx += nthreads) {
     double comm, total;
     int trans;
-    uniform_entry<M, CONT, RESCALE>(p, st, r, c, comm, total, trans);
+    uniform_entry<M, CONT, RESCALE>(p, a.lay, st, r, c, comm, total, trans);
     store_entry<OUT>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
                      trans);
     c += dc;
@@ -1167,8 +1237,9 @@ __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const 
       double comm;
       int trans = 0;
       const uint32_t src = st.colh[c].x, cinfo = st.colh[c].y;
-      const uint32_t tgt = st.row[r].x, tinfo = st.row[r].y;
-      if (no_producer || !(cinfo & tinfo & 1u)) {
+      const RowRecord row = st.row[r];
+      const uint32_t tgt = row.codes;
+      if (no_producer || !(cinfo & 1u) || (row.slots & 0xFFu) == kRowNotASpec) {
         comm = a.pt_values[v.pt_begin + local];
       } else {
         trans = (src != tgt) ? p.transition_scale : 0;
@@ -1185,7 +1256,7 @@ __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const 
       }
       if (v.flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;
       const int64_t o = v.entry_begin + local;
-      total = comm + st.cpa[r] + (double)trans;
+      total = comm + row.cpa + (double)trans;
       if (a.comm_out) a.comm_out[o] = comm;
       if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
       if (a.cost_out) a.cost_out[o] = total;

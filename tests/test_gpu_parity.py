@@ -432,15 +432,20 @@ def test_graph_replay_of_one_pass_matches_eager(gpu_device, launches):
             assert torch.equal(v, want[k]), (replay, k)
 
 
-@pytest.mark.parametrize("mesh", [(6,), (4, 8), (16, 2, 4), (2, 2, 2, 2)])
+@pytest.mark.parametrize("mesh", [(6,), (4, 8), (16, 2, 4), (2, 2, 2, 2), (5, 2, 3, 2)])
 @pytest.mark.parametrize("contiguous", [True, False])
-def test_every_placement_pair(gpu_device, mesh, contiguous):
+@pytest.mark.parametrize("threads", [None, 64, 128, 256])
+def test_every_placement_pair(gpu_device, mesh, contiguous, threads, monkeypatch):
     """Brute force over the placement algebra: every producer placement against every consumer
     placement (Replicate, Partial(sum), Partial(avg), Shard of each tensor dim, on every mesh
-    dim; a sample of 300 x 300 on the 4-D mesh), for a contiguous and a transposed tensor, with
-    and without the gradient rescale.  Kernel == C oracle bit for bit on all of them, == the
-    scalar Python oracle on the 1-D and 2-D meshes."""
+    dim; a sample of 300 x 300 on the 4-D meshes), for a contiguous and a transposed tensor, with
+    and without the gradient rescale, with the wavefronts per tile the library picks and with
+    each of its three instantiations forced.  Kernel == C oracle bit for bit on all of them, ==
+    the scalar Python oracle on the 1-D and 2-D meshes."""
     import itertools
+
+    if threads is not None:
+        monkeypatch.setenv("APC_TILE_THREADS", str(threads))
 
     M = len(mesh)
     options = [0, partial_code(0), partial_code(1), shard_code(0), shard_code(1), shard_code(2)]
