@@ -1954,11 +1954,12 @@ static int redistribute_tables_impl(const apc_params *params, const int64_t *ten
   hipStream_t s = (hipStream_t)stream;
   // Wavefronts per tile by the mean number of values a tile stores (n_entries counts the
   // copies written for de-duplicated edges too: work per tile either way): one below 512,
-  // two up to 1536, four above.  Measured on tables of 290 .. 1800 values per tile: more
-  // wavefronts drain a long tile sooner, fewer leave more tiles resident per compute unit.
+  // two up to 4096, four above.  Measured on tables of 290 .. 1800 values per tile: more
+  // wavefronts drain a long tile sooner, fewer leave more tiles resident per compute unit
+  // (1800 values per tile, Llama-3-70B: 169 / 154 / 179 us with one / two / four).
   const dim3 grid((unsigned)(((n_tiles + (1 << xs) - 1) >> xs) << xs));  // rounded up for xcd_chunked_unit
   const int64_t per_tile = n_entries / n_tiles;
-  int threads = per_tile >= 1536 ? 256 : per_tile >= 512 ? 128 : 64;
+  int threads = per_tile >= 4096 ? 256 : per_tile >= 512 ? 128 : 64;
   if (const char *env = getenv("APC_TILE_THREADS")) threads = atoi(env);  // tuning override
   const int om = out_mode(params->mesh_ndim, comm_out, trans_out, cost_out);
 #define APC_LAUNCH_T(KERNEL_, M_, OUT_)                                                                               \

@@ -52,8 +52,11 @@ EDGE_NO_PRODUCER = _native.EDGE_NO_PRODUCER
 # up to 64 x 64 entries is best served by one tile (its producer specs and cost terms are
 # staged once); a table that would then have too few tiles to fill the chip several times
 # over is cut finer (fewer copies per tiled edge first, then smaller tiles), as long as a
-# tile still stores a few thousand entries.
-AUTO_MIN_TILES = 32768
+# tile still stores a few thousand entries.  (Llama-3-70B on (8, 8, 8), 73 M entries: 126 us with
+# 11 732 tiles of 2048 entries and 4 copies; 134 us with 8 130 of 4096 / 4, 130 us with 16 192 of
+# 4096 / 2, 140 us with 23 376 of 2048 / 2, 155 us with 40 727 of 1024 / 2, 164 us with 2 085 of
+# 4096 / 16.)
+AUTO_MIN_TILES = 10000
 AUTO_MIN_STORED_PER_TILE = 2048
 AUTO_MIN_TILE_ENTRIES = 512
 # A table this small is bound by the latency of one workgroup, not by work: it keeps the largest
@@ -302,7 +305,11 @@ class CostTables:
                 if n == 0 or n >= AUTO_MIN_TILES or self.n_entries / n <= AUTO_MIN_STORED_PER_TILE \
                         or self.n_entries <= AUTO_SMALL_TABLE_ENTRIES:
                     break
-                if dedupe and mc > 2:
+                if dedupe and mc > 4:
+                    mc //= 2
+                elif te > 2048:
+                    te //= 2
+                elif dedupe and mc > 2:
                     mc //= 2
                 elif te > AUTO_MIN_TILE_ENTRIES:
                     te //= 2
