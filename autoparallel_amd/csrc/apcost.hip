@@ -926,8 +926,8 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
       // the gathered bytes.  (Power-of-two layout: that shift is part of the word's base.)
       const uint32_t k = (uint32_t)States<M>::index(i, 0, 0) + (mask << i);
       const uint32_t k2 = (uint32_t)States<M>::index(i + 1, 0, 0) + (mask << (i + 1)) + (1u << i);
-      const uint32_t at = (E != 0 ? j0 : k) * (uint32_t)lay.state_stride;
-      const uint32_t at0 = (E != 0 ? j0 : cls >= 2 ? k2 : k) * (uint32_t)lay.state_stride;
+      const uint32_t at = __umul24(E != 0 ? j0 : k, (uint32_t)lay.state_stride);
+      const uint32_t at0 = __umul24(E != 0 ? j0 : cls >= 2 ? k2 : k, (uint32_t)lay.state_stride);
       uint32_t *w = st.words + jc * (M * kWordsPerDim + 1) + i * kWordsPerDim;
       w[0] = base.x + at0;
       w[1] = base.y + at;
@@ -973,7 +973,7 @@ __device__ __forceinline__ void uniform_entry(const apc_params &p, const TermLay
   const RowRecord row = st.row[r];
   const uint32_t tgt = row.codes;
   const uint32_t x = src ^ tgt;
-  const char *words = reinterpret_cast<const char *>(st.words) + c * ((M * kWordsPerDim + 1) * 4);
+  const char *words = reinterpret_cast<const char *>(st.words) + __umul24((uint32_t)c, (M * kWordsPerDim + 1) * 4);
   const char *terms = reinterpret_cast<const char *>(st.terms);
   // ---- integer part: which term at which running index each mesh dim adds -------------------
   uint32_t at = 0;  // byte offset of the running index (history of the earlier dims / exponent steps), mod 2^32
@@ -988,7 +988,7 @@ __device__ __forceinline__ void uniform_entry(const apc_params &p, const TermLay
     term_at[i] = (w & 0xFFFFu) + at;
     rw_at[i] = term_at[i] + (uint32_t)(int32_t)(int8_t)(w >> 16);
     if (!CONT) nc_at[i] = *reinterpret_cast<const uint32_t *>(words + (kWordsPerDim * i + 5) * 4) + at;
-    at += (uint32_t)(((int32_t)w >> 24) * lay.state_stride);
+    at += (uint32_t)__mul24((int32_t)w >> 24, lay.state_stride);  // (24-bit multiplies issue at full rate)
   }
   // ---- lookups ------------------------------------------------------------------------------
   double term[M], rw[M], nc[M];
