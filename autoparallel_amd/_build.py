@@ -22,6 +22,9 @@ HIPCC_FLAGS = [
     "-ffp-contract=off",
     "-fPIC",
     "-shared",
+    # (the torch layer names the library by this soname: whichever build of it is in the process
+    # first, APCOST_LIBRARY's included, serves both bindings)
+    "-Wl,-soname,libapcost.so",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
@@ -39,6 +42,31 @@ def build_library(verbose: bool = False) -> str:
     if verbose and err.strip():
         print(err)
     return LIB_PATH
+
+
+TORCH_EXT_SOURCE = os.path.join(_PKG, "csrc", "apcost_torch.cpp")
+TORCH_EXT_PATH = os.path.join(_PKG, "libapcost_torch.so")
+
+
+def build_torch_extension(verbose: bool = False) -> str:
+    """The torch layer over the C ABI (operators of the ``apcost`` namespace), compiled against
+    the installed torch and linked to libapcost.so beside it.  Host code only."""
+    import torch
+    from torch.utils import cpp_extension
+
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    includes = [f"-I{d}" for d in cpp_extension.include_paths("cuda")]
+    cmd = [hipcc, "-x", "c++", "-std=c++17", "-O2", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", *includes, f"-I{INCLUDE}",
+           "-o", TORCH_EXT_PATH, TORCH_EXT_SOURCE, f"-L{_PKG}", "-lapcost", f"-L{torch_lib}", "-lc10", "-lc10_hip",
+           "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{proc.stderr}")
+    return TORCH_EXT_PATH
 
 
 ABI_CONSUMER_SOURCE = os.path.join(_ROOT, "tests", "abi_consumer.cpp")
@@ -63,4 +91,5 @@ def build_abi_consumer(verbose: bool = False) -> str:
 
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_torch_extension(verbose=True))
     print(build_abi_consumer(verbose=True))

@@ -9,7 +9,7 @@ from __future__ import annotations
 import ctypes
 import os
 
-from ._build import LIB_PATH
+from ._build import LIB_PATH, TORCH_EXT_PATH
 
 APC_MAX_RANK = 8
 APC_MAX_MESH = 4
@@ -105,7 +105,7 @@ def lib() -> ctypes.CDLL:
                 f"{LIB_PATH} is missing: the HIP library has not been built "
                 "(run `python -m autoparallel_amd._build`). There is no CPU fallback."
             )
-        l = ctypes.CDLL(LIB_PATH)
+        l = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
         for name in EXPORTS:
             if not hasattr(l, name):
                 raise RuntimeError(f"{LIB_PATH} does not export {name}")
@@ -115,6 +115,37 @@ def lib() -> ctypes.CDLL:
                 getattr(l, name).restype = ctypes.c_int
         _lib = l
     return _lib
+
+
+_ops = None
+
+
+def torch_ops():
+    """The ``apcost`` operator namespace of the torch layer (csrc/apcost_torch.cpp): operators
+    over torch tensors on the HIP device, bound to the same library.  Raises if it has not
+    been built."""
+    global _ops
+    if _ops is None:
+        import torch
+
+        lib()  # the C-ABI library first: the extension resolves its symbols against it
+        if not os.path.exists(TORCH_EXT_PATH):
+            raise RuntimeError(
+                f"{TORCH_EXT_PATH} is missing: the torch layer has not been built "
+                "(run `python -m autoparallel_amd._build`). There is no CPU fallback."
+            )
+        torch.ops.load_library(TORCH_EXT_PATH)
+        _ops = torch.ops.apcost
+        if int(_ops.abi_version()) != int(lib().apc_version()):
+            raise RuntimeError("the torch layer and the C-ABI library are different builds")
+    return _ops
+
+
+def params_tensor(c_params: "ApcParams"):
+    """``struct apc_params`` as the CPU uint8 tensor the operators take."""
+    import torch
+
+    return torch.frombuffer(bytearray(bytes(c_params)), dtype=torch.uint8)
 
 
 def check(rc: int, what: str) -> None:

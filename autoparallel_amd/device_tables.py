@@ -1,20 +1,19 @@
 """Device-resident cost tables: uploads a ``CostTables`` encoding to HBM once and
-runs the HIP kernels of libapcost.so over it through the C ABI.
+runs the HIP kernels of libapcost.so over it through the operators of the torch layer
+(``torch.ops.apcost``, csrc/apcost_torch.cpp: tensors in, tensors out, argument checks,
+current stream and device guard on the C++ side).
 
-torch is used for device memory and the current HIP stream only; every
-computation is a kernel of the library.  Without a HIP device (or without the
-built library) construction raises: there is no CPU path.
+torch is used for device memory and streams only; every computation is a kernel of the
+library.  Without a HIP device (or without the built libraries) construction raises: there
+is no CPU path.
 """
 
 from __future__ import annotations
-
-import ctypes
 
 import numpy as np
 import torch
 
 from . import _native
-from ._native import APC_MAX_RANK, vp
 from .cost_model import CostModelParams
 from .encoding import CostTables
 
@@ -61,13 +60,14 @@ class DeviceCostTables:
     def __init__(self, tables: CostTables, params: CostModelParams, device="cuda:0", validate=True):
         if not torch.cuda.is_available():
             raise RuntimeError("DeviceCostTables needs a HIP device; there is no CPU path")
-        self.lib = _native.lib()
+        self.ops = _native.torch_ops()
         self.tables = tables
         self.params = params
         self.device = torch.device(device)
         if validate:
             tables.validate(params)
         self.c_params = params.to_c()
+        self.p = _native.params_tensor(self.c_params)  # struct apc_params as the operators take it
         with torch.cuda.device(self.device):
             self.d = {k: _to_device(getattr(tables, k), self.device) for k in _UPLOAD}
         self.tensor_bytes = None
@@ -89,65 +89,48 @@ class DeviceCostTables:
                 self.d[k] = _to_device(getattr(self.tables, k), self.device)
 
     # ---- helpers -------------------------------------------------------------------------
+    def _empty(self, shape, dtype):
+        return torch.empty(shape, dtype=dtype, device=self.device)
+
+    # (for the entry points of the C ABI that have no operator: raw pointers and the stream handle)
+    @property
+    def lib(self):
+        return _native.lib()
+
     def _stream(self):
-        return vp(torch.cuda.current_stream(self.device).cuda_stream)
+        return _native.vp(torch.cuda.current_stream(self.device).cuda_stream)
 
     def _p(self, key):
         t = self.d[key] if isinstance(key, str) else key
-        return vp(t.data_ptr() if t is not None and t.numel() else 0)
+        return _native.vp(t.data_ptr() if t is not None and t.numel() else 0)
 
-    def _empty(self, shape, dtype):
-        return torch.empty(shape, dtype=dtype, device=self.device)
+    def _tensor_table(self):
+        d = self.d
+        return d["tensor_rank"], d["tensor_itemsize"], d["tensor_shape"], d["tensor_stride"]
+
+    def _strategy_table(self):
+        d = self.d
+        return d["strat_flops"], d["strat_rw_bytes"], d["strat_dtype"], d["strat_zero_cost"], d["strat_num_args"]
 
     # ---- integer tables ------------------------------------------------------------------
     @_guarded
     def run_tensor_tables(self):
-        n = self.tables.n_tensors
-        self.tensor_bytes = self._empty((n,), torch.int64)
-        self.tensor_contiguous = self._empty((n,), torch.uint8)
-        with torch.cuda.device(self.device):
-            rc = self.lib.apc_tensor_tables(
-                ctypes.c_int64(n), self._p("tensor_rank"), self._p("tensor_itemsize"), self._p("tensor_shape"),
-                self._p("tensor_stride"), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
-                self._stream())
-        _native.check(rc, "apc_tensor_tables")
+        self.tensor_bytes, self.tensor_contiguous = self.ops.tensor_tables(*self._tensor_table())
         return self.tensor_bytes, self.tensor_contiguous
 
     @_guarded
     def run_spec_tables(self):
-        n = self.tables.n_specs
         width = self.tables.shape_width()  # rows as wide as the largest rank needs, not APC_MAX_RANK
-        out = {
-            "num_shards": self._empty((n,), torch.int64),
-            "local_shape": self._empty((n, width), torch.int64),
-            "local_stride": self._empty((n, width), torch.int64),
-            "local_numel": self._empty((n,), torch.int64),
-            "local_bytes": self._empty((n,), torch.int64),
-        }
-        with torch.cuda.device(self.device):
-            rc = self.lib.apc_spec_tables(
-                ctypes.byref(self.c_params), ctypes.c_int64(n), self._p("spec_codes"), self._p("spec_tensor"),
-                self._p("tensor_rank"), self._p("tensor_itemsize"), self._p("tensor_shape"),
-                self._p("tensor_stride"), self._p(out["num_shards"]), self._p(out["local_shape"]),
-                self._p(out["local_stride"]), ctypes.c_int32(width), self._p(out["local_numel"]),
-                self._p(out["local_bytes"]), self._stream())
-        _native.check(rc, "apc_spec_tables")
+        names = ("num_shards", "local_shape", "local_stride", "local_numel", "local_bytes")
+        out = dict(zip(names, self.ops.shard_shapes_bytes(self.p, self.d["spec_codes"], self.d["spec_tensor"],
+                                                          *self._tensor_table(), width)))
         self.spec_out = out
         return out
 
     # ---- per-strategy compute cost ---------------------------------------------------------
     @_guarded
     def run_compute_costs(self):
-        n = self.tables.n_strategies
-        self.compute_cost = self._empty((n,), torch.float64)
-        self.compute_cost_per_arg = self._empty((n,), torch.float64)
-        err = torch.zeros((1,), dtype=torch.int32, device=self.device)
-        with torch.cuda.device(self.device):
-            rc = self.lib.apc_compute_costs(
-                ctypes.byref(self.c_params), ctypes.c_int64(n), self._p("strat_flops"), self._p("strat_rw_bytes"),
-                self._p("strat_dtype"), self._p("strat_zero_cost"), self._p("strat_num_args"),
-                self._p(self.compute_cost), self._p(self.compute_cost_per_arg), self._p(err), self._stream())
-        _native.check(rc, "apc_compute_costs")
+        self.compute_cost, self.compute_cost_per_arg, err = self.ops.compute_cost(self.p, *self._strategy_table())
         if int(err.item()) != 0:
             # compute_estimation.py:198-201
             raise ValueError(f"a strategy with non-zero flops uses a dtype not supported on {self.params.device_name}")
@@ -161,26 +144,25 @@ class DeviceCostTables:
         self.transition = self._empty((n,), torch.uint8) if transition else None
         self.cost = self._empty((n,), torch.float64) if cost else None
 
+    def _bind_redistribute_tables(self, comm, transition, cost, rows=None):
+        """A bound launch of the table kernel over the tables already built, writing the given
+        per-entry arrays (None: not written) and, with ``rows = (edge_row_begin, row_min,
+        row_argmin)``, the row minima."""
+        d = self.d
+        erb, rmin, rarg = rows if rows is not None else (None, None, None)
+        return self.ops.bind_redistribute_tables(
+            self.p, self.tensor_bytes, self.tensor_contiguous, d["spec_codes"], d["spec_tensor"], d["pt_values"],
+            self.compute_cost_per_arg, d["tile_records"], d["dup_entry_begin"], self.tables.n_entries, comm, transition, cost,
+            erb, d["dup_row_begin"] if rows is not None else None, rmin, rarg)
+
     @_guarded
     def launch_redistribute_tables(self, row_min=False):
-        """One enqueue of the table kernel over pre-allocated outputs (no allocation,
-        no synchronisation).  ``row_min``: the launch also writes ``row_min`` / ``row_argmin``
-        (allocated by ``run_redistribute_tables``)."""
-        args = (ctypes.byref(self.c_params), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
-                self._p("spec_codes"), self._p("spec_tensor"), self._p("pt_values"),
-                self._p(self.compute_cost_per_arg), ctypes.c_int64(self.tables.n_tiles), self._p("tile_records"),
-                self._p("dup_entry_begin"), ctypes.c_int64(self.tables.n_entries), self._p(self.comm),
-                self._p(self.transition), self._p(self.cost))
-        with torch.cuda.device(self.device):
-            if row_min:
-                edge_row_begin = _to_device(self.tables.edge_row_begin(), self.device)
-                rows = _native.ApcRowMinima(self._p(edge_row_begin), self._p("dup_row_begin"), self._p(self.row_min),
-                                            self._p(self.row_argmin))
-                rc = self.lib.apc_redistribute_tables_row_min(*args, ctypes.byref(rows), self._stream())
-                self._rows_keepalive = (edge_row_begin, rows)  # until the stream has run the launch
-            else:
-                rc = self.lib.apc_redistribute_tables(*args, self._stream())
-        _native.check(rc, "apc_redistribute_tables")
+        """One enqueue of the table kernel over pre-allocated outputs.  ``row_min``: the launch
+        also writes ``row_min`` / ``row_argmin`` (allocated by ``run_redistribute_tables``)."""
+        rows = None
+        if row_min:
+            rows = (_to_device(self.tables.edge_row_begin(), self.device), self.row_min, self.row_argmin)
+        self._bind_redistribute_tables(self.comm, self.transition, self.cost, rows).run()
 
     @_guarded
     def run_redistribute_tables(self, comm=True, transition=True, cost=True, row_min=None):
@@ -298,81 +280,64 @@ class DeviceCostTables:
         spec = self._alloc_input_tables(spec_table)
         self.alloc_outputs("comm" in outputs, "transition" in outputs, "cost" in outputs)
         self.row_min = self.row_argmin = None
-        lib, P, cp = self.lib, self._p, ctypes.byref(self.c_params)
-        stream = self._stream()
-        tb = self.tables
+        ops, d, tb = self.ops, self.d, self.tables
         err = torch.zeros((1,), dtype=torch.int32, device=self.device)
         self._step_keepalive = [err, spec]
-        null = vp(0)
-        a_tensor = (ctypes.c_int64(tb.n_tensors), P("tensor_rank"), P("tensor_itemsize"), P("tensor_shape"),
-                    P("tensor_stride"), P(self.tensor_bytes), P(self.tensor_contiguous), stream)
-        spec_outs = (P(spec["num_shards"]), P(spec["local_shape"]), P(spec["local_stride"]),
-                     ctypes.c_int32(spec["local_shape"].shape[1]), P(spec["local_numel"]), P(spec["local_bytes"])) \
-            if spec_table else (null, null, null, ctypes.c_int32(tb.shape_width()), null, null)
-        a_spec = (cp, ctypes.c_int64(tb.n_specs), P("spec_codes"), P("spec_tensor"), P("tensor_rank"),
-                  P("tensor_itemsize"), P("tensor_shape"), P("tensor_stride")) + spec_outs + (stream,)
-        a_compute = (cp, ctypes.c_int64(tb.n_strategies), P("strat_flops"), P("strat_rw_bytes"), P("strat_dtype"),
-                     P("strat_zero_cost"), P("strat_num_args"), P(self.compute_cost), P(self.compute_cost_per_arg),
-                     P(err), stream)
-        a_tables = (cp, P(self.tensor_bytes), P(self.tensor_contiguous), P("spec_codes"), P("spec_tensor"),
-                    P("pt_values"), P(self.compute_cost_per_arg), ctypes.c_int64(tb.n_tiles), P("tile_records"),
-                    P("dup_entry_begin"), ctypes.c_int64(tb.n_entries), P(self.comm), P(self.transition), P(self.cost), stream)
+        spec_outputs = [spec[k] for k in ("num_shards", "local_shape", "local_stride", "local_numel", "local_bytes")] \
+            if spec_table else []
+        width = spec["local_shape"].shape[1] if spec_table else tb.shape_width()
+        input_tables = (self.p, *self._tensor_table(), self.tensor_bytes, self.tensor_contiguous, d["spec_codes"],
+                        d["spec_tensor"], spec_outputs, width, *self._strategy_table(), self.compute_cost,
+                        self.compute_cost_per_arg, err)
 
-        def bind(fn, args, what):
-            head = args[:-1]
+        def bind(bound):
+            # a launcher only looks up the current stream (or takes the given one) and enqueues
+            run, run_on = bound.run, bound.run_on
 
             def launch(on_stream=None):
-                rc = fn(*args) if on_stream is None else fn(*head, on_stream)
-                if rc != 0:
-                    _native.check(rc, what)
+                if on_stream is None:
+                    run()
+                else:
+                    run_on(int(on_stream.cuda_stream))
+            launch.bound = bound
             return launch
 
-        rows_arg = ()
+        rows = None
         if row_min:
             self.row_min = self._empty((tb.n_rows,), torch.float64)
             self.row_argmin = self._empty((tb.n_rows,), torch.int32)
         if row_min_in_tiles:
-            edge_row_begin = _to_device(tb.edge_row_begin(), self.device)
-            self._step_keepalive.append(edge_row_begin)
-            rows = _native.ApcRowMinima(P(edge_row_begin), P("dup_row_begin"), P(self.row_min), P(self.row_argmin))
-            self._step_keepalive.append(rows)
-            rows_arg = (ctypes.byref(rows),)
-        table_fn = (lib.apc_redistribute_tables_row_min, "apc_redistribute_tables_row_min") if row_min_in_tiles \
-            else (lib.apc_redistribute_tables, "apc_redistribute_tables")
-        all_fn = (lib.apc_build_tables_row_min, "apc_build_tables_row_min") if row_min_in_tiles \
-            else (lib.apc_build_tables, "apc_build_tables")
-        a_tables = a_tables[:-1] + rows_arg + (stream,)
+            rows = (_to_device(tb.edge_row_begin(), self.device), self.row_min, self.row_argmin)
+        erb, rmin, rarg = rows if rows is not None else (None, None, None)
+        dup_rows = d["dup_row_begin"] if rows is not None else None
         if one_launch:
-            a_all = (cp,) + a_tensor[:-1] + (a_spec[1], a_spec[2], a_spec[3]) + a_spec[8:-1] + a_compute[1:-1] + \
-                (a_tables[5],) + a_tables[7:]
-            step = {"build_tables": bind(all_fn[0], a_all, all_fn[1])}
+            step = {"build_tables": bind(ops.bind_cost_tables(
+                *input_tables, d["pt_values"], d["tile_records"], d["dup_entry_begin"], tb.n_entries, self.comm,
+                self.transition, self.cost, erb, dup_rows, rmin, rarg))}
         elif fused_inputs:
-            a_inputs = (cp,) + a_tensor[:-1] + (a_spec[1], a_spec[2], a_spec[3]) + a_spec[8:-1] + a_compute[1:]
-            step = {"input_tables": bind(lib.apc_input_tables, a_inputs, "apc_input_tables")}
+            step = {"input_tables": bind(ops.bind_input_tables(*input_tables))}
         else:
             step = {
-                "tensor_tables": bind(lib.apc_tensor_tables, a_tensor, "apc_tensor_tables"),
-                "spec_tables": bind(lib.apc_spec_tables, a_spec, "apc_spec_tables"),
-                "compute_costs": bind(lib.apc_compute_costs, a_compute, "apc_compute_costs"),
+                "tensor_tables": bind(ops.bind_tensor_tables(*self._tensor_table(), self.tensor_bytes,
+                                                             self.tensor_contiguous)),
+                "spec_tables": bind(ops.bind_spec_tables(self.p, d["spec_codes"], d["spec_tensor"],
+                                                         *self._tensor_table(), spec_outputs, width)),
+                "compute_costs": bind(ops.bind_compute_costs(self.p, *self._strategy_table(), self.compute_cost,
+                                                             self.compute_cost_per_arg, err)),
             }
         if not one_launch:
-            step["redistribute_tables"] = bind(table_fn[0], a_tables, table_fn[1])
+            step["redistribute_tables"] = bind(self._bind_redistribute_tables(self.comm, self.transition, self.cost, rows))
         if row_min and not row_min_in_tiles:
             row_ptr = torch.from_numpy(tb.row_ptr()).to(self.device)
-            n_seg = row_ptr.numel() - 1
-            assert n_seg == self.row_min.numel()
-            self._step_keepalive.append(row_ptr)
+            assert row_ptr.numel() - 1 == self.row_min.numel()
             copies = self._row_copies()
             if copies is not None:  # identical edges: every distinct row is read once, its minimum stored to all
                 selected, copy_ptr, copy_rows, n_read = copies
-                self._step_keepalive.append(copies)
-                a_min = (P(self.cost), P(row_ptr), ctypes.c_int64(selected.numel()), P(selected), P(copy_ptr),
-                         P(copy_rows), ctypes.c_int64(n_read), P(self.row_min), P(self.row_argmin), stream)
-                step["segmented_min"] = bind(lib.apc_segmented_min_copies, a_min, "apc_segmented_min_copies")
+                step["segmented_min"] = bind(ops.bind_segmented_min(self.cost, row_ptr, selected, copy_ptr, copy_rows,
+                                                                    n_read, self.row_min, self.row_argmin))
             else:
-                a_min = (P(self.cost), P(row_ptr), ctypes.c_int64(n_seg), ctypes.c_int64(tb.n_entries), P(self.row_min),
-                         P(self.row_argmin), stream)
-                step["segmented_min"] = bind(lib.apc_segmented_min, a_min, "apc_segmented_min")
+                step["segmented_min"] = bind(ops.bind_segmented_min(self.cost, row_ptr, None, None, None, 0,
+                                                                    self.row_min, self.row_argmin))
         self._step_error_flag = err
         return step
 
@@ -413,14 +378,7 @@ class DeviceCostTables:
             raise RuntimeError("no table pass has run yet")
         n = self.tables.n_entries
         out = self._empty((n,), torch.uint8 if name == "transition" else torch.float64)
-        ptrs = {k: self._p(out) if k == name else vp(0) for k in have}
-        with torch.cuda.device(self.device):
-            rc = self.lib.apc_redistribute_tables(
-                ctypes.byref(self.c_params), self._p(self.tensor_bytes), self._p(self.tensor_contiguous),
-                self._p("spec_codes"), self._p("spec_tensor"), self._p("pt_values"), self._p(self.compute_cost_per_arg),
-                ctypes.c_int64(self.tables.n_tiles), self._p("tile_records"), self._p("dup_entry_begin"),
-                ctypes.c_int64(n), ptrs["comm"], ptrs["transition"], ptrs["cost"], self._stream())
-        _native.check(rc, "apc_redistribute_tables")
+        self._bind_redistribute_tables(*(out if k == name else None for k in have)).run()
         setattr(self, name, out)
         return out
 
@@ -437,16 +395,7 @@ class DeviceCostTables:
         if n_groups and (int(group_var_begin[0]) != 0 or int(group_var_begin[-1]) != n_vars
                          or int(group_member_begin[-1]) != len(member_entry_begin)):
             raise ValueError("group pointers do not span the variables / members")
-        cost = self.fetch("cost")
-        obj = self._empty((n_vars,), torch.float64)
-        forced = self._empty((n_vars,), torch.uint8)
-        with torch.cuda.device(self.device):
-            rc = self.lib.apc_cost_objective(ctypes.c_int64(n_vars), ctypes.c_int64(n_groups), self._p(gv), self._p(gm),
-                                             self._p(me), self._p(cost), ctypes.c_double(self.params.inf_replacement_cost),
-                                             self._p(obj), self._p(forced), self._stream())
-        _native.check(rc, "apc_cost_objective")
-        self._objective_keepalive = (gv, gm, me)
-        return obj, forced
+        return self.ops.cost_objective(int(n_vars), gv, gm, me, self.fetch("cost"), float(self.params.inf_replacement_cost))
 
     @_guarded
     def capture_step_graph(self, step):
@@ -466,19 +415,19 @@ class DeviceCostTables:
             for b in branches:
                 b.wait_stream(main)
             if "build_tables" in step:
-                step["build_tables"](ctypes.c_void_p(main.cuda_stream))
+                step["build_tables"](main)
             elif "input_tables" in step:
-                step["input_tables"](ctypes.c_void_p(main.cuda_stream))
+                step["input_tables"](main)
             else:
-                step["spec_tables"](ctypes.c_void_p(main.cuda_stream))
-                step["tensor_tables"](ctypes.c_void_p(branches[0].cuda_stream))
-                step["compute_costs"](ctypes.c_void_p(branches[1].cuda_stream))
+                step["spec_tables"](main)
+                step["tensor_tables"](branches[0])
+                step["compute_costs"](branches[1])
             for b in branches:
                 main.wait_stream(b)
             if "redistribute_tables" in step:
-                step["redistribute_tables"](ctypes.c_void_p(main.cuda_stream))
+                step["redistribute_tables"](main)
             if "segmented_min" in step:
-                step["segmented_min"](ctypes.c_void_p(main.cuda_stream))
+                step["segmented_min"](main)
         self._step_keepalive.append(branches)
         return graph
 
@@ -515,11 +464,7 @@ class DeviceCostTables:
         n_rows = row_ptr.numel() - 1
         mins = self._empty((n_rows,), torch.float64)
         args = self._empty((n_rows,), torch.int32)
-        with torch.cuda.device(self.device):
-            rc = self.lib.apc_segmented_min_copies(self._p(self.fetch("cost")), self._p(row_ptr),
-                                                   ctypes.c_int64(selected.numel()), self._p(selected), self._p(copy_ptr), self._p(copy_rows),
-                                                   ctypes.c_int64(n_read), self._p(mins), self._p(args), self._stream())
-        _native.check(rc, "apc_segmented_min_copies")
+        self.ops.bind_segmented_min(self.fetch("cost"), row_ptr, selected, copy_ptr, copy_rows, n_read, mins, args).run()
         return mins, args  # (the index arrays stay cached with the tables)
 
     @_guarded
@@ -538,14 +483,7 @@ class DeviceCostTables:
             ok = bool((seg_ptr[1:] >= seg_ptr[:-1]).all()) and int(seg_ptr[0]) >= 0 and int(seg_ptr[-1]) <= values.numel()
             if not ok:
                 raise ValueError("seg_ptr must be non-decreasing and end within the value array")
-        mins = self._empty((n_seg,), torch.float64)
-        args = self._empty((n_seg,), torch.int32)
-        with torch.cuda.device(self.device):
-            rc = self.lib.apc_segmented_min(self._p(values), self._p(seg_ptr), ctypes.c_int64(n_seg),
-                                            ctypes.c_int64(values.numel()), self._p(mins), self._p(args),
-                                            self._stream())
-        _native.check(rc, "apc_segmented_min")
-        return mins, args
+        return self.ops.segmented_min(values, seg_ptr)
 
     # ---- dual ascent over the planning program's labelling form ---------------------------------
     @_guarded
@@ -561,16 +499,10 @@ class DeviceCostTables:
         d = cached[1]
         th = torch.from_numpy(np.ascontiguousarray(theta, np.float64)).to(self.device)
         un = torch.from_numpy(np.ascontiguousarray(unary, np.float64)).to(self.device)
-        color_begin = np.ascontiguousarray(graph.color_begin, np.int64)
+        color_begin = torch.from_numpy(np.ascontiguousarray(graph.color_begin, np.int64))
         max_labels = int(np.diff(graph.label_begin).max()) if graph.n_classes else 0
-        with torch.cuda.device(self.device):
-            rc = self.lib.apc_diffusion_sweeps(
-                ctypes.c_int32(int(n_sweeps)), ctypes.c_int32(len(color_begin) - 1),
-                color_begin.ctypes.data_as(ctypes.c_void_p), self._p(d["color_nodes"]), ctypes.c_int64(graph.n_classes),
-                self._p(d["label_begin"]), self._p(d["inc_begin"]), self._p(d["inc_edge"]), self._p(d["inc_side"]),
-                self._p(d["edge_begin"]), self._p(d["edge_i"]), self._p(d["edge_j"]), ctypes.c_int32(max_labels),
-                self._p(th), self._p(un), self._stream())
-        _native.check(rc, "apc_diffusion_sweeps")
+        self.ops.diffusion_sweeps_(int(n_sweeps), color_begin, d["color_nodes"], d["label_begin"], d["inc_begin"],
+                                   d["inc_edge"], d["inc_side"], d["edge_begin"], d["edge_i"], d["edge_j"], max_labels, th, un)
         return th.cpu().numpy(), un.cpu().numpy()
 
     def strategy_bounds(self, row_min: torch.Tensor) -> torch.Tensor:
@@ -585,14 +517,8 @@ class DeviceCostTables:
             self._bound_index = {k: _to_device(v, self.device) for k, v in t.strategy_bound_index().items()}
             self._bound_index["node_strat_begin"] = _to_device(np.ascontiguousarray(t.node_strat_begin, np.int64), self.device)
         ix = self._bound_index
-        bound = self._empty((t.n_strategies,), torch.float64)
-        with torch.cuda.device(self.device):
-            rc = self.lib.apc_strategy_bounds(ctypes.c_int64(t.n_strategies), self._p(ix["strat_node"]),
-                                              self._p(ix["node_strat_begin"]), self._p(ix["node_edge_begin"]),
-                                              self._p(ix["edges_by_node"]), self._p(ix["edge_row_begin"]),
-                                              self._p(row_min), self._p(bound), self._stream())
-        _native.check(rc, "apc_strategy_bounds")
-        return bound
+        return self.ops.strategy_bounds(ix["strat_node"], ix["node_strat_begin"], ix["node_edge_begin"], ix["edges_by_node"],
+                                        ix["edge_row_begin"], row_min)
 
     def greedy_strategies(self, row_min: torch.Tensor):
         """-> (bound per strategy, min per node, argmin per node): the cheapest strategy of every

@@ -1,0 +1,133 @@
+"""The torch layer over the C ABI (``torch.ops.apcost``, csrc/apcost_torch.cpp): it loads, exports
+its operators with named schemas, rejects malformed arguments with RuntimeError before anything
+is launched, and its operators give the oracle's bits on the HIP device."""
+
+import numpy as np
+import pytest
+import torch
+
+from autoparallel_amd import CostModelParams, _native
+from autoparallel_amd.device_tables import DeviceCostTables, _to_device
+from autoparallel_amd.synthetic import stress_dag
+from oracle import c_oracle
+from oracle import cost_oracle as po
+
+OPERATORS = (
+    "abi_version", "tensor_tables", "shard_shapes_bytes", "compute_cost", "segmented_min", "cost_objective",
+    "redistribute_cost_tables", "strategy_bounds", "diffusion_sweeps_", "bind_tensor_tables", "bind_spec_tables",
+    "bind_compute_costs", "bind_segmented_min", "bind_redistribute_tables", "bind_input_tables", "bind_cost_tables",
+)
+
+
+def test_the_extension_loads_and_exports_its_operators():
+    ops = _native.torch_ops()
+    assert int(ops.abi_version()) == int(_native.lib().apc_version())
+    for name in OPERATORS:
+        schema = str(getattr(ops, name).default._schema)
+        assert schema.startswith(f"apcost::{name}("), schema
+        assert "_0" not in schema, f"{name}: arguments are named"
+    assert "Tensor(a!) theta" in str(ops.diffusion_sweeps_.default._schema)
+    assert "BoundLaunch" in str(ops.bind_cost_tables.default._schema)
+
+
+def test_arguments_are_checked_before_any_launch():
+    ops = _native.torch_ops()
+    f64, i64 = torch.zeros(3, dtype=torch.float64), torch.zeros(2, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="must be on the HIP device"):
+        ops.segmented_min(f64, i64)
+    params = _native.params_tensor(CostModelParams.from_mesh((4, 2)).to_c())
+    assert params.dtype == torch.uint8 and params.numel() == 296  # sizeof(struct apc_params)
+    i32 = torch.zeros(1, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="struct apc_params"):
+        ops.shard_shapes_bytes(params[:-8], i32, i32, i32, i32, i64, i64, 8)
+    with pytest.raises(RuntimeError, match="struct apc_params"):
+        ops.compute_cost(params.to(torch.float32), i64, i64, i32, i32, i32)
+    with pytest.raises(RuntimeError, match="must be on the HIP device"):
+        ops.compute_cost(params, i64, i64, i32, i32, i32)
+
+
+@pytest.fixture(scope="module")
+def small_table(gpu_device):
+    mesh = (4, 4, 2)
+    tb = stress_dag(seed=5, n_nodes=400, mesh_sizes=mesh, frac_nonspec_nodes=0.02, frac_noncontiguous=0.2)
+    params = CostModelParams.from_mesh(mesh, rescale=2.2)
+    dev = {k: _to_device(getattr(tb, k), gpu_device) for k in (
+        "tensor_rank", "tensor_itemsize", "tensor_shape", "tensor_stride", "spec_codes", "spec_tensor", "strat_flops",
+        "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "strat_num_args", "pt_values", "tile_records", "dup_entry_begin")}
+    want = c_oracle.build_tables(tb.as_dict(), po.make_params(mesh, rescale=2.2))
+    return mesh, tb, _native.params_tensor(params.to_c()), dev, want
+
+
+@pytest.mark.gpu
+def test_operators_match_the_oracle(small_table):
+    """The operators named by the extension's contract, called directly: shard shapes and byte
+    counts, compute costs, the cost matrices and the row minima."""
+    mesh, tb, p, d, want = small_table
+    ops = _native.torch_ops()
+    table = (d["tensor_rank"], d["tensor_itemsize"], d["tensor_shape"], d["tensor_stride"])
+    nbytes, contiguous = ops.tensor_tables(*table)
+    wb, wc = c_oracle.tensor_tables(tb.as_dict())
+    assert np.array_equal(nbytes.cpu().numpy(), wb) and np.array_equal(contiguous.cpu().numpy(), wc)
+    got = ops.shard_shapes_bytes(p, d["spec_codes"], d["spec_tensor"], *table, 8)
+    for g, w in zip(got, c_oracle.spec_tables(tb.as_dict(), mesh)):
+        assert np.array_equal(g.cpu().numpy().reshape(np.asarray(w).shape), w)
+    compute, per_arg, err = ops.compute_cost(p, d["strat_flops"], d["strat_rw_bytes"], d["strat_dtype"], d["strat_zero_cost"],
+                                             d["strat_num_args"])
+    assert int(err.item()) == 0
+    want_compute, want_per_arg = c_oracle.compute_costs(tb.as_dict(), po.make_params(mesh, rescale=2.2))[:2]
+    assert np.array_equal(compute.cpu().numpy(), want_compute) and np.array_equal(per_arg.cpu().numpy(), want_per_arg)
+    comm, transition, cost = ops.redistribute_cost_tables(p, nbytes, contiguous, d["spec_codes"], d["spec_tensor"], d["pt_values"],
+                                                          per_arg, d["tile_records"], d["dup_entry_begin"], tb.n_entries)
+    assert np.array_equal(comm.cpu().numpy(), want["comm"])
+    assert np.array_equal(transition.cpu().numpy(), want["transition"])
+    assert np.array_equal(cost.cpu().numpy(), want["cost"])
+    mins, args = ops.segmented_min(cost, torch.from_numpy(tb.row_ptr()).to(cost.device))
+    wm, wa = c_oracle.segmented_min(want["cost"], tb.row_ptr())
+    assert np.array_equal(mins.cpu().numpy(), wm) and np.array_equal(args.cpu().numpy(), wa)
+
+
+@pytest.mark.gpu
+def test_lengths_that_disagree_are_rejected(small_table):
+    mesh, tb, p, d, want = small_table
+    ops = _native.torch_ops()
+    with pytest.raises(RuntimeError, match="tensor_itemsize has"):
+        ops.tensor_tables(d["tensor_rank"], d["tensor_itemsize"][:-1], d["tensor_shape"], d["tensor_stride"])
+    with pytest.raises(RuntimeError, match="one row per strategy"):
+        ops.compute_cost(p, d["strat_flops"], d["strat_rw_bytes"][:-1], d["strat_dtype"], d["strat_zero_cost"], d["strat_num_args"])
+    with pytest.raises(RuntimeError, match="must be Long"):
+        ops.segmented_min(torch.zeros(4, dtype=torch.float64, device=d["pt_values"].device),
+                          torch.zeros(2, dtype=torch.int32, device=d["pt_values"].device))
+    with pytest.raises(RuntimeError, match="must be contiguous"):
+        ops.tensor_tables(d["tensor_rank"], d["tensor_itemsize"], d["tensor_shape"].t(), d["tensor_stride"])
+    nbytes, contiguous = ops.tensor_tables(d["tensor_rank"], d["tensor_itemsize"], d["tensor_shape"], d["tensor_stride"])
+    cost = torch.empty(tb.n_entries + 1, dtype=torch.float64, device=nbytes.device)
+    with pytest.raises(RuntimeError, match="a per-entry output has"):
+        ops.bind_redistribute_tables(p, nbytes, contiguous, d["spec_codes"], d["spec_tensor"], d["pt_values"], None,
+                                     d["tile_records"], d["dup_entry_begin"], tb.n_entries, None, None, cost, None, None, None, None)
+    with pytest.raises(RuntimeError, match="cost_out needs compute_cost_per_arg"):  # the library's own check, as RuntimeError
+        ops.bind_redistribute_tables(p, nbytes, contiguous, d["spec_codes"], d["spec_tensor"], d["pt_values"], None,
+                                     d["tile_records"], d["dup_entry_begin"], tb.n_entries, None, None, cost[:-1], None, None, None,
+                                     None).run()
+
+
+@pytest.mark.gpu
+def test_a_bound_launch_follows_the_current_stream(small_table, gpu_device):
+    """A bound launch enqueues on whatever stream is current when it runs (and on a given
+    stream handle): the same values from a side stream as from the default stream."""
+    mesh, tb, p, d, want = small_table
+    dev = DeviceCostTables(tb, CostModelParams.from_mesh(mesh, rescale=2.2), device=gpu_device)
+    step = dev.planner_pass()
+    side = torch.cuda.Stream(device=dev.device)  # default priority
+    for name, launch in step.items():
+        assert launch.bound.name().startswith("apc_"), name
+    with torch.cuda.stream(side):
+        for launch in step.values():
+            launch()
+    side.synchronize()
+    assert np.array_equal(dev.cost.cpu().numpy(), want["cost"])
+    dev.cost.zero_()
+    torch.cuda.synchronize()
+    for launch in step.values():
+        launch(side)
+    side.synchronize()
+    assert np.array_equal(dev.cost.cpu().numpy(), want["cost"])
