@@ -81,6 +81,7 @@ EXPORTS = (
     "apc_validate_row_minima_host",
     "apc_diffusion_sweeps",
     "apc_redistribute_tables_static",
+    "apc_strategy_inputs",
 )
 
 _lib = None

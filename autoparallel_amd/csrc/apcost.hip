@@ -405,6 +405,73 @@ __global__ __launch_bounds__(kBlock) void compute_costs_kernel(apc_params p, Com
   compute_costs_block<kBlock>(blockIdx.x, p, a);
 }
 
+// ------------------------------------------------------------------------------------------
+// a9, integer part: flop and byte counts per (node, strategy) from the local shard shapes.
+// The reference runs every operator on fake tensors of the local shard shapes under torch's
+// FlopCounterMode and adds the bytes of all tensor arguments and outputs
+// (compute_estimation.py:232-299, 334-349).  For the operators torch's counter knows in the
+// planned graphs the count is a closed form of the local shapes (torch/utils/flop_counter.py:
+// mm_flop, bmm_flop, sdpa_flop_count, sdpa_backward_flop_count), and the bytes are the local
+// bytes of the strategy's input and output specs (the rows of the spec table) plus a per-node
+// constant (outputs of factories, tensor constants).  One recipe per node, written by the
+// host; one thread per strategy.
+// ------------------------------------------------------------------------------------------
+struct StrategyInputArgs {
+  int64_t n;
+  const int32_t *strat_node;
+  const int64_t *node_strat_begin;
+  const int32_t *node_kind;        // APC_NODE_*
+  const int8_t *node_dtype;
+  const int64_t *node_const_bytes;
+  const int64_t *node_row_begin;   // CSR over byte_rows
+  const int32_t *byte_rows;        // first spec rows of the node's argument and output slots (strategy ss reads row + ss)
+  const int32_t *node_flop_rows;   // [n_nodes, 4]: first spec rows of the tensors the flop formula reads
+  const int64_t *local_shape;      // [n_specs, width]
+  int32_t width;
+  const int64_t *local_bytes;      // [n_specs]
+  int64_t *flops, *rw_bytes;
+  int8_t *dtype;
+  uint8_t *zero_cost;
+};
+
+// b * m * n * 2 * k, in torch's order of multiplications (exact in int64 below 2^63)
+__device__ __forceinline__ int64_t bmm_flops(int64_t b, int64_t m, int64_t k, int64_t n) { return b * m * n * 2 * k; }
+
+__global__ __launch_bounds__(kBlock) void strategy_inputs_kernel(StrategyInputArgs a) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= a.n) return;
+  const int node = a.strat_node[i];
+  const int64_t ss = i - a.node_strat_begin[node];
+  const int kind = a.node_kind[node];
+  int64_t flops = 0, bytes = 0;
+  if (kind != APC_NODE_ZERO_COST) {
+    bytes = a.node_const_bytes[node];
+    for (int64_t r = a.node_row_begin[node]; r < a.node_row_begin[node + 1]; ++r) bytes += a.local_bytes[a.byte_rows[r] + ss];
+    const int32_t *rows = a.node_flop_rows + (int64_t)node * 4;
+    const int w = a.width;
+    // (a dim past the row's width reads as 1: the host checks ranks, this keeps the load inside the table)
+    auto dim = [&](int t, int d) { return d < w ? a.local_shape[(rows[t] + ss) * w + d] : (int64_t)1; };
+    if (kind == APC_NODE_MM) {  // [m, k] x [k, n]
+      flops = dim(0, 0) * dim(1, 1) * 2 * dim(0, 1);
+    } else if (kind == APC_NODE_BMM) {  // [b, m, k] x [b, k, n]
+      flops = bmm_flops(dim(0, 0), dim(0, 1), dim(0, 2), dim(1, 2));
+    } else if (kind == APC_NODE_SDPA || kind == APC_NODE_SDPA_BACKWARD) {
+      // rows: query [b, h, s_q, d_q], key [b, h, s_k, d_q], value [b, h, s_k, d_v]
+      const int64_t bh = dim(0, 0) * dim(0, 1), s_q = dim(0, 2), d_q = dim(0, 3), s_k = dim(1, 2), d_v = dim(2, 3);
+      if (kind == APC_NODE_SDPA) {
+        flops = bmm_flops(bh, s_q, d_q, s_k) + bmm_flops(bh, s_q, s_k, d_v);
+      } else {  // recomputed scores, gradScores, gradV, gradQ, gradK
+        flops = bmm_flops(bh, s_q, d_q, s_k) + bmm_flops(bh, s_q, d_v, s_k) + bmm_flops(bh, s_k, s_q, d_v) +
+                bmm_flops(bh, s_q, s_k, d_q) + bmm_flops(bh, d_q, s_q, s_k);
+      }
+    }
+  }
+  a.flops[i] = flops;
+  a.rw_bytes[i] = bytes;
+  a.dtype[i] = a.node_dtype[node];
+  a.zero_cost[i] = kind == APC_NODE_ZERO_COST ? 1 : 0;
+}
+
 // The three tables above in one launch: workgroups [0, spec_blocks) take the spec table (the
 // largest), the next tensor_blocks the tensor table, the rest the compute costs.  None of the
 // three reads another's output.
@@ -1876,6 +1943,24 @@ int apc_compute_costs(const apc_params *params, int64_t n, const int64_t *flops,
                      *params,
                      ComputeCostArgs{n, flops, rw_bytes, dtype, zero_cost, num_args, compute, per_arg, error_flag});
   return check_launch("apc_compute_costs");
+}
+
+int apc_strategy_inputs(int64_t n_strategies, const int32_t *strat_node, int64_t n_nodes, const int64_t *node_strat_begin,
+                        const int32_t *node_kind, const int8_t *node_dtype, const int64_t *node_const_bytes,
+                        const int64_t *node_row_begin, const int32_t *byte_rows, const int32_t *node_flop_rows,
+                        const int64_t *local_shape, int32_t shape_width, const int64_t *local_bytes, int64_t *flops,
+                        int64_t *rw_bytes, int8_t *dtype_code, uint8_t *zero_cost, void *stream) {
+  if (n_strategies < 0 || n_nodes < 0) return fail(-1, "apc_strategy_inputs: negative count");
+  if (n_strategies == 0) return 0;
+  if (int rc = check_width(shape_width)) return rc;
+  if (!strat_node || !node_strat_begin || !node_kind || !node_dtype || !node_const_bytes || !node_row_begin ||
+      !node_flop_rows || !local_shape || !local_bytes || !flops || !rw_bytes || !dtype_code || !zero_cost)
+    return fail(-1, "apc_strategy_inputs: NULL array");
+  hipLaunchKernelGGL(strategy_inputs_kernel, dim3(blocks_for(n_strategies, kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
+                     StrategyInputArgs{n_strategies, strat_node, node_strat_begin, node_kind, node_dtype, node_const_bytes,
+                                       node_row_begin, byte_rows, node_flop_rows, local_shape, shape_width, local_bytes, flops,
+                                       rw_bytes, dtype_code, zero_cost});
+  return check_launch("apc_strategy_inputs");
 }
 
 int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t *rank, const int32_t *itemsize,

@@ -588,6 +588,43 @@ void diffusion_sweeps_(int64_t n_sweeps, const Tensor &color_begin, const Tensor
   });
 }
 
+// Flop and byte counts of every (node, strategy) from the spec table's local shapes and the
+// per-node recipes (compute_estimation.py:232-299, 334-349; apc_strategy_inputs).
+std::tuple<Tensor, Tensor, Tensor, Tensor> strategy_inputs(const Tensor &strat_node, const Tensor &node_strat_begin,
+                                                           const Tensor &node_kind, const Tensor &node_dtype,
+                                                           const Tensor &node_const_bytes, const Tensor &node_row_begin,
+                                                           const Tensor &byte_rows, const Tensor &node_flop_rows,
+                                                           const Tensor &local_shape, const Tensor &local_bytes) {
+  const int32_t *sn = dev<int32_t>(strat_node, at::kInt, "strat_node");
+  const int64_t *nsb = dev<int64_t>(node_strat_begin, at::kLong, "node_strat_begin");
+  const int32_t *kind = dev<int32_t>(node_kind, at::kInt, "node_kind");
+  const int8_t *dt = dev<int8_t>(node_dtype, at::kChar, "node_dtype");
+  const int64_t *cb = dev<int64_t>(node_const_bytes, at::kLong, "node_const_bytes");
+  const int64_t *rb = dev<int64_t>(node_row_begin, at::kLong, "node_row_begin");
+  const int32_t *rows = dev<int32_t>(byte_rows, at::kInt, "byte_rows");
+  const int32_t *fr = dev<int32_t>(node_flop_rows, at::kInt, "node_flop_rows");
+  const int64_t *ls = dev<int64_t>(local_shape, at::kLong, "local_shape");
+  const int64_t *lb = dev<int64_t>(local_bytes, at::kLong, "local_bytes");
+  const int64_t n = strat_node.numel(), n_nodes = node_kind.numel();
+  TORCH_CHECK(node_strat_begin.numel() == n_nodes + 1 && node_row_begin.numel() == n_nodes + 1,
+              "apcost: node_strat_begin / node_row_begin need n_nodes + 1 rows");
+  TORCH_CHECK(node_dtype.numel() == n_nodes && node_const_bytes.numel() == n_nodes && node_flop_rows.numel() == 4 * n_nodes,
+              "apcost: the recipe arrays need one row per node (node_flop_rows four values per node)");
+  TORCH_CHECK(local_shape.dim() == 2 && local_shape.size(0) == local_bytes.numel(),
+              "apcost: local_shape must be [n_specs, shape_width] with one row per row of local_bytes");
+  for (const Tensor *t : {&node_strat_begin, &node_kind, &node_dtype, &node_const_bytes, &node_row_begin, &byte_rows, &node_flop_rows,
+                          &local_shape, &local_bytes})
+    same_device(strat_node, *t, "a recipe array");
+  Tensor flops = empty_like_device(strat_node, {n}, at::kLong), rw_bytes = empty_like_device(strat_node, {n}, at::kLong),
+         dtype = empty_like_device(strat_node, {n}, at::kChar), zero_cost = empty_like_device(strat_node, {n}, at::kByte);
+  on_current_stream(strat_node.device(), "apc_strategy_inputs", [&](void *s) {
+    return apc_strategy_inputs(n, sn, n_nodes, nsb, kind, dt, cb, rb, rows, fr, ls, (int32_t)local_shape.size(1), lb,
+                               n ? static_cast<int64_t *>(flops.data_ptr()) : nullptr, n ? static_cast<int64_t *>(rw_bytes.data_ptr()) : nullptr,
+                               n ? static_cast<int8_t *>(dtype.data_ptr()) : nullptr, n ? zero_cost.data_ptr<uint8_t>() : nullptr, s);
+  });
+  return {flops, rw_bytes, dtype, zero_cost};
+}
+
 int64_t abi_version() { return apc_version(); }
 
 }  // namespace
@@ -611,6 +648,10 @@ TORCH_LIBRARY(apcost, m) {
   m.def("compute_cost(Tensor params, " APCOST_STRATEGY_TABLE
         ") -> (Tensor compute_cost, Tensor compute_cost_per_arg, Tensor error_flag)",
         &compute_cost);
+  m.def("strategy_inputs(Tensor strat_node, Tensor node_strat_begin, Tensor node_kind, Tensor node_dtype, Tensor node_const_bytes, "
+        "Tensor node_row_begin, Tensor byte_rows, Tensor node_flop_rows, Tensor local_shape, Tensor local_bytes) "
+        "-> (Tensor flops, Tensor rw_bytes, Tensor dtype_code, Tensor zero_cost)",
+        &strategy_inputs);
   m.def("segmented_min(Tensor values, Tensor seg_ptr) -> (Tensor seg_min, Tensor seg_argmin)", &segmented_min);
   m.def("cost_objective(int n_vars, Tensor group_var_begin, Tensor group_member_begin, Tensor member_entry_begin, Tensor cost, "
         "float inf_replacement) -> (Tensor objective, Tensor forced_zero)",

@@ -127,6 +127,43 @@ class DeviceCostTables:
         self.spec_out = out
         return out
 
+    # ---- per-strategy flop / byte counts -----------------------------------------------------
+    @_guarded
+    def run_strategy_inputs(self, recipes):
+        """Flop and byte counts of every (node, strategy) from the spec table and the per-node
+        ``recipes`` (``graphs.cost_inputs.StrategyRecipes``), on the device; the strategy table
+        of later launches reads the results where they are.  -> (flops, rw_bytes, dtype_code,
+        zero_cost) device tensors."""
+        tb = self.tables
+        spec = getattr(self, "spec_out", None) or self.run_spec_tables()
+        n_nodes = tb.n_nodes
+        for name in ("node_kind", "node_dtype", "node_const_bytes"):
+            if len(getattr(recipes, name)) != n_nodes:
+                raise ValueError(f"recipes.{name} must have one row per node")
+        # every row a recipe names, plus the node's strategies, lies inside the spec table; the
+        # tensors of a flop formula have the rank it reads
+        n_strat = np.diff(tb.node_strat_begin).astype(np.int64)
+        per_node = np.repeat(n_strat, np.diff(recipes.node_row_begin))
+        if len(recipes.byte_rows) and int((recipes.byte_rows.astype(np.int64) + per_node).max()) > tb.n_specs:
+            raise ValueError("a recipe's spec rows run past the spec table")
+        with_formula = recipes.node_kind >= 2
+        if with_formula.any():
+            if int((recipes.node_flop_rows[with_formula].astype(np.int64).max(axis=1) + n_strat[with_formula]).max()) > tb.n_specs:
+                raise ValueError("a flop formula's spec rows run past the spec table")
+            need = 4 if (recipes.node_kind >= 4).any() else 3 if (recipes.node_kind == 3).any() else 2
+            if spec["local_shape"].shape[1] < need:
+                raise ValueError("the spec table's shape rows are narrower than a flop formula's tensors")
+        strat_node = _to_device(np.repeat(np.arange(n_nodes, dtype=np.int32), n_strat), self.device)
+        up = {k: _to_device(np.ascontiguousarray(getattr(recipes, k)), self.device) for k in (
+            "node_kind", "node_dtype", "node_const_bytes", "node_row_begin", "byte_rows", "node_flop_rows")}
+        node_strat_begin = _to_device(np.ascontiguousarray(tb.node_strat_begin, np.int64), self.device)
+        out = self.ops.strategy_inputs(strat_node, node_strat_begin, up["node_kind"], up["node_dtype"], up["node_const_bytes"],
+                                       up["node_row_begin"], up["byte_rows"], up["node_flop_rows"].reshape(-1),
+                                       spec["local_shape"], spec["local_bytes"])
+        for key, t in zip(("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost"), out):
+            self.d[key] = t
+        return out
+
     # ---- per-strategy compute cost ---------------------------------------------------------
     @_guarded
     def run_compute_costs(self):

@@ -43,6 +43,116 @@ def _const_key(x):
     return repr(x)
 
 
+# what a node's flop count is to the device kernel (APC_NODE_* of include/apcost.h)
+NODE_ZERO_COST, NODE_BYTES_ONLY, NODE_MM, NODE_BMM, NODE_SDPA, NODE_SDPA_BACKWARD = range(6)
+
+# operator packet -> (kind, positions among the node's tensor arguments of the tensors the
+# formula reads, the rank it expects of them): torch/utils/flop_counter.py mm_flop, addmm_flop,
+# bmm_flop, baddbmm_flop, sdpa_flop, sdpa_backward_flop
+_aten = torch.ops.aten
+_CLOSED_FORMS = {
+    _aten.mm: (NODE_MM, (0, 1), 2),
+    _aten.addmm: (NODE_MM, (1, 2), 2),
+    _aten.bmm: (NODE_BMM, (0, 1), 3),
+    _aten.baddbmm: (NODE_BMM, (1, 2), 3),
+    _aten._scaled_dot_product_flash_attention: (NODE_SDPA, (0, 1, 2), 4),
+    _aten._scaled_dot_product_efficient_attention: (NODE_SDPA, (0, 1, 2), 4),
+    _aten._scaled_dot_product_cudnn_attention: (NODE_SDPA, (0, 1, 2), 4),
+    _aten._scaled_dot_product_flash_attention_backward: (NODE_SDPA_BACKWARD, (1, 2, 3), 4),
+    _aten._scaled_dot_product_efficient_attention_backward: (NODE_SDPA_BACKWARD, (1, 2, 3), 4),
+    _aten._scaled_dot_product_cudnn_attention_backward: (NODE_SDPA_BACKWARD, (1, 2, 3), 4),
+}
+
+
+class StrategyRecipes:
+    """Per-node recipes from which the device computes the flop and byte count of every
+    (node, strategy) out of the spec table (``apc_strategy_inputs``): ``node_kind``,
+    ``node_dtype``, ``node_const_bytes``, ``node_row_begin`` / ``byte_rows`` (CSR of first spec
+    rows whose local bytes add up) and ``node_flop_rows`` [n_nodes, 4].  ``host_nodes`` lists
+    the nodes no recipe covers (an operator torch's flop counter knows but the kernel has no
+    formula for, or one that decomposes under the counter): with any of them the planner takes
+    the host path (``fill_flops_and_bytes``) for the whole graph."""
+
+    def __init__(self, n_nodes: int):
+        self.node_kind = np.zeros(n_nodes, np.int32)
+        self.node_dtype = np.ones(n_nodes, np.int8)  # the strategy table's initial dtype code
+        self.node_const_bytes = np.zeros(n_nodes, np.int64)
+        self.node_row_begin = np.zeros(n_nodes + 1, np.int64)
+        self.byte_rows = np.zeros(0, np.int32)
+        self.node_flop_rows = np.zeros((n_nodes, 4), np.int32)
+        self.host_nodes: list = []
+
+
+def strategy_recipes(encoded, strats) -> StrategyRecipes:
+    """One recipe per graph node (no per-strategy work on the host).  What the reference does
+    per strategy (compute_estimation.py:232-299, 334-349): run the operator on fake tensors of
+    the local shard shapes under ``FlopCounterMode`` and add the bytes of every tensor among
+    the arguments and the outputs.  Per node that is: the local bytes of the strategy's input
+    specs and output specs (rows of the spec table) plus the bytes of tensor constants; for an
+    operator without tensor arguments (a factory) the operator runs on its own arguments, so
+    its output is the global tensor whatever the strategy: a constant; flops as the closed
+    form of the operator's entry in torch's flop registry, zero outside the registry."""
+    from torch.utils.flop_counter import flop_registry
+
+    n_nodes = len(encoded.nodes)
+    rc = StrategyRecipes(n_nodes)
+    rows: list = []
+    slots_of: dict = {}
+    for (s_i, slot), row in encoded.output_spec_row.items():
+        slots_of.setdefault(s_i, []).append(row)
+    for s_i, node in enumerate(encoded.nodes):
+        rc.node_row_begin[s_i] = len(rows)
+        if node.op == "output" or has_zero_cost(node):
+            continue  # NODE_ZERO_COST, dtype code 1
+        flat_args, treespec = tree_flatten(node.args)
+        vals = [a.meta["val"] if isinstance(a, torch.fx.Node) else a for a in flat_args]
+        tensor_pos = [i for i, v in enumerate(vals) if isinstance(v, torch.Tensor)]
+        kw_flat, kw_spec = tree_flatten(node.kwargs)
+        kw_vals = [a.meta["val"] if isinstance(a, torch.fx.Node) else a for a in kw_flat]
+        for v in kw_vals:
+            # compute_estimation.py:254-256: tensors are expected in args only
+            assert not isinstance(v, torch.Tensor), f"{node}: tensor keyword arguments are not supported"
+        rc.node_kind[s_i] = NODE_BYTES_ONLY
+        dtype = vals[tensor_pos[0]].dtype if tensor_pos else torch.float32
+        rc.node_dtype[s_i] = _DTYPE_TO_CODE.get(dtype, UNSUPPORTED_DTYPE_CODE)
+        packet = node.target.overloadpacket
+        if not tensor_pos:
+            # a factory: the reference runs it on its own (global) arguments for every strategy
+            mode = getattr(node.meta.get("val"), "fake_mode", None)
+            flops, rw_bytes, code = _evaluate(node.target, vals, [], [], treespec, kw_vals, kw_spec, mode)
+            if flops != 0:
+                rc.host_nodes.append(node)
+            rc.node_const_bytes[s_i] = rw_bytes
+            rc.node_dtype[s_i] = code
+            continue
+        node_args = [i for i in tensor_pos if isinstance(flat_args[i], torch.fx.Node)]
+        if len(node_args) != encoded.num_args[s_i]:
+            rc.host_nodes.append(node)  # input specs do not line up with the tensor arguments
+            continue
+        for i in tensor_pos:
+            if not isinstance(flat_args[i], torch.fx.Node):  # a tensor constant keeps its size
+                rc.node_const_bytes[s_i] += vals[i].numel() * vals[i].element_size()
+        arg_rows = [encoded.input_spec_row[(s_i, k)] for k in range(len(node_args))]
+        rows.extend(arg_rows)
+        rows.extend(slots_of.get(s_i, []))
+        form = _CLOSED_FORMS.get(packet)
+        if form is not None:
+            kind, positions, rank = form
+            reads = [tensor_pos[p] for p in positions] if max(positions) < len(tensor_pos) else None
+            if reads is None or any(not isinstance(flat_args[i], torch.fx.Node) or vals[i].dim() != rank for i in reads):
+                rc.host_nodes.append(node)
+                continue
+            rc.node_kind[s_i] = kind
+            for t, i in enumerate(reads):
+                rc.node_flop_rows[s_i, t] = arg_rows[node_args.index(i)]
+        elif packet in flop_registry or torch._C._dispatch_has_kernel_for_dispatch_key(
+                node.target.name(), "CompositeImplicitAutograd"):
+            rc.host_nodes.append(node)  # counted by torch, no formula here (or decomposes under the counter)
+    rc.node_row_begin[n_nodes] = len(rows)
+    rc.byte_rows = np.asarray(rows, np.int32)
+    return rc
+
+
 def fill_flops_and_bytes(encoded, strats, local_shape: np.ndarray, local_stride: np.ndarray, stats=None) -> None:
     """Writes strat_flops / strat_rw_bytes / strat_dtype / strat_zero_cost of
     ``encoded.tables`` in place.  ``local_shape`` / ``local_stride`` are the [n_specs, width]

@@ -38,7 +38,7 @@ from torch.distributed.tensor._dtensor_spec import DTensorSpec
 from torch.distributed.tensor.placement_types import Placement, Replicate, Shard
 
 from .cost_model import CostModelParams
-from .graphs.cost_inputs import fill_flops_and_bytes
+from .graphs.cost_inputs import fill_flops_and_bytes, strategy_recipes
 from .graphs.encode import EncodedGraph, all_input_nodes, encode_graph
 from .graphs.strategies import StrategyEnumerator
 from .ilp import BinaryProgram, next_name
@@ -68,12 +68,30 @@ class DeviceBackend:
             out = self.dev.run_spec_tables()
             return out["local_shape"].cpu().numpy(), out["local_stride"].cpu().numpy()
 
+    def strategy_inputs(self, recipes):
+        """Flop and byte counts of every strategy on the device (spec table, then
+        ``apc_strategy_inputs`` over the per-node recipes); the host's strategy table receives
+        copies (identical edges are found on the host, and flop / byte counts are part of an
+        edge's identity)."""
+        from .device_tables import _real_tensors
+
+        with _real_tensors():
+            flops, rw_bytes, dtype, zero = self.dev.run_strategy_inputs(recipes)
+            tb = self.dev.tables
+            tb.strat_flops[:] = flops.cpu().numpy()
+            tb.strat_rw_bytes[:] = rw_bytes.cpu().numpy()
+            tb.strat_dtype[:] = dtype.cpu().numpy()
+            tb.strat_zero_cost[:] = zero.cpu().numpy()
+        self._strategy_inputs_on_device = True
+
     def upload_strategy_inputs(self, tables, tile_entries=None, dedupe=True, max_copies=16):
         """The strategy table is final: tile the edges (identical edges once) and send both."""
         tables.build_tiles(tile_entries, dedupe=dedupe, max_copies=max_copies)
         tables.validate(self.dev.params)
-        self.dev.refresh("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost", "tile_records",
-                         "dup_entry_begin", "dup_row_begin")
+        names = ("tile_records", "dup_entry_begin", "dup_row_begin")
+        if not getattr(self, "_strategy_inputs_on_device", False):
+            names = ("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost") + names
+        self.dev.refresh(*names)
 
     def launch_tables(self):
         """Enqueues the planner's table pass (``DeviceCostTables.planner_pass``) and returns."""
@@ -294,6 +312,10 @@ class ShardingOptimizer:
     # during enumeration torch's own redistribute_cost (whose values the table build replaces) is
     # stubbed by a constant; False leaves it alone (same tables, slower enumeration)
     cheap_enumeration_costs = True
+    # flop / byte counts of the strategies from per-node recipes on the device (apc_strategy_inputs);
+    # False: on the host, every distinct (operator, local shapes) on fake tensors under torch's
+    # flop counter, as the reference does
+    strategy_inputs_on_device = True
     node_choice_variables = True
     compact_constraints = True  # with choice variables: the structural constraints written through them
     # Before the solver runs: a dual ascent over the program's labelling form (row / column minima
@@ -388,12 +410,23 @@ class ShardingOptimizer:
         tb = self.encoded.tables
         t0 = time.perf_counter()
         self.backend = self.backend_cls(tb, self.params, self.device)
-        local_shape, local_stride = self.backend.local_shapes()
+        self.cost_input_stats = {}
+        # flop / byte counts of every strategy (compute_estimation.py:232-299, 334-349): on the
+        # device from per-node recipes; on the host, operator by operator on fake tensors of the
+        # local shapes, when the graph holds an operator no recipe covers (or the backend has
+        # no device)
+        recipes = strategy_recipes(self.encoded, self.strats) if self.strategy_inputs_on_device else None
+        on_device = recipes is not None and not recipes.host_nodes and hasattr(self.backend, "strategy_inputs")
+        self.cost_input_stats["strategy_inputs"] = "device" if on_device else "host"
+        if on_device:
+            self.backend.strategy_inputs(recipes)
+        else:
+            local_shape, local_stride = self.backend.local_shapes()
         self.timings["upload_and_shapes_s"] = time.perf_counter() - t0
         logger.info("%s %.3f s", "upload_and_shapes_s", self.timings["upload_and_shapes_s"])
         t0 = time.perf_counter()
-        self.cost_input_stats = {}
-        fill_flops_and_bytes(self.encoded, self.strats, local_shape, local_stride, self.cost_input_stats)
+        if not on_device:
+            fill_flops_and_bytes(self.encoded, self.strats, local_shape, local_stride, self.cost_input_stats)
         self.backend.upload_strategy_inputs(tb, self.tile_entries, self.dedupe, self.max_copies)
         self.timings["flops_bytes_s"] = time.perf_counter() - t0
         logger.info("%s %.3f s", "flops_bytes_s", self.timings["flops_bytes_s"])

@@ -157,11 +157,38 @@ int apc_compute_costs(const apc_params *params, int64_t n_strategies, const int6
                       const int32_t *num_args, double *compute_cost, double *compute_cost_per_arg,
                       int32_t *error_flag, void *stream);
 
+/* a9, integer part: flop and byte counts of every (node, strategy) from the local shard shapes
+ * (replaces the fake-tensor run of compute_estimation.py:232-299, 334-349 for the operators whose
+ * flop count torch/utils/flop_counter.py gives in closed form).  One recipe per node:
+ *   node_kind         what the flop formula is (APC_NODE_*); APC_NODE_ZERO_COST rows get
+ *                     flops = rw_bytes = 0 and zero_cost = 1 (compute_estimation.py:279-291)
+ *   node_dtype        dtype code of the node's first tensor argument (written to every strategy)
+ *   node_const_bytes  bytes that do not depend on the strategy (factory outputs, tensor constants)
+ *   node_row_begin / byte_rows   CSR: first spec rows of the node's tensor arguments and output
+ *                     slots; strategy ss adds local_bytes[row + ss] of each
+ *   node_flop_rows    [n_nodes, 4] first spec rows of the tensors the formula reads (mm: mat1,
+ *                     mat2; bmm: batch1, batch2; attention: query, key, value), unused slots 0
+ * local_shape [n_specs, shape_width] / local_bytes [n_specs] are outputs of apc_spec_tables.
+ * The caller guarantees that every row + ss lies inside the spec table and that the tensors a
+ * formula reads have the rank it expects (2 / 3 / 4).  Outputs: one row per strategy. */
+#define APC_NODE_ZERO_COST 0
+#define APC_NODE_BYTES_ONLY 1 /* not counted by torch's flop counter: flops = 0 */
+#define APC_NODE_MM 2         /* aten.mm, aten.addmm:    m * n * 2 * k */
+#define APC_NODE_BMM 3        /* aten.bmm, aten.baddbmm: b * m * n * 2 * k */
+#define APC_NODE_SDPA 4       /* _scaled_dot_product_{flash,efficient,cudnn}_attention */
+#define APC_NODE_SDPA_BACKWARD 5
+int apc_strategy_inputs(int64_t n_strategies, const int32_t *strat_node, int64_t n_nodes,
+                        const int64_t *node_strat_begin, const int32_t *node_kind, const int8_t *node_dtype,
+                        const int64_t *node_const_bytes, const int64_t *node_row_begin, const int32_t *byte_rows,
+                        const int32_t *node_flop_rows, const int64_t *local_shape, int32_t shape_width,
+                        const int64_t *local_bytes, int64_t *flops, int64_t *rw_bytes, int8_t *dtype_code,
+                        uint8_t *zero_cost, void *stream);
+
 /* apc_tensor_tables + apc_spec_tables + apc_compute_costs in ONE launch (none of the three
  * reads another's output): same arguments, same results, two launches fewer.  For a caller that
  * already holds the per-strategy flop / byte counts, e.g. when the tables of a graph are
  * rebuilt under another cost model.  (A planner that still has to infer those counts from the
- * local shard shapes, compute_estimation.py:244-300, calls apc_spec_tables first and alone.)
+ * local shard shapes calls apc_spec_tables and apc_strategy_inputs first.)
  * The five spec-table outputs may all be NULL: the spec table is then skipped. */
 int apc_input_tables(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
                      const int32_t *tensor_itemsize, const int64_t *tensor_shape, const int64_t *tensor_stride,

@@ -334,6 +334,47 @@ def sdpa_backward_flop(b, h, s_q, s_k, d_q, d_v):
     return total
 
 
+NODE_ZERO_COST, NODE_BYTES_ONLY, NODE_MM, NODE_BMM, NODE_SDPA, NODE_SDPA_BACKWARD = range(6)
+
+
+def strategy_inputs(strat_node, node_strat_begin, node_kind, node_dtype, node_const_bytes, node_row_begin, byte_rows,
+                    node_flop_rows, local_shape, local_bytes):
+    """ref: compute_estimation.py:232-299, 334-349 per (node, strategy), on the encoded form:
+    the bytes of every tensor argument and output on its local shard (rows of the spec table)
+    plus the node's constant bytes, and the flops torch's counter gives the operator on the
+    local shapes (mm / bmm / attention formulas above; zero for operators outside its registry;
+    zero-cost nodes :279-291 get nothing).
+    -> (flops, rw_bytes, dtype_code, zero_cost), one row per strategy."""
+    n = len(strat_node)
+    flops, rw, dtype, zero = [0] * n, [0] * n, [0] * n, [0] * n
+    for i in range(n):
+        node = int(strat_node[i])
+        ss = i - int(node_strat_begin[node])
+        kind = int(node_kind[node])
+        dtype[i] = int(node_dtype[node])
+        zero[i] = 1 if kind == NODE_ZERO_COST else 0
+        if kind == NODE_ZERO_COST:
+            continue
+        total = int(node_const_bytes[node])
+        for r in range(int(node_row_begin[node]), int(node_row_begin[node + 1])):
+            total += int(local_bytes[int(byte_rows[r]) + ss])
+        rw[i] = total
+
+        def shape(t):
+            return [int(x) for x in local_shape[int(node_flop_rows[node][t]) + ss]]
+
+        if kind == NODE_MM:
+            (m, k), (_, nn) = shape(0)[:2], shape(1)[:2]
+            flops[i] = mm_flop(m, k, nn)
+        elif kind == NODE_BMM:
+            (b, m, k), (_, _, nn) = shape(0)[:3], shape(1)[:3]
+            flops[i] = bmm_flop(b, m, k, nn)
+        elif kind in (NODE_SDPA, NODE_SDPA_BACKWARD):
+            (b, h, s_q, d_q), s_k, d_v = shape(0)[:4], shape(1)[2], shape(2)[3]
+            flops[i] = (sdpa_flop if kind == NODE_SDPA else sdpa_backward_flop)(b, h, s_q, s_k, d_q, d_v)
+    return flops, rw, dtype, zero
+
+
 def compute_cost(zero_cost: bool, flops: int, rw_bytes: int, dtype_code: int, p: CostParams):
     """ref: compute_estimation.py:334-365 tail (after flops / bytes are known)."""
     if zero_cost:

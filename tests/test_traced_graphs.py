@@ -192,16 +192,19 @@ def test_device_tables_match_oracle_on_benchmark_configurations(gpu_device, fake
             assert not o._host_arrays, "no per-entry array has left the backend so far"
             out.update(comm=o.comm_cost.copy(), transition=o.transition_cost.copy(), cost=o.cost.copy(),
                        per_arg=o.compute_cost_per_arg.copy(), n_entries=tb.n_entries,
-                       backend=type(o.backend).__name__)
+                       backend=type(o.backend).__name__, inputs=o.cost_input_stats["strategy_inputs"])
             out["row_min"], out["row_argmin"] = o.row_minima()
             return out
 
     d = snapshot(AutoParallelPlanner)
     o = snapshot(OraclePlanner)
     assert d["backend"] == "DeviceBackend" and o["backend"] == "OracleBackend"
+    # flop / byte counts: the device's kernel over per-node recipes against torch's own flop
+    # counter and shape functions on fake tensors of the local shapes (the reference's way)
+    assert d["inputs"] == "device" and o["inputs"] == "host"
     assert d["n_entries"] == o["n_entries"] > 0
     for name in d:
-        if name not in ("backend", "n_entries"):
+        if name not in ("backend", "n_entries", "inputs"):
             assert np.array_equal(d[name], o[name]), name
     # something was actually costed: finite positive comm and compute costs exist
     assert (d["comm"][np.isfinite(d["comm"])] > 0).any() and (d["per_arg"] > 0).any()
@@ -311,3 +314,47 @@ def test_split_tensor_rule(fake_pg):
     with pytest.raises(NotImplementedError, match="Partial"):
         enum.placement_options(aten.split.Tensor, [OpStrategy([OpSpec(partial, input_specs=[partial], redistribute_cost=[[0.0]])]), 4, 1],
                                [x, 4, 1], {})
+
+
+@pytest.mark.parametrize("case", ["llama3_8b_1layer_mesh32x8", "dsv3_moe_tiny_mesh64x4", "block_1k_batch8_mesh64"])
+def test_strategy_recipes_give_the_flop_counter_path(fake_pg, case):
+    """The per-node recipes the device computes flop / byte counts from, evaluated by the
+    oracle's restatement of that kernel on the oracle's spec table, against the host path that
+    (like the reference, compute_estimation.py:232-299, 334-349) runs every distinct operator
+    call on fake tensors of the local shapes under torch's FlopCounterMode: equal on every
+    (node, strategy), factories and attention included."""
+    from autoparallel_amd.graphs.cost_inputs import strategy_recipes
+    from oracle import c_oracle
+    from oracle import cost_oracle as po
+
+    cfg, mesh, batch, seq = CASES[case]
+    with _planner(OraclePlanner, cfg, mesh, batch, seq, block=case.startswith("block")) as autop:
+        o = autop.sharding_optimizer
+        assert o.cost_input_stats["strategy_inputs"] == "host"  # the oracle backend has no device
+        enc, tb = o.encoded, o.encoded.tables
+        rc = strategy_recipes(enc, o.strats)
+        assert not rc.host_nodes
+        _, lshape, _, _, lbytes = c_oracle.spec_tables(tb.as_dict(), mesh)
+        strat_node = np.repeat(np.arange(len(enc.nodes)), np.diff(tb.node_strat_begin))
+        got = po.strategy_inputs(strat_node, tb.node_strat_begin, rc.node_kind, rc.node_dtype, rc.node_const_bytes,
+                                 rc.node_row_begin, rc.byte_rows, rc.node_flop_rows, np.asarray(lshape), np.asarray(lbytes))
+        assert int(np.count_nonzero(tb.strat_flops)) > 0
+        for name, g in zip(("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost"), got):
+            assert np.array_equal(np.asarray(g), getattr(tb, name)), name
+
+
+def test_an_operator_without_a_recipe_takes_the_host_path(fake_pg):
+    """A node whose operator torch's flop counter knows but no recipe covers is reported, and
+    the planner then counts flops and bytes on the host for the whole graph."""
+    from autoparallel_amd.graphs import cost_inputs
+
+    cfg, mesh, batch, seq = CASES["block_1k_batch8_mesh64"]
+    saved = dict(cost_inputs._CLOSED_FORMS)
+    try:
+        del cost_inputs._CLOSED_FORMS[torch.ops.aten.mm]
+        with _planner(OraclePlanner, cfg, mesh, batch, seq, block=True) as autop:
+            o = autop.sharding_optimizer
+            rc = cost_inputs.strategy_recipes(o.encoded, o.strats)
+            assert rc.host_nodes and all(n.target.overloadpacket == torch.ops.aten.mm for n in rc.host_nodes)
+    finally:
+        cost_inputs._CLOSED_FORMS.update(saved)
