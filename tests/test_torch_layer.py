@@ -13,7 +13,7 @@ from oracle import c_oracle
 from oracle import cost_oracle as po
 
 OPERATORS = (
-    "abi_version", "tensor_tables", "shard_shapes_bytes", "compute_cost", "segmented_min", "cost_objective",
+    "abi_version", "tensor_tables", "shard_shapes_bytes", "strategy_inputs", "compute_cost", "segmented_min", "cost_objective",
     "redistribute_cost_tables", "strategy_bounds", "diffusion_sweeps_", "bind_tensor_tables", "bind_spec_tables",
     "bind_compute_costs", "bind_segmented_min", "bind_redistribute_tables", "bind_input_tables", "bind_cost_tables",
 )
