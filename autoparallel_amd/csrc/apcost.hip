@@ -1195,23 +1195,26 @@ __device__ __forceinline__ void row_min_chunk(double (&rmin)[2][APC_TILE_MAX_ROW
 // parts and stores minimum and first argmin to the row of the tile's edge and of every
 // identical edge.  (Called by every thread of the workgroup.)
 template <int M>
-__device__ __forceinline__ void row_min_finish(const TableArgs &a, TileStage<M, true> &st, const TileView &v, int tid) {
+__device__ __forceinline__ void row_min_finish(const TableArgs &a, TileStage<M, true> &st, const TileView &v, int tid,
+                                               int nthreads) {
   __syncthreads();
-  if (tid >= v.rows) return;
-  double m = st.rmin[0][tid];
-  int mc = st.rarg[0][tid];
-  const double m1 = st.rmin[1][tid];
+  // lane = row, wavefront w takes the copies w, w + waves, ...: copy 0 is the tile's own edge, copy
+  // d > 0 the d-th identical edge (a tile of many copies ends with a short store phase in every
+  // wavefront instead of a long one in the first)
+  const int row = tid & 63;
+  if (row >= v.rows) return;
+  double m = st.rmin[0][row];
+  int mc = st.rarg[0][row];
+  const double m1 = st.rmin[1][row];
   if (m1 < m) {  // the later part wins only if strictly smaller
     m = m1;
-    mc = st.rarg[1][tid];
+    mc = st.rarg[1][row];
   }
-  const int64_t row = st.row_out + v.row_begin + tid;
-  a.row_min_out[row] = m;
-  a.row_arg_out[row] = v.col_begin + mc;
-  for (int d = 0; d < v.dup_count; ++d) {
-    const int64_t rd = st.dup_row[d] + v.row_begin + tid;
-    a.row_min_out[rd] = m;
-    a.row_arg_out[rd] = v.col_begin + mc;
+  const int waves = nthreads >> 6;
+  for (int d = tid >> 6; d <= v.dup_count; d += waves) {
+    const int64_t out = (d == 0 ? st.row_out : st.dup_row[d - 1]) + v.row_begin + row;
+    a.row_min_out[out] = m;
+    a.row_arg_out[out] = v.col_begin + mc;
   }
 }
 
@@ -1251,7 +1254,7 @@ __device__ __forceinline__ void uniform_tile_entries_row_min(const apc_params &p
       }
     }
   }
-  row_min_finish<M>(a, st, v, tid);
+  row_min_finish<M>(a, st, v, tid, nthreads);
 }
 
 // The per-entry loop of such a tile for `nthreads` threads (this one is `tid`): a flattened
@@ -1344,7 +1347,7 @@ __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const 
       }
     }
   }
-  if constexpr (ROW_MIN && RM) row_min_finish<M>(a, st, v, tid);
+  if constexpr (ROW_MIN && RM) row_min_finish<M>(a, st, v, tid, nthreads);
 }
 
 // All entries of a staged tile.  Row minima are taken when the caller wants them and the tile
