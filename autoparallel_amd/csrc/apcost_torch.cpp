@@ -625,6 +625,43 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> strategy_inputs(const Tensor &strat_n
   return {flops, rw_bytes, dtype, zero_cost};
 }
 
+// Structural check of the flattened tables on the host (apc_validate_tables_host; the kernels
+// trust their indices): CPU tensors, RuntimeError naming the first malformed row
+// (non-monotone pointers, placement codes out of range, rank above the maximum, tiles that
+// leave their edge, ...).
+template <typename T>
+const T *host(const Tensor &t, at::ScalarType dtype, const char *name) {
+  TORCH_CHECK(t.defined() && t.device().is_cpu(), "apcost: ", name, " must be a CPU tensor (host-side validation)");
+  TORCH_CHECK(t.scalar_type() == dtype, "apcost: ", name, " must be ", dtype, " (got ", t.scalar_type(), ")");
+  TORCH_CHECK(t.is_contiguous(), "apcost: ", name, " must be contiguous");
+  return t.numel() ? static_cast<const T *>(t.data_ptr()) : nullptr;
+}
+
+void validate_tables(const Tensor &params, const Tensor &tensor_rank, const Tensor &spec_codes, const Tensor &spec_tensor,
+                     const Tensor &edge_src_begin, const Tensor &edge_n_src, const Tensor &edge_tgt_begin,
+                     const Tensor &edge_n_tgt, const Tensor &edge_flags, const Tensor &edge_pt_begin,
+                     const Tensor &edge_entry_begin, const Tensor &edge_strat_begin, int64_t n_pt, int64_t n_strategies,
+                     const Tensor &tiles, const Tensor &dup_entry_begin) {
+  const apc_params p = params_of(params);
+  const int64_t n_edges = edge_src_begin.numel();
+  for (const Tensor *t : {&edge_n_src, &edge_tgt_begin, &edge_n_tgt, &edge_flags, &edge_pt_begin, &edge_strat_begin})
+    TORCH_CHECK(t->numel() == n_edges, "apcost: the edge arrays must have one row per edge (", n_edges, ")");
+  TORCH_CHECK(edge_entry_begin.numel() == n_edges + 1, "apcost: edge_entry_begin needs n_edges + 1 rows");
+  TORCH_CHECK(spec_tensor.numel() == spec_codes.numel(), "apcost: spec_tensor and spec_codes differ in length");
+  constexpr int64_t kWords = sizeof(apc_tile) / 4;
+  TORCH_CHECK(tiles.numel() % kWords == 0, "apcost: tiles must be [n_tiles, ", kWords, "] int32 words (struct apc_tile)");
+  const int rc = apc_validate_tables_host(
+      &p, tensor_rank.numel(), host<int32_t>(tensor_rank, at::kInt, "tensor_rank"), spec_codes.numel(),
+      reinterpret_cast<const uint32_t *>(host<int32_t>(spec_codes, at::kInt, "spec_codes")), host<int32_t>(spec_tensor, at::kInt, "spec_tensor"),
+      n_edges, host<int32_t>(edge_src_begin, at::kInt, "edge_src_begin"), host<int32_t>(edge_n_src, at::kInt, "edge_n_src"),
+      host<int32_t>(edge_tgt_begin, at::kInt, "edge_tgt_begin"), host<int32_t>(edge_n_tgt, at::kInt, "edge_n_tgt"),
+      host<int32_t>(edge_flags, at::kInt, "edge_flags"), host<int64_t>(edge_pt_begin, at::kLong, "edge_pt_begin"),
+      host<int64_t>(edge_entry_begin, at::kLong, "edge_entry_begin"), host<int32_t>(edge_strat_begin, at::kInt, "edge_strat_begin"), n_pt,
+      n_strategies, tiles.numel() / kWords, reinterpret_cast<const apc_tile *>(host<int32_t>(tiles, at::kInt, "tiles")),
+      dup_entry_begin.numel(), host<int64_t>(dup_entry_begin, at::kLong, "dup_entry_begin"));
+  check_rc(rc, "apc_validate_tables_host");
+}
+
 int64_t abi_version() { return apc_version(); }
 
 }  // namespace
@@ -641,6 +678,10 @@ TORCH_LIBRARY(apcost, m) {
   "Tensor? comm, Tensor? transition, Tensor? cost, Tensor? edge_row_begin, Tensor? dup_row_begin, Tensor? row_min, " \
   "Tensor? row_argmin"
   m.def("abi_version() -> int", &abi_version);
+  m.def("validate_tables(Tensor params, Tensor tensor_rank, Tensor spec_codes, Tensor spec_tensor, Tensor edge_src_begin, "
+        "Tensor edge_n_src, Tensor edge_tgt_begin, Tensor edge_n_tgt, Tensor edge_flags, Tensor edge_pt_begin, "
+        "Tensor edge_entry_begin, Tensor edge_strat_begin, int n_pt, int n_strategies, Tensor tiles, Tensor dup_entry_begin) -> ()",
+        &validate_tables);
   m.def("tensor_tables(" APCOST_TENSOR_TABLE ") -> (Tensor tensor_bytes, Tensor tensor_contiguous)", &tensor_tables);
   m.def("shard_shapes_bytes(Tensor params, Tensor spec_codes, Tensor spec_tensor, " APCOST_TENSOR_TABLE
         ", int shape_width) -> (Tensor num_shards, Tensor local_shape, Tensor local_stride, Tensor local_numel, Tensor local_bytes)",

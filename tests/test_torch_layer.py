@@ -13,7 +13,7 @@ from oracle import c_oracle
 from oracle import cost_oracle as po
 
 OPERATORS = (
-    "abi_version", "tensor_tables", "shard_shapes_bytes", "strategy_inputs", "compute_cost", "segmented_min", "cost_objective",
+    "abi_version", "validate_tables", "tensor_tables", "shard_shapes_bytes", "strategy_inputs", "compute_cost", "segmented_min", "cost_objective",
     "redistribute_cost_tables", "strategy_bounds", "diffusion_sweeps_", "bind_tensor_tables", "bind_spec_tables",
     "bind_compute_costs", "bind_segmented_min", "bind_redistribute_tables", "bind_input_tables", "bind_cost_tables",
 )
@@ -131,3 +131,40 @@ def test_a_bound_launch_follows_the_current_stream(small_table, gpu_device):
         launch(side)
     side.synchronize()
     assert np.array_equal(dev.cost.cpu().numpy(), want["cost"])
+
+
+def _host_tables(tb):
+    from autoparallel_amd.device_tables import _to_device
+
+    names = ("tensor_rank", "spec_codes", "spec_tensor", "edge_src_begin", "edge_n_src", "edge_tgt_begin", "edge_n_tgt",
+             "edge_flags", "edge_pt_begin", "edge_entry_begin", "edge_strat_begin")
+    t = [_to_device(np.ascontiguousarray(getattr(tb, k)), "cpu") for k in names]
+    return t, _to_device(tb.tile_records, "cpu"), _to_device(np.ascontiguousarray(tb.dup_entry_begin), "cpu")
+
+
+@pytest.mark.parametrize("mutate, message", [
+    (None, None),
+    (lambda t: t.tensor_rank.__setitem__(0, 9), "rank"),                                            # rank above the maximum
+    (lambda t: t.spec_codes.__setitem__(0, 0xC0), "no meaning"),                                    # placement code out of range
+    (lambda t: t.spec_codes.__setitem__(0, 0x800000), "beyond mesh ndim"),
+    (lambda t: t.edge_entry_begin.__setitem__(2, int(t.edge_entry_begin[2]) + 1), "entry_begin"),  # pointer that does not follow the sizes
+    (lambda t: t.edge_src_begin.__setitem__(1, t.n_specs), "producer spec range"),
+])
+def test_malformed_tables_raise_runtime_error_through_the_operator(mutate, message):
+    """The host-side validator behind ``torch.ops.apcost.validate_tables``: malformed flattened
+    tables (rank above the maximum, placement codes without a meaning, pointers that do not
+    follow the sizes, ranges outside a table) are RuntimeErrors that name the row."""
+    ops = _native.torch_ops()
+    tb = stress_dag(seed=3, n_nodes=30, mesh_sizes=(4, 2), max_strategies=6)
+    tb.build_tiles()
+    if mutate is not None:
+        mutate(tb)
+        tb.pack_tile_records()
+    arrays, tiles, dups = _host_tables(tb)
+    params = _native.params_tensor(CostModelParams.from_mesh((4, 2)).to_c())
+    call = lambda: ops.validate_tables(params, *arrays, len(tb.pt_values), tb.n_strategies, tiles, dups)  # noqa: E731
+    if mutate is None:
+        call()
+    else:
+        with pytest.raises(RuntimeError, match=message):
+            call()
