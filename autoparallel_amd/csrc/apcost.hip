@@ -589,9 +589,6 @@ __host__ __device__ constexpr uint32_t pair_action(int c, int t) {
   if (c == 1) return t == 0 ? AR : (RS | (tn << 3) | UPD);
   return t == 0 ? (AG | (cn << 3) | UPD) : (A2A | ((cn + tn) << 3));
 }
-__host__ __device__ constexpr uint32_t pair_row(int c) {
-  return pair_action(c, 0) | (pair_action(c, 1) << 8) | (pair_action(c, 2) << 16) | (pair_action(c, 3) << 24);
-}
 __device__ __forceinline__ int placement_class(uint32_t code) {
   const int k = kind_of(code);
   return k == 2 ? 2 + (dim_of(code) != 0 ? 1 : 0) : k;
