@@ -6,6 +6,10 @@ current stream and device guard on the C++ side).
 torch is used for device memory and streams only; every computation is a kernel of the
 library.  Without a HIP device (or without the built libraries) construction raises: there
 is no CPU path.
+
+Every method that allocates, launches or copies runs on the package's device thread
+(``_device_thread``), where no dispatch mode of the caller (a graph capture's fake-tensor
+mode) is active; the launchers of ``prepare_step`` enqueue from whichever thread calls them.
 """
 
 from __future__ import annotations
@@ -14,6 +18,7 @@ import numpy as np
 import torch
 
 from . import _native
+from ._device_thread import on_device_thread as _guarded
 from .cost_model import CostModelParams
 from .encoding import CostTables
 
@@ -24,25 +29,6 @@ _UPLOAD = (
     "edge_entry_begin", "edge_strat_begin", "pt_values", "tile_records", "dup_entry_begin",
     "dup_row_begin",
 )
-
-
-def _real_tensors():
-    """The planner is usually called while a graph-capture context keeps a FakeTensorMode
-    (or another dispatch mode) active; device buffers must be real allocations."""
-    from torch.utils._python_dispatch import _disable_current_modes
-
-    return _disable_current_modes()
-
-
-def _guarded(fn):
-    import functools
-
-    @functools.wraps(fn)
-    def wrapper(*args, **kwargs):
-        with _real_tensors():
-            return fn(*args, **kwargs)
-
-    return wrapper
 
 
 def _to_device(a: np.ndarray, device) -> torch.Tensor:
@@ -394,6 +380,7 @@ class DeviceCostTables:
         return self.prepare_step(row_min=self.row_min_in_tiles_pays(), fused_inputs=True,
                                  outputs=self.PLANNER_OUTPUTS, spec_table=False)
 
+    @_guarded
     def check_error_flag(self):
         """After a synchronisation: raises if a strategy with flops had an unsupported dtype."""
         err = getattr(self, "_step_error_flag", None)
@@ -542,6 +529,7 @@ class DeviceCostTables:
                                    d["inc_edge"], d["inc_side"], d["edge_begin"], d["edge_i"], d["edge_j"], max_labels, th, un)
         return th.cpu().numpy(), un.cpu().numpy()
 
+    @_guarded
     def strategy_bounds(self, row_min: torch.Tensor) -> torch.Tensor:
         """Per-(node, strategy) sum of the row minima of the node's edges (``row_min`` in the
         order of ``CostTables.row_ptr()``)."""
@@ -557,6 +545,7 @@ class DeviceCostTables:
         return self.ops.strategy_bounds(ix["strat_node"], ix["node_strat_begin"], ix["node_edge_begin"], ix["edges_by_node"],
                                         ix["edge_row_begin"], row_min)
 
+    @_guarded
     def greedy_strategies(self, row_min: torch.Tensor):
         """-> (bound per strategy, min per node, argmin per node): the cheapest strategy of every
         node when each of its edges is charged its row minimum."""

@@ -37,6 +37,7 @@ import torch
 from torch.distributed.tensor._dtensor_spec import DTensorSpec
 from torch.distributed.tensor.placement_types import Placement, Replicate, Shard
 
+from ._device_thread import on_device_thread
 from .cost_model import CostModelParams
 from .graphs.cost_inputs import fill_flops_and_bytes, strategy_recipes
 from .graphs.encode import EncodedGraph, all_input_nodes, encode_graph
@@ -52,7 +53,10 @@ class DeviceBackend:
     The table pass is enqueued and left running while the host numbers the ILP variables;
     what comes back afterwards is one objective coefficient and one forced-to-zero flag per
     variable plus the per-strategy compute costs.  The per-entry arrays stay in HBM and are
-    copied (``comm`` and ``transition`` are even computed) only when a report asks for them."""
+    copied (``comm`` and ``transition`` are even computed) only when a report asks for them.
+
+    Methods that handle device tensors run on the package's device thread: the planner calls
+    them under the fake-tensor mode of its graph capture, which that thread does not see."""
 
     def __init__(self, tables, params: CostModelParams, device="cuda:0"):
         from .device_tables import DeviceCostTables
@@ -61,27 +65,23 @@ class DeviceBackend:
         self.timings = {}
         self.launches = ()
 
+    @on_device_thread
     def local_shapes(self):
-        from .device_tables import _real_tensors
+        out = self.dev.run_spec_tables()
+        return out["local_shape"].cpu().numpy(), out["local_stride"].cpu().numpy()
 
-        with _real_tensors():
-            out = self.dev.run_spec_tables()
-            return out["local_shape"].cpu().numpy(), out["local_stride"].cpu().numpy()
-
+    @on_device_thread
     def strategy_inputs(self, recipes):
         """Flop and byte counts of every strategy on the device (spec table, then
         ``apc_strategy_inputs`` over the per-node recipes); the host's strategy table receives
         copies (identical edges are found on the host, and flop / byte counts are part of an
         edge's identity)."""
-        from .device_tables import _real_tensors
-
-        with _real_tensors():
-            flops, rw_bytes, dtype, zero = self.dev.run_strategy_inputs(recipes)
-            tb = self.dev.tables
-            tb.strat_flops[:] = flops.cpu().numpy()
-            tb.strat_rw_bytes[:] = rw_bytes.cpu().numpy()
-            tb.strat_dtype[:] = dtype.cpu().numpy()
-            tb.strat_zero_cost[:] = zero.cpu().numpy()
+        flops, rw_bytes, dtype, zero = self.dev.run_strategy_inputs(recipes)
+        tb = self.dev.tables
+        tb.strat_flops[:] = flops.cpu().numpy()
+        tb.strat_rw_bytes[:] = rw_bytes.cpu().numpy()
+        tb.strat_dtype[:] = dtype.cpu().numpy()
+        tb.strat_zero_cost[:] = zero.cpu().numpy()
         self._strategy_inputs_on_device = True
 
     def upload_strategy_inputs(self, tables, tile_entries=None, dedupe=True, max_copies=16):
@@ -93,89 +93,77 @@ class DeviceBackend:
             names = ("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost") + names
         self.dev.refresh(*names)
 
+    @on_device_thread
     def launch_tables(self):
         """Enqueues the planner's table pass (``DeviceCostTables.planner_pass``) and returns."""
-        from .device_tables import _real_tensors
+        d = self.dev
+        step = d.planner_pass()
+        self.launches = tuple(step)
+        self._events = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+        with torch.cuda.device(d.device):
+            self._events[0].record()
+            for launch in step.values():
+                launch()
+            self._events[1].record()
 
-        with _real_tensors():
-            d = self.dev
-            step = d.planner_pass()
-            self.launches = tuple(step)
-            self._events = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-            with torch.cuda.device(d.device):
-                self._events[0].record()
-                for launch in step.values():
-                    launch()
-                self._events[1].record()
-
+    @on_device_thread
     def finish(self, n_vars, group_var_begin, group_member_begin, member_entry_begin):
         """Sums the ILP objective on the device and copies back what the planner needs:
         -> {"objective", "forced_zero", "compute", "compute_per_arg"} (host arrays)."""
-        from .device_tables import _real_tensors
-
-        with _real_tensors():
-            d = self.dev
-            with torch.cuda.device(d.device):
-                obj, forced = d.cost_objective(n_vars, group_var_begin, group_member_begin, member_entry_begin)
-                torch.cuda.synchronize(d.device)
-            d.check_error_flag()
-            self.timings["kernels_s"] = self._events[0].elapsed_time(self._events[1]) * 1e-3
-            t0 = time.perf_counter()
-            out = {
-                "objective": obj.cpu().numpy(),
-                "forced_zero": forced.cpu().numpy().astype(bool),
-                "compute": d.compute_cost.cpu().numpy(),
-                "compute_per_arg": d.compute_cost_per_arg.cpu().numpy(),
-            }
-            self.timings["copy_back_s"] = time.perf_counter() - t0
+        d = self.dev
+        with torch.cuda.device(d.device):
+            obj, forced = d.cost_objective(n_vars, group_var_begin, group_member_begin, member_entry_begin)
+            torch.cuda.synchronize(d.device)
+        d.check_error_flag()
+        self.timings["kernels_s"] = self._events[0].elapsed_time(self._events[1]) * 1e-3
+        t0 = time.perf_counter()
+        out = {
+            "objective": obj.cpu().numpy(),
+            "forced_zero": forced.cpu().numpy().astype(bool),
+            "compute": d.compute_cost.cpu().numpy(),
+            "compute_per_arg": d.compute_cost_per_arg.cpu().numpy(),
+        }
+        self.timings["copy_back_s"] = time.perf_counter() - t0
         for k in ("kernels_s", "copy_back_s"):
             logger.info("%s %.6f s", k, self.timings[k])
         return out
 
+    @on_device_thread
     def host_array(self, name):
         """``comm`` / ``transition`` / ``cost`` of every entry, copied (computed first, if the
         table pass did not write it) now."""
-        from .device_tables import _real_tensors
+        return self.dev.fetch(name).cpu().numpy()
 
-        with _real_tensors():
-            return self.dev.fetch(name).cpu().numpy()
-
+    @on_device_thread
     def gather(self, name, entries):
         """The values of a few entries of ``comm`` / ``transition`` / ``cost``."""
-        from .device_tables import _real_tensors
-
-        with _real_tensors():
-            idx = torch.from_numpy(np.ascontiguousarray(entries, np.int64)).to(self.dev.device)
-            return self.dev.fetch(name)[idx].cpu().numpy()
+        idx = torch.from_numpy(np.ascontiguousarray(entries, np.int64)).to(self.dev.device)
+        return self.dev.fetch(name)[idx].cpu().numpy()
 
     def diffusion_sweeps(self, graph, theta, unary, n_sweeps):
         """Sweeps of the dual ascent that prunes the program (pruning.py), on the device."""
         return self.dev.diffusion_sweeps(graph, theta, unary, n_sweeps)
 
+    @on_device_thread
     def row_min(self, row_ptr):
-        from .device_tables import _real_tensors
-
-        with _real_tensors():
-            if self._are_matrix_rows(row_ptr):  # taken by the table launch, or one read of every distinct row
-                mins, args = self.dev.row_minima()
-            else:
-                mins, args = self.dev.segmented_min(self.dev.fetch("cost"), row_ptr)
-            return mins.cpu().numpy(), args.cpu().numpy()
+        if self._are_matrix_rows(row_ptr):  # taken by the table launch, or one read of every distinct row
+            mins, args = self.dev.row_minima()
+        else:
+            mins, args = self.dev.segmented_min(self.dev.fetch("cost"), row_ptr)
+        return mins.cpu().numpy(), args.cpu().numpy()
 
     def _are_matrix_rows(self, row_ptr) -> bool:
         tb = self.dev.tables
         return len(row_ptr) == tb.n_rows + 1 and np.array_equal(row_ptr, tb.row_ptr())
 
+    @on_device_thread
     def greedy(self, row_ptr):
         """-> (bound per strategy, min per node, argmin per node) from the row minima of the cost table"""
-        from .device_tables import _real_tensors
-
-        with _real_tensors():
-            if self._are_matrix_rows(row_ptr):
-                mins, _ = self.dev.row_minima()
-            else:
-                mins, _ = self.dev.segmented_min(self.dev.fetch("cost"), row_ptr)
-            return tuple(x.cpu().numpy() for x in self.dev.greedy_strategies(mins))
+        if self._are_matrix_rows(row_ptr):
+            mins, _ = self.dev.row_minima()
+        else:
+            mins, _ = self.dev.segmented_min(self.dev.fetch("cost"), row_ptr)
+        return tuple(x.cpu().numpy() for x in self.dev.greedy_strategies(mins))
 
 
 class CostRecords(Mapping):

@@ -469,15 +469,16 @@ def measure(name, args, log, steps, warmup, main_run):
     import numpy as np
     import torch
 
-    from autoparallel_amd.device_tables import DeviceCostTables, _real_tensors
+    from autoparallel_amd._device_thread import call as on_device_thread
+    from autoparallel_amd.device_tables import DeviceCostTables
 
     t_setup = time.perf_counter()
     tables, params, desc, dev, planner, host_timings = build_workload(name, args)
-    # a traced workload keeps its capture context (a fake-tensor mode) open until the plan is
-    # solved; the measurements below work on real device buffers
-    guard = _real_tensors()
-    guard.__enter__()
-    try:
+
+    # a traced workload keeps its capture context (a fake-tensor mode) open in this thread until
+    # the plan is solved; the measurements work on real device buffers, so they run where the
+    # package's own device work runs
+    def on_real_tensors(dev):
         t0 = time.perf_counter()
         if dev is None:
             if args.tile_entries:
@@ -537,8 +538,9 @@ def measure(name, args, log, steps, warmup, main_run):
         }
         if main_run and not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline(tables, params, args.cpu_seconds)
-    finally:
-        guard.__exit__(None, None, None)
+        return out
+
+    out = on_device_thread(on_real_tensors, dev)
     return out, planner, tables, host_timings
 
 
@@ -599,12 +601,9 @@ def main():
     if "cpu_baseline" in out:
         result["cpu_baseline"] = out["cpu_baseline"]
     if not args.no_traffic:
-        from autoparallel_amd.device_tables import _real_tensors
-
-        with _real_tensors():
-            t0 = time.perf_counter()
-            read = measure_traffic(tables, out["params"], args.pass_kind, out["roofline"]["kernel"], log)
-            log.info("traffic reading: %.1f s", time.perf_counter() - t0)
+        t0 = time.perf_counter()
+        read = measure_traffic(tables, out["params"], args.pass_kind, out["roofline"]["kernel"], log)
+        log.info("traffic reading: %.1f s", time.perf_counter() - t0)
         if read is not None:
             result["roofline"].update(read)
             result["roofline"]["traffic_over_bytes_per_launch"] = read["traffic"] / result["roofline"]["bytes_per_launch"]

@@ -1,0 +1,89 @@
+"""The helper thread the planner's device work runs on: no dispatch mode of the caller is
+active there, nested calls run in place, exceptions and results come back unchanged, the
+caller's current stream is carried over."""
+
+import threading
+
+import pytest
+import torch
+from torch._subclasses.fake_tensor import FakeTensor, FakeTensorMode
+
+from autoparallel_amd import _device_thread
+from autoparallel_amd._device_thread import call, on_device_thread
+
+
+def test_caller_modes_are_not_active_on_the_device_thread():
+    def make():
+        t = torch.arange(4.0)
+        return t, threading.current_thread().name
+
+    with FakeTensorMode():
+        assert isinstance(torch.arange(4.0), FakeTensor)
+        t, name = call(make)
+    assert not isinstance(t, FakeTensor) and t.sum().item() == 6.0
+    assert name.startswith("apcost-device")
+
+
+def test_nested_calls_run_in_place_and_one_thread_serves_all():
+    seen = []
+
+    @on_device_thread
+    def inner():
+        seen.append(threading.get_ident())
+        return 7
+
+    @on_device_thread
+    def outer():
+        seen.append(threading.get_ident())
+        return inner() + 1  # would deadlock a one-worker pool if it were queued
+
+    assert outer() == 8 and inner() == 7
+    assert len(set(seen)) == 1 and seen[0] != threading.get_ident()
+    assert seen[0] == _device_thread._worker_ident
+
+
+def test_exceptions_come_back_to_the_caller():
+    class Marker(Exception):
+        pass
+
+    def fail():
+        raise Marker("from the device thread")
+
+    with pytest.raises(Marker, match="from the device thread"):
+        call(fail)
+    assert call(lambda: 3) == 3  # the thread survives
+
+
+def test_device_tables_fail_loudly_without_a_device():
+    if torch.cuda.is_available():
+        pytest.skip("a device is present")
+    from autoparallel_amd import CostModelParams
+    from autoparallel_amd.device_tables import DeviceCostTables
+    from autoparallel_amd.synthetic import stress_dag
+
+    tables = stress_dag(seed=1, n_nodes=20, mesh_sizes=(2, 2))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        DeviceCostTables(tables, CostModelParams.from_mesh((2, 2)))
+
+
+@pytest.mark.gpu
+def test_real_tables_under_a_fake_tensor_mode_and_the_callers_stream():
+    from autoparallel_amd import CostModelParams
+    from autoparallel_amd.device_tables import DeviceCostTables
+    from autoparallel_amd.synthetic import stress_dag
+
+    tables = stress_dag(seed=5, n_nodes=300, mesh_sizes=(4, 2))
+    params = CostModelParams.from_mesh((4, 2))
+    plain = DeviceCostTables(tables, params)
+    plain.build_all()
+    want = plain.cost.cpu()
+    side = torch.cuda.Stream()  # default priority
+    with FakeTensorMode():
+        dev = DeviceCostTables(tables, params)
+        with torch.cuda.stream(side):
+            dev.build_all()
+            seen = call(lambda: torch.cuda.current_stream().cuda_stream)
+        assert seen == side.cuda_stream
+        assert not isinstance(dev.cost, FakeTensor)
+    side.synchronize()
+    assert torch.equal(dev.cost.cpu(), want)
