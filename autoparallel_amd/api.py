@@ -50,6 +50,24 @@ class AutoParallelPlanner:
 
     def __enter__(self):
         assert self.active is False
+        # Capture and construction allocate millions of long-lived objects (graph nodes,
+        # strategies, specs): the cyclic collector's passes over them find nothing worth the
+        # time (5 % of the capture, and a pass over everything when it is switched on again).
+        # It is paused here, and what exists when construction ends is moved out of its sight
+        # (gc.freeze) until __exit__, so the solve's own collections stay short too.
+        import gc
+
+        collector_was_on = gc.isenabled()
+        gc.disable()
+        try:
+            return self._enter()
+        finally:
+            gc.freeze()
+            self._frozen = True
+            if collector_was_on:
+                gc.enable()
+
+    def _enter(self):
         t0 = time.perf_counter()
         self._ctx = capture_joint_graph(self.model, self.input_fn, param_dtype=self.param_dtype,
                                         device=self.trace_device, dynamo=self.dynamo)
@@ -75,6 +93,11 @@ class AutoParallelPlanner:
 
     def __exit__(self, *exc):
         self.active = None
+        if getattr(self, "_frozen", False):
+            import gc
+
+            self._frozen = False
+            gc.unfreeze()  # (the collector sees everything again; cycles left by planning go at its next pass)
         return self._ctx.__exit__(*exc)
 
     def add_parameter_memory_constraint(self, low=None, high=None):

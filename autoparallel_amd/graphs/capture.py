@@ -82,15 +82,16 @@ def cast_parameters_(model: nn.Module, dtype: torch.dtype) -> nn.Module:
 
 
 def cleanup_graph(gm: torch.fx.GraphModule) -> None:
+    """Dead code, no-op and assert removal on ``gm.graph``.  The module's Python code is not
+    regenerated here (a quarter of a second per pass on a 10 000-node graph, and planning only
+    reads the graph): the caller recompiles once when the graph is final."""
     from torch._inductor.fx_passes.post_grad import remove_assert_ops, remove_noop_ops
 
     gm.graph.eliminate_dead_code()
-    gm.recompile()
     remove_noop_ops(gm.graph)
     remove_assert_ops(gm.graph)
     gm.graph.eliminate_dead_code()
     gm.graph.lint()
-    gm.recompile()
 
 
 def add_alias_nodes(gm: torch.fx.GraphModule) -> torch.fx.GraphModule:
@@ -177,4 +178,6 @@ def capture_joint_graph(model: nn.Module, input_fn, param_dtype: torch.dtype | N
             cleanup_graph(gm)
             if add_aliases:
                 add_alias_nodes(gm)
+            else:
+                gm.recompile()
         yield gm, joint

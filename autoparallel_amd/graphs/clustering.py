@@ -50,8 +50,15 @@ def cluster_nodes(graph: torch.fx.Graph, strats: dict, rounds: int = 2) -> dict:
     """node -> representative node, for every call_function node that shares its final key
     with an earlier node (placeholders and the output node are never linked)."""
     interned: dict = {}
+    known: dict = {}  # (node, output_only) -> id: a producer is asked about once per consumer
 
     def strategy_id(node, output_only: bool) -> int:
+        found = known.get((node, output_only))
+        if found is None:
+            found = known[(node, output_only)] = intern_strategies(node, output_only)
+        return found
+
+    def intern_strategies(node, output_only: bool) -> int:
         s = strats[node]
         if not hasattr(s, "strategies"):
             return -1
