@@ -198,6 +198,38 @@ def test_parameter_smaller_than_the_mesh_stays_replicated(meshes):
             assert placement[node].output_specs.placements == (Replicate(),)
 
 
+def test_collector_is_paused_while_planning_and_restored_afterwards(meshes):
+    """Objects made by capture and construction are frozen out of the cyclic collector's sight
+    inside the ``with`` block and handed back at exit; the collector's on / off state is the
+    caller's again as soon as ``__enter__`` returns (also when construction raises)."""
+    import gc
+
+    mesh = meshes["1d"]
+    model_fn, input_fn = make_model_and_inputs(mesh, "small_param")
+    with torch.device("meta"):
+        model = model_fn()
+    gc.unfreeze()  # (a planner that an earlier test entered and never left)
+    assert gc.isenabled() and gc.get_freeze_count() == 0
+    with OraclePlanner(model, input_fn, mesh) as autop:
+        assert gc.isenabled() and gc.get_freeze_count() > 0
+        autop.add_input_constraints([(Shard(0),)])
+        autop.optimize_placement()
+    assert gc.isenabled() and gc.get_freeze_count() == 0
+
+    class Failing(OraclePlanner):
+        def _enter(self):
+            raise ValueError("construction failed")
+
+    gc.disable()
+    try:
+        with pytest.raises(ValueError, match="construction failed"):
+            Failing(model, input_fn, mesh).__enter__()
+        assert not gc.isenabled()
+    finally:
+        gc.unfreeze()
+        gc.enable()
+
+
 def test_unsolvable_problem_raises(meshes):
     model_fn, input_fn = make_model_and_inputs(meshes["2d"], "ffn")
     with torch.device("meta"):
