@@ -58,10 +58,21 @@ def cluster_nodes(graph: torch.fx.Graph, strats: dict, rounds: int = 2) -> dict:
             found = known[(node, output_only)] = intern_strategies(node, output_only)
         return found
 
+    by_origin: dict = {}  # nodes enumerated from one memo entry hold the same strategy list
+
     def intern_strategies(node, output_only: bool) -> int:
         s = strats[node]
         if not hasattr(s, "strategies"):
             return -1
+        origin = getattr(s, "_apc_origin", None)
+        if origin is None:
+            return intern_list(s, output_only)
+        found = by_origin.get((id(origin), output_only))
+        if found is None:
+            found = by_origin[(id(origin), output_only)] = intern_list(s, output_only)
+        return found
+
+    def intern_list(s, output_only: bool) -> int:
         rows = []
         for st in s.strategies:
             outs = st.output_specs

@@ -115,18 +115,46 @@ def encode_graph(graph: torch.fx.Graph, strats: dict, mesh_sizes, grad_param_nod
     spec_tensor: list = []
     spec_cache: dict = {}
 
-    def add_spec(spec) -> None:
+    def row_of(spec) -> tuple:
+        """(placement codes, tensor row) of a spec; (0, -1) for what is not a DTensorSpec"""
         if not isinstance(spec, DTensorSpec):
-            spec_codes.append(0)
-            spec_tensor.append(-1)
-            return
+            return 0, -1
         hit = spec_cache.get(id(spec))
         if hit is None:
             codes = pack_codes([coder.code(p) for p in spec.placements])
             hit = (codes, tensor_row(spec.tensor_meta))
             spec_cache[id(spec)] = hit
-        spec_codes.append(hit[0])
-        spec_tensor.append(hit[1])
+        return hit
+
+    def block_of(specs) -> tuple:
+        rows = [row_of(spec) for spec in specs]
+        return [r[0] for r in rows], [r[1] for r in rows]
+
+    def add_block(block) -> None:
+        spec_codes.extend(block[0])
+        spec_tensor.extend(block[1])
+
+    # Nodes enumerated from one memo entry (``_apc_origin``) share their OpSpec objects: their
+    # spec rows are worked out once and appended per node.
+    blocks_of_origin: dict = {}
+
+    def spec_blocks(strategy) -> tuple:
+        """-> (one block per output slot, one block per argument) of a node's strategies"""
+        origin = getattr(strategy, "_apc_origin", None)
+        if origin is not None:
+            hit = blocks_of_origin.get(id(origin))
+            if hit is not None:
+                return hit
+        strategies = strategy.strategies
+        outs0 = strategies[0].output_specs
+        if isinstance(outs0, (list, tuple)):
+            outs = [block_of([s.output_specs[slot] for s in strategies]) for slot in range(len(outs0))]
+        else:
+            outs = [block_of([s.output_specs for s in strategies])]
+        ins = [block_of([s.input_specs[argi] for s in strategies]) for argi in range(len(strategies[0].redistribute_cost))]
+        if origin is not None:
+            blocks_of_origin[id(origin)] = (outs, ins)
+        return outs, ins
 
     strat_begin: dict = {}
     output_spec_row: dict = {}
@@ -151,21 +179,14 @@ def encode_graph(graph: torch.fx.Graph, strats: dict, mesh_sizes, grad_param_nod
         na = len(strategies[0].input_specs)
         num_args[s_i] = na
         strat_num_args.extend([na] * len(strategies))
-        outs0 = strategies[0].output_specs
-        if isinstance(outs0, (list, tuple)):
-            for slot in range(len(outs0)):
-                output_spec_row[(s_i, slot)] = len(spec_codes)
-                for s in strategies:
-                    add_spec(s.output_specs[slot])
-        else:
-            output_spec_row[(s_i, 0)] = len(spec_codes)
-            for s in strategies:
-                add_spec(s.output_specs)
+        outs, ins = spec_blocks(strats[node])
+        for slot, block in enumerate(outs):
+            output_spec_row[(s_i, slot)] = len(spec_codes)
+            add_block(block)
         for argi, row in enumerate(strategies[0].redistribute_cost):
             num_inp_out[(s_i, argi)] = {"num_input_strat": len(row), "num_output_strat": len(strategies)}
             input_spec_row[(s_i, argi)] = len(spec_codes)
-            for s in strategies:
-                add_spec(s.input_specs[argi])
+            add_block(ins[argi])
 
     node_index = {n: i for i, n in enumerate(nodes)}
     # producer-less pseudo arguments read a block of always-invalid spec rows appended below

@@ -19,8 +19,9 @@ once on the node's fake arguments, strategies that shard a dim unevenly are drop
 duplicates (same input and output specs) are removed, first occurrence kept.
 
 Transformer layers repeat: results are memoised on (op, the input strategies' output
-specs, the non-tensor arguments), and a hit hands out fresh ``OpSpec`` shells (own
-``redistribute_cost`` lists) around the shared spec objects.
+specs, the non-tensor arguments), and every node with the same key gets its own
+``OpStrategy`` around the memo entry's ``OpSpec`` objects (shared read-only;
+``StrategyEnumerator.own_specs`` un-shares a node's before anything is written into them).
 """
 
 from __future__ import annotations
@@ -272,9 +273,16 @@ class StrategyEnumerator:
             val = x.meta.get("val")
             meta = (tuple(val.shape), tuple(val.stride()), val.dtype) if isinstance(val, torch.Tensor) else repr(val)
             s = strats[x]
-            if not hasattr(s, "_apc_sig"):
-                s._apc_sig = self._signature(s)
-            return ("node", s._apc_sig, meta)
+            sig = getattr(s, "_apc_sig", None)
+            if sig is None:
+                origin = getattr(s, "_apc_origin", None)  # (the same list for every node of the memo entry)
+                sig = getattr(origin, "_apc_sig", None) if origin is not None else None
+                if sig is None:
+                    sig = self._signature(s)
+                    if origin is not None:
+                        origin._apc_sig = sig
+                s._apc_sig = sig
+            return ("node", sig, meta)
         if isinstance(x, (list, tuple)):
             return (type(x).__name__,) + tuple(self._arg_key(y, strats) for y in x)
         if isinstance(x, dict):
@@ -283,13 +291,26 @@ class StrategyEnumerator:
 
     @staticmethod
     def _fresh_copy(strategy: OpStrategy) -> OpStrategy:
-        out = []
-        for s in strategy.strategies:
-            # the outer list is the node's own (rows are replaced per argument when the computed
-            # costs are written back); the rows themselves are shared read-only with the memo
-            rc = None if s.redistribute_cost is None else list(s.redistribute_cost)
-            out.append(OpSpec(s.output_specs, input_specs=s.input_specs, redistribute_cost=rc))
-        return OpStrategy(out)
+        """The node's own OpStrategy around the memo's OpSpec objects, which every node with
+        the same key shares read-only (a planner that writes costs into
+        ``OpSpec.redistribute_cost`` un-shares them first: ``own_specs``).  ``_apc_origin``
+        names the memo entry, so that later passes (output signature, clustering key, spec
+        encoding) do per distinct strategy list what they would otherwise do per node."""
+        out = OpStrategy(list(strategy.strategies))
+        out._apc_origin = strategy
+        return out
+
+    @staticmethod
+    def own_specs(strategy: OpStrategy) -> None:
+        """Replaces the shared OpSpec objects of a node's OpStrategy by copies of its own (with
+        their own ``redistribute_cost`` lists)."""
+        if getattr(strategy, "_apc_origin", None) is None:
+            return
+        strategy.strategies = [
+            OpSpec(s.output_specs, input_specs=s.input_specs,
+                   redistribute_cost=None if s.redistribute_cost is None else list(s.redistribute_cost))
+            for s in strategy.strategies]
+        strategy._apc_origin = None
 
     def _placeholder(self, val) -> OpStrategy:
         key = ("placeholder", tuple(val.shape), tuple(val.stride()), val.dtype)

@@ -35,6 +35,7 @@ from typing import Optional
 import numpy as np
 import torch
 from torch.distributed.tensor._dtensor_spec import DTensorSpec
+from torch.distributed.tensor._op_schema import OpStrategy
 from torch.distributed.tensor.placement_types import Placement, Replicate, Shard
 
 from ._device_thread import on_device_thread
@@ -506,15 +507,22 @@ class ShardingOptimizer:
         begin = tb.edge_entry_begin.astype(np.int64)
         sizes = begin[1:] - begin[:-1]
         edge_rep = np.arange(n_edges, dtype=np.int64)
+        edge_of = self.encoded.edge_of
+        linked, roots = [], []
         for node, rep in self.node_representative.items():
             s1, s0 = self.node_map[node], self.node_map[rep]
             assert self.num_args[s1] == self.num_args[s0], f"clustering linked {node} and {rep} with different arity"
             for argi in range(self.num_args[s1]):
-                e1, e0 = self.encoded.edge_of[(s1, argi)], self.encoded.edge_of[(s0, argi)]
-                assert (tb.edge_n_tgt[e1], tb.edge_n_src[e1]) == (tb.edge_n_tgt[e0], tb.edge_n_src[e0]), (
-                    f"Problem with graph clustering: {rep} and {node} don't have the same number of input/output "
-                    "placements. Please report a bug")
-                edge_rep[e1] = e0
+                linked.append(edge_of[(s1, argi)])
+                roots.append(edge_of[(s0, argi)])
+        linked, roots = np.asarray(linked, np.int64), np.asarray(roots, np.int64)
+        differ = (tb.edge_n_tgt[linked] != tb.edge_n_tgt[roots]) | (tb.edge_n_src[linked] != tb.edge_n_src[roots])
+        if differ.any():
+            e1, e0 = int(linked[differ][0]), int(roots[differ][0])
+            node, rep = (self.nodes[self.encoded.edge_keys[e][0]] for e in (e1, e0))
+            raise AssertionError(f"Problem with graph clustering: {rep} and {node} don't have the same number of "
+                                 "input/output placements. Please report a bug")
+        edge_rep[linked] = roots
         while not np.array_equal(edge_rep[edge_rep], edge_rep):  # representatives are roots already; be safe
             edge_rep = edge_rep[edge_rep]
         is_root = edge_rep == np.arange(n_edges)
@@ -531,21 +539,23 @@ class ShardingOptimizer:
         self.choice_var_of_strategy = None
         self.node_choice_base = {}
         if self.node_choice_variables:
-            sb = self.encoded.strat_begin
-            choice = np.zeros(tb.n_strategies, np.int64)
-            next_free = self.n_variables
-            for s_i, node in enumerate(self.nodes):
-                if node.op == "output" or node in self.node_representative:
-                    continue
-                n = len(self.strats[node].strategies)
-                self.node_choice_base[s_i] = next_free
-                choice[sb[s_i]:sb[s_i] + n] = np.arange(next_free, next_free + n)
-                next_free += n
+            # the strategies of every node that represents itself, numbered in node order; a linked
+            # node's strategies take its representative's numbers
+            nsb = np.asarray(tb.node_strat_begin, np.int64)
+            n_strat = nsb[1:] - nsb[:-1]
+            own = np.array([node.op != "output" and node not in self.node_representative for node in self.nodes], bool)
+            node_base = np.full(len(self.nodes), -1, np.int64)
+            node_base[own] = self.n_variables + np.cumsum(n_strat[own]) - n_strat[own]
+            next_free = self.n_variables + int(n_strat[own].sum())
             for node, rep in self.node_representative.items():
                 s1, s0 = self.node_map[node], self.node_map[rep]
-                n = len(self.strats[node].strategies)
-                self.node_choice_base[s1] = self.node_choice_base[s0]
-                choice[sb[s1]:sb[s1] + n] = choice[sb[s0]:sb[s0] + n]
+                assert n_strat[s1] == n_strat[s0]
+                node_base[s1] = node_base[s0]
+            has = node_base >= 0
+            self.node_choice_base = {int(s_i): int(node_base[s_i]) for s_i in np.nonzero(has)[0]}
+            strat_node = np.repeat(np.arange(len(self.nodes)), n_strat)
+            choice = node_base[strat_node] + (np.arange(tb.n_strategies, dtype=np.int64) - nsb[:-1][strat_node])
+            choice[~has[strat_node]] = 0
             self.choice_var_of_strategy = choice
             self.n_choice_variables = next_free - self.n_variables
 
@@ -556,6 +566,9 @@ class ShardingOptimizer:
         is made only on request, or at construction with ``write_back_redistribute_cost = True``."""
         tb = self.encoded.tables
         comm = self.comm_cost
+        for strategy in self.strats.values():  # nodes of one memo entry share their OpSpec objects until now
+            if isinstance(strategy, OpStrategy):
+                StrategyEnumerator.own_specs(strategy)
         for e, (s_i, argi) in enumerate(self.encoded.edge_keys):
             ns, nt = int(tb.edge_n_src[e]), int(tb.edge_n_tgt[e])
             b = int(tb.edge_entry_begin[e])

@@ -198,6 +198,34 @@ def test_parameter_smaller_than_the_mesh_stays_replicated(meshes):
             assert placement[node].output_specs.placements == (Replicate(),)
 
 
+def test_cost_rows_are_written_into_specs_each_node_owns(meshes):
+    """optimize_sharding.py:361-363 on request: ``OpSpec.redistribute_cost[argi][ii]`` of every
+    strategy holds the recomputed communication cost.  Nodes enumerated from one memo entry
+    share their OpSpec objects until then; the write-back gives each node its own."""
+    mesh = meshes["2d"]
+    model_fn, input_fn = make_model_and_inputs(mesh, "block")
+    with torch.device("meta"):
+        model = model_fn()
+    with OraclePlanner(model, input_fn, mesh) as autop:
+        opt = autop.sharding_optimizer
+        nodes = [n for n in opt.nodes if n.op != "output"]
+        shared_before = len({id(s) for n in nodes for s in opt.strats[n].strategies})
+        total = sum(len(opt.strats[n].strategies) for n in nodes)
+        assert shared_before < total  # (some nodes do share: the memo had hits)
+        opt.materialize_redistribute_costs()
+        assert len({id(s) for n in nodes for s in opt.strats[n].strategies}) == total
+        tb, comm = opt.encoded.tables, opt.comm_cost
+        for e, (s_i, argi) in enumerate(opt.encoded.edge_keys):
+            ns, nt, b = int(tb.edge_n_src[e]), int(tb.edge_n_tgt[e]), int(tb.edge_entry_begin[e])
+            rows = [s.redistribute_cost[argi] for s in opt.strats[opt.nodes[s_i]].strategies]
+            assert len(rows) == nt and all(len(r) == ns for r in rows)
+            assert np.array_equal(np.asarray(rows, np.float64).reshape(-1), comm[b:b + ns * nt])
+        # the plan is the same afterwards
+        autop.add_parameter_memory_constraint(low=0, high=None)
+        placement = autop.optimize_placement()
+        _check_2d(autop, placement, "block")
+
+
 def test_collector_is_paused_while_planning_and_restored_afterwards(meshes):
     """Objects made by capture and construction are frozen out of the cyclic collector's sight
     inside the ``with`` block and handed back at exit; the collector's on / off state is the
