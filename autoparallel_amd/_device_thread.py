@@ -54,6 +54,12 @@ def call(fn, *args, **kwargs):
     return _executor().submit(task).result()
 
 
+def submit(fn, *args, **kwargs):
+    """Queues ``fn(*args, **kwargs)`` on the device thread and returns its future without
+    waiting (work that may overlap the caller's: the device's first-use costs)."""
+    return _executor().submit(fn, *args, **kwargs)
+
+
 def on_device_thread(fn):
     """Decorator form of ``call``."""
 

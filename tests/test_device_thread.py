@@ -87,3 +87,25 @@ def test_real_tables_under_a_fake_tensor_mode_and_the_callers_stream():
         assert not isinstance(dev.cost, FakeTensor)
     side.synchronize()
     assert torch.equal(dev.cost.cpu(), want)
+
+
+def test_warm_up_returns_at_once_and_never_raises():
+    """The planner starts the device's first-use costs before it captures the graph; without a
+    device (or with one) the future completes with None and construction reports any problem."""
+    from autoparallel_amd.optimize_sharding import DeviceBackend
+
+    assert DeviceBackend.warm_up().result(timeout=120) is None
+
+
+@pytest.mark.gpu
+def test_tables_after_a_warm_up():
+    from autoparallel_amd import CostModelParams
+    from autoparallel_amd.device_tables import DeviceCostTables
+    from autoparallel_amd.optimize_sharding import DeviceBackend
+    from autoparallel_amd.synthetic import stress_dag
+
+    DeviceBackend.warm_up()  # (not waited for: the construction below queues behind it)
+    tables = stress_dag(seed=6, n_nodes=200, mesh_sizes=(4, 2))
+    dev = DeviceCostTables(tables, CostModelParams.from_mesh((4, 2)))
+    dev.build_all()
+    assert torch.isfinite(dev.compute_cost).all()
