@@ -1385,14 +1385,14 @@ __device__ __forceinline__ void tile_entries(const apc_params &p, const TableArg
 }
 
 template <int M, int kTileThreads, bool RM, int OUT>
-__device__ __forceinline__ void redistribute_tile(const apc_params &p, const TableArgs &a, int n_tiles, int xcd_shift,
-                                                  TileStage<M, RM> &stage) {
+__device__ __forceinline__ void redistribute_tile(const apc_params &p, const TableArgs &a, const apc_tile *tiles, int n_tiles,
+                                                  int xcd_shift, TileStage<M, RM> &stage) {
   const int64_t tile_id = xcd_chunked_unit(xcd_shift);
   if (tile_id >= n_tiles) return;
   static_assert(kTileThreads == 64 || kTileThreads == 128 || kTileThreads == 256, "wavefronts per tile: 1, 2 or 4");
   static_assert(kTileThreads >= APC_TILE_MAX_COLS && kTileThreads >= APC_TILE_MAX_ROWS &&
                 2 * kTileThreads > APC_TILE_MAX_DUPS, "one staging round covers a tile");
-  const apc_tile tile = a.tiles[tile_id];
+  const apc_tile tile = tiles[tile_id];
   stage_tile<M, false, RM>(p, a, tile, stage, threadIdx.x, kTileThreads);
   __syncthreads();
   tile_entries<M, false, RM, OUT>(p, a, stage, view_of(tile), threadIdx.x, kTileThreads);
@@ -1412,9 +1412,9 @@ constexpr int tile_waves_per_simd(int mesh_ndim, int threads) {
 
 template <int M, int kTileThreads, int OUT>
 __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads), 8)))
-void redistribute_tiles_kernel(apc_params p, TableArgs a, int n_tiles, int xcd_shift) {
+void redistribute_tiles_kernel(const apc_tile *tiles, int n_tiles, int xcd_shift, apc_params p, TableArgs a) {
   extern __shared__ __align__(16) unsigned char s_stage_bytes[];  // stage_lds_bytes<M, false>
-  redistribute_tile<M, kTileThreads, false, OUT>(p, a, n_tiles, xcd_shift,
+  redistribute_tile<M, kTileThreads, false, OUT>(p, a, tiles, n_tiles, xcd_shift,
                                                  *reinterpret_cast<TileStage<M, false> *>(s_stage_bytes));
 }
 
@@ -1422,9 +1422,9 @@ void redistribute_tiles_kernel(apc_params p, TableArgs a, int n_tiles, int xcd_s
 template <int M, int kTileThreads, int OUT>
 __global__ __launch_bounds__(kTileThreads)
 __attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads), 8)))
-void redistribute_tiles_row_min_kernel(apc_params p, TableArgs a, int n_tiles, int xcd_shift) {
+void redistribute_tiles_row_min_kernel(const apc_tile *tiles, int n_tiles, int xcd_shift, apc_params p, TableArgs a) {
   extern __shared__ __align__(16) unsigned char s_stage_bytes[];  // stage_lds_bytes<M, true>
-  redistribute_tile<M, kTileThreads, true, OUT>(p, a, n_tiles, xcd_shift,
+  redistribute_tile<M, kTileThreads, true, OUT>(p, a, tiles, n_tiles, xcd_shift,
                                                 *reinterpret_cast<TileStage<M, true> *>(s_stage_bytes));
 }
 
@@ -1442,10 +1442,9 @@ void redistribute_tiles_row_min_kernel(apc_params p, TableArgs a, int n_tiles, i
 // uncapped; 20.3 us capped at 3 or when asked for 8.  The mixture-of-experts table: no change.)
 template <int M, int kThreads, bool RM, int OUT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(M <= 2 ? 5 : 1, M <= 2 ? 5 : 8)))
-void build_tables_kernel(apc_params p, TableArgs a, TensorTableArgs t,
-                                                                SpecTableArgs sp, ComputeCostArgs c, int n_tiles,
-                                                                int64_t tile_blocks, int64_t spec_blocks,
-                                                                int64_t tensor_blocks, int xcd_shift) {
+void build_tables_kernel(const apc_tile *tiles, int n_tiles, int xcd_shift, int64_t tile_blocks, apc_params p, TableArgs a,
+                         TensorTableArgs t, SpecTableArgs sp, ComputeCostArgs c, int64_t spec_blocks,
+                         int64_t tensor_blocks) {
   constexpr size_t kRowBytes = (size_t)kThreads * (APC_MAX_RANK + 1) * sizeof(int64_t);
   constexpr size_t kLds = sizeof(TileStage<M, RM>) > kRowBytes ? sizeof(TileStage<M, RM>) : kRowBytes;
   __shared__ __align__(16) unsigned char s_raw[kLds];
@@ -1456,7 +1455,7 @@ void build_tables_kernel(apc_params p, TableArgs a, TensorTableArgs t,
     const int64_t tile_id = (b & ((1 << xcd_shift) - 1)) * per + (b >> xcd_shift);
     if (tile_id >= n_tiles) return;
     TileStage<M, RM> &stage = *reinterpret_cast<TileStage<M, RM> *>(s_raw);
-    const apc_tile tile = a.tiles[tile_id];
+    const apc_tile tile = tiles[tile_id];
     stage_tile<M, true, RM>(p, a, tile, stage, threadIdx.x, kThreads);
     __syncthreads();
     tile_entries<M, true, RM, OUT>(p, a, stage, view_of(tile), threadIdx.x, kThreads);
@@ -2049,9 +2048,9 @@ static int redistribute_tables_impl(const apc_params *params, const int64_t *ten
   const int om = out_mode(params->mesh_ndim, comm_out, trans_out, cost_out);
 #define APC_LAUNCH_T(KERNEL_, M_, OUT_)                                                                               \
   const size_t lds = rows ? stage_lds_bytes<M_, true>(a.lay) : stage_lds_bytes<M_, false>(a.lay);                      \
-  if (threads >= 256) hipLaunchKernelGGL((KERNEL_<M_, 256, OUT_>), grid, dim3(256), lds, s, *params, a, nt, xs);      \
-  else if (threads >= 128) hipLaunchKernelGGL((KERNEL_<M_, 128, OUT_>), grid, dim3(128), lds, s, *params, a, nt, xs); \
-  else hipLaunchKernelGGL((KERNEL_<M_, 64, OUT_>), grid, dim3(64), lds, s, *params, a, nt, xs)
+  if (threads >= 256) hipLaunchKernelGGL((KERNEL_<M_, 256, OUT_>), grid, dim3(256), lds, s, a.tiles, nt, xs, *params, a);      \
+  else if (threads >= 128) hipLaunchKernelGGL((KERNEL_<M_, 128, OUT_>), grid, dim3(128), lds, s, a.tiles, nt, xs, *params, a); \
+  else hipLaunchKernelGGL((KERNEL_<M_, 64, OUT_>), grid, dim3(64), lds, s, a.tiles, nt, xs, *params, a)
 #define APC_LAUNCH_K(KERNEL_, M_)                                   \
   if (om == kOutAll) { APC_LAUNCH_T(KERNEL_, M_, kOutAll); }        \
   else if (om == kOutCost) { APC_LAUNCH_T(KERNEL_, M_, kOutCost); } \
@@ -2132,9 +2131,9 @@ static int build_tables_impl(const apc_params *params, int64_t n_tensors, const 
   const int nt = (int)n_tiles;
   const int om = out_mode(params->mesh_ndim, comm_out, trans_out, cost_out);
 #define APC_LAUNCH_ALL_T(M_, RM_, OUT_)                                                                                 \
-  if (threads == 256) hipLaunchKernelGGL((build_tables_kernel<M_, 256, RM_, OUT_>), grid, dim3(256), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
-  else if (threads == 128) hipLaunchKernelGGL((build_tables_kernel<M_, 128, RM_, OUT_>), grid, dim3(128), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs); \
-  else hipLaunchKernelGGL((build_tables_kernel<M_, 64, RM_, OUT_>), grid, dim3(64), 0, s, *params, a, ta, sa, ca, nt, tile_blocks, sb, tb, xs)
+  if (threads == 256) hipLaunchKernelGGL((build_tables_kernel<M_, 256, RM_, OUT_>), grid, dim3(256), 0, s, a.tiles, nt, xs, tile_blocks, *params, a, ta, sa, ca, sb, tb); \
+  else if (threads == 128) hipLaunchKernelGGL((build_tables_kernel<M_, 128, RM_, OUT_>), grid, dim3(128), 0, s, a.tiles, nt, xs, tile_blocks, *params, a, ta, sa, ca, sb, tb); \
+  else hipLaunchKernelGGL((build_tables_kernel<M_, 64, RM_, OUT_>), grid, dim3(64), 0, s, a.tiles, nt, xs, tile_blocks, *params, a, ta, sa, ca, sb, tb)
 #define APC_LAUNCH_ALL_RM(M_, RM_)                                   \
   if (om == kOutAll) { APC_LAUNCH_ALL_T(M_, RM_, kOutAll); }         \
   else if (om == kOutCost) { APC_LAUNCH_ALL_T(M_, RM_, kOutCost); }  \
