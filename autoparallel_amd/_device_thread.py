@@ -15,6 +15,7 @@ caller unchanged.
 from __future__ import annotations
 
 import functools
+import os
 import threading
 from concurrent.futures import ThreadPoolExecutor
 
@@ -35,6 +36,16 @@ def _executor() -> ThreadPoolExecutor:
             _pool = ThreadPoolExecutor(max_workers=1, thread_name_prefix="apcost-device",
                                        initializer=_remember_ident)
         return _pool
+
+
+def _forget_thread():
+    # a forked child has the parent's pool object but none of its threads
+    global _pool, _worker_ident
+    _pool = None
+    _worker_ident = None
+
+
+os.register_at_fork(after_in_child=_forget_thread)
 
 
 def call(fn, *args, **kwargs):

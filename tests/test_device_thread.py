@@ -109,3 +109,27 @@ def test_tables_after_a_warm_up():
     dev = DeviceCostTables(tables, CostModelParams.from_mesh((4, 2)))
     dev.build_all()
     assert torch.isfinite(dev.compute_cost).all()
+
+
+def test_a_forked_child_starts_its_own_thread():
+    import os
+
+    assert call(lambda: 1) == 1  # the parent's thread exists
+    r, w = os.pipe()
+    pid = os.fork()
+    if pid == 0:  # child: the parent's worker did not come along
+        try:
+            ok = call(lambda: threading.current_thread().name).startswith("apcost-device")
+            os.write(w, b"1" if ok else b"0")
+        finally:
+            os._exit(0)
+    os.close(w)
+    import select
+
+    ready, _, _ = select.select([r], [], [], 30)
+    got = os.read(r, 1) if ready else b"timeout"
+    os.close(r)
+    if not ready:
+        os.kill(pid, 9)
+    os.waitpid(pid, 0)
+    assert got == b"1"
