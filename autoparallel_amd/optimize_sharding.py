@@ -339,6 +339,15 @@ class ShardingOptimizer:
     prune_before_solve = True
     prune_sweep_chunks = (40, 40, 80, 80, 160)
     prune_gap = 2e-4
+    # Where the rounding does not reach the bound (the relaxation has a gap, or the ascent is not
+    # through: a mixture-of-experts graph has four times the classes of a Llama graph), the
+    # ascent goes on in doubling chunks while a chunk still lifts the bound by more than
+    # ``prune_gap / 4`` (relative), up to ``prune_max_sweeps`` in all; then the program is solved
+    # restricted to the variables whose bound is within a slack of the lower bound, slack =
+    # ``prune_slacks`` x |bound| in turn, capped by the incumbent's distance.  A restricted optimum
+    # that is itself within the slack is the optimum: everything left out costs more.
+    prune_max_sweeps = 3200
+    prune_slacks = (1e-4, 1e-3, 1e-2)
     # copy ``comm`` back and write it into every OpSpec.redistribute_cost at construction
     # (optimize_sharding.py:361-363); off: ``materialize_redistribute_costs()`` does it on request
     write_back_redistribute_cost = False
@@ -796,11 +805,17 @@ class ShardingOptimizer:
         obj[:self.n_variables] = self.objective_vector
         self.prob.objective = obj
         self.solve_stats = {"columns": int((self.prob.upper > 0).sum())}
+        self._solved_while_pruning = False
         if self.prune_before_solve and self.node_choice_variables:
             self.prune()
         t0 = time.perf_counter()
-        status = self.prob.solve(verbose=verbose, time_limit=self.solver_time_limit, mip_rel_gap=self.solver_rel_gap)
-        self.solve_stats.update(solver_s=time.perf_counter() - t0, solved_by=self.prob.solved_by,
+        if self._solved_while_pruning:  # (the restricted program's optimum, proven to be the program's)
+            status = self.prob.status
+            solver_s = self.solve_stats["near_bound_solver_s"]
+        else:
+            status = self.prob.solve(verbose=verbose, time_limit=self.solver_time_limit, mip_rel_gap=self.solver_rel_gap)
+            solver_s = time.perf_counter() - t0 + self.solve_stats.get("near_bound_solver_s", 0.0)
+        self.solve_stats.update(solver_s=solver_s, solved_by=self.prob.solved_by,
                                 columns_solved=getattr(self.prob, "cols_after_fixing", None))
         if status == -1:
             print(self.get_violated_constraints_log())
@@ -931,11 +946,14 @@ class ShardingOptimizer:
         return x
 
     def prune(self):
-        """Fixes to zero the variables that the bound proves to be in no optimal plan."""
+        """Fixes to zero the variables that the bound proves to be in no optimal plan; where the
+        incumbent stays above the bound, solves the program restricted to the variables near the
+        bound (``prune_slacks``) and keeps the solution once it is proven optimal."""
         from . import pruning
 
         t0 = time.perf_counter()
         stats = self.solve_stats
+        self._solved_while_pruning = False
         graph = self._label_graph()
         stats["prune_graph_s"] = time.perf_counter() - t0
         t_sweeps = t_round = 0.0
@@ -944,14 +962,19 @@ class ShardingOptimizer:
             return
         theta, unary = graph.theta.copy(), graph.unary.copy()
         best_ub, best_x, sweeps, bound = math.inf, None, 0, -math.inf
-        for chunk in self.prune_sweep_chunks:
+        chunks = list(self.prune_sweep_chunks)
+        k = 0
+        while k < len(chunks):
+            chunk = chunks[k]
+            k += 1
             t1 = time.perf_counter()
             theta, unary = self.backend.diffusion_sweeps(graph, theta, unary, chunk)
             t_sweeps += time.perf_counter() - t1
             t1 = time.perf_counter()
             sweeps += chunk
+            before = bound
             bound = pruning.lower_bound(graph, theta, unary)[0]
-            labels = pruning.decode(graph, theta, unary)
+            labels = pruning.refine(graph, theta, unary, pruning.decode(graph, theta, unary))
             x = self._plan_vector(graph, labels)
             if (x <= self.prob.upper).all() and not self.prob.violated_constraints(x):
                 ub = float(self.prob.objective @ x)
@@ -960,28 +983,80 @@ class ShardingOptimizer:
             t_round += time.perf_counter() - t1
             if best_ub - bound <= self.prune_gap * abs(best_ub):
                 break
+            if k == len(chunks) and sweeps + 2 * chunk <= self.prune_max_sweeps and \
+                    bound - before > 0.25 * self.prune_gap * abs(bound):
+                chunks.append(2 * chunk)  # the ascent is not through
         stats.update(prune_sweeps_s=t_sweeps, prune_rounding_s=t_round)
         stats.update(prune_sweeps=sweeps, lower_bound=bound, incumbent=best_ub if best_x is not None else None,
                      label_classes=graph.n_classes, label_edges=graph.n_edges)
         if best_x is not None:
-            dead_label, dead_pair = pruning.prune_masks(graph, theta, unary, best_ub)
-            lb = graph.label_begin
-            off = []
-            for c, bases in enumerate(graph.members):
-                d = np.nonzero(dead_label[lb[c]:lb[c + 1]])[0]
-                off.extend(cb + d for cb in bases)
-            for b in graph.blocks:
-                dead = dead_label[lb[b.row_class]:lb[b.row_class + 1]][:, None] & np.ones((1, b.ns), bool)
-                if b.col_class >= 0:
-                    pair = graph.matrix(dead_pair, b.edge)
-                    dead = dead | (pair.T if b.transposed else pair)
-                off.append(b.var_begin + np.nonzero(dead.ravel())[0])
-            off = np.concatenate(off) if off else np.zeros(0, np.int64)
-            assert not best_x[off].any(), "the incumbent uses a variable the bound rules out"
-            self.prob.force_zero(off)
             self.incumbent = best_x
+            state = (graph, theta, unary)
+            if best_ub - bound <= self.prune_gap * abs(best_ub) or not self.prune_slacks:
+                self._fix_above(state, best_ub, best_x)
+            else:
+                self._solve_near_the_bound(state, bound, best_ub, best_x)
         stats["columns_after_pruning"] = int((self.prob.upper > 0).sum())
         stats["prune_s"] = time.perf_counter() - t0
+
+    def _fix_above(self, state, limit, feasible_x=None):
+        """Upper bound 0 for every variable whose bound (min-marginal of its strategy / strategy
+        pair under the reparametrised costs) exceeds ``limit``."""
+        from . import pruning
+
+        graph, theta, unary = state
+        dead_label, dead_pair = pruning.prune_masks(graph, theta, unary, limit)
+        lb = graph.label_begin
+        off = []
+        for c, bases in enumerate(graph.members):
+            d = np.nonzero(dead_label[lb[c]:lb[c + 1]])[0]
+            off.extend(cb + d for cb in bases)
+        for b in graph.blocks:
+            dead = dead_label[lb[b.row_class]:lb[b.row_class + 1]][:, None] & np.ones((1, b.ns), bool)
+            if b.col_class >= 0:
+                pair = graph.matrix(dead_pair, b.edge)
+                dead = dead | (pair.T if b.transposed else pair)
+            off.append(b.var_begin + np.nonzero(dead.ravel())[0])
+        off = np.concatenate(off) if off else np.zeros(0, np.int64)
+        if feasible_x is not None:
+            assert not feasible_x[off].any(), "the incumbent uses a variable the bound rules out"
+        self.prob.force_zero(off)
+
+    def _solve_near_the_bound(self, state, bound, best_ub, best_x):
+        """Solves the program restricted to the variables whose bound is at most ``bound +
+        slack`` for growing slacks.  A plan that uses a variable left out costs more than ``bound
+        + slack``, so a restricted optimum of at most that value is an optimum of the full
+        program (and no optimal plan was left out).  The last slack is the incumbent's distance,
+        where that always holds: the incumbent itself lies inside."""
+        stats = self.solve_stats
+        upper0 = self.prob.upper.copy()
+        tries = []
+        t_solver = 0.0
+        for rel in tuple(self.prune_slacks) + (math.inf,):
+            slack = min(rel * abs(bound), best_ub - bound)
+            last = slack >= best_ub - bound
+            self.prob.upper = upper0.copy()
+            self._fix_above(state, bound + slack, best_x if last else None)
+            t1 = time.perf_counter()
+            status = self.prob.solve(time_limit=self.solver_time_limit, mip_rel_gap=self.solver_rel_gap)
+            dt = time.perf_counter() - t1
+            t_solver += dt
+            value = self.prob.objective_value if status == 1 else None
+            tries.append({"slack": slack, "columns": int(self.prob.cols_after_fixing), "seconds": dt, "value": value,
+                          "solved_by": self.prob.solved_by})
+            if value is not None and value <= bound + slack:
+                self._solved_while_pruning = True
+                break
+            if value is not None and value < best_ub:  # a better incumbent: the cap of the next slack
+                best_ub, best_x = value, self.prob.x.astype(np.float64)
+                self.incumbent = best_x
+            if last:
+                break
+        stats["near_bound_solves"] = tries
+        stats["near_bound_solver_s"] = t_solver
+        if not self._solved_while_pruning:  # (a solver time limit: leave the decision to the full solve)
+            self.prob.upper = upper0.copy()
+            self._fix_above(state, best_ub, best_x)
 
     def objective_value(self) -> float:
         return float(self._values("cost", self.res_entries).sum())

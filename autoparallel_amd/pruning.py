@@ -15,12 +15,16 @@ free:
     tables, applied to the reparametrised matrices) and hands the sum back in equal shares.
     Every update leaves the cost of every labelling unchanged and never lowers the bound
     ``LB = sum_classes min unary + sum_edges min matrix``;
-  * ``decode`` rounds the reparametrised costs to a labelling; if that labelling satisfies every
-    row of the program it is an incumbent with cost ``UB``;
+  * ``decode`` rounds the reparametrised costs to a labelling and ``refine`` improves it by local
+    search; if the labelling satisfies every row of the program it is an incumbent with cost ``UB``;
   * ``prune`` fixes to zero every strategy whose min-marginal bound, and every strategy pair
     whose entry bound, exceeds ``UB``: such a variable is in no optimal plan, so the set of
     optimal plans, and the optimum, are unchanged, and the solver receives a program a tenth
     (Llama-3-8B) of the size.
+
+Where the rounded labelling stays above the bound, the planner solves the program restricted to the
+variables whose bound lies within a slack of ``LB`` (``ShardingOptimizer._solve_near_the_bound``): an
+optimum of the restricted program that is itself within the slack is an optimum of the program.
 
 Constraints the labelling form does not model are simply left out of the bound (it stays a
 valid lower bound of the constrained program); the incumbent is checked against ALL rows.
@@ -183,6 +187,31 @@ def decode(g: LabelGraph, theta: np.ndarray, unary: np.ndarray) -> np.ndarray:
             other = int(g.edge_j[k]) if side == 0 else int(g.edge_i[k])
             score = score + (m[:, lab[other]] if lab[other] >= 0 else m.min(axis=1))
         lab[c] = int(np.argmin(score)) if len(score) else -1
+    return lab
+
+
+def refine(g: LabelGraph, theta: np.ndarray, unary: np.ndarray, labels: np.ndarray, max_rounds: int = 10) -> np.ndarray:
+    """Local search from a labelling: class by class, the label that is cheapest given the labels
+    of all its neighbours, until a round changes nothing.  Never raises the labelling's cost."""
+    lab = labels.copy()
+    lb = g.label_begin
+    for _ in range(max_rounds):
+        changed = False
+        for c in range(g.n_classes):
+            if lab[c] < 0:
+                continue
+            score = unary[lb[c]:lb[c + 1]].copy()
+            for t in range(int(g.inc_begin[c]), int(g.inc_begin[c + 1])):
+                k, side = int(g.inc_edge[t]), int(g.inc_side[t])
+                m = g.matrix(theta, k)
+                other = int(g.edge_j[k]) if side == 0 else int(g.edge_i[k])
+                score = score + (m[:, lab[other]] if side == 0 else m[lab[other], :])
+            best = int(np.argmin(score))
+            if score[best] < score[lab[c]]:
+                lab[c] = best
+                changed = True
+        if not changed:
+            break
     return lab
 
 

@@ -343,6 +343,46 @@ def test_pruning_before_the_solve_changes_neither_plan_nor_objective(meshes, kin
             _check_1d(autop, plan, kind, high_mem)
 
 
+@pytest.mark.parametrize("kind,mesh_key", [("ffn", "2d"), ("block", "2d"), ("block", "1d")])
+def test_solve_near_the_bound_is_the_programs_optimum(meshes, kind, mesh_key):
+    """With an ascent cut short the incumbent stays above the bound; the program restricted to
+    the variables near the bound is solved for growing slacks and the first restricted optimum
+    within its slack is taken: it equals the full program's optimum, and the plan is a feasible
+    plan of the full program."""
+
+    class ShortAscent(OracleOptimizer):
+        prune_sweep_chunks = (2,)
+        prune_max_sweeps = 2
+        prune_slacks = (1e-6, 1e-3, 1e-1)
+
+    class ShortAscentPlanner(AutoParallelPlanner):
+        optimizer_cls = ShortAscent
+
+    class FullOptimizer(OracleOptimizer):
+        prune_before_solve = False
+
+    class FullPlanner(AutoParallelPlanner):
+        optimizer_cls = FullOptimizer
+
+    a, plan_a = _plan(ShortAscentPlanner, meshes[mesh_key], kind, None)
+    b, plan_b = _plan(FullPlanner, meshes[mesh_key], kind, None)
+    oa, ob = a.sharding_optimizer, b.sharding_optimizer
+    sa = oa.solve_stats
+    assert sa["prune_sweeps"] == 2 and sa["incumbent"] - sa["lower_bound"] > oa.prune_gap * abs(sa["incumbent"]), sa
+    tries = sa["near_bound_solves"]
+    assert tries and tries[-1]["value"] is not None and tries[-1]["value"] <= sa["lower_bound"] + tries[-1]["slack"]
+    assert [t["slack"] for t in tries] == sorted(t["slack"] for t in tries)
+    assert all(t["value"] is None or t["value"] > sa["lower_bound"] + t["slack"] for t in tries[:-1])
+    assert sa["columns_solved"] < sa["columns"]
+    assert math.isclose(oa.objective_value(), ob.objective_value(), rel_tol=1e-13)
+    assert not ob.prob.violated_constraints(oa.prob.x)
+    assert math.isclose(float(ob.prob.objective @ oa.prob.x), ob.prob.objective_value, rel_tol=1e-12)
+    if mesh_key == "2d":
+        _check_2d(a, plan_a, kind)
+    else:
+        _check_1d(a, plan_a, kind, None)
+
+
 @pytest.mark.parametrize("kind,mesh_key", [("ffn", "2d"), ("block", "1d")])
 def test_node_choice_variables_do_not_change_the_optimum(meshes, kind, mesh_key):
     """Declaring only the per-(node, strategy) variables integral is a reformulation: the
