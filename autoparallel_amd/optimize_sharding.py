@@ -215,7 +215,7 @@ class CostRecords(Mapping):
         s_i, argi, ss, _ = key
         full = o.strats[o.nodes[s_i]].strategies[ss]
         return {
-            "va": int(o.var_of_entry[idx]),
+            "va": int(o.vars_of(idx)),
             "cost": float(o.cost[idx]),
             "compute_cost": float(o.compute_cost_per_arg[o.encoded.strat_begin[s_i] + ss]),
             "comm_cost": float(o.comm_cost[idx]),
@@ -459,7 +459,6 @@ class ShardingOptimizer:
         self.timings["launch_tables_s"] = time.perf_counter() - t0
         self._host_arrays = {}
         self._inf_entries = None
-        self.var_of_entry = np.arange(tb.n_entries, dtype=np.int64)
         if self.write_back_redistribute_cost:
             self.materialize_redistribute_costs()
         return CostRecords(self), self.encoded.num_inp_out, self.encoded.num_args
@@ -564,7 +563,7 @@ class ShardingOptimizer:
         self.edge_var_base = base[edge_rep]
         self.edge_rep = edge_rep
         self.edge_is_representative = is_root
-        self.var_of_entry = np.repeat(self.edge_var_base - begin[:-1], sizes) + np.arange(tb.n_entries, dtype=np.int64)
+        self._var_of_entry = None  # (one number per entry: made when somebody asks, see var_of_entry)
         self.n_variables = int(sizes[is_root].sum())
         self.n_linked_entries = int(sizes[~is_root].sum())
         # choice variables: one per (node, strategy), shared with the node's representative
@@ -591,6 +590,40 @@ class ShardingOptimizer:
             choice[~has[strat_node]] = 0
             self.choice_var_of_strategy = choice
             self.n_choice_variables = next_free - self.n_variables
+
+    # ---- entries <-> ILP variables -------------------------------------------------------------
+    def vars_of(self, entries):
+        """ILP variables of the given entries (an entry of a linked edge has its representative's)."""
+        begin = self.encoded.tables.edge_entry_begin
+        entries = np.asarray(entries, np.int64)
+        e = np.searchsorted(begin, entries, side="right") - 1  # (an empty edge shares its begin with the next one)
+        return self.edge_var_base[e] + (entries - begin[e])
+
+    @property
+    def var_of_entry(self):
+        """The variable of every entry, as one array (n_entries numbers: planning itself asks
+        ``vars_of`` about the few entries it needs)."""
+        if getattr(self, "_var_of_entry", None) is None:
+            self._var_of_entry = self.vars_of(np.arange(self.encoded.tables.n_entries, dtype=np.int64))
+        return self._var_of_entry
+
+    def _chosen_entries(self):
+        """Entries whose variable is 1 in the solution, ascending.  Every edge's block of
+        variables holds exactly one (its unique-decision row), so each edge, linked ones included,
+        contributes the entry at that offset; anything else falls back to a pass over all entries."""
+        tb = self.encoded.tables
+        begin = tb.edge_entry_begin.astype(np.int64)
+        sizes = begin[1:] - begin[:-1]
+        ones = np.nonzero(self.prob.x[:self.n_variables] == 1)[0]
+        roots = np.nonzero(self.edge_is_representative & (sizes > 0))[0]
+        root_base = self.edge_var_base[roots]  # ascending: blocks are numbered in edge order
+        block = np.searchsorted(root_base, ones, side="right") - 1
+        if len(ones) != len(roots) or not np.array_equal(block, np.arange(len(roots))):
+            return np.nonzero(self.prob.x[self.var_of_entry] == 1)[0]
+        offset_of_root = np.zeros(tb.n_edges, np.int64)
+        offset_of_root[roots] = ones - root_base
+        live = np.nonzero(sizes > 0)[0]
+        return begin[:-1][live] + offset_of_root[self.edge_rep[live]]
 
     def materialize_redistribute_costs(self):
         """Writes the recomputed communication costs into ``OpSpec.redistribute_cost`` of every
@@ -820,7 +853,7 @@ class ShardingOptimizer:
         if status == -1:
             print(self.get_violated_constraints_log())
             raise RuntimeError("Unsolvable problem")
-        chosen = np.nonzero(self.prob.x[self.var_of_entry] == 1)[0]
+        chosen = self._chosen_entries()
         self.res = self.ds.keys_of_entries(chosen)
         self.res_entries = chosen
 
@@ -1077,7 +1110,7 @@ class ShardingOptimizer:
         for argi in range(self.num_args[s_i]):
             b, nt, ns = self._edge(s_i, argi)
             idx = (b + rows[:, None] * ns + np.arange(ns)[None, :]).ravel()
-            self.prob.add_row(self.var_of_entry[idx], 1.0, 1.0, 1.0, next_name(constraint_name))
+            self.prob.add_row(self.vars_of(idx), 1.0, 1.0, 1.0, next_name(constraint_name))
 
     def add_grad_param_constraints(self):
         """A parameter and its gradient choose the same placement."""
@@ -1103,7 +1136,7 @@ class ShardingOptimizer:
                 g = bg + ooi * nsg + np.arange(num_inp_g)
                 cols = np.concatenate([g, [bp + oi * nsp]])
                 vals = np.concatenate([np.ones(num_inp_g), [-1.0]])
-                self.prob.add_row(self.var_of_entry[cols], vals, 0.0, 0.0, next_name("grad_param_constraint"))
+                self.prob.add_row(self.vars_of(cols), vals, 0.0, 0.0, next_name("grad_param_constraint"))
 
     def add_parameter_memory_constraint(self, memory_factor_low: float, memory_factor_high: float):
         """Sum over parameters of (local size / global size) stays within [low, high] x #params."""
@@ -1131,7 +1164,7 @@ class ShardingOptimizer:
                 ratios.append(math.prod(shape) / old)
             vals.extend(ratios)
             per_node.append((s_i, ratios) if ns == 1 else None)
-        cols = self.var_of_entry[np.asarray(cols, np.int64)]
+        cols = self.vars_of(np.asarray(cols, np.int64))
         self.prob.add_row(cols, vals, -np.inf, memory_factor_high * considered, "memory_constraint_high")
         self.prob.add_row(cols, vals, memory_factor_low * considered, np.inf, "memory_constraint_low")
         if all(x is not None for x in per_node):  # (a parameter's only column is its own strategy)

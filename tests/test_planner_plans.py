@@ -116,6 +116,7 @@ def test_reference_golden_plans_2d_with_oracle_tables(meshes, kind):
     opt = autop.sharding_optimizer
     # every (node, argument) picked exactly one entry and nothing infinite was chosen
     assert len(opt.res) == opt.encoded.tables.n_edges
+    assert np.array_equal(opt.res_entries, np.nonzero(opt.prob.x[opt.var_of_entry] == 1)[0])
     assert np.isfinite(opt.comm_cost[opt.res_entries]).all()
     assert not opt.prob.violated_constraints()
     # ds is a mapping over the flat arrays with the reference's record fields

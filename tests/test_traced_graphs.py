@@ -105,6 +105,12 @@ def test_tiny_llama_tables_and_clustering(fake_pg):
         # and here 0.3 % above it
         assert opt.objective_value() >= free_objective - 1e-6
         assert opt.objective_value() <= free_objective * 1.01
+        # the chosen entries, worked out edge by edge (linked edges take their representative's
+        # choice), are the entries whose variable is 1
+        assert opt.n_linked_entries > 0
+        assert np.array_equal(opt.res_entries, np.nonzero(opt.prob.x[opt.var_of_entry] == 1)[0])
+        some = np.arange(0, opt.encoded.tables.n_entries, 97)
+        assert np.array_equal(opt.vars_of(some), opt.var_of_entry[some])
         # linked nodes chose the same strategy as their representative
         for node, rep in opt.node_representative.items():
             assert str(plan[node]) == str(plan[rep])
