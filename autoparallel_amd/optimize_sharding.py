@@ -837,6 +837,8 @@ class ShardingOptimizer:
         obj = np.zeros(self.prob.n_vars, np.float64)
         obj[:self.n_variables] = self.objective_vector
         self.prob.objective = obj
+        if getattr(self, "_upper_unpruned", None) is not None:  # (a second solve, maybe under more constraints)
+            self.prob.upper = self._upper_unpruned.copy()
         self.solve_stats = {"columns": int((self.prob.upper > 0).sum())}
         self._solved_while_pruning = False
         if self.prune_before_solve and self.node_choice_variables:
@@ -987,6 +989,11 @@ class ShardingOptimizer:
         t0 = time.perf_counter()
         stats = self.solve_stats
         self._solved_while_pruning = False
+        # what an earlier call fixed was decided under the constraints of that call: start again
+        # from the bounds of the unpruned program (nothing but pruning changes them after construction)
+        if getattr(self, "_upper_unpruned", None) is not None:
+            self.prob.upper = self._upper_unpruned.copy()
+        self._upper_unpruned = self.prob.upper.copy()
         graph = self._label_graph()
         stats["prune_graph_s"] = time.perf_counter() - t0
         t_sweeps = t_round = 0.0

@@ -344,6 +344,46 @@ def test_pruning_before_the_solve_changes_neither_plan_nor_objective(meshes, kin
             _check_1d(autop, plan, kind, high_mem)
 
 
+def test_a_second_solve_under_more_constraints_starts_from_the_unpruned_program(meshes):
+    """What the first solve pruned was ruled out under its constraints only: after a new
+    constraint the second solve finds what a fresh planner with both constraints finds."""
+    mesh = meshes["2d"]
+    model_fn, input_fn = make_model_and_inputs(mesh, "ffn")
+
+    def planner():
+        with torch.device("meta"):
+            model = model_fn()
+        p = OraclePlanner(model, input_fn, mesh)
+        p.__enter__()
+        p.add_parameter_memory_constraint(low=0, high=None)
+        return p
+
+    a = planner()
+    first_plan = a.optimize_placement()
+    oa = a.sharding_optimizer
+    first = oa.objective_value()
+    assert oa.solve_stats["columns_after_pruning"] < oa.solve_stats["columns"]
+    node = get_param_nodes(a.gm.graph)[0]
+
+    def plan_of(_, n):
+        return first_plan[n].output_specs.placements
+
+    assert plan_of(a, node) == (Shard(0), Shard(0))
+    forced = (Shard(0), Shard(1))  # not what the first plan chose: its variables were pruned
+    oa.add_node_constraint(node, forced)
+    plan = a.optimize_placement()
+    assert plan[node].output_specs.placements == forced
+    second, columns = oa.objective_value(), oa.solve_stats["columns"]
+    a.__exit__(None, None, None)
+    b = planner()
+    b.sharding_optimizer.add_node_constraint(get_param_nodes(b.gm.graph)[0], forced)
+    b.optimize_placement()
+    assert math.isclose(second, b.sharding_optimizer.objective_value(), rel_tol=1e-13)
+    assert second > first
+    assert columns == b.sharding_optimizer.solve_stats["columns"]
+    b.__exit__(None, None, None)
+
+
 @pytest.mark.parametrize("kind,mesh_key", [("ffn", "2d"), ("block", "2d"), ("block", "1d")])
 def test_solve_near_the_bound_is_the_programs_optimum(meshes, kind, mesh_key):
     """With an ascent cut short the incumbent stays above the bound; the program restricted to
