@@ -16,7 +16,7 @@ APC_MAX_MESH = 4
 APC_MAX_DTYPES = 8
 APC_TILE_MAX_COLS = 64
 APC_TILE_MAX_ROWS = 64
-APC_TILE_MAX_DUPS = 127
+APC_TILE_MAX_DUPS = 32
 
 EDGE_GRAD_RESCALE = 1
 EDGE_NO_PRODUCER = 2

@@ -755,23 +755,34 @@ struct TileStage : std::conditional_t<RM, RowMinStage, NoRowMinStage> {
   // that the lanes of consecutive producer specs hit different banks
   uint32_t words[APC_TILE_MAX_COLS * (M * kWordsPerDim + 1)];
   alignas(16) uint32_t pair_base[M * 16];  // TermLayout::pair of the launch
-  // per staging wavefront (power-of-two layout): B and the value constants of every computed array
-  double chain[4][kMaxTermArrays];
-  TermValueConstants value_of[4][kMaxTermArrays];
   int64_t dup[APC_TILE_MAX_DUPS];  // first entries of the identical edges
   double gb_unsharded;  // bytes / 1024^3 of the tile's tensor
   int mixed[4];         // per staging wavefront: some spec is not a DTensorSpec on the tile's tensor (generic loop)
   int cont;             // the tile's tensor is contiguous
   // Last: the tile kernels size their LDS per launch for the entries the layout in use needs
   // (stage_lds_bytes), so that the small power-of-two layout leaves room for more workgroups.
+  // In front of the entries, one StagingScratch per wavefront of the workgroup (a compile-time
+  // number in every kernel, so the entries still sit at a fixed offset): term_base.
   alignas(16) double terms[TermTable<M>::kEntries];
 };
 
+// What one wavefront keeps while it stages the term arrays of the power-of-two layout.
+struct alignas(16) StagingScratch {
+  double chain[kMaxTermArrays];
+  TermValueConstants value_of[kMaxTermArrays];
+};
+// Where the term arrays of a stage start, for a workgroup of `nthreads` threads.
+template <typename Stage>
+__device__ __forceinline__ char *term_base(Stage &st, int nthreads) {
+  return const_cast<char *>(reinterpret_cast<const char *>(st.terms)) + sizeof(StagingScratch) * (size_t)(nthreads >> 6);
+}
+
 // LDS bytes of a tile stage whose term arrays hold what the launch's layout needs.
 template <int M, bool RM>
-static size_t stage_lds_bytes(const TermLayout &lay) {
+static size_t stage_lds_bytes(const TermLayout &lay, int threads) {
   const size_t entries = lay.exponents ? (size_t)(kPow2Stride / 8) * lay.exponents : (size_t)TermTable<M>::kGeneral;
-  return sizeof(TileStage<M, RM>) - sizeof(double) * TermTable<M>::kEntries + sizeof(double) * entries;
+  return sizeof(TileStage<M, RM>) - sizeof(double) * TermTable<M>::kEntries + sizeof(StagingScratch) * (size_t)(threads / 64) +
+         sizeof(double) * entries;
 }
 
 // The fields of a tile record the entry loops use.
@@ -855,15 +866,13 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
     row_zero = a.zero_cost[sr];
     row_args = a.num_args[sr];
   }
-  // (dup_count <= APC_TILE_MAX_DUPS < 2 * nthreads)
-  const bool has_dup0 = tid < tile.dup_count, has_dup1 = tid + nthreads < tile.dup_count;
-  int64_t dup0 = 0, dup1 = 0;
+  // (dup_count <= APC_TILE_MAX_DUPS <= nthreads)
+  const bool has_dup0 = tid < tile.dup_count;
+  int64_t dup0 = 0;
   if (has_dup0) dup0 = a.dup_entry_begin[tile.dup_begin + tid];
-  if (has_dup1) dup1 = a.dup_entry_begin[tile.dup_begin + tid + nthreads];
-  int64_t dup_row0 = 0, dup_row1 = 0, row_out = 0;
+  int64_t dup_row0 = 0, row_out = 0;
   if constexpr (RM) {
     if (has_dup0) dup_row0 = a.dup_row_begin[tile.dup_begin + tid];
-    if (has_dup1) dup_row1 = a.dup_row_begin[tile.dup_begin + tid + nthreads];
     row_out = a.edge_row_begin[tile.edge];  // wave-uniform: a scalar load
   }
   // the contiguity byte of the tile's tensor, read as the aligned word around it (which lies
@@ -889,21 +898,22 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
     // bytes (every wavefront its own copy: no barrier), then a lane per (array, exponent) the
     // value.
     const double fbytes = (double)tensor_nbytes;
+    StagingScratch &mine = reinterpret_cast<StagingScratch *>(st.terms)[wave];
     if (lane < kComputed) {
-      st.chain[wave][lane] = div_by(div_by(fbytes * chain_of.hops, chain_of.div1, chain_of.inv_div1) * 1e6,
-                                    chain_of.div2, chain_of.inv_div2);
-      st.value_of[wave][lane] = TermValueConstants{chain_of.lat, chain_of.floor, chain_of.scale, chain_of.shift, 0};
+      mine.chain[lane] = div_by(div_by(fbytes * chain_of.hops, chain_of.div1, chain_of.inv_div1) * 1e6, chain_of.div2,
+                                chain_of.inv_div2);
+      mine.value_of[lane] = TermValueConstants{chain_of.lat, chain_of.floor, chain_of.scale, chain_of.shift, 0};
     }
     __builtin_amdgcn_wave_barrier();  // (LDS operations of one wavefront complete in order)
     // (The value constants go through LDS as well.  Read from the kernel arguments by a per-lane
     // index inside the loop below, `lat + ldexp(..)` was compiled to `x + x` in the 4-D
     // instantiations by hipcc 7.2: the placement-pair tests on 4-D power-of-two meshes show it.)
-    char *terms = reinterpret_cast<char *>(st.terms);
+    char *terms = term_base(st, nthreads);
     for (int t = tid; t < kComputed * E; t += nthreads) {
       const int arr = (int)(((uint32_t)t * lay.exponent_magic) >> 16);  // t / E
       const int j = t - arr * E;  // the running bytes are bytes x 2^(j - L - 30)
-      const TermValueConstants k = st.value_of[wave][arr];
-      double v = k.lat + __builtin_ldexp(st.chain[wave][arr], j + k.shift);
+      const TermValueConstants k = mine.value_of[arr];
+      double v = k.lat + __builtin_ldexp(mine.chain[arr], j + k.shift);
       v = v > k.floor ? v : k.floor;
       v = v * k.scale;
       *reinterpret_cast<double *>(terms + j * kPow2Stride + (arr + 2) * 8) = v;
@@ -943,7 +953,7 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
       double a2a = rs;
       a2a *= p.a2a_scale;
       const double rw = rw_time_r(gb * 2 * 1073741824.0, p);
-      double *e = st.terms + k * (kGeneralStride / 8);
+      double *e = reinterpret_cast<double *>(term_base(st, nthreads)) + k * (kGeneralStride / 8);
       e[kZerosArray] = 0.0;
       e[kInfArray] = __builtin_inf();
       e[kRw1Array] = rw;
@@ -961,10 +971,8 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   if (tid == 0) st.cont = contiguous != 0;
   if (tid < 16 * M) st.pair_base[tid] = pair_word;
   if (has_dup0) st.dup[tid] = dup0;
-  if (has_dup1) st.dup[tid + nthreads] = dup1;
   if constexpr (RM) {
     if (has_dup0) st.dup_row[tid] = dup_row0;
-    if (has_dup1) st.dup_row[tid + nthreads] = dup_row1;
     if (tid < APC_TILE_MAX_ROWS) st.rmin[1][tid] = __builtin_inf();  // (slot 0 of every row is always written)
     if (tid == 0) st.row_out = row_out;
   }
@@ -1032,13 +1040,13 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
 // are issued together; no vector memory loads.
 template <int M, bool CONT, bool RESCALE, bool RM>
 __device__ __forceinline__ void uniform_entry(const apc_params &p, const TermLayout &lay, const TileStage<M, RM> &st,
-                                              int r, int c, double &comm_o, double &total_o, int &trans_o) {
+                                              const char *terms, int r, int c, double &comm_o, double &total_o,
+                                              int &trans_o) {
   const uint32_t src = st.col_codes[c];
   const RowRecord row = st.row[r];
   const uint32_t tgt = row.codes;
   const uint32_t x = src ^ tgt;
   const char *words = reinterpret_cast<const char *>(st.words) + __umul24((uint32_t)c, (M * kWordsPerDim + 1) * 4);
-  const char *terms = reinterpret_cast<const char *>(st.terms);
   // ---- integer part: which term at which running index each mesh dim adds -------------------
   uint32_t at = 0;  // byte offset of the running index (history of the earlier dims / exponent steps), mod 2^32
   uint32_t term_at[M], rw_at[M], nc_at[M];
@@ -1237,7 +1245,7 @@ __device__ __forceinline__ void uniform_tile_entries_row_min(const apc_params &p
     double comm, total = 0.0;
     int trans;
     if (active) {
-      uniform_entry<M, CONT, RESCALE>(p, a.lay, st, r, c, comm, total, trans);
+      uniform_entry<M, CONT, RESCALE>(p, a.lay, st, term_base(st, nthreads), r, c, comm, total, trans);
       store_entry<OUT>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
                        trans);
     }
@@ -1273,7 +1281,7 @@ __device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const 
   for (int idx = first; idx < n; idx += nthreads) {
     double comm, total;
     int trans;
-    uniform_entry<M, CONT, RESCALE>(p, a.lay, st, r, c, comm, total, trans);
+    uniform_entry<M, CONT, RESCALE>(p, a.lay, st, term_base(st, nthreads), r, c, comm, total, trans);
     store_entry<OUT>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
                      trans);
     c += dc;
@@ -1391,7 +1399,7 @@ __device__ __forceinline__ void redistribute_tile(const apc_params &p, const Tab
   if (tile_id >= n_tiles) return;
   static_assert(kTileThreads == 64 || kTileThreads == 128 || kTileThreads == 256, "wavefronts per tile: 1, 2 or 4");
   static_assert(kTileThreads >= APC_TILE_MAX_COLS && kTileThreads >= APC_TILE_MAX_ROWS &&
-                2 * kTileThreads > APC_TILE_MAX_DUPS, "one staging round covers a tile");
+                kTileThreads >= APC_TILE_MAX_DUPS, "one staging round covers a tile");
   const apc_tile tile = tiles[tile_id];
   stage_tile<M, false, RM>(p, a, tile, stage, threadIdx.x, kTileThreads);
   __syncthreads();
@@ -1404,14 +1412,16 @@ __device__ __forceinline__ void redistribute_tile(const apc_params &p, const Tab
 // use otherwise: the row-minimum kernel got 97 registers and 4 wavefronts on a 3-D mesh where 67
 // registers do without spilling (stress table 2.94 -> 2.58 ms); the kernel without the minima
 // gains 1 - 2 % (same box: stress 1.93 -> 1.88 ms, Llama-3-70B 251 -> 248 us).
-constexpr int tile_waves_per_simd(int mesh_ndim, int threads) {
+constexpr int tile_waves_per_simd(int mesh_ndim, int threads, bool row_min) {
   if (mesh_ndim >= 4) return threads >= 256 ? 4 : threads >= 128 ? 3 : 2;
   if (threads < 128) return mesh_ndim <= 1 ? 7 : mesh_ndim == 2 ? 6 : 4;
-  return 7;
+  // two-wavefront tiles without the minima fit sixteen to a compute unit (under 10 KB of LDS
+  // each on a power-of-two mesh): all eight wavefront slots of a SIMD, 64 registers
+  return threads == 128 && !row_min ? 8 : 7;
 }
 
 template <int M, int kTileThreads, int OUT>
-__global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads), 8)))
+__global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads, false), 8)))
 void redistribute_tiles_kernel(const apc_tile *tiles, int n_tiles, int xcd_shift, apc_params p, TableArgs a) {
   extern __shared__ __align__(16) unsigned char s_stage_bytes[];  // stage_lds_bytes<M, false>
   redistribute_tile<M, kTileThreads, false, OUT>(p, a, tiles, n_tiles, xcd_shift,
@@ -1421,7 +1431,7 @@ void redistribute_tiles_kernel(const apc_tile *tiles, int n_tiles, int xcd_shift
 // The same with the row minima.
 template <int M, int kTileThreads, int OUT>
 __global__ __launch_bounds__(kTileThreads)
-__attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads), 8)))
+__attribute__((amdgpu_waves_per_eu(tile_waves_per_simd(M, kTileThreads, true), 8)))
 void redistribute_tiles_row_min_kernel(const apc_tile *tiles, int n_tiles, int xcd_shift, apc_params p, TableArgs a) {
   extern __shared__ __align__(16) unsigned char s_stage_bytes[];  // stage_lds_bytes<M, true>
   redistribute_tile<M, kTileThreads, true, OUT>(p, a, tiles, n_tiles, xcd_shift,
@@ -1446,7 +1456,8 @@ void build_tables_kernel(const apc_tile *tiles, int n_tiles, int xcd_shift, int6
                          TensorTableArgs t, SpecTableArgs sp, ComputeCostArgs c, int64_t spec_blocks,
                          int64_t tensor_blocks) {
   constexpr size_t kRowBytes = (size_t)kThreads * (APC_MAX_RANK + 1) * sizeof(int64_t);
-  constexpr size_t kLds = sizeof(TileStage<M, RM>) > kRowBytes ? sizeof(TileStage<M, RM>) : kRowBytes;
+  constexpr size_t kStage = sizeof(TileStage<M, RM>) + sizeof(StagingScratch) * (kThreads / 64);
+  constexpr size_t kLds = kStage > kRowBytes ? kStage : kRowBytes;
   __shared__ __align__(16) unsigned char s_raw[kLds];
   static_assert(kThreads == 64 || kThreads == 128 || kThreads == 256, "wavefronts per workgroup: 1, 2 or 4");
   const int64_t b = blockIdx.x;
@@ -2047,7 +2058,8 @@ static int redistribute_tables_impl(const apc_params *params, const int64_t *ten
   if (const char *env = getenv("APC_TILE_THREADS")) threads = atoi(env);  // tuning override
   const int om = out_mode(params->mesh_ndim, comm_out, trans_out, cost_out);
 #define APC_LAUNCH_T(KERNEL_, M_, OUT_)                                                                               \
-  const size_t lds = rows ? stage_lds_bytes<M_, true>(a.lay) : stage_lds_bytes<M_, false>(a.lay);                      \
+  const int wg = threads >= 256 ? 256 : threads >= 128 ? 128 : 64;                                                     \
+  const size_t lds = rows ? stage_lds_bytes<M_, true>(a.lay, wg) : stage_lds_bytes<M_, false>(a.lay, wg);              \
   if (threads >= 256) hipLaunchKernelGGL((KERNEL_<M_, 256, OUT_>), grid, dim3(256), lds, s, a.tiles, nt, xs, *params, a);      \
   else if (threads >= 128) hipLaunchKernelGGL((KERNEL_<M_, 128, OUT_>), grid, dim3(128), lds, s, a.tiles, nt, xs, *params, a); \
   else hipLaunchKernelGGL((KERNEL_<M_, 64, OUT_>), grid, dim3(64), lds, s, a.tiles, nt, xs, *params, a)

@@ -55,7 +55,8 @@ extern "C" {
 #define APC_MAX_DTYPES 8
 #define APC_TILE_MAX_COLS 64 /* producer specs staged in LDS per tile */
 #define APC_TILE_MAX_ROWS 64 /* consumer specs staged in LDS per tile */
-#define APC_TILE_MAX_DUPS 127 /* identical edges served by one tile (offsets staged in LDS) */
+#define APC_TILE_MAX_DUPS 32 /* identical edges served by one tile (offsets staged in LDS); a larger group of
+                              identical edges is served by several tiled edges */
 #define APC_MAX_STRATEGIES (1 << 22) /* strategies of one node: a tile's rows span < 4 GiB of fp64 */
 
 #define APC_EDGE_GRAD_RESCALE 1 /* consumer is a parameter-gradient node (optimize_sharding.py:358-359) */

@@ -94,6 +94,25 @@ def test_tables_match_oracle_on_seeded_dags(gpu_device, mesh):
     assert got["local_shape"].shape[1] == tb.shape_width() <= 8
 
 
+@pytest.mark.parametrize("mesh,threads", [((4, 2), None), ((8, 4, 2), "64"), ((8, 4, 2), "256"), ((3, 2), "128")])
+def test_tiles_with_the_maximum_number_of_identical_edges(gpu_device, mesh, threads, monkeypatch):
+    """A tile lists at most APC_TILE_MAX_DUPS identical edges (their first entries, and first
+    matrix rows for the minima, are staged in LDS): 64 copies of a graph are served by two tiled
+    edges per group, whatever ``max_copies`` asks for."""
+    from autoparallel_amd._native import APC_TILE_MAX_DUPS
+    from test_abi_and_encoding import twin_graph
+
+    if threads:
+        monkeypatch.setenv("APC_TILE_THREADS", threads)
+    tb = stress_dag(seed=31, n_nodes=40, mesh_sizes=mesh, max_strategies=12, frac_nonspec_nodes=0.05,
+                    frac_noncontiguous=0.2)
+    for _ in range(6):  # 64 copies of every edge
+        tb = twin_graph(tb)
+    tb.build_tiles(None, dedupe=True, max_copies=100)
+    assert int(tb.tile_records["dup_count"].max()) == APC_TILE_MAX_DUPS == 32 and tb.rows_fit_tiles()
+    _run_and_compare(tb, mesh, 2.2, gpu_device)
+
+
 @pytest.mark.parametrize("mesh", [(32, 8), (16, 8, 4), (2, 4, 2, 2)])
 def test_per_state_term_arrays_on_power_of_two_meshes(gpu_device, mesh, monkeypatch):
     """The term arrays every mesh can use give the same bits on the meshes that normally take
