@@ -445,6 +445,49 @@ def test_node_choice_variables_do_not_change_the_optimum(meshes, kind, mesh_key)
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kind,mesh_key", [("block", "2d"), ("ffn", "2d")])
+def test_solve_near_the_bound_from_device_sweeps(gpu_device, meshes, kind, mesh_key):
+    """The ascent cut short on the device as on its CPU restatement: the same bound, the same
+    tries near the bound, the same optimum as the full program's."""
+
+    class ShortDevice(ShardingOptimizer):
+        prune_sweep_chunks = (2,)
+        prune_max_sweeps = 2
+        prune_slacks = (1e-6, 1e-3, 1e-1)
+
+    class ShortDevicePlanner(AutoParallelPlanner):
+        optimizer_cls = ShortDevice
+
+    class ShortOracle(OracleOptimizer):
+        prune_sweep_chunks = (2,)
+        prune_max_sweeps = 2
+        prune_slacks = (1e-6, 1e-3, 1e-1)
+
+    class ShortOraclePlanner(AutoParallelPlanner):
+        optimizer_cls = ShortOracle
+
+    class FullOptimizer(OracleOptimizer):
+        prune_before_solve = False
+
+    class FullPlanner(AutoParallelPlanner):
+        optimizer_cls = FullOptimizer
+
+    a, plan_a = _plan(ShortDevicePlanner, meshes[mesh_key], kind, None)
+    b, _ = _plan(ShortOraclePlanner, meshes[mesh_key], kind, None)
+    c, _ = _plan(FullPlanner, meshes[mesh_key], kind, None)
+    oa, ob, oc = a.sharding_optimizer, b.sharding_optimizer, c.sharding_optimizer
+    assert type(oa.backend).__name__ == "DeviceBackend"
+    sa, sb = oa.solve_stats, ob.solve_stats
+    assert sa["near_bound_solves"] and len(sa["near_bound_solves"]) == len(sb["near_bound_solves"])
+    assert math.isclose(sa["lower_bound"], sb["lower_bound"], rel_tol=1e-12)
+    for ta, tb_ in zip(sa["near_bound_solves"], sb["near_bound_solves"]):
+        assert ta["columns"] == tb_["columns"] and math.isclose(ta["slack"], tb_["slack"], rel_tol=1e-9)
+    assert math.isclose(oa.objective_value(), oc.objective_value(), rel_tol=1e-13)
+    assert not oc.prob.violated_constraints(oa.prob.x)
+    _check_2d(a, plan_a, kind)
+
+
+@pytest.mark.gpu
 def test_local_map_plan_from_device_tables(gpu_device, meshes):
     dev_autop, dev_plan = _plan_local_map(AutoParallelPlanner, meshes["3d"])
     ora_autop, ora_plan = _plan_local_map(OraclePlanner, meshes["3d"])
