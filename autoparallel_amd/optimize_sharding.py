@@ -341,8 +341,8 @@ class ShardingOptimizer:
     prune_gap = 2e-4
     # Where the rounding does not reach the bound (the relaxation has a gap, or the ascent is not
     # through: a mixture-of-experts graph has four times the classes of a Llama graph), the
-    # ascent goes on in doubling chunks while a chunk still lifts the bound by more than
-    # ``prune_gap / 4`` (relative), up to ``prune_max_sweeps`` in all; then the program is solved
+    # ascent goes on in chunks twice the last one's size while a chunk still lifts the bound by more
+    # than ``prune_gap / 4`` (relative), up to ``prune_max_sweeps`` in all; then the program is solved
     # restricted to the variables whose bound is within a slack of the lower bound, slack =
     # ``prune_slacks`` x |bound| in turn, capped by the incumbent's distance.  A restricted optimum
     # that is itself within the slack is the optimum: everything left out costs more.
@@ -1023,9 +1023,10 @@ class ShardingOptimizer:
             t_round += time.perf_counter() - t1
             if best_ub - bound <= self.prune_gap * abs(best_ub):
                 break
-            if k == len(chunks) and sweeps + 2 * chunk <= self.prune_max_sweeps and \
-                    bound - before > 0.25 * self.prune_gap * abs(bound):
-                chunks.append(2 * chunk)  # the ascent is not through
+            if k == len(chunks) and bound - before > 0.25 * self.prune_gap * abs(bound):  # the ascent is not through
+                more = 2 * chunk if k == len(self.prune_sweep_chunks) else chunk  # (twice the last planned chunk, repeated)
+                if sweeps + more <= self.prune_max_sweeps:
+                    chunks.append(more)
         stats.update(prune_sweeps_s=t_sweeps, prune_rounding_s=t_round)
         stats.update(prune_sweeps=sweeps, lower_bound=bound, incumbent=best_ub if best_x is not None else None,
                      label_classes=graph.n_classes, label_edges=graph.n_edges)
