@@ -192,26 +192,31 @@ def decode(g: LabelGraph, theta: np.ndarray, unary: np.ndarray) -> np.ndarray:
 
 def refine(g: LabelGraph, theta: np.ndarray, unary: np.ndarray, labels: np.ndarray, max_rounds: int = 10) -> np.ndarray:
     """Local search from a labelling: class by class, the label that is cheapest given the labels
-    of all its neighbours, until a round changes nothing.  Never raises the labelling's cost."""
+    of all its neighbours, until a round changes nothing (after the first round only classes with
+    a changed neighbour are looked at again).  Never raises the labelling's cost."""
     lab = labels.copy()
     lb = g.label_begin
+    todo = np.ones(g.n_classes, bool)
     for _ in range(max_rounds):
-        changed = False
-        for c in range(g.n_classes):
+        again = np.zeros(g.n_classes, bool)
+        for c in np.nonzero(todo)[0]:
             if lab[c] < 0:
                 continue
             score = unary[lb[c]:lb[c + 1]].copy()
+            others = []
             for t in range(int(g.inc_begin[c]), int(g.inc_begin[c + 1])):
                 k, side = int(g.inc_edge[t]), int(g.inc_side[t])
                 m = g.matrix(theta, k)
                 other = int(g.edge_j[k]) if side == 0 else int(g.edge_i[k])
+                others.append(other)
                 score = score + (m[:, lab[other]] if side == 0 else m[lab[other], :])
             best = int(np.argmin(score))
             if score[best] < score[lab[c]]:
                 lab[c] = best
-                changed = True
-        if not changed:
+                again[others] = True
+        if not again.any():
             break
+        todo = again
     return lab
 
 

@@ -122,3 +122,24 @@ def test_device_sweeps_equal_the_cpu_restatement(gpu_device, seed, n, max_labels
         want_t, want_u = _sweep(g, theta, unary, chunk)
         theta, unary = dev.diffusion_sweeps(g, theta, unary, chunk)
         assert np.array_equal(theta, want_t) and np.array_equal(unary, want_u), chunk
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_refine_never_raises_the_cost_and_ends_where_no_single_change_helps(seed):
+    g, sizes = _random_problem(100 + seed, n=7, p_inf=0.0)
+    theta, unary = _sweep(g, g.theta, g.unary, 2)
+    rng = np.random.default_rng(seed)
+    start = np.asarray([int(rng.integers(0, s)) for s in sizes], np.int64)
+    if not np.isfinite(_energy(g, theta, unary, start)):  # (a masked label of class 0)
+        start[0] = 0
+    end = pruning.refine(g, theta, unary, start)
+    e0, e1 = _energy(g, theta, unary, start), _energy(g, theta, unary, end)
+    assert e1 <= e0 + 1e-9
+    for c in range(g.n_classes):  # a local optimum: no class alone can do better
+        for lab in range(sizes[c]):
+            other = end.copy()
+            other[c] = lab
+            assert _energy(g, theta, unary, other) >= e1 - 1e-9
+    # the labelling decode proposes is only ever improved
+    d = pruning.decode(g, theta, unary)
+    assert _energy(g, theta, unary, pruning.refine(g, theta, unary, d)) <= _energy(g, theta, unary, d) + 1e-9
