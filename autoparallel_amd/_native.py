@@ -11,6 +11,7 @@ import os
 
 from ._build import LIB_PATH, TORCH_EXT_PATH
 
+APC_ABI_VERSION = 2  # include/apcost.h: the interface this binding's structs and limits mirror
 APC_MAX_RANK = 8
 APC_MAX_MESH = 4
 APC_MAX_DTYPES = 8
@@ -111,6 +112,10 @@ def lib() -> ctypes.CDLL:
             if not hasattr(l, name):
                 raise RuntimeError(f"{LIB_PATH} does not export {name}")
         l.apc_last_error.restype = ctypes.c_char_p
+        l.apc_version.restype = ctypes.c_int
+        if int(l.apc_version()) != APC_ABI_VERSION:
+            raise RuntimeError(f"{LIB_PATH} implements interface version {int(l.apc_version())}, this binding "
+                               f"mirrors version {APC_ABI_VERSION} of include/apcost.h: rebuild the library")
         for name in EXPORTS:
             if name != "apc_last_error":
                 getattr(l, name).restype = ctypes.c_int
@@ -137,8 +142,10 @@ def torch_ops():
             )
         torch.ops.load_library(TORCH_EXT_PATH)
         _ops = torch.ops.apcost
-        if int(_ops.abi_version()) != int(lib().apc_version()):
-            raise RuntimeError("the torch layer and the C-ABI library are different builds")
+        if int(_ops.abi_version()) != APC_ABI_VERSION or int(_ops.library_abi_version()) != APC_ABI_VERSION:
+            raise RuntimeError(f"the torch layer was compiled against interface version {int(_ops.abi_version())} and "
+                               f"sees a library of version {int(_ops.library_abi_version())}; this binding mirrors "
+                               f"version {APC_ABI_VERSION}: rebuild both")
     return _ops
 
 

@@ -59,14 +59,32 @@ class AutoParallelPlanner:
         import gc
 
         collector_was_on = gc.isenabled()
+        # An application that froze its own objects (a server after start-up) keeps its frozen
+        # set: this planner then neither freezes nor, on exit, thaws.
+        host_has_frozen = gc.get_freeze_count() != 0
         gc.disable()
         try:
-            return self._enter()
-        finally:
-            gc.freeze()
-            self._frozen = True
+            out = self._enter()
+        except BaseException:
+            # `with` does not call __exit__ after a failing __enter__: nothing may stay frozen,
+            # and the capture context that was entered is left here
             if collector_was_on:
                 gc.enable()
+            ctx, self._ctx = self._ctx, None
+            if ctx is not None and getattr(self, "gm", None) is not None:
+                import sys
+
+                try:
+                    ctx.__exit__(*sys.exc_info())
+                except Exception:  # (the failure being reported is the one that matters)
+                    logger.debug("closing the capture context after a failed construction raised", exc_info=True)
+            raise
+        if not host_has_frozen:
+            gc.freeze()
+            self._frozen = True
+        if collector_was_on:
+            gc.enable()
+        return out
 
     def _enter(self):
         # the device's first-use costs (a fifth of a second) overlap the capture
@@ -104,7 +122,8 @@ class AutoParallelPlanner:
 
             self._frozen = False
             gc.unfreeze()  # (the collector sees everything again; cycles left by planning go at its next pass)
-        return self._ctx.__exit__(*exc)
+        ctx, self._ctx = self._ctx, None
+        return ctx.__exit__(*exc) if ctx is not None else None
 
     def add_parameter_memory_constraint(self, low=None, high=None):
         self._assert_entered()

@@ -48,6 +48,127 @@ constexpr int kBlock = 256;
 __device__ __forceinline__ int kind_of(uint32_t c) { return (int)(c >> 6); }  // 0 R, 1 P, 2 S
 __device__ __forceinline__ int dim_of(uint32_t c) { return (int)(c & 0x0F); }
 
+// A load from a wave-uniform address of a table that no kernel of this library writes while it
+// reads it (the uploaded encoding): through the constant address space, i.e. the scalar cache,
+// into scalar registers.  (Left as a plain load the compiler takes such an address through vector
+// memory, where the load queues behind the wavefront's other vector loads.)
+#define APC_CONSTANT __attribute__((address_space(4)))
+template <typename T>
+__device__ __forceinline__ T uniform_load(const T *p) {
+  return *(const APC_CONSTANT T *)p;
+}
+typedef int32_t i32x16 __attribute__((ext_vector_type(16)));
+typedef int64_t i64x8 __attribute__((ext_vector_type(8)));
+
+// The value lane `lane` (wave-uniform) holds.
+__device__ __forceinline__ int64_t value_of_lane(int64_t x, int lane) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)x, lane);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)((uint64_t)x >> 32), lane);
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+// Kernel arguments a wavefront will need, fetched now: the compiler loads an argument where it
+// is first used, each behind the wait of whatever came before it, and a chain of such loads in
+// front of a tile's own loads cost more than the loads themselves.  Naming the values as scalar
+// operands of an (empty) asm statement puts their loads here, together, under one wait.
+// One statement for all of them: a load may be moved past an asm statement that does not name it.
+template <typename T0>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0) {
+  __asm__ volatile("" ::"s"(v0));
+}
+template <typename T0, typename T1>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1));
+}
+template <typename T0, typename T1, typename T2>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2));
+}
+template <typename T0, typename T1, typename T2, typename T3>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12, typename T13>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12, T13 v13) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12), "s"(v13));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12, typename T13, typename T14>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12, T13 v13, T14 v14) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12), "s"(v13), "s"(v14));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12, typename T13, typename T14, typename T15>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12, T13 v13, T14 v14, T15 v15) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12), "s"(v13), "s"(v14), "s"(v15));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12, typename T13, typename T14, typename T15, typename T16>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12, T13 v13, T14 v14, T15 v15, T16 v16) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12), "s"(v13), "s"(v14), "s"(v15), "s"(v16));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12, typename T13, typename T14, typename T15, typename T16, typename T17>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12, T13 v13, T14 v14, T15 v15, T16 v16, T17 v17) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12), "s"(v13), "s"(v14), "s"(v15), "s"(v16), "s"(v17));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12, typename T13, typename T14, typename T15, typename T16, typename T17, typename T18>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12, T13 v13, T14 v14, T15 v15, T16 v16, T17 v17, T18 v18) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12), "s"(v13), "s"(v14), "s"(v15), "s"(v16), "s"(v17), "s"(v18));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12, typename T13, typename T14, typename T15, typename T16, typename T17, typename T18, typename T19>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12, T13 v13, T14 v14, T15 v15, T16 v16, T17 v17, T18 v18, T19 v19) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12), "s"(v13), "s"(v14), "s"(v15), "s"(v16), "s"(v17), "s"(v18), "s"(v19));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12, typename T13, typename T14, typename T15, typename T16, typename T17, typename T18, typename T19, typename T20>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12, T13 v13, T14 v14, T15 v15, T16 v16, T17 v17, T18 v18, T19 v19, T20 v20) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12), "s"(v13), "s"(v14), "s"(v15), "s"(v16), "s"(v17), "s"(v18), "s"(v19), "s"(v20));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12, typename T13, typename T14, typename T15, typename T16, typename T17, typename T18, typename T19, typename T20, typename T21>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12, T13 v13, T14 v14, T15 v15, T16 v16, T17 v17, T18 v18, T19 v19, T20 v20, T21 v21) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12), "s"(v13), "s"(v14), "s"(v15), "s"(v16), "s"(v17), "s"(v18), "s"(v19), "s"(v20), "s"(v21));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12, typename T13, typename T14, typename T15, typename T16, typename T17, typename T18, typename T19, typename T20, typename T21, typename T22>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12, T13 v13, T14 v14, T15 v15, T16 v16, T17 v17, T18 v18, T19 v19, T20 v20, T21 v21, T22 v22) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12), "s"(v13), "s"(v14), "s"(v15), "s"(v16), "s"(v17), "s"(v18), "s"(v19), "s"(v20), "s"(v21), "s"(v22));
+}
+template <typename T0, typename T1, typename T2, typename T3, typename T4, typename T5, typename T6, typename T7, typename T8, typename T9, typename T10, typename T11, typename T12, typename T13, typename T14, typename T15, typename T16, typename T17, typename T18, typename T19, typename T20, typename T21, typename T22, typename T23>
+__device__ __forceinline__ void fetch_arguments_now(T0 v0, T1 v1, T2 v2, T3 v3, T4 v4, T5 v5, T6 v6, T7 v7, T8 v8, T9 v9, T10 v10, T11 v11, T12 v12, T13 v13, T14 v14, T15 v15, T16 v16, T17 v17, T18 v18, T19 v19, T20 v20, T21 v21, T22 v22, T23 v23) {
+  __asm__ volatile("" ::"s"(v0), "s"(v1), "s"(v2), "s"(v3), "s"(v4), "s"(v5), "s"(v6), "s"(v7), "s"(v8), "s"(v9), "s"(v10), "s"(v11), "s"(v12), "s"(v13), "s"(v14), "s"(v15), "s"(v16), "s"(v17), "s"(v18), "s"(v19), "s"(v20), "s"(v21), "s"(v22), "s"(v23));
+}
+
 // compute_estimation.py:302-314
 __device__ __forceinline__ double rw_time(double bytes, const apc_params &p) {
   double t = bytes / p.hbm_bw * 1e6;
@@ -193,18 +314,11 @@ struct TensorTableArgs {
   uint8_t *cont;
 };
 
-// Bytes and contiguity of one tensor row (torch _collective_utils.py:230-232,
-// _prims_common/__init__.py:252-292).
-__device__ __forceinline__ void tensor_bytes_and_contiguity(int r, int64_t itemsize, const int64_t *sh, const int64_t *st,
-                                                            int64_t &nbytes, bool &contiguous) {
-  // the whole (zero-padded) rows are read at once, before the scan: one round of loads
-  // instead of one per dim
-  int64_t x[APC_MAX_RANK], y[APC_MAX_RANK];
-#pragma unroll
-  for (int i = 0; i < APC_MAX_RANK; ++i) {
-    x[i] = sh[i];
-    y[i] = st[i];
-  }
+// Bytes and contiguity of one tensor (torch _collective_utils.py:230-232,
+// _prims_common/__init__.py:252-292) from its zero-padded shape and stride rows, held in registers.
+template <typename Row>
+__device__ __forceinline__ void tensor_bytes_and_contiguity_of(int r, int64_t itemsize, const Row &x, const Row &y,
+                                                               int64_t &nbytes, bool &contiguous) {
   nbytes = itemsize;
   int64_t expected = 1, expected_max = 1;
   bool ok = true;
@@ -218,6 +332,19 @@ __device__ __forceinline__ void tensor_bytes_and_contiguity(int r, int64_t items
     expected *= x[i];
   }
   contiguous = ok;
+}
+
+__device__ __forceinline__ void tensor_bytes_and_contiguity(int r, int64_t itemsize, const int64_t *sh, const int64_t *st,
+                                                            int64_t &nbytes, bool &contiguous) {
+  // the whole (zero-padded) rows are read at once, before the scan: one round of loads
+  // instead of one per dim
+  int64_t x[APC_MAX_RANK], y[APC_MAX_RANK];
+#pragma unroll
+  for (int i = 0; i < APC_MAX_RANK; ++i) {
+    x[i] = sh[i];
+    y[i] = st[i];
+  }
+  tensor_bytes_and_contiguity_of(r, itemsize, x, y, nbytes, contiguous);
 }
 
 template <int BS>
@@ -572,6 +699,7 @@ __device__ __forceinline__ void tensor_info(const TableArgs &a, int t, int64_t &
   }
 }
 
+
 // What one mesh dim contributes, by (producer class, consumer class) with classes
 // 0 Replicate, 1 Partial, 2 Shard(0), 3 Shard(d != 0); only consulted when the two placement
 // codes differ.  One byte per pair:
@@ -720,13 +848,11 @@ static TermLayout term_layout(const apc_params &p) {
 // What a tile that also takes its row minima keeps in LDS beside the rest (a launch that does
 // not want them is a different instantiation and does not pay for the space).
 struct RowMinStage {
-  int64_t dup_row[APC_TILE_MAX_DUPS];  // first matrix rows of the identical edges
   // A row of at most 64 entries meets at most two of the 64-entry chunks the wavefronts
   // walk.  Slot 0 takes the part that holds the row's first column, slot 1 the part that
   // starts a chunk: one writer per slot, no atomics.
   double rmin[2][APC_TILE_MAX_ROWS];
   int rarg[2][APC_TILE_MAX_ROWS];
-  int64_t row_out;  // first matrix row of the tile's edge
 };
 struct NoRowMinStage {};
 
@@ -755,7 +881,6 @@ struct TileStage : std::conditional_t<RM, RowMinStage, NoRowMinStage> {
   // that the lanes of consecutive producer specs hit different banks
   uint32_t words[APC_TILE_MAX_COLS * (M * kWordsPerDim + 1)];
   alignas(16) uint32_t pair_base[M * 16];  // TermLayout::pair of the launch
-  int64_t dup[APC_TILE_MAX_DUPS];  // first entries of the identical edges
   double gb_unsharded;  // bytes / 1024^3 of the tile's tensor
   int mixed[4];         // per staging wavefront: some spec is not a DTensorSpec on the tile's tensor (generic loop)
   int cont;             // the tile's tensor is contiguous
@@ -784,6 +909,16 @@ static size_t stage_lds_bytes(const TermLayout &lay, int threads) {
   return sizeof(TileStage<M, RM>) - sizeof(double) * TermTable<M>::kEntries + sizeof(StagingScratch) * (size_t)(threads / 64) +
          sizeof(double) * entries;
 }
+
+// Where the copies of a tile's values go: lane k of EVERY wavefront holds the first entry and the
+// first matrix row of the k-th identical edge (k < dup_count <= APC_TILE_MAX_DUPS <= 64), read
+// back one by one as scalars (value_of_lane) when a value is stored to all copies: no LDS, no
+// load in the store loop.  row_out (wave-uniform) is the first matrix row of the tile's own edge.
+struct TileCopies {
+  int64_t entry0, row0;
+  int64_t row_out;
+};
+static_assert(APC_TILE_MAX_DUPS <= 64, "one lane per identical edge");
 
 // The fields of a tile record the entry loops use.
 struct TileView {
@@ -821,7 +956,7 @@ __device__ __forceinline__ double ring_at(double gb, const apc_params &p, int d,
 // the compute unit, so the number of rounds, not of loads, is what staging costs.
 template <int M, bool DERIVE, bool RM>
 __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs &a, const apc_tile &tile,
-                                           TileStage<M, RM> &st, int tid, int nthreads) {
+                                           TileStage<M, RM> &st, int tid, int nthreads, TileCopies &copies) {
   constexpr int NS = States<M>::kCount;
   const int rows = tile.counts & 0xFFFF, cols = tile.counts >> 16;
   const int t0 = tile.tensor;  // spec_tensor of the tile's first producer spec (checked by the host)
@@ -830,6 +965,7 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   bool mixed = !terms_wanted;
   const TermLayout &lay = a.lay;
   const int E = lay.exponents;  // wave-uniform; 0: general layout
+  const int lane = tid & 63, wave = tid >> 6;
   // (written and read by the first wavefront only, which stages the producer specs: in order.
   // A kernel argument indexed by the lane: one vector load, part of the round below.)
   uint32_t pair_word = 0;
@@ -837,7 +973,6 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   // power-of-two layout: the constants of array 2 + lane (whose chain this lane computes) and of
   // the array of the first value this thread computes, also read by lane
   constexpr int kComputed = 3 * M + 2;
-  const int lane = tid & 63, wave = tid >> 6;
   TermArrayConstants chain_of{};
   if (E != 0 && lane < kComputed) chain_of = lay.arrays[lane];
   // ---- the round of vector loads ------------------------------------------------------------
@@ -866,31 +1001,37 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
     row_zero = a.zero_cost[sr];
     row_args = a.num_args[sr];
   }
-  // (dup_count <= APC_TILE_MAX_DUPS <= nthreads)
-  const bool has_dup0 = tid < tile.dup_count;
-  int64_t dup0 = 0;
-  if (has_dup0) dup0 = a.dup_entry_begin[tile.dup_begin + tid];
-  int64_t dup_row0 = 0, row_out = 0;
+  // (every wavefront its own copy of the identical edges' offsets, in lanes 0 .. dup_count - 1)
+  const bool has_dup0 = lane < tile.dup_count;
+  copies.entry0 = copies.row0 = copies.row_out = 0;
+  if (has_dup0) copies.entry0 = a.dup_entry_begin[tile.dup_begin + lane];
   if constexpr (RM) {
-    if (has_dup0) dup_row0 = a.dup_row_begin[tile.dup_begin + tid];
-    row_out = a.edge_row_begin[tile.edge];  // wave-uniform: a scalar load
+    if (has_dup0) copies.row0 = a.dup_row_begin[tile.dup_begin + lane];
   }
-  // the contiguity byte of the tile's tensor, read as the aligned word around it (which lies
-  // in the byte's own page): a wave-uniform word goes through the scalar cache
+  // ---- the scalar loads of the round (wave-uniform addresses), issued together ---------------------
+  // The tile's tensor (row 0 when the tile has none: unconditional loads, the values are not
+  // used then) and the first matrix row of its edge.  The contiguity byte is read as the aligned
+  // word around it (which lies in the byte's own page).
+  const int t0c = t0 >= 0 ? t0 : 0;
   uint32_t contiguous = 1;
   int64_t tensor_nbytes = 0;
-  if (terms_wanted) {
-    if (!DERIVE) {
-      const uint8_t *flag = a.tensor_contiguous + t0;
-      const uint32_t byte = (uint32_t)(reinterpret_cast<uintptr_t>(flag) & 3);
-      const uint32_t word = *reinterpret_cast<const uint32_t *>(flag - byte);
-      contiguous = (word >> (8 * byte)) & 0xFFu;
-      tensor_nbytes = a.tensor_bytes[t0];
-    } else {  // (t0 is wave-uniform: scalar loads and scalar arithmetic)
-      bool ok;
-      tensor_info<true>(a, t0, tensor_nbytes, ok);
-      contiguous = ok ? 1u : 0u;
-    }
+  if constexpr (!DERIVE) {
+    const uint8_t *flag = a.tensor_contiguous + t0c;
+    const uint32_t byte = (uint32_t)(reinterpret_cast<uintptr_t>(flag) & 3);
+    const uint32_t word = uniform_load(reinterpret_cast<const uint32_t *>(flag - byte));
+    tensor_nbytes = uniform_load(a.tensor_bytes + t0c);
+    if constexpr (RM) copies.row_out = uniform_load(a.edge_row_begin + tile.edge);
+    fetch_arguments_now(word, tensor_nbytes, copies.row_out);
+    contiguous = (word >> (8 * byte)) & 0xFFu;
+  } else {
+    const int t_rank = uniform_load(a.rank + t0c), t_item = uniform_load(a.itemsize + t0c);
+    const i64x8 t_shape = uniform_load(reinterpret_cast<const i64x8 *>(a.shape + (int64_t)t0c * APC_MAX_RANK));
+    const i64x8 t_stride = uniform_load(reinterpret_cast<const i64x8 *>(a.stride + (int64_t)t0c * APC_MAX_RANK));
+    if constexpr (RM) copies.row_out = uniform_load(a.edge_row_begin + tile.edge);
+    fetch_arguments_now(t_rank, t_item, t_shape[0], t_stride[0], copies.row_out);
+    bool ok;
+    tensor_bytes_and_contiguity_of(t_rank, t_item, t_shape, t_stride, tensor_nbytes, ok);
+    contiguous = ok ? 1u : 0u;
   }
   // ---- term arrays (scalar operands only) ---------------------------------------------------
   if (terms_wanted && E != 0) {
@@ -970,11 +1111,8 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   // ---- what the loads brought, to LDS ---------------------------------------------------------
   if (tid == 0) st.cont = contiguous != 0;
   if (tid < 16 * M) st.pair_base[tid] = pair_word;
-  if (has_dup0) st.dup[tid] = dup0;
   if constexpr (RM) {
-    if (has_dup0) st.dup_row[tid] = dup_row0;
     if (tid < APC_TILE_MAX_ROWS) st.rmin[1][tid] = __builtin_inf();  // (slot 0 of every row is always written)
-    if (tid == 0) st.row_out = row_out;
   }
   if (has_col) {
     // info: bit0 valid spec, bit1 fully replicated, bits 4.. mask of sharded mesh dims
@@ -1113,20 +1251,26 @@ struct TileOut {
 // is checked per store.
 enum : int { kOutAny = 0, kOutAll = 1, kOutCost = 2 };
 
-// Stores one entry's values to its edge and to every identical edge.
+// Stores one entry's values to its edge and to every identical edge.  Called by every lane of
+// the wavefront (`active`: this lane holds an entry), so that the copies' offsets are read from
+// their lanes under uniform control flow.
 template <int OUT>
-__device__ __forceinline__ void store_entry(const TileOut &o, int dup_count, const int64_t *s_dup, uint32_t local,
-                                            double comm, double total, int trans) {
+__device__ __forceinline__ void store_entry(const TileOut &o, int dup_count, const TileCopies &copies, bool active,
+                                            uint32_t local, double comm, double total, int trans) {
   constexpr bool ALL = OUT == kOutAll, COST = OUT == kOutCost;
   const uint32_t off8 = local * 8u;
-  if (ALL || (!COST && o.comm)) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.comm) + off8) = comm;
-  if (ALL || (!COST && o.trans)) o.trans[local] = (uint8_t)trans;
-  if (ALL || COST || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost) + off8) = total;
+  if (active) {
+    if (ALL || (!COST && o.comm)) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.comm) + off8) = comm;
+    if (ALL || (!COST && o.trans)) o.trans[local] = (uint8_t)trans;
+    if (ALL || COST || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost) + off8) = total;
+  }
   for (int d = 0; d < dup_count; ++d) {
-    const int64_t delta = uniform_i64(s_dup[d]) - o.entry_begin;
-    if (ALL || (!COST && o.comm)) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.comm + delta) + off8) = comm;
-    if (ALL || (!COST && o.trans)) (o.trans + delta)[local] = (uint8_t)trans;
-    if (ALL || COST || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost + delta) + off8) = total;
+    const int64_t delta = value_of_lane(copies.entry0, d) - o.entry_begin;
+    if (active) {
+      if (ALL || (!COST && o.comm)) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.comm + delta) + off8) = comm;
+      if (ALL || (!COST && o.trans)) (o.trans + delta)[local] = (uint8_t)trans;
+      if (ALL || COST || o.cost) *reinterpret_cast<double *>(reinterpret_cast<char *>(o.cost + delta) + off8) = total;
+    }
   }
 }
 
@@ -1200,26 +1344,33 @@ __device__ __forceinline__ void row_min_chunk(double (&rmin)[2][APC_TILE_MAX_ROW
 // parts and stores minimum and first argmin to the row of the tile's edge and of every
 // identical edge.  (Called by every thread of the workgroup.)
 template <int M>
-__device__ __forceinline__ void row_min_finish(const TableArgs &a, TileStage<M, true> &st, const TileView &v, int tid,
-                                               int nthreads) {
+__device__ __forceinline__ void row_min_finish(const TableArgs &a, TileStage<M, true> &st, const TileView &v,
+                                               const TileCopies &copies, int tid, int nthreads) {
   __syncthreads();
   // lane = row, wavefront w takes the copies w, w + waves, ...: copy 0 is the tile's own edge, copy
   // d > 0 the d-th identical edge (a tile of many copies ends with a short store phase in every
   // wavefront instead of a long one in the first)
   const int row = tid & 63;
-  if (row >= v.rows) return;
-  double m = st.rmin[0][row];
-  int mc = st.rarg[0][row];
-  const double m1 = st.rmin[1][row];
-  if (m1 < m) {  // the later part wins only if strictly smaller
-    m = m1;
-    mc = st.rarg[1][row];
+  const bool live = row < v.rows;
+  double m = __builtin_inf();
+  int mc = 0;
+  if (live) {
+    m = st.rmin[0][row];
+    mc = st.rarg[0][row];
+    const double m1 = st.rmin[1][row];
+    if (m1 < m) {  // the later part wins only if strictly smaller
+      m = m1;
+      mc = st.rarg[1][row];
+    }
   }
   const int waves = nthreads >> 6;
-  for (int d = tid >> 6; d <= v.dup_count; d += waves) {
-    const int64_t out = (d == 0 ? st.row_out : st.dup_row[d - 1]) + v.row_begin + row;
-    a.row_min_out[out] = m;
-    a.row_arg_out[out] = v.col_begin + mc;
+  for (int d = uniform_i32(tid >> 6); d <= v.dup_count; d += waves) {
+    const int64_t first = d == 0 ? copies.row_out : value_of_lane(copies.row0, d - 1);  // (uniform control flow)
+    if (live) {
+      const int64_t out = first + v.row_begin + row;
+      a.row_min_out[out] = m;
+      a.row_arg_out[out] = v.col_begin + mc;
+    }
   }
 }
 
@@ -1229,7 +1380,8 @@ __device__ __forceinline__ void row_min_finish(const TableArgs &a, TileStage<M, 
 // wrapping round), so that the lanes of one pass hold consecutive entries.
 template <int M, bool CONT, bool RESCALE, int OUT>
 __device__ __forceinline__ void uniform_tile_entries_row_min(const apc_params &p, const TableArgs &a, TileStage<M, true> &st,
-                                                             const TileView &v, int tid, int nthreads) {
+                                                             const TileView &v, const TileCopies &copies, int tid,
+                                                             int nthreads) {
   const int n = v.rows * v.cols;
   const int dr = nthreads / v.cols, dc = nthreads - dr * v.cols;
   const int64_t tile_base = v.entry_begin + (int64_t)v.row_begin * v.n_src + v.col_begin;
@@ -1242,13 +1394,11 @@ __device__ __forceinline__ void uniform_tile_entries_row_min(const apc_params &p
                     a.cost_out ? a.cost_out + tile_base : nullptr, v.entry_begin};
   for (int wave_first = tid - lane - shift; wave_first < n; wave_first += nthreads, idx += nthreads) {
     const bool active = idx >= 0 && idx < n;
-    double comm, total = 0.0;
-    int trans;
-    if (active) {
-      uniform_entry<M, CONT, RESCALE>(p, a.lay, st, term_base(st, nthreads), r, c, comm, total, trans);
-      store_entry<OUT>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
-                       trans);
-    }
+    double comm = 0.0, total = 0.0;
+    int trans = 0;
+    if (active) uniform_entry<M, CONT, RESCALE>(p, a.lay, st, term_base(st, nthreads), r, c, comm, total, trans);
+    store_entry<OUT>(out, v.dup_count, copies, active, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
+                     trans);
     row_min_chunk(st.rmin, st.rarg, active, total, r, c, v.cols, lane);
     if (active) {
       c += dc;
@@ -1259,58 +1409,65 @@ __device__ __forceinline__ void uniform_tile_entries_row_min(const apc_params &p
       }
     }
   }
-  row_min_finish<M>(a, st, v, tid, nthreads);
+  row_min_finish<M>(a, st, v, copies, tid, nthreads);
 }
 
 // The per-entry loop of such a tile for `nthreads` threads (this one is `tid`): a flattened
 // (row, column) walk, so a wavefront writes 64 consecutive entries.
 template <int M, bool CONT, bool RESCALE, int OUT, bool RM>
 __device__ __forceinline__ void uniform_tile_entries(const apc_params &p, const TableArgs &a, const TileStage<M, RM> &st,
-                                                     const TileView &v, int tid, int nthreads) {
+                                                     const TileView &v, const TileCopies &copies, int tid, int nthreads) {
   const int n = v.rows * v.cols;
   const int dr = nthreads / v.cols, dc = nthreads - dr * v.cols;
   const int64_t tile_base = v.entry_begin + (int64_t)v.row_begin * v.n_src + v.col_begin;
   // A full-width tile is one contiguous run of entries: lanes are shifted so that every
   // wavefront store starts on a 64-entry boundary of the output arrays (whole 128-byte lines
-  // of the fp64 streams) instead of straddling one more line than it fills.
-  int first = tid - (v.cols == v.n_src ? (int)(tile_base & 63) : 0);
-  if (first < 0) first += nthreads;
+  // of the fp64 streams) instead of straddling one more line than it fills.  Every lane of a
+  // wavefront makes the same number of passes (a lane in front of the tile's first entry idles
+  // in the first one), so the copies' offsets are read under uniform control flow.
+  const int shift = v.cols == v.n_src ? (int)(tile_base & 63) : 0;
+  const int lane = tid & 63;
+  int idx = tid - shift;
+  const int first = idx < 0 ? idx + nthreads : idx;
   int r = first / v.cols, c = first - r * v.cols;
   const TileOut out{a.comm_out ? a.comm_out + tile_base : nullptr, a.trans_out ? a.trans_out + tile_base : nullptr,
                     a.cost_out ? a.cost_out + tile_base : nullptr, v.entry_begin};
-  for (int idx = first; idx < n; idx += nthreads) {
-    double comm, total;
-    int trans;
-    uniform_entry<M, CONT, RESCALE>(p, a.lay, st, term_base(st, nthreads), r, c, comm, total, trans);
-    store_entry<OUT>(out, v.dup_count, st.dup, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
+  for (int wave_first = tid - lane - shift; wave_first < n; wave_first += nthreads, idx += nthreads) {
+    const bool active = idx >= 0 && idx < n;
+    double comm = 0.0, total = 0.0;
+    int trans = 0;
+    if (active) uniform_entry<M, CONT, RESCALE>(p, a.lay, st, term_base(st, nthreads), r, c, comm, total, trans);
+    store_entry<OUT>(out, v.dup_count, copies, active, __umul24((uint32_t)r, (uint32_t)v.n_src) + (uint32_t)c, comm, total,
                      trans);
-    c += dc;
-    r += dr;
-    if (c >= v.cols) {
-      c -= v.cols;
-      r += 1;
+    if (active) {
+      c += dc;
+      r += dr;
+      if (c >= v.cols) {
+        c -= v.cols;
+        r += 1;
+      }
     }
   }
 }
 
 // Generic loop: pass-through edges and edges whose producer specs name different tensors.
-// ROW_MIN (tiles of whole rows only): every lane of a wavefront makes the same number of
-// passes and the row minima are taken on the way.
+// Every lane of a wavefront makes the same number of passes; ROW_MIN (tiles of whole rows only):
+// the row minima are taken on the way.
 template <int M, bool DERIVE, bool ROW_MIN, bool RM>
 __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const TableArgs &a, TileStage<M, RM> &st,
-                                                     const TileView &v, int tid, int nthreads) {
+                                                     const TileView &v, const TileCopies &copies, int tid, int nthreads) {
   const int n = v.rows * v.cols;
   const int lane = tid & 63;
   int r = tid / v.cols, c = tid - r * v.cols;
   const int dr = nthreads / v.cols, dc = nthreads - dr * v.cols;
   const bool no_producer = (v.flags & APC_EDGE_NO_PRODUCER) != 0;
-  for (int idx = tid; ROW_MIN ? idx - lane < n : idx < n; idx += nthreads) {
-    const bool active = !ROW_MIN || idx < n;
-    double total = 0.0;
+  for (int idx = tid; idx - lane < n; idx += nthreads) {
+    const bool active = idx < n;
+    double total = 0.0, comm = 0.0;
+    int trans = 0;
+    int64_t o = 0;
     if (active) {
       const int64_t local = (int64_t)(v.row_begin + r) * v.n_src + (v.col_begin + c);
-      double comm;
-      int trans = 0;
       const uint32_t src = st.colh[c].x, cinfo = st.colh[c].y;
       const RowRecord row = st.row[r];
       const uint32_t tgt = row.codes;
@@ -1330,16 +1487,18 @@ __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const 
         comm = entry_cost<M>(src, tgt, gb, sten_contiguous, p);
       }
       if (v.flags & APC_EDGE_GRAD_RESCALE) comm = comm / p.rescale;
-      const int64_t o = v.entry_begin + local;
+      o = v.entry_begin + local;
       total = comm + row.cpa + (double)trans;
       if (a.comm_out) a.comm_out[o] = comm;
       if (a.trans_out) a.trans_out[o] = (uint8_t)trans;
       if (a.cost_out) a.cost_out[o] = total;
-      for (int d = 0; d < v.dup_count; ++d) {
-        const int64_t od = o + (st.dup[d] - v.entry_begin);
-        if (a.comm_out) a.comm_out[od] = comm;
-        if (a.trans_out) a.trans_out[od] = (uint8_t)trans;
-        if (a.cost_out) a.cost_out[od] = total;
+    }
+    for (int d = 0; d < v.dup_count; ++d) {
+      const int64_t delta = value_of_lane(copies.entry0, d) - v.entry_begin;  // (uniform control flow)
+      if (active) {
+        if (a.comm_out) a.comm_out[o + delta] = comm;
+        if (a.trans_out) a.trans_out[o + delta] = (uint8_t)trans;
+        if (a.cost_out) a.cost_out[o + delta] = total;
       }
     }
     if constexpr (ROW_MIN && RM) row_min_chunk(st.rmin, st.rarg, active, total, r, c, v.cols, lane);
@@ -1352,25 +1511,25 @@ __device__ __forceinline__ void generic_tile_entries(const apc_params &p, const 
       }
     }
   }
-  if constexpr (ROW_MIN && RM) row_min_finish<M>(a, st, v, tid, nthreads);
+  if constexpr (ROW_MIN && RM) row_min_finish<M>(a, st, v, copies, tid, nthreads);
 }
 
 // All entries of a staged tile.  Row minima are taken when the caller wants them and the tile
 // holds whole rows (which the host arranges for every tile of a table before asking).
 template <int M, bool DERIVE, bool RM, int OUT>
 __device__ __forceinline__ void tile_entries(const apc_params &p, const TableArgs &a, TileStage<M, RM> &st,
-                                             const TileView &v, int tid, int nthreads) {
+                                             const TileView &v, const TileCopies &copies, int tid, int nthreads) {
   int mixed = st.mixed[0];
   for (int w = 1; w < nthreads / 64; ++w) mixed |= st.mixed[w];
   const bool row_minima = RM && v.cols == v.n_src;
   if (uniform_i32(mixed)) {
     if constexpr (RM) {
       if (row_minima) {
-        generic_tile_entries<M, DERIVE, true>(p, a, st, v, tid, nthreads);
+        generic_tile_entries<M, DERIVE, true>(p, a, st, v, copies, tid, nthreads);
         return;
       }
     }
-    generic_tile_entries<M, DERIVE, false>(p, a, st, v, tid, nthreads);
+    generic_tile_entries<M, DERIVE, false>(p, a, st, v, copies, tid, nthreads);
     return;
   }
   const bool rescale = (v.flags & APC_EDGE_GRAD_RESCALE) != 0;
@@ -1378,11 +1537,11 @@ __device__ __forceinline__ void tile_entries(const apc_params &p, const TableArg
   do {                                                                                            \
     if constexpr (RM) {                                                                           \
       if (row_minima) {                                                                           \
-        uniform_tile_entries_row_min<M, CONT_, RESCALE_, OUT>(p, a, st, v, tid, nthreads);        \
+        uniform_tile_entries_row_min<M, CONT_, RESCALE_, OUT>(p, a, st, v, copies, tid, nthreads); \
         break;                                                                                    \
       }                                                                                           \
     }                                                                                             \
-    uniform_tile_entries<M, CONT_, RESCALE_, OUT>(p, a, st, v, tid, nthreads);                    \
+    uniform_tile_entries<M, CONT_, RESCALE_, OUT>(p, a, st, v, copies, tid, nthreads);            \
   } while (0)
   if (uniform_i32(st.cont)) {
     if (rescale) { APC_TILE_LOOP(true, true); } else { APC_TILE_LOOP(true, false); }
@@ -1390,6 +1549,36 @@ __device__ __forceinline__ void tile_entries(const apc_params &p, const TableArg
     if (rescale) { APC_TILE_LOOP(false, true); } else { APC_TILE_LOOP(false, false); }
   }
 #undef APC_TILE_LOOP
+}
+
+// A tile record (64 bytes, wave-uniform) as one scalar load.
+__device__ __forceinline__ apc_tile load_tile_record(const apc_tile *tiles, int64_t tile_id) {
+  static_assert(sizeof(apc_tile) == sizeof(i32x16), "one 64-byte scalar load per record");
+  const i32x16 raw = uniform_load(reinterpret_cast<const i32x16 *>(tiles + tile_id));
+  apc_tile tile;
+  __builtin_memcpy(&tile, &raw, sizeof(tile));
+  return tile;
+}
+
+// A tile's record and the table addresses its wavefronts use, all fetched on entry under one wait
+// (fetch_arguments_now): the record's address needs only arguments that arrive in registers.
+template <bool DERIVE, bool RM, int OUT>
+__device__ __forceinline__ apc_tile fetch_tile(const apc_tile *tiles, int64_t tile_id, const TableArgs &a) {
+  const apc_tile tile = load_tile_record(tiles, tile_id);
+  if constexpr (DERIVE && RM && OUT == kOutCost)
+    fetch_arguments_now(tile.counts, a.lay.exponents, a.spec_codes, a.spec_tensor, a.dup_entry_begin, a.cost_out, a.rank, a.itemsize, a.shape,
+                        a.stride, a.flops, a.rw_bytes, a.dtype, a.zero_cost, a.num_args, a.edge_row_begin, a.dup_row_begin,
+                        a.row_min_out, a.row_arg_out);
+  else if constexpr (DERIVE)
+    fetch_arguments_now(tile.counts, a.lay.exponents, a.spec_codes, a.spec_tensor, a.dup_entry_begin, a.rank, a.itemsize, a.shape, a.stride,
+                        a.flops, a.rw_bytes, a.dtype, a.zero_cost, a.num_args);
+  else if constexpr (RM)
+    fetch_arguments_now(tile.counts, a.lay.exponents, a.spec_codes, a.spec_tensor, a.dup_entry_begin, a.tensor_bytes, a.tensor_contiguous,
+                        a.per_arg, a.edge_row_begin, a.dup_row_begin);
+  else
+    fetch_arguments_now(tile.counts, a.lay.exponents, a.spec_codes, a.spec_tensor, a.dup_entry_begin, a.tensor_bytes, a.tensor_contiguous,
+                        a.per_arg);
+  return tile;
 }
 
 template <int M, int kTileThreads, bool RM, int OUT>
@@ -1400,10 +1589,13 @@ __device__ __forceinline__ void redistribute_tile(const apc_params &p, const Tab
   static_assert(kTileThreads == 64 || kTileThreads == 128 || kTileThreads == 256, "wavefronts per tile: 1, 2 or 4");
   static_assert(kTileThreads >= APC_TILE_MAX_COLS && kTileThreads >= APC_TILE_MAX_ROWS &&
                 kTileThreads >= APC_TILE_MAX_DUPS, "one staging round covers a tile");
-  const apc_tile tile = tiles[tile_id];
-  stage_tile<M, false, RM>(p, a, tile, stage, threadIdx.x, kTileThreads);
+  const apc_tile tile = fetch_tile<false, RM, OUT>(tiles, tile_id, a);
+  // a record the host validator would have rejected (more identical edges than lanes hold): skipped
+  if ((unsigned)tile.dup_count > (unsigned)APC_TILE_MAX_DUPS) return;
+  TileCopies copies;
+  stage_tile<M, false, RM>(p, a, tile, stage, threadIdx.x, kTileThreads, copies);
   __syncthreads();
-  tile_entries<M, false, RM, OUT>(p, a, stage, view_of(tile), threadIdx.x, kTileThreads);
+  tile_entries<M, false, RM, OUT>(p, a, stage, view_of(tile), copies, threadIdx.x, kTileThreads);
 }
 
 // Wavefronts per SIMD the tile kernels ask for: what the LDS of their larger, row-minimum
@@ -1466,10 +1658,12 @@ void build_tables_kernel(const apc_tile *tiles, int n_tiles, int xcd_shift, int6
     const int64_t tile_id = (b & ((1 << xcd_shift) - 1)) * per + (b >> xcd_shift);
     if (tile_id >= n_tiles) return;
     TileStage<M, RM> &stage = *reinterpret_cast<TileStage<M, RM> *>(s_raw);
-    const apc_tile tile = tiles[tile_id];
-    stage_tile<M, true, RM>(p, a, tile, stage, threadIdx.x, kThreads);
+    const apc_tile tile = fetch_tile<true, RM, OUT>(tiles, tile_id, a);
+    if ((unsigned)tile.dup_count > (unsigned)APC_TILE_MAX_DUPS) return;  // (see redistribute_tile)
+    TileCopies copies;
+    stage_tile<M, true, RM>(p, a, tile, stage, threadIdx.x, kThreads, copies);
     __syncthreads();
-    tile_entries<M, true, RM, OUT>(p, a, stage, view_of(tile), threadIdx.x, kThreads);
+    tile_entries<M, true, RM, OUT>(p, a, stage, view_of(tile), copies, threadIdx.x, kThreads);
     return;
   }
   const int64_t tb = b - tile_blocks;
@@ -1810,7 +2004,7 @@ int check_params(const apc_params *p) {
 
 extern "C" {
 
-int apc_version(void) { return 1; }
+int apc_version(void) { return APC_ABI_VERSION; }
 
 const char *apc_last_error(void) { return g_err; }
 
@@ -2115,6 +2309,8 @@ static int build_tables_impl(const apc_params *params, int64_t n_tensors, const 
     return fail(-1, "apc_build_tables: NULL strategy array");
   if (n_tiles > 0 && (!spec_codes || !spec_tensor || !tiles || !rank || !itemsize || !shape || !stride))
     return fail(-1, "apc_build_tables: NULL table");
+  // (a tile without a tensor still loads row 0 of the tensor table: unconditional loads)
+  if (n_tiles > 0 && n_tensors == 0) return fail(-1, "apc_build_tables: tiles need a tensor table with at least one row");
   const int xs = xcd_shift();
   int threads = 256;
   if (n_tiles > 0) {

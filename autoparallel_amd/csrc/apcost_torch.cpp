@@ -662,7 +662,10 @@ void validate_tables(const Tensor &params, const Tensor &tensor_rank, const Tens
   check_rc(rc, "apc_validate_tables_host");
 }
 
-int64_t abi_version() { return apc_version(); }
+// The interface version this layer was compiled against; the binding compares it with what the
+// loaded library reports (apc_version) before the first call.
+int64_t abi_version() { return APC_ABI_VERSION; }
+int64_t library_abi_version() { return apc_version(); }
 
 }  // namespace
 
@@ -678,6 +681,7 @@ TORCH_LIBRARY(apcost, m) {
   "Tensor? comm, Tensor? transition, Tensor? cost, Tensor? edge_row_begin, Tensor? dup_row_begin, Tensor? row_min, " \
   "Tensor? row_argmin"
   m.def("abi_version() -> int", &abi_version);
+  m.def("library_abi_version() -> int", &library_abi_version);
   m.def("validate_tables(Tensor params, Tensor tensor_rank, Tensor spec_codes, Tensor spec_tensor, Tensor edge_src_begin, "
         "Tensor edge_n_src, Tensor edge_tgt_begin, Tensor edge_n_tgt, Tensor edge_flags, Tensor edge_pt_begin, "
         "Tensor edge_entry_begin, Tensor edge_strat_begin, int n_pt, int n_strategies, Tensor tiles, Tensor dup_entry_begin) -> ()",

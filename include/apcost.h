@@ -50,13 +50,20 @@
 extern "C" {
 #endif
 
+/* Version of this interface: the value apc_version() of a matching library returns.  It changes
+ * whenever a struct layout, a limit below or the meaning of an argument changes (2: at most 32
+ * identical edges per tile instead of 127; the row-minimum entry points write the minima of the
+ * assembled cost whichever arrays are stored).  A binding compares the two before its first call. */
+#define APC_ABI_VERSION 2
+
 #define APC_MAX_RANK 8
 #define APC_MAX_MESH 4
 #define APC_MAX_DTYPES 8
 #define APC_TILE_MAX_COLS 64 /* producer specs staged in LDS per tile */
 #define APC_TILE_MAX_ROWS 64 /* consumer specs staged in LDS per tile */
 #define APC_TILE_MAX_DUPS 32 /* identical edges served by one tile (offsets staged in LDS); a larger group of
-                              identical edges is served by several tiled edges */
+                              identical edges is served by several tiled edges.  apc_validate_tables_host
+                              rejects a tile with more; the kernels leave such a tile unwritten */
 #define APC_MAX_STRATEGIES (1 << 22) /* strategies of one node: a tile's rows span < 4 GiB of fp64 */
 
 #define APC_EDGE_GRAD_RESCALE 1 /* consumer is a parameter-gradient node (optimize_sharding.py:358-359) */

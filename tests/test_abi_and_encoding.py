@@ -26,7 +26,9 @@ def test_library_exports_every_declared_symbol():
     for name in sorted(declared):
         assert hasattr(lib, name), f"{name} declared in apcost.h but not exported"
     assert declared == set(_native.EXPORTS)
-    assert lib.apc_version() == 1
+    # the header's constant, the library's answer and the binding's mirror agree
+    version = int(re.search(r"#define APC_ABI_VERSION (\d+)", header).group(1))
+    assert lib.apc_version() == version == _native.APC_ABI_VERSION
 
 
 def test_params_struct_layout_matches_header(tmp_path):
@@ -284,6 +286,22 @@ def test_validator_rejects_tile_record_that_disagrees_with_its_edge():
     tb.tile_records["edge"][0] = tb.n_edges
     with pytest.raises(RuntimeError, match="out of range"):
         tb.validate(CostModelParams.from_mesh((4, 2)))
+
+
+def test_validator_rejects_a_tile_with_more_identical_edges_than_the_kernels_stage():
+    """The tile kernels stage APC_TILE_MAX_DUPS offsets of identical edges in LDS; a record with
+    more (a tile array built against an older header, which allowed 127) is refused on the host."""
+    tb = twin_graph(stress_dag(seed=8, n_nodes=60, mesh_sizes=(4, 2), max_strategies=10))
+    tb.build_tiles(256, dedupe=True)
+    params = CostModelParams.from_mesh((4, 2))
+    tb.validate(params)
+    t = int(np.nonzero(tb.tile_records["dup_count"] > 0)[0][0])
+    assert int(re.search(r"#define APC_TILE_MAX_DUPS (\d+)", open(os.path.join(ROOT, "include", "apcost.h")).read()).group(1)) \
+        == _native.APC_TILE_MAX_DUPS == 32
+    for bad in (_native.APC_TILE_MAX_DUPS + 1, 127, -1):
+        tb.tile_records["dup_count"][t] = bad
+        with pytest.raises(RuntimeError, match="duplicate list"):
+            tb.validate(params)
 
 
 def test_validator_needs_pass_through_values_for_producerless_edges():

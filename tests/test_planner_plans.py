@@ -237,7 +237,6 @@ def test_collector_is_paused_while_planning_and_restored_afterwards(meshes):
     model_fn, input_fn = make_model_and_inputs(mesh, "small_param")
     with torch.device("meta"):
         model = model_fn()
-    gc.unfreeze()  # (a planner that an earlier test entered and never left)
     assert gc.isenabled() and gc.get_freeze_count() == 0
     with OraclePlanner(model, input_fn, mesh) as autop:
         assert gc.isenabled() and gc.get_freeze_count() > 0
@@ -249,14 +248,42 @@ def test_collector_is_paused_while_planning_and_restored_afterwards(meshes):
         def _enter(self):
             raise ValueError("construction failed")
 
-    gc.disable()
+    # `with` does not call __exit__ after a failing __enter__: nothing stays frozen, the
+    # collector is in the caller's state
+    for on in (False, True):
+        (gc.enable if on else gc.disable)()
+        try:
+            with pytest.raises(ValueError, match="construction failed"):
+                with Failing(model, input_fn, mesh):
+                    pass
+            assert gc.isenabled() == on and gc.get_freeze_count() == 0
+        finally:
+            gc.enable()
+
+    class FailsAfterCapture(OraclePlanner):
+        class optimizer_cls(OracleOptimizer):
+            def __init__(self, *a, **k):
+                raise ValueError("optimizer failed")
+
+    with pytest.raises(ValueError, match="optimizer failed"):
+        with FailsAfterCapture(model, input_fn, mesh):
+            pass
+    assert gc.isenabled() and gc.get_freeze_count() == 0
+    # the capture context was closed: a new planner can enter
+    with OraclePlanner(model, input_fn, mesh) as autop:
+        assert autop.active is True
+
+    # an application that froze its own objects keeps them frozen: the planner neither adds to
+    # the frozen set nor thaws it
+    gc.freeze()
     try:
-        with pytest.raises(ValueError, match="construction failed"):
-            Failing(model, input_fn, mesh).__enter__()
-        assert not gc.isenabled()
+        theirs = gc.get_freeze_count()
+        assert theirs > 0
+        with OraclePlanner(model, input_fn, mesh) as autop:
+            assert gc.get_freeze_count() == theirs
+        assert gc.get_freeze_count() == theirs
     finally:
         gc.unfreeze()
-        gc.enable()
 
 
 def test_unsolvable_problem_raises(meshes):
