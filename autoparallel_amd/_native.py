@@ -11,13 +11,14 @@ import os
 
 from ._build import LIB_PATH, TORCH_EXT_PATH
 
-APC_ABI_VERSION = 2  # include/apcost.h: the interface this binding's structs and limits mirror
+APC_ABI_VERSION = 3  # include/apcost.h: the interface this binding's structs and limits mirror
 APC_MAX_RANK = 8
 APC_MAX_MESH = 4
 APC_MAX_DTYPES = 8
 APC_TILE_MAX_COLS = 64
 APC_TILE_MAX_ROWS = 64
 APC_TILE_MAX_DUPS = 32
+APC_PACKED_MAX_DUPS = 16
 
 EDGE_GRAD_RESCALE = 1
 EDGE_NO_PRODUCER = 2
@@ -42,6 +43,8 @@ class ApcParams(ctypes.Structure):
         ("inv_mesh", ctypes.c_double * APC_MAX_MESH),
         ("inv_hbm_bw", ctypes.c_double),
         ("inv_rw_eff", ctypes.c_double),
+        ("inv_compute_eff", ctypes.c_double),
+        ("inv_gpu_flops", ctypes.c_double * APC_MAX_DTYPES),
     ]
 
 
@@ -83,6 +86,10 @@ EXPORTS = (
     "apc_diffusion_sweeps",
     "apc_redistribute_tables_static",
     "apc_strategy_inputs",
+    "apc_validate_packed_tiles_host",
+    "apc_build_tables_packed",
+    "apc_calibrate_launch",
+    "apc_calibrate_fill",
 )
 
 _lib = None

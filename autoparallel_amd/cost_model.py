@@ -142,4 +142,7 @@ class CostModelParams:
             c.inv_mesh[i] = 1.0 / float(self.mesh_sizes[i])
         c.inv_hbm_bw = 1.0 / self.hbm_bw
         c.inv_rw_eff = 1.0 / self.rw_eff
+        c.inv_compute_eff = 1.0 / self.compute_eff
+        for i, g in enumerate(self.gpu_flops):
+            c.inv_gpu_flops[i] = 1.0 / g if g else 0.0
         return c

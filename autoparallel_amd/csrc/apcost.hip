@@ -14,6 +14,7 @@
 
 #include <cmath>
 #include <cstdarg>
+#include <cstddef>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -517,6 +518,19 @@ __device__ __forceinline__ double compute_cost_of(const apc_params &p, bool zero
   return t > rw ? t : rw;
 }
 
+// The same value with the divisions taken through the checked reciprocals (div_by): gf / inv_gf =
+// the device row's throughput for the strategy's dtype and its reciprocal, 0 when unsupported.
+__device__ __forceinline__ double compute_cost_through_reciprocals(const apc_params &p, bool zero_cost, int64_t rw_bytes,
+                                                                   int64_t flops, double gf, double inv_gf) {
+  if (zero_cost) return 0.0;
+  const double rw = rw_time_r((double)rw_bytes, p);
+  if (flops == 0) return rw;
+  if (gf == 0.0) return NAN;  // compute_estimation.py:198-201 raises ValueError (flagged by compute_costs_block)
+  double t = div_by((double)flops, gf, inv_gf) * 1e6;
+  t = div_by(t, p.compute_eff, p.inv_compute_eff);
+  return t > rw ? t : rw;
+}
+
 template <int BS>
 __device__ __forceinline__ void compute_costs_block(int64_t block, const apc_params &p, const ComputeCostArgs &a) {
   const int64_t s = block * BS + threadIdx.x;
@@ -913,12 +927,20 @@ static size_t stage_lds_bytes(const TermLayout &lay, int threads) {
 // Where the copies of a tile's values go: lane k of EVERY wavefront holds the first entry and the
 // first matrix row of the k-th identical edge (k < dup_count <= APC_TILE_MAX_DUPS <= 64), read
 // back one by one as scalars (value_of_lane) when a value is stored to all copies: no LDS, no
-// load in the store loop.  row_out (wave-uniform) is the first matrix row of the tile's own edge.
+// load in the store loop.  row_out (the same in every lane) is the first matrix row of the tile's own edge.
 struct TileCopies {
   int64_t entry0, row0;
   int64_t row_out;
 };
 static_assert(APC_TILE_MAX_DUPS <= 64, "one lane per identical edge");
+
+// Waits for the loads of `copies` now.  On this hardware loads and stores share one counter of
+// outstanding vector-memory operations, and a wait for a load behind which stores were issued
+// can only be a wait for all of them: offsets first touched inside the store loop would make
+// every wavefront sit out the full round trip of its first store.  Called before the stores begin.
+__device__ __forceinline__ void settle(TileCopies &copies) {
+  __asm__ volatile("" : "+v"(copies.entry0), "+v"(copies.row0), "+v"(copies.row_out));
+}
 
 // The fields of a tile record the entry loops use.
 struct TileView {
@@ -1007,6 +1029,9 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
   if (has_dup0) copies.entry0 = a.dup_entry_begin[tile.dup_begin + lane];
   if constexpr (RM) {
     if (has_dup0) copies.row0 = a.dup_row_begin[tile.dup_begin + lane];
+    // (wave-uniform, but needed last: with the vector loads of the round, so that the scalar
+    // loads the term arrays wait for are one round and not two)
+    copies.row_out = a.edge_row_begin[tile.edge];
   }
   // ---- the scalar loads of the round (wave-uniform addresses), issued together ---------------------
   // The tile's tensor (row 0 when the tile has none: unconditional loads, the values are not
@@ -1020,15 +1045,13 @@ __device__ __forceinline__ void stage_tile(const apc_params &p, const TableArgs 
     const uint32_t byte = (uint32_t)(reinterpret_cast<uintptr_t>(flag) & 3);
     const uint32_t word = uniform_load(reinterpret_cast<const uint32_t *>(flag - byte));
     tensor_nbytes = uniform_load(a.tensor_bytes + t0c);
-    if constexpr (RM) copies.row_out = uniform_load(a.edge_row_begin + tile.edge);
-    fetch_arguments_now(word, tensor_nbytes, copies.row_out);
+    fetch_arguments_now(word, tensor_nbytes);
     contiguous = (word >> (8 * byte)) & 0xFFu;
   } else {
     const int t_rank = uniform_load(a.rank + t0c), t_item = uniform_load(a.itemsize + t0c);
     const i64x8 t_shape = uniform_load(reinterpret_cast<const i64x8 *>(a.shape + (int64_t)t0c * APC_MAX_RANK));
     const i64x8 t_stride = uniform_load(reinterpret_cast<const i64x8 *>(a.stride + (int64_t)t0c * APC_MAX_RANK));
-    if constexpr (RM) copies.row_out = uniform_load(a.edge_row_begin + tile.edge);
-    fetch_arguments_now(t_rank, t_item, t_shape[0], t_stride[0], copies.row_out);
+    fetch_arguments_now(t_rank, t_item, t_shape[0], t_stride[0]);
     bool ok;
     tensor_bytes_and_contiguity_of(t_rank, t_item, t_shape, t_stride, tensor_nbytes, ok);
     contiguous = ok ? 1u : 0u;
@@ -1298,10 +1321,11 @@ __device__ __forceinline__ double value_of_lane(double x, int lane) {  // lane: 
 // the end of its 16 lanes.  Lanes 16, 32 and 48 hold such a part for a row that came in from the
 // lanes before them: their values are read as scalars and joined, in lane order, by the lanes
 // whose row reaches them.  The first lane of every run of one row writes the row's slot.
-__device__ __forceinline__ void row_min_chunk(double (&rmin)[2][APC_TILE_MAX_ROWS], int (&rarg)[2][APC_TILE_MAX_ROWS],
-                                              bool active, double value, int r, int c, int cols, int lane) {
-  double m = active ? value : __builtin_inf();
-  int mc = c;
+// row_min_in_wave: the reduction itself; on return a lane holds minimum and first argmin of its
+// row's entries from itself to the row's end within the wavefront (the whole row for c == 0).
+__device__ __forceinline__ void row_min_in_wave(bool active, double value, int c, int cols, int lane, double &m, int &mc) {
+  m = active ? value : __builtin_inf();
+  mc = c;
   const int in_row16 = lane & 15;
 #define APC_ROW_MIN_STEP(N_)                                                            \
   if (N_ < cols) { /* (cols is wave-uniform) */                                         \
@@ -1333,6 +1357,13 @@ __device__ __forceinline__ void row_min_chunk(double (&rmin)[2][APC_TILE_MAX_ROW
     APC_ROW_MIN_JOIN(48)
   }
 #undef APC_ROW_MIN_JOIN
+}
+
+__device__ __forceinline__ void row_min_chunk(double (&rmin)[2][APC_TILE_MAX_ROWS], int (&rarg)[2][APC_TILE_MAX_ROWS],
+                                              bool active, double value, int r, int c, int cols, int lane) {
+  double m;
+  int mc;
+  row_min_in_wave(active, value, c, cols, lane, m, mc);
   if (active && (c == 0 || lane == 0)) {
     const int slot = c == 0 ? 0 : 1;
     rmin[slot][r] = m;
@@ -1365,7 +1396,7 @@ __device__ __forceinline__ void row_min_finish(const TableArgs &a, TileStage<M, 
   }
   const int waves = nthreads >> 6;
   for (int d = uniform_i32(tid >> 6); d <= v.dup_count; d += waves) {
-    const int64_t first = d == 0 ? copies.row_out : value_of_lane(copies.row0, d - 1);  // (uniform control flow)
+    const int64_t first = d == 0 ? uniform_i64(copies.row_out) : value_of_lane(copies.row0, d - 1);  // (uniform control flow)
     if (live) {
       const int64_t out = first + v.row_begin + row;
       a.row_min_out[out] = m;
@@ -1594,6 +1625,7 @@ __device__ __forceinline__ void redistribute_tile(const apc_params &p, const Tab
   if ((unsigned)tile.dup_count > (unsigned)APC_TILE_MAX_DUPS) return;
   TileCopies copies;
   stage_tile<M, false, RM>(p, a, tile, stage, threadIdx.x, kTileThreads, copies);
+  settle(copies);
   __syncthreads();
   tile_entries<M, false, RM, OUT>(p, a, stage, view_of(tile), copies, threadIdx.x, kTileThreads);
 }
@@ -1662,6 +1694,7 @@ void build_tables_kernel(const apc_tile *tiles, int n_tiles, int xcd_shift, int6
     if ((unsigned)tile.dup_count > (unsigned)APC_TILE_MAX_DUPS) return;  // (see redistribute_tile)
     TileCopies copies;
     stage_tile<M, true, RM>(p, a, tile, stage, threadIdx.x, kThreads, copies);
+    settle(copies);
     __syncthreads();
     tile_entries<M, true, RM, OUT>(p, a, stage, view_of(tile), copies, threadIdx.x, kThreads);
     return;
@@ -1670,6 +1703,355 @@ void build_tables_kernel(const apc_tile *tiles, int n_tiles, int xcd_shift, int6
   if (tb < spec_blocks) spec_tables_block<kThreads>(tb, p, sp, reinterpret_cast<int64_t *>(s_raw));
   else if (tb < spec_blocks + tensor_blocks) tensor_tables_block<kThreads>(tb - spec_blocks, t);
   else compute_costs_block<kThreads>(tb - spec_blocks - tensor_blocks, p, c);
+}
+
+// ------------------------------------------------------------------------------------------
+// Packed tiles: the planner's pass over a small table, every wavefront on its own.
+//
+// A table of a few million entries is bound by the latency of one workgroup: all workgroups are
+// resident at once, stage and then store in step, and the chain of dependent loads in front of
+// the first store decides the launch.  Here a workgroup's loads depend on nothing but its index
+// (one fixed-size record per tile, copied out of the tables by the host: apc_packed_tile), and
+// nothing is staged in LDS: lane j of every wavefront holds producer spec j, consumer spec j and
+// the compute cost / num_args of consumer strategy j; a wavefront walks whole matrix rows,
+// fetches an entry's two specs from their lanes, evaluates the entry directly
+// (collective_runtime_estimation.py:37-153 in the reference's operation order, divisions through
+// the checked reciprocals), reduces the row minima across its lanes and stores values and minima to
+// the tile's edge and to every identical edge.  No barrier, no second pass over the rows.
+// ------------------------------------------------------------------------------------------
+struct DimConstants {  // of one mesh dim, wave-uniform
+  double n, inv_n, bw, inv_bw;
+  double hops1, lat1;  // all-gather, reduce-scatter, all-to-all: n - 1 hops (torch _collective_utils.py:281-301)
+  double hops2, lat2;  // all-reduce: 2 (n - 1) hops (:304-313)
+};
+template <int M>
+struct FlatConstants {
+  DimConstants dim[M];
+};
+
+template <int M>
+__device__ __forceinline__ FlatConstants<M> flat_constants(const apc_params &p) {
+  FlatConstants<M> k;
+#pragma unroll
+  for (int i = 0; i < M; ++i) {
+    DimConstants &d = k.dim[i];
+    d.n = (double)p.mesh_size[i];
+    d.inv_n = p.inv_mesh[i];
+    d.bw = p.bw[i];
+    d.inv_bw = p.inv_bw[i];
+    d.hops1 = (double)(p.mesh_size[i] - 1);
+    d.hops2 = (double)(2 * (p.mesh_size[i] - 1));
+    d.lat1 = p.base_latency + d.hops1 * p.lat[i];
+    d.lat2 = p.base_latency + d.hops2 * p.lat[i];
+  }
+  return k;
+}
+
+// entry_cost without branches: every lane of a wavefront evaluates its own (producer spec,
+// consumer spec) pair, whatever collectives the pair needs.  What a mesh dim adds is selected,
+// not branched on: the ring term of the one collective the dim can need (none: + 0.0, which
+// leaves a non-negative sum unchanged), 0, 1 or 2 read+write reshuffles ((double)copies x rw:
+// 0.0, rw, 2.0 x rw).  FIRST = 1 (2-D meshes): dim 1 before dim 0 (:146-151).  CONT: the tensor
+// is contiguous (no lane ever adds the non-contiguity term).  gb = bytes / num_shards / 1024^3.
+template <int M, int FIRST, bool CONT>
+__device__ __forceinline__ double entry_cost_flat(uint32_t srcp, uint32_t tgtp, double gb, const apc_params &p,
+                                                  const FlatConstants<M> &k) {
+  double cost = 0.0;
+  bool banned = false, cont = CONT;
+  bool tgt_partial = false;
+#pragma unroll
+  for (int s = 0; s < M; ++s) {
+    const int i = (M == 2 && FIRST == 1) ? 1 - s : s;
+    const DimConstants &d = k.dim[i];
+    const uint32_t c = (srcp >> (8 * i)) & 0xFF, t = (tgtp >> (8 * i)) & 0xFF;
+    const bool neq = c != t;
+    const uint32_t ck = c >> 6, tk = t >> 6;
+    tgt_partial |= tk == 1;
+    const bool from_shard = neq && ck == 2, from_partial = neq && ck == 1;
+    const bool is_ag = from_shard && tk == 0, is_a2a = from_shard && tk == 2;  // :83-113
+    const bool is_ar = from_partial && tk == 0, is_rs = from_partial && tk == 2;  // :115-130
+    banned |= neq && tk == 1 && ck != 1;  // :131-138
+    if (!CONT) {  // :81-82: charged once, on the bytes before this dim
+      const double rw_before = rw_time_r(gb * 2 * 1073741824.0, p);
+      cost += (neq && !cont) ? rw_before : 0.0;
+      cont = cont || neq;  // :141
+    }
+    const double x = is_ag ? gb * d.n : gb;  // an all-gather is charged on the gathered bytes (:86)
+    const double hops = is_ar ? d.hops2 : d.hops1;
+    const double ring0 = (is_ar ? d.lat2 : d.lat1) + div_by(div_by(x * hops, d.n, d.inv_n), d.bw, d.inv_bw) * 1e6;
+    const double ring = is_a2a ? ring0 * p.a2a_scale : ring0;  // :22-32
+    cost += (from_shard || from_partial) && tk != 1 ? ring : 0.0;
+    const double rw = rw_time_r(x * 2 * 1073741824.0, p);
+    const uint32_t cn = (c & 0x0F) != 0 ? 1u : 0u, tn = (t & 0x0F) != 0 ? 1u : 0u;
+    const uint32_t copies = is_ag ? cn : is_a2a ? cn + tn : is_rs ? tn : 0u;
+    cost += copies == 0u ? 0.0 : copies == 1u ? rw : 2.0 * rw;
+    gb = is_ag ? x : is_rs ? div_by(gb, d.n, d.inv_n) : gb;  // :86, :128
+  }
+  if (srcp == 0u) return tgt_partial ? __builtin_inf() : 0.0;  // :56-62
+  return banned ? __builtin_inf() : cost;
+}
+
+// The same entry on a mesh whose sizes are all powers of two (TermLayout::exponents != 0; "Term
+// arrays" above): the running bytes are the tensor's bytes x 2^(j - L - 30) for an integer j a lane
+// carries from dim to dim, and every term is one ldexp of a wave-uniform chain value: no division
+// per entry.  R / B[d]: the chains of the read+write and of dim d's one-hop ring on the tensor's
+// bytes (TermArrayConstants of arrays 2 and 4 + 3 d).
+template <int M>
+struct Pow2Constants {
+  double R, B[M];
+  double lat1[M], lat2[M];
+  int lg[M], shift[M];  // log2 n_d; -L - 30 - log2 n_d
+  int rw_shift;         // -L - 30 + 31
+  double floor;         // launch floor of a read+write
+};
+
+template <int M, int FIRST, bool CONT>
+__device__ __forceinline__ double entry_cost_pow2(uint32_t srcp, uint32_t tgtp, int j, double a2a_scale, const Pow2Constants<M> &k) {
+  double cost = 0.0;
+  bool banned = false, cont = CONT, tgt_partial = false;
+#pragma unroll
+  for (int s = 0; s < M; ++s) {
+    const int i = (M == 2 && FIRST == 1) ? 1 - s : s;
+    const uint32_t c = (srcp >> (8 * i)) & 0xFF, t = (tgtp >> (8 * i)) & 0xFF;
+    const bool neq = c != t;
+    const uint32_t ck = c >> 6, tk = t >> 6;
+    tgt_partial |= tk == 1;
+    const bool from_shard = neq && ck == 2, from_partial = neq && ck == 1;
+    const bool is_ag = from_shard && tk == 0, is_a2a = from_shard && tk == 2;
+    const bool is_ar = from_partial && tk == 0, is_rs = from_partial && tk == 2;
+    banned |= neq && tk == 1 && ck != 1;
+    if (!CONT) {
+      const double before = __builtin_ldexp(k.R, j + k.rw_shift);
+      cost += (neq && !cont) ? (before > k.floor ? before : k.floor) : 0.0;
+      cont = cont || neq;
+    }
+    const int jx = is_ag ? j + k.lg[i] : j;  // an all-gather is charged on the gathered bytes
+    const double ring0 = (is_ar ? k.lat2[i] : k.lat1[i]) + __builtin_ldexp(k.B[i], jx + k.shift[i] + (is_ar ? 1 : 0));
+    const double ring = is_a2a ? ring0 * a2a_scale : ring0;
+    cost += (from_shard || from_partial) && tk != 1 ? ring : 0.0;
+    const double rw0 = __builtin_ldexp(k.R, jx + k.rw_shift);
+    const double rw = rw0 > k.floor ? rw0 : k.floor;
+    const uint32_t cn = (c & 0x0F) != 0 ? 1u : 0u, tn = (t & 0x0F) != 0 ? 1u : 0u;
+    const uint32_t copies = is_ag ? cn : is_a2a ? cn + tn : is_rs ? tn : 0u;
+    cost += copies == 0u ? 0.0 : copies == 1u ? rw : 2.0 * rw;
+    j = is_ag ? jx : is_rs ? j - k.lg[i] : j;
+  }
+  if (srcp == 0u) return tgt_partial ? __builtin_inf() : 0.0;
+  return banned ? __builtin_inf() : cost;
+}
+
+__device__ __forceinline__ int from_lane(int v, int lane) { return __builtin_amdgcn_ds_bpermute(lane << 2, v); }
+__device__ __forceinline__ double from_lane(double v, int lane) {
+  return __hiloint2double(from_lane(__double2hiint(v), lane), from_lane(__double2loint(v), lane));
+}
+__device__ __forceinline__ int64_t from_lane_i64(int64_t v, int lane) {
+  const uint32_t lo = (uint32_t)from_lane((int)(uint32_t)v, lane), hi = (uint32_t)from_lane((int)(uint32_t)((uint64_t)v >> 32), lane);
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+// value -> *(double *)((char *)base + byte_offset) for a wave-uniform base: the address stays a
+// scalar register pair plus a 32-bit lane offset (left to the compiler, the sum is re-associated
+// into per-lane 64-bit arithmetic inside a loop over bases).  A store needs no wait before the
+// wavefront ends, and a wait by count for an older load stays correct with younger stores in
+// flight (loads return in order among themselves).
+// (s_nop 4: a vector-memory instruction may read a scalar register a vector instruction wrote,
+// such as a value fetched from a lane, only five cycles later; the compiler inserts that wait
+// for its own instructions and does not look inside an asm statement.)
+__device__ __forceinline__ void store_at(double *base, uint32_t byte_offset, double value) {
+  __asm__ volatile("s_nop 4\n\tglobal_store_dwordx2 %0, %1, %2" ::"v"(byte_offset), "v"(value), "s"(base) : "memory");
+}
+
+struct PackedArgs {
+  // the wavefronts of the tiles read their own copy of the parameters: a value both kinds of
+  // workgroup load from one place is loaded on entry, for all of them, before the first branch
+  apc_params p;
+  double *row_min_out;
+  int32_t *row_arg_out;
+  const double *pt_values;
+  // the tensor table: a tile whose producer specs name several tensors reads it entry by entry
+  const int32_t *rank, *itemsize;
+  const int64_t *shape, *stride;
+  double inv_rescale;  // 1.0 / params.rescale
+  // every mesh size a power of two (term_layout): log2 of the sizes and of their product; else exponents = 0
+  int32_t exponents, lg_total, lg[APC_MAX_MESH];
+};
+
+template <int M, bool POW2>
+__device__ __forceinline__ void packed_tile(const apc_packed_tile *T, double *cost_out, const PackedArgs &a) {
+  const apc_params &p = a.p;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
+  // ---- the one round of loads: nothing here depends on another load ---------------------------
+  const i32x16 h = uniform_load(reinterpret_cast<const i32x16 *>(T));
+  const i64x8 t_shape = uniform_load(reinterpret_cast<const i64x8 *>(T->tensor_shape));
+  const i64x8 t_stride = uniform_load(reinterpret_cast<const i64x8 *>(T->tensor_stride));
+  TileCopies copies;
+  copies.entry0 = T->dup_entry_begin[lane & (APC_PACKED_MAX_DUPS - 1)];
+  copies.row0 = T->dup_row_begin[lane & (APC_PACKED_MAX_DUPS - 1)];
+  copies.row_out = 0;
+  const uint32_t col_code = T->col_codes[lane], row_code = T->row_codes[lane];
+  const int col_tensor = T->col_tensor[lane], row_tensor = T->row_tensor[lane];
+  const int64_t row_flops = T->row_flops[lane], row_rw = T->row_rw_bytes[lane];
+  const int row_meta = T->row_meta[lane];
+  // (lane j holds the throughput of dtype code j & 7: fetched by the lanes that need it, below)
+  const double gf_of_lane = a.p.gpu_flops[lane & (APC_MAX_DTYPES - 1)], inv_gf_of_lane = a.p.inv_gpu_flops[lane & (APC_MAX_DTYPES - 1)];
+  // (kernel arguments the wavefront needs first or in its store loops, under the same wait)
+  fetch_arguments_now(h[0], t_shape[0], t_stride[0], a.row_min_out, a.row_arg_out, p.hbm_bw, p.inv_hbm_bw, p.rw_eff, p.inv_rw_eff,
+                      p.launch_floor, p.compute_eff, p.inv_compute_eff, a.inv_rescale, p.rescale, p.a2a_scale, p.base_latency);
+  const int rows = h[0], cols = h[1], flags = h[2], dup_count = h[3], t0 = h[4];
+  if ((unsigned)rows > (unsigned)APC_TILE_MAX_ROWS || (unsigned)(cols - 1) >= (unsigned)APC_TILE_MAX_COLS ||
+      (unsigned)dup_count > (unsigned)APC_PACKED_MAX_DUPS)
+    return;  // a record the host validator would have rejected
+  const int64_t entry_begin = ((int64_t)h[9] << 32) | (uint32_t)h[8], row_begin = ((int64_t)h[11] << 32) | (uint32_t)h[10];
+  const int64_t pt_begin = ((int64_t)h[13] << 32) | (uint32_t)h[12];
+  const uint32_t magic = (65536u + (uint32_t)cols - 1u) / (uint32_t)cols;  // x / cols = (x magic) >> 16 for x <= 64
+  const int rows_per_pass = (int)((64u * magic) >> 16);
+  if (wave * rows_per_pass >= rows) return;  // a wavefront without rows (a tile of fewer rows than the workgroup walks at once)
+  // ---- per wavefront: the tensor's bytes, the rows' compute costs -------------------------------
+  int64_t nbytes;
+  bool contiguous;
+  tensor_bytes_and_contiguity_of(h[5], h[6], t_shape, t_stride, nbytes, contiguous);
+  const double fbytes = (double)nbytes;
+  const int dt = (int)(int8_t)(row_meta & 0xFF);
+  const bool known_dtype = dt >= 0 && dt < APC_MAX_DTYPES;
+  const double gf = from_lane(gf_of_lane, dt & (APC_MAX_DTYPES - 1)), inv_gf = from_lane(inv_gf_of_lane, dt & (APC_MAX_DTYPES - 1));
+  const double cpa = compute_cost_through_reciprocals(p, ((row_meta >> 8) & 0xFF) != 0, row_rw, row_flops, known_dtype ? gf : 0.0,
+                                                      known_dtype ? inv_gf : 0.0) /
+                     (double)(row_meta >> 16);  // (lanes past the tile's rows: never read)
+  settle(copies);
+  FlatConstants<M> k;
+  constexpr bool pow2 = POW2;
+  Pow2Constants<M> k2;
+  if constexpr (!POW2) k = flat_constants<M>(p);
+  if constexpr (POW2) {  // the chains of TermArrayConstants arrays 2 (read+write) and 4 + 3 d (one-hop ring of dim d)
+    k2.R = div_by(div_by(fbytes, p.hbm_bw, p.inv_hbm_bw) * 1e6, p.rw_eff, p.inv_rw_eff);
+    k2.rw_shift = 1 - a.lg_total;
+    k2.floor = p.launch_floor;
+#pragma unroll
+    for (int i = 0; i < M; ++i) {
+      const double hops1 = (double)(p.mesh_size[i] - 1), hops2 = (double)(2 * (p.mesh_size[i] - 1));
+      k2.B[i] = div_by(fbytes * hops1, p.bw[i], p.inv_bw[i]) * 1e6;
+      k2.lat1[i] = p.base_latency + hops1 * p.lat[i];
+      k2.lat2[i] = p.base_latency + hops2 * p.lat[i];
+      k2.lg[i] = a.lg[i];
+      k2.shift[i] = -a.lg_total - 30 - a.lg[i];
+    }
+  }
+  // ---- whole rows: cols lanes per row, 64 / cols rows per pass, wavefront w the passes w, w + waves, ...
+  const int r_local = (int)(((uint32_t)lane * magic) >> 16), c = lane - r_local * cols;
+  const bool in_pass = r_local < rows_per_pass;
+  // (for the stores of the row minima: lane -> (row of the pass, copy))
+  const uint32_t magic_rows = (65536u + (uint32_t)rows_per_pass - 1u) / (uint32_t)rows_per_pass;
+  const int copies_per_store = (int)((64u * magic_rows) >> 16);
+  const int copy_slot = (int)(((uint32_t)lane * magic_rows) >> 16), q = lane - copy_slot * rows_per_pass;
+  const int q_first_lane = q * cols;
+  const bool rescale = (flags & APC_EDGE_GRAD_RESCALE) != 0, no_producer = (flags & APC_EDGE_NO_PRODUCER) != 0;
+  const bool entry_by_entry = (flags & APC_PACKED_MIXED) != 0 || no_producer || t0 < 0;
+  double *const cost_base = cost_out + entry_begin;
+  for (int row0 = wave * rows_per_pass; row0 < rows; row0 += waves * rows_per_pass) {
+    const int r = row0 + r_local;
+    const bool active = in_pass && r < rows;
+    const uint32_t src = (uint32_t)from_lane((int)col_code, c), tgt = (uint32_t)from_lane((int)row_code, r);
+    const double row_cpa = from_lane(cpa, r);
+    const uint32_t local = (uint32_t)(r * cols + c);
+    double comm = 0.0;
+    int trans = 0;
+    if (!entry_by_entry) {
+      const bool flip = M == 2 && src == 0x4040u && ((tgt >> 6) & 3u) == 2u && ((tgt >> 14) & 3u) == 2u;
+      const bool some_flip = M == 2 && __ballot(flip && active) != 0;  // (Partial, Partial) -> all Shard walks dim 1 first (:146-151)
+      if constexpr (pow2) {
+        int j = a.lg_total;  // bytes / num_shards = bytes x 2^(j - L): exact on such a mesh
+#pragma unroll
+        for (int i = 0; i < M; ++i) j -= ((src >> (8 * i + 6)) & 3u) == 2u ? k2.lg[i] : 0;
+        comm = contiguous ? entry_cost_pow2<M, 0, true>(src, tgt, j, p.a2a_scale, k2) : entry_cost_pow2<M, 0, false>(src, tgt, j, p.a2a_scale, k2);
+        if (some_flip) {
+          const double other = contiguous ? entry_cost_pow2<M, 1, true>(src, tgt, j, p.a2a_scale, k2)
+                                          : entry_cost_pow2<M, 1, false>(src, tgt, j, p.a2a_scale, k2);
+          comm = flip ? other : comm;
+        }
+      } else {
+        double shards = 1.0;  // exact: a product of mesh sizes (torch _dtensor_spec.py:555-561)
+#pragma unroll
+        for (int i = 0; i < M; ++i) shards *= ((src >> (8 * i + 6)) & 3u) == 2u ? (double)p.mesh_size[i] : 1.0;
+        const double gb = fbytes / shards * 0x1p-30;  // / 1024 / 1024 / 1024 (:66-68)
+        comm = contiguous ? entry_cost_flat<M, 0, true>(src, tgt, gb, p, k) : entry_cost_flat<M, 0, false>(src, tgt, gb, p, k);
+        if (some_flip) {
+          const double other = contiguous ? entry_cost_flat<M, 1, true>(src, tgt, gb, p, k)
+                                          : entry_cost_flat<M, 1, false>(src, tgt, gb, p, k);
+          comm = flip ? other : comm;
+        }
+      }
+      trans = src != tgt ? p.transition_scale : 0;  // optimize_sharding.py:345-351
+      // :358-359; the quotient through the reciprocal is the division's (div_by), +inf stays +inf
+      if (rescale) comm = comm < __builtin_inf() ? div_by(comm, p.rescale, a.inv_rescale) : comm;
+    } else {
+      // pass-through edges and tiles whose specs are not all DTensorSpecs on one tensor: the
+      // rule-provided value, or the direct evaluation on the entry's own tensor
+      const int sten = from_lane(col_tensor, c), tten = from_lane(row_tensor, r);
+      if (active) {
+        if (no_producer || sten < 0 || tten < 0) {
+          comm = a.pt_values[pt_begin + local];
+        } else {
+          trans = src != tgt ? p.transition_scale : 0;
+          int64_t shards = 1;
+#pragma unroll
+          for (int i = 0; i < M; ++i)
+            if (kind_of((src >> (8 * i)) & 0xFF) == 2) shards *= p.mesh_size[i];
+          int64_t sten_bytes;
+          bool sten_contiguous;
+          tensor_bytes_and_contiguity(a.rank[sten], a.itemsize[sten], a.shape + (int64_t)sten * APC_MAX_RANK,
+                                      a.stride + (int64_t)sten * APC_MAX_RANK, sten_bytes, sten_contiguous);
+          const double gb = (double)sten_bytes / (double)shards / 1024 / 1024 / 1024;
+          comm = entry_cost<M>(src, tgt, gb, sten_contiguous, p);
+        }
+        if (rescale) comm = comm / p.rescale;
+      }
+    }
+    const double total = comm + row_cpa + (double)trans;  // optimize_sharding.py:368-372
+    // ---- the entry, to the tile's edge and to every identical edge ----------------------------------
+    const uint32_t off8 = local * 8u;
+    if (active) store_at(cost_base, off8, total);
+    for (int d = 0; d < dup_count; ++d) {  // per copy: the offset out of its lane, scalar address arithmetic, the store
+      double *const base = cost_out + value_of_lane(copies.entry0, d);
+      if (active) store_at(base, off8, total);
+    }
+    // ---- the rows' minima ----------------------------------------------------------------------------
+    double m;
+    int mc;
+    row_min_in_wave(active, total, c, cols, lane, m, mc);
+    // A row's minimum sits in the row's first lane.  Stored to all copies at once: lane (q, copy) =
+    // (lane mod rows per pass, lane / rows per pass) fetches row q's result and writes it to its
+    // copy (copy 0 = the tile's own edge), 64 / rows-per-pass copies per store instruction.
+    const double m_q = from_lane(m, q_first_lane);
+    const int mc_q = from_lane(mc, q_first_lane);
+    const bool row_live = row0 + q < rows;
+    for (int copy0 = 0; copy0 <= dup_count; copy0 += copies_per_store) {
+      const int copy = copy0 + copy_slot;
+      const int64_t first_row = from_lane_i64(copies.row0, copy - 1);  // (every lane takes part)
+      if (row_live && copy_slot < copies_per_store && copy <= dup_count) {
+        const int64_t out = (copy == 0 ? row_begin : first_row) + row0 + q;
+        a.row_min_out[out] = m_q;
+        a.row_arg_out[out] = mc_q;
+      }
+    }
+  }
+}
+
+template <int M, bool POW2>
+__global__ __launch_bounds__(kBlock) void build_tables_packed_kernel(const apc_packed_tile *tiles, int n_tiles, int xcd_shift,
+                                                                     int64_t tile_blocks, double *cost_out, PackedArgs a,
+                                                                     apc_params p, TensorTableArgs t, ComputeCostArgs c,
+                                                                     int64_t tensor_blocks) {
+  const int64_t b = blockIdx.x;
+  if (b < tile_blocks) {
+    const int64_t per = tile_blocks >> xcd_shift;
+    const int64_t tile_id = (b & ((1 << xcd_shift) - 1)) * per + (b >> xcd_shift);
+    if (tile_id >= n_tiles) return;
+    packed_tile<M, POW2>(tiles + tile_id, cost_out, a);
+    return;
+  }
+  const int64_t tb = b - tile_blocks;
+  if (tb < tensor_blocks) tensor_tables_block<kBlock>(tb, t);
+  else compute_costs_block<kBlock>(tb - tensor_blocks, p, c);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1995,8 +2377,11 @@ int check_params(const apc_params *p) {
     if (p->inv_mesh[i] != 1.0 / (double)p->mesh_size[i] || p->inv_bw[i] != 1.0 / p->bw[i])
       return fail(-1, "inv_mesh[%d] / inv_bw[%d] are not 1.0 / mesh_size, 1.0 / bw", i, i);
   }
-  if (p->inv_hbm_bw != 1.0 / p->hbm_bw || p->inv_rw_eff != 1.0 / p->rw_eff)
-    return fail(-1, "inv_hbm_bw / inv_rw_eff are not 1.0 / hbm_bw, 1.0 / rw_eff");
+  if (p->inv_hbm_bw != 1.0 / p->hbm_bw || p->inv_rw_eff != 1.0 / p->rw_eff || p->inv_compute_eff != 1.0 / p->compute_eff)
+    return fail(-1, "inv_hbm_bw / inv_rw_eff / inv_compute_eff are not 1.0 / hbm_bw, 1.0 / rw_eff, 1.0 / compute_eff");
+  for (int i = 0; i < APC_MAX_DTYPES; ++i)
+    if (p->inv_gpu_flops[i] != (p->gpu_flops[i] != 0.0 ? 1.0 / p->gpu_flops[i] : 0.0))
+      return fail(-1, "inv_gpu_flops[%d] is not 1.0 / gpu_flops[%d] (0 for an unsupported dtype)", i, i);
   return 0;
 }
 
@@ -2599,6 +2984,181 @@ int apc_redistribute_tables_static(const apc_params *params, int64_t n_tensors, 
     return rc;
   return redistribute_tables_impl(params, tensor_bytes, tensor_contiguous, spec_codes, spec_tensor, pt_values, per_arg, n_tiles,
                                   tiles, dup_entry_begin, n_entries, comm_out, trans_out, cost_out, nullptr, stream);
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------------------------------------
+// Packed tiles: host-side check and launch.
+// ------------------------------------------------------------------------------------------
+static_assert(sizeof(apc_packed_tile) == 2752 && sizeof(apc_packed_tile) % 64 == 0, "apc_packed_tile layout");
+static_assert(offsetof(apc_packed_tile, entry_begin) == 32 && offsetof(apc_packed_tile, tensor_shape) == 64,
+              "the header is the record's first 64 bytes");
+
+extern "C" {
+
+int apc_validate_packed_tiles_host(int64_t n_tensors, const int32_t *tensor_rank, const int32_t *tensor_itemsize,
+                                   const int64_t *tensor_shape, const int64_t *tensor_stride, int64_t n_specs,
+                                   const uint32_t *spec_codes, const int32_t *spec_tensor, int64_t n_strategies,
+                                   const int64_t *flops, const int64_t *rw_bytes, const int8_t *dtype_code,
+                                   const uint8_t *zero_cost, const int32_t *num_args, int64_t n_edges,
+                                   const int64_t *edge_row_begin, int64_t n_tiles, const apc_tile *tiles, int64_t n_dups,
+                                   const int64_t *dup_entry_begin, const int64_t *dup_row_begin,
+                                   const apc_packed_tile *packed) {
+  if (n_tiles < 0 || n_tensors < 0 || n_specs < 0 || n_strategies < 0 || n_edges < 0 || n_dups < 0)
+    return fail(-1, "apc_validate_packed_tiles_host: negative count");
+  if (n_tiles == 0) return 0;
+  if (!tiles || !packed || !spec_codes || !spec_tensor || !edge_row_begin || !flops || !rw_bytes || !dtype_code || !zero_cost ||
+      !num_args || (n_dups > 0 && (!dup_entry_begin || !dup_row_begin)) ||
+      (n_tensors > 0 && (!tensor_rank || !tensor_itemsize || !tensor_shape || !tensor_stride)))
+    return fail(-1, "apc_validate_packed_tiles_host: NULL array");
+  for (int64_t t = 0; t < n_tiles; ++t) {
+    const apc_tile &tl = tiles[t];
+    const apc_packed_tile &pk = packed[t];
+    const int rows = tl.counts & 0xFFFF, cols = tl.counts >> 16;
+    if (tl.edge < 0 || tl.edge >= n_edges) return fail(-2, "tile %lld: edge %d out of range", (long long)t, tl.edge);
+    if (tl.col_begin != 0 || cols != tl.n_src || cols < 1 || cols > APC_TILE_MAX_COLS || rows < 1 || rows > APC_TILE_MAX_ROWS)
+      return fail(-2, "tile %lld: a packed tile holds 1 .. %d whole rows of at most %d columns (%d rows, columns [%d, +%d) of %d)",
+                  (long long)t, APC_TILE_MAX_ROWS, APC_TILE_MAX_COLS, rows, tl.col_begin, cols, tl.n_src);
+    if (tl.dup_count < 0 || tl.dup_count > APC_PACKED_MAX_DUPS || tl.dup_begin < 0 || (int64_t)tl.dup_begin + tl.dup_count > n_dups)
+      return fail(-2, "tile %lld: %d identical edges, a packed tile serves at most %d", (long long)t, tl.dup_count,
+                  APC_PACKED_MAX_DUPS);
+    if (tl.src_begin < 0 || (int64_t)tl.src_begin + cols > n_specs || tl.tgt_begin < 0 ||
+        (int64_t)tl.tgt_begin + tl.row_begin + rows > n_specs || tl.strat_begin < 0 ||
+        (int64_t)tl.strat_begin + tl.row_begin + rows > n_strategies)
+      return fail(-2, "tile %lld: spec or strategy rows outside their tables", (long long)t);
+    const int64_t first = (int64_t)tl.row_begin * cols;
+    bool mixed = false;
+    for (int j = 0; j < cols; ++j) {
+      const int64_t sp = (int64_t)tl.src_begin + j;
+      if (pk.col_codes[j] != spec_codes[sp] || pk.col_tensor[j] != spec_tensor[sp])
+        return fail(-2, "packed tile %lld: producer spec %d differs from the spec table", (long long)t, j);
+      mixed |= spec_tensor[sp] < 0 || spec_tensor[sp] != tl.tensor;
+    }
+    for (int j = 0; j < rows; ++j) {
+      const int64_t ts = (int64_t)tl.tgt_begin + tl.row_begin + j, sr = (int64_t)tl.strat_begin + tl.row_begin + j;
+      if (pk.row_codes[j] != spec_codes[ts] || pk.row_tensor[j] != spec_tensor[ts])
+        return fail(-2, "packed tile %lld: consumer spec %d differs from the spec table", (long long)t, j);
+      mixed |= spec_tensor[ts] < 0;
+      if (num_args[sr] < 1 || num_args[sr] > 0x7FFF)
+        return fail(-2, "packed tile %lld: num_args %d of consumer strategy %d does not fit its 15 bits", (long long)t,
+                    num_args[sr], j);
+      const int32_t meta = (int32_t)(uint8_t)dtype_code[sr] | ((int32_t)(zero_cost[sr] != 0) << 8) | (num_args[sr] << 16);
+      if (pk.row_flops[j] != flops[sr] || pk.row_rw_bytes[j] != rw_bytes[sr] || pk.row_meta[j] != meta)
+        return fail(-2, "packed tile %lld: consumer strategy %d differs from the strategy table", (long long)t, j);
+    }
+    if (pk.rows != rows || pk.cols != cols || pk.dup_count != tl.dup_count || pk.tensor != tl.tensor || pk.edge != tl.edge ||
+        pk.flags != (tl.flags | (mixed ? APC_PACKED_MIXED : 0)) || pk.entry_begin != tl.entry_begin + first ||
+        pk.row_begin != edge_row_begin[tl.edge] + tl.row_begin || pk.pt_begin != (tl.pt_begin < 0 ? -1 : tl.pt_begin + first))
+      return fail(-2, "packed tile %lld: header does not repeat the fields of tile record %lld", (long long)t, (long long)t);
+    if (tl.tensor >= 0) {
+      if (tl.tensor >= n_tensors) return fail(-2, "tile %lld: tensor %d out of range", (long long)t, tl.tensor);
+      if (pk.tensor_rank != tensor_rank[tl.tensor] || pk.tensor_itemsize != tensor_itemsize[tl.tensor] ||
+          memcmp(pk.tensor_shape, tensor_shape + (int64_t)tl.tensor * APC_MAX_RANK, sizeof(pk.tensor_shape)) != 0 ||
+          memcmp(pk.tensor_stride, tensor_stride + (int64_t)tl.tensor * APC_MAX_RANK, sizeof(pk.tensor_stride)) != 0)
+        return fail(-2, "packed tile %lld: tensor row differs from the tensor table", (long long)t);
+    }
+    for (int d = 0; d < tl.dup_count; ++d)
+      if (pk.dup_entry_begin[d] != dup_entry_begin[tl.dup_begin + d] + first ||
+          pk.dup_row_begin[d] != dup_row_begin[tl.dup_begin + d] + tl.row_begin)
+        return fail(-2, "packed tile %lld: identical edge %d differs from the duplicate lists", (long long)t, d);
+  }
+  return 0;
+}
+
+int apc_build_tables_packed(const apc_params *params, int64_t n_tensors, const int32_t *rank, const int32_t *itemsize,
+                            const int64_t *shape, const int64_t *stride, int64_t *tensor_bytes, uint8_t *tensor_contiguous,
+                            int64_t n_strategies, const int64_t *flops, const int64_t *rw_bytes, const int8_t *dtype,
+                            const uint8_t *zero_cost, const int32_t *num_args, double *compute, double *per_arg,
+                            int32_t *error_flag, const double *pt_values, int64_t n_tiles, const apc_packed_tile *packed,
+                            int64_t n_entries, double *cost_out, double *row_min, int32_t *row_argmin, void *stream) {
+  if (int rc = check_params(params)) return rc;
+  if (n_tensors < 0 || n_strategies < 0 || n_entries < 0) return fail(-1, "apc_build_tables_packed: negative count");
+  if (n_tiles < 0 || n_tiles > (1 << 30)) return fail(-1, "n_tiles %lld out of range", (long long)n_tiles);
+  if (n_tensors > 0 && (!rank || !itemsize || !shape || !stride || !tensor_bytes || !tensor_contiguous))
+    return fail(-1, "apc_build_tables_packed: NULL tensor array");
+  if (n_strategies > 0 && (!flops || !rw_bytes || !dtype || !zero_cost || !num_args))
+    return fail(-1, "apc_build_tables_packed: NULL strategy array");
+  if (n_tiles > 0 && (!packed || !cost_out || !row_min || !row_argmin))
+    return fail(-1, "apc_build_tables_packed: NULL tile records or outputs");
+  if ((reinterpret_cast<uintptr_t>(packed) & 63) != 0) return fail(-1, "apc_build_tables_packed: packed tiles must be 64-byte aligned");
+  const int xs = xcd_shift();
+  const int64_t tile_blocks = ((n_tiles + (1 << xs) - 1) >> xs) << xs;
+  const int64_t tb = blocks_for(n_tensors, kBlock), cb = blocks_for(n_strategies, kBlock);
+  const int64_t blocks = tile_blocks + tb + cb;
+  if (blocks == 0) return 0;
+  if (blocks > INT32_MAX) return fail(-1, "apc_build_tables_packed: too many rows for one launch");
+  const TermLayout lay = term_layout(*params);
+  PackedArgs a{*params, row_min, row_argmin, pt_values, rank, itemsize, shape, stride, 1.0 / params->rescale, lay.exponents,
+               lay.lg_total, {0, 0, 0, 0}};
+  for (int i = 0; i < APC_MAX_MESH; ++i) a.lg[i] = lay.lg[i];
+  const TensorTableArgs ta{n_tensors, rank, itemsize, shape, stride, tensor_bytes, tensor_contiguous};
+  const ComputeCostArgs ca{n_strategies, flops, rw_bytes, dtype, zero_cost, num_args, compute, per_arg, error_flag};
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)blocks);
+  const int nt = (int)n_tiles;
+#define APC_LAUNCH_PACKED(M_)                                                                                                    \
+  if (lay.exponents)                                                                                                           \
+    hipLaunchKernelGGL((build_tables_packed_kernel<M_, true>), grid, dim3(kBlock), 0, s, packed, nt, xs, tile_blocks, cost_out, a, \
+                       *params, ta, ca, tb);                                                                                   \
+  else                                                                                                                         \
+    hipLaunchKernelGGL((build_tables_packed_kernel<M_, false>), grid, dim3(kBlock), 0, s, packed, nt, xs, tile_blocks, cost_out, a, \
+                       *params, ta, ca, tb)
+  switch (params->mesh_ndim) {
+    case 1: APC_LAUNCH_PACKED(1); break;
+    case 2: APC_LAUNCH_PACKED(2); break;
+    case 3: APC_LAUNCH_PACKED(3); break;
+    default: APC_LAUNCH_PACKED(4); break;
+  }
+#undef APC_LAUNCH_PACKED
+  return check_launch("apc_build_tables_packed");
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------------------------------------
+// Measurement aids (no counterpart in the reference): what a launch costs on this system
+// before it does any work, and what the store path gives a kernel that does nothing but write.
+// A benchmark prices the table launches against both.
+// ------------------------------------------------------------------------------------------
+namespace {
+
+__global__ void calibrate_empty_kernel() {}
+
+// Workgroup b writes doubles [b * per_workgroup, (b + 1) * per_workgroup) of out (clipped to n),
+// 16 bytes per lane and store instruction, consecutive lanes consecutive addresses.
+__global__ __launch_bounds__(kBlock) void calibrate_fill_kernel(double *__restrict__ out, int64_t n, int64_t per_workgroup,
+                                                                double value) {
+  typedef double pair_t __attribute__((ext_vector_type(2)));
+  const int64_t begin = (int64_t)blockIdx.x * per_workgroup;
+  const int64_t end = begin + per_workgroup < n ? begin + per_workgroup : n;
+  const pair_t v = {value, value};
+  int64_t i = begin + 2 * (int64_t)threadIdx.x;
+  for (; i + 1 < end; i += 2 * kBlock) *reinterpret_cast<pair_t *>(out + i) = v;
+  if (i < end) out[i] = value;
+}
+
+}  // namespace
+
+extern "C" {
+
+int apc_calibrate_launch(int64_t n_workgroups, int32_t threads, void *stream) {
+  if (n_workgroups < 1 || n_workgroups > INT32_MAX || threads < 1 || threads > 1024)
+    return fail(-1, "apc_calibrate_launch: %lld workgroups of %d threads", (long long)n_workgroups, threads);
+  hipLaunchKernelGGL(calibrate_empty_kernel, dim3((unsigned)n_workgroups), dim3((unsigned)threads), 0, (hipStream_t)stream);
+  return check_launch("apc_calibrate_launch");
+}
+
+int apc_calibrate_fill(double *out, int64_t n, int64_t per_workgroup, double value, void *stream) {
+  if (n < 0 || per_workgroup < 2 || (per_workgroup & 1)) return fail(-1, "apc_calibrate_fill: n >= 0, per_workgroup even and >= 2");
+  if (n == 0) return 0;
+  if (!out) return fail(-1, "apc_calibrate_fill: NULL array");
+  if ((reinterpret_cast<uintptr_t>(out) & 15) != 0) return fail(-1, "apc_calibrate_fill: out must be 16-byte aligned");
+  const int64_t blocks = (n + per_workgroup - 1) / per_workgroup;
+  if (blocks > INT32_MAX) return fail(-1, "apc_calibrate_fill: too many workgroups");
+  hipLaunchKernelGGL(calibrate_fill_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, (hipStream_t)stream, out, n, per_workgroup,
+                     value);
+  return check_launch("apc_calibrate_fill");
 }
 
 }  // extern "C"

@@ -432,6 +432,52 @@ c10::intrusive_ptr<BoundLaunch> bind_cost_tables(APCOST_INPUT_TABLE_PARAMS, cons
   return b;
 }
 
+// apc_build_tables_packed: the planner's pass over packed tiles (one record of int32 words per tile).
+c10::intrusive_ptr<BoundLaunch> bind_cost_tables_packed(const Tensor &params, const Tensor &rank, const Tensor &itemsize,
+                                                        const Tensor &shape, const Tensor &stride, const Tensor &tensor_bytes,
+                                                        const Tensor &tensor_contiguous, const Tensor &flops,
+                                                        const Tensor &rw_bytes, const Tensor &dtype, const Tensor &zero_cost,
+                                                        const Tensor &num_args, const Tensor &compute, const Tensor &per_arg,
+                                                        const Tensor &error_flag, const Tensor &pt_values, const Tensor &packed,
+                                                        int64_t n_entries, int64_t n_rows, const Tensor &cost,
+                                                        const Tensor &row_min, const Tensor &row_argmin) {
+  auto b = c10::make_intrusive<BoundLaunch>();
+  const apc_params p = params_of(params);
+  const TensorTable t = tensor_table(rank, itemsize, shape, stride);
+  int64_t *bytes = dev<int64_t>(tensor_bytes, at::kLong, "tensor_bytes");
+  uint8_t *contiguous = dev<uint8_t>(tensor_contiguous, at::kByte, "tensor_contiguous");
+  TORCH_CHECK(tensor_bytes.numel() == t.n && tensor_contiguous.numel() == t.n, "apcost: tensor_bytes / tensor_contiguous need one row per tensor");
+  const StrategyTable st = strategy_table(flops, rw_bytes, dtype, zero_cost, num_args);
+  double *cc = dev<double>(compute, at::kDouble, "compute_cost"), *cpa = dev<double>(per_arg, at::kDouble, "compute_cost_per_arg");
+  TORCH_CHECK(compute.numel() == st.n && per_arg.numel() == st.n, "apcost: compute_cost / compute_cost_per_arg need one row per strategy");
+  int32_t *err = dev<int32_t>(error_flag, at::kInt, "error_flag");
+  TORCH_CHECK(error_flag.numel() >= 1, "apcost: error_flag needs one element");
+  const double *pt = dev<double>(pt_values, at::kDouble, "pt_values");
+  constexpr int64_t kWords = (int64_t)(sizeof(apc_packed_tile) / sizeof(int32_t));
+  TORCH_CHECK(packed.dim() == 2 && packed.size(1) == kWords, "apcost: packed tiles must be [n_tiles, ", kWords, "] int32 words (struct apc_packed_tile)");
+  const apc_packed_tile *tiles = reinterpret_cast<const apc_packed_tile *>(dev<int32_t>(packed, at::kInt, "packed"));
+  const int64_t n_tiles = packed.size(0);
+  TORCH_CHECK(n_entries >= 0 && n_rows >= 0, "apcost: negative count");
+  double *cost_out = dev<double>(cost, at::kDouble, "cost");
+  double *mins = dev<double>(row_min, at::kDouble, "row_min");
+  int32_t *args = dev<int32_t>(row_argmin, at::kInt, "row_argmin");
+  TORCH_CHECK(cost.numel() == n_entries, "apcost: cost needs one value per entry");
+  TORCH_CHECK(row_min.numel() == n_rows && row_argmin.numel() == n_rows, "apcost: row_min / row_argmin need one value per matrix row");
+  for (const Tensor *x : {&rank, &itemsize, &shape, &stride, &tensor_bytes, &tensor_contiguous, &flops, &rw_bytes, &dtype, &zero_cost,
+                          &num_args, &compute, &per_arg, &error_flag, &pt_values, &packed, &cost, &row_min, &row_argmin}) {
+    same_device(rank, *x, "a table");
+    b->keep.push_back(*x);
+  }
+  b->what = "apc_build_tables_packed";
+  b->device = rank.device();
+  b->launch = [=](void *s) {
+    return apc_build_tables_packed(&p, t.n, t.rank, t.itemsize, t.shape, t.stride, bytes, contiguous, st.n, st.flops, st.rw_bytes,
+                                   st.dtype, st.zero_cost, st.num_args, cc, cpa, err, pt, n_tiles, tiles, n_entries, cost_out, mins,
+                                   args, s);
+  };
+  return b;
+}
+
 // The matrices as fresh tensors: (comm, transition, cost) of apc_redistribute_tables.
 std::tuple<Tensor, Tensor, Tensor> redistribute_cost_tables(const Tensor &params, const Tensor &tensor_bytes,
                                                             const Tensor &tensor_contiguous, const Tensor &spec_codes,
@@ -731,4 +777,9 @@ TORCH_LIBRARY(apcost, m) {
   m.def("bind_cost_tables(" APCOST_INPUT_TABLES ", Tensor pt_values, Tensor tiles, Tensor dup_entry_begin, int n_entries, "
         APCOST_TABLE_OUTPUTS ") -> __torch__.torch.classes.apcost.BoundLaunch",
         &bind_cost_tables);
+  m.def("bind_cost_tables_packed(Tensor params, " APCOST_TENSOR_TABLE ", Tensor tensor_bytes, Tensor tensor_contiguous, "
+        APCOST_STRATEGY_TABLE ", Tensor compute_cost, Tensor compute_cost_per_arg, Tensor error_flag, Tensor pt_values, "
+        "Tensor packed, int n_entries, int n_rows, Tensor cost, Tensor row_min, Tensor row_argmin) "
+        "-> __torch__.torch.classes.apcost.BoundLaunch",
+        &bind_cost_tables_packed);
 }

@@ -268,9 +268,32 @@ class DeviceCostTables:
             total += 12 * tb.n_rows
         return total
 
+    # A table up to this many entries is bound by the latency of one workgroup: its planner pass
+    # runs over packed tiles (every wavefront on its own, one round of loads, no LDS staging).
+    # Above, the per-entry arithmetic of that kernel (direct evaluation) costs more than the
+    # staging it saves.
+    PACKED_MAX_ENTRIES = 4_000_000
+
+    def packed_pass_pays(self) -> bool:
+        tb = self.tables
+        return tb.n_entries <= self.PACKED_MAX_ENTRIES and tb.packable()
+
+    def _packed_tiles(self):
+        """The device copy of ``CostTables.pack_tiles()`` (checked against the tables by the
+        library's host-side validator), made once per tiling."""
+        cached = getattr(self, "_packed_cache", None)
+        if cached is not None and cached[0] is self.tables.tile_records:
+            return cached[1]
+        packed = self.tables.pack_tiles()
+        self.tables.validate_packed(packed)
+        with torch.cuda.device(self.device):
+            dev = _to_device(packed, self.device)
+        self._packed_cache = (self.tables.tile_records, dev)
+        return dev
+
     @_guarded
     def prepare_step(self, row_min=True, fused_inputs=False, one_launch=None, row_min_in_tiles=None,
-                     outputs=("comm", "transition", "cost"), spec_table=True):
+                     outputs=("comm", "transition", "cost"), spec_table=True, packed=None):
         """Allocates every output once and returns ``{kernel name: zero-argument launcher}``
         in launch order.  A launcher only enqueues (no allocation, no synchronisation), so a
         timed loop measures the kernels and not Python argument marshalling.  With
@@ -283,7 +306,9 @@ class DeviceCostTables:
         (``CostTables.rows_fit_tiles``), and ``None`` takes it when ``row_min_in_tiles_pays``.
         ``outputs``: which of the per-entry arrays the pass writes; ``spec_table=False`` leaves
         the local shard shapes out (a planner has computed them before it could fill in the
-        flop / byte counts this pass reads)."""
+        flop / byte counts this pass reads).  ``packed``: the one launch runs over packed tiles
+        (``apc_build_tables_packed``: the assembled cost and the row minima, no spec table);
+        ``None`` takes them when the pass is of that kind and ``packed_pass_pays``."""
         outputs = tuple(outputs)
         if not outputs or any(o not in ("comm", "transition", "cost") for o in outputs):
             raise ValueError(f"outputs must name some of comm, transition, cost: {outputs}")
@@ -300,6 +325,12 @@ class DeviceCostTables:
         total = self.pass_bytes(outputs, spec_table, row_min_in_tiles)
         if one_launch is None:
             one_launch = bool(fused_inputs) and total <= self.ONE_LAUNCH_MAX_BYTES
+        packed_kind = bool(one_launch) and row_min_in_tiles and outputs == ("cost",) and not spec_table
+        if packed is None:
+            packed = packed_kind and self.packed_pass_pays()
+        elif packed and not (packed_kind and self.tables.packable()):
+            raise ValueError("a pass over packed tiles is one launch that writes the assembled cost and the row minima, "
+                             "without the spec table, over tiles of whole rows")
         spec = self._alloc_input_tables(spec_table)
         self.alloc_outputs("comm" in outputs, "transition" in outputs, "cost" in outputs)
         self.row_min = self.row_argmin = None
@@ -333,7 +364,12 @@ class DeviceCostTables:
             rows = (_to_device(tb.edge_row_begin(), self.device), self.row_min, self.row_argmin)
         erb, rmin, rarg = rows if rows is not None else (None, None, None)
         dup_rows = d["dup_row_begin"] if rows is not None else None
-        if one_launch:
+        if packed:
+            step = {"build_tables_packed": bind(ops.bind_cost_tables_packed(
+                self.p, *self._tensor_table(), self.tensor_bytes, self.tensor_contiguous, *self._strategy_table(),
+                self.compute_cost, self.compute_cost_per_arg, err, d["pt_values"], self._packed_tiles(), tb.n_entries, tb.n_rows,
+                self.cost, self.row_min, self.row_argmin))}
+        elif one_launch:
             step = {"build_tables": bind(ops.bind_cost_tables(
                 *input_tables, d["pt_values"], d["tile_records"], d["dup_entry_begin"], tb.n_entries, self.comm,
                 self.transition, self.cost, erb, dup_rows, rmin, rarg))}
@@ -348,7 +384,7 @@ class DeviceCostTables:
                 "compute_costs": bind(ops.bind_compute_costs(self.p, *self._strategy_table(), self.compute_cost,
                                                              self.compute_cost_per_arg, err)),
             }
-        if not one_launch:
+        if not one_launch and not packed:
             step["redistribute_tables"] = bind(self._bind_redistribute_tables(self.comm, self.transition, self.cost, rows))
         if row_min and not row_min_in_tiles:
             row_ptr = torch.from_numpy(tb.row_ptr()).to(self.device)
@@ -367,7 +403,7 @@ class DeviceCostTables:
     # ---- the planner's table build -------------------------------------------------------------
     PLANNER_OUTPUTS = ("cost",)
 
-    def planner_pass(self):
+    def planner_pass(self, packed=None):
         """The launches ``ShardingOptimizer.build_ds`` issues once the flop / byte counts are in
         the strategy table (optimize_sharding.py:270-380 in one pass): the tensor and
         compute-cost tables and the assembled cost of every entry, the array the ILP objective
@@ -378,7 +414,7 @@ class DeviceCostTables:
         shapes before it could count flops); ``comm`` and ``transition`` are written only when a
         report asks (``fetch``)."""
         return self.prepare_step(row_min=self.row_min_in_tiles_pays(), fused_inputs=True,
-                                 outputs=self.PLANNER_OUTPUTS, spec_table=False)
+                                 outputs=self.PLANNER_OUTPUTS, spec_table=False, packed=packed)
 
     @_guarded
     def check_error_flag(self):

@@ -36,7 +36,7 @@ from typing import Optional
 import numpy as np
 
 from . import _native
-from ._native import APC_MAX_RANK, APC_TILE_MAX_COLS, APC_TILE_MAX_DUPS, APC_TILE_MAX_ROWS
+from ._native import APC_MAX_RANK, APC_PACKED_MAX_DUPS, APC_TILE_MAX_COLS, APC_TILE_MAX_DUPS, APC_TILE_MAX_ROWS
 
 REPLICATE = 0x00
 PARTIAL_SUM = 0x40
@@ -71,6 +71,21 @@ TILE_DTYPE = np.dtype([
     ("tensor", "<i4"), ("entry_begin", "<i8"), ("pt_begin", "<i8"), ("dup_begin", "<i4"), ("dup_count", "<i4"),
 ])
 assert TILE_DTYPE.itemsize == 64
+
+
+# numpy mirror of the C struct apc_packed_tile: everything one tile reads, in one record
+PACKED_MIXED = 0x100
+PACKED_TILE_DTYPE = np.dtype([
+    ("rows", "<i4"), ("cols", "<i4"), ("flags", "<i4"), ("dup_count", "<i4"), ("tensor", "<i4"), ("tensor_rank", "<i4"),
+    ("tensor_itemsize", "<i4"), ("edge", "<i4"), ("entry_begin", "<i8"), ("row_begin", "<i8"), ("pt_begin", "<i8"),
+    ("reserved", "<i8"), ("tensor_shape", "<i8", (APC_MAX_RANK,)), ("tensor_stride", "<i8", (APC_MAX_RANK,)),
+    ("dup_entry_begin", "<i8", (APC_PACKED_MAX_DUPS,)), ("dup_row_begin", "<i8", (APC_PACKED_MAX_DUPS,)),
+    ("col_codes", "<u4", (APC_TILE_MAX_COLS,)), ("col_tensor", "<i4", (APC_TILE_MAX_COLS,)),
+    ("row_codes", "<u4", (APC_TILE_MAX_ROWS,)), ("row_tensor", "<i4", (APC_TILE_MAX_ROWS,)),
+    ("row_flops", "<i8", (APC_TILE_MAX_ROWS,)), ("row_rw_bytes", "<i8", (APC_TILE_MAX_ROWS,)),
+    ("row_meta", "<i4", (APC_TILE_MAX_ROWS,)),
+])
+assert PACKED_TILE_DTYPE.itemsize == 2752
 
 
 def shard_code(dim: int, variant: int = 0) -> int:
@@ -287,7 +302,7 @@ class CostTables:
         return out
 
     def build_tiles(self, tile_entries: Optional[int] = None, dedupe: bool = False, max_copies: int = 16,
-                    signatures=None) -> None:
+                    signatures=None, rows_per_wavefront_pass: Optional[int] = None) -> None:
         """Cuts every edge matrix into rectangles of about ``tile_entries`` entries:
         whole rows when a row fits the LDS column budget, column chunks otherwise.  With
         ``dedupe`` only the first of every group of identical edges is tiled; its tiles
@@ -295,12 +310,17 @@ class CostTables:
         the compute-cost inputs are part of an edge's identity.)  One tiled edge serves at
         most ``max_copies - 1`` duplicates, so a long run of identical edges still spreads
         over many workgroups.  ``tile_entries=None`` chooses tile size and copies per tiled
-        edge from the table (``tiling`` records the choice)."""
+        edge from the table (``tiling`` records the choice).  ``rows_per_wavefront_pass = w``: a
+        tile of whole rows holds at most ``w * (64 // columns)`` of them, what ``w`` wavefronts that
+        each walk ``64 // columns`` whole rows at a time cover in one pass (the packed-tile launch
+        of a small table, whose slowest workgroup decides the launch; the automatic choice sets it
+        to 4 for such a table)."""
         if tile_entries is None:
             sigs = self.edge_signatures() if dedupe and self.n_edges else None
             te, mc = APC_TILE_MAX_ROWS * APC_TILE_MAX_COLS, int(max_copies)
+            small = self.n_entries <= AUTO_SMALL_TABLE_ENTRIES
             while True:
-                self.build_tiles(te, dedupe, mc, signatures=sigs)
+                self.build_tiles(te, dedupe, mc, signatures=sigs, rows_per_wavefront_pass=4 if small else None)
                 n = self.n_tiles
                 if n == 0 or n >= AUTO_MIN_TILES or self.n_entries / n <= AUTO_MIN_STORED_PER_TILE \
                         or self.n_entries <= AUTO_SMALL_TABLE_ENTRIES:
@@ -317,6 +337,8 @@ class CostTables:
                     break
             return
         self.tiling = {"tile_entries": int(tile_entries), "max_copies": int(max_copies) if dedupe else 1}
+        if rows_per_wavefront_pass:
+            self.tiling["rows_per_wavefront_pass"] = int(rows_per_wavefront_pass)
         ns = self.edge_n_src.astype(np.int64)
         nt = self.edge_n_tgt.astype(np.int64)
         canonical = np.arange(self.n_edges, dtype=np.int64)
@@ -345,6 +367,8 @@ class CostTables:
         ncc = -(-ns1 // APC_TILE_MAX_COLS)  # column chunks per edge
         cw = -(-ns1 // ncc)  # chunk width
         rpt = np.clip(tile_entries // cw, 1, APC_TILE_MAX_ROWS)
+        if rows_per_wavefront_pass:
+            rpt = np.where(ncc == 1, np.minimum(rpt, int(rows_per_wavefront_pass) * np.maximum(64 // cw, 1)), rpt)
         nrt = -(-nt1 // rpt)  # row tiles per edge
         rpt = -(-nt1 // nrt)  # balanced rows per tile
         per_edge = np.where(live, ncc * nrt, 0)
@@ -394,6 +418,92 @@ class CostTables:
             first = np.clip(self.edge_src_begin[tc].astype(np.int64) + self.tile_col_begin, 0, self.n_specs - 1)
             rec["tensor"] = self.spec_tensor[first]
         self.tile_records = rec
+
+    # ---- packed tiles ------------------------------------------------------------------
+    def packable(self) -> bool:
+        """Every tile holds whole rows of at most APC_TILE_MAX_COLS columns and serves at most
+        APC_PACKED_MAX_DUPS identical edges: the table can be built from packed tiles."""
+        if self.n_tiles == 0 or not self.rows_fit_tiles():
+            return False
+        if int(self.tile_records["dup_count"].max()) > APC_PACKED_MAX_DUPS:
+            return False
+        return bool(self.n_strategies == 0 or int(self.strat_num_args.max()) <= 0x7FFF)
+
+    def pack_tiles(self) -> np.ndarray:
+        """One ``apc_packed_tile`` record per tile: the tile's header, its tensor's row, the
+        first entries / rows of its identical edges, its producer and consumer specs and its
+        consumer strategies' rows of the strategy table, copied out of the tables (after the
+        strategy table is final).  A workgroup then loads nothing whose address depends on
+        another load."""
+        if not self.packable():
+            raise RuntimeError("packed tiles need whole rows in every tile and at most "
+                               f"{APC_PACKED_MAX_DUPS} identical edges per tile")
+        rec = self.tile_records
+        n = len(rec)
+        pk = np.zeros(n, PACKED_TILE_DTYPE)
+        rows = (rec["counts"] & 0xFFFF).astype(np.int64)
+        cols = (rec["counts"] >> 16).astype(np.int64)
+        rb = rec["row_begin"].astype(np.int64)
+        edge = rec["edge"].astype(np.int64)
+        first = rb * cols
+        pk["rows"], pk["cols"], pk["dup_count"], pk["tensor"], pk["edge"] = rows, cols, rec["dup_count"], rec["tensor"], rec["edge"]
+        pk["entry_begin"] = rec["entry_begin"] + first
+        pk["row_begin"] = self.edge_row_begin()[edge] + rb
+        pk["pt_begin"] = np.where(rec["pt_begin"] < 0, -1, rec["pt_begin"] + first)
+        t = rec["tensor"].astype(np.int64)
+        has = t >= 0
+        tc = np.where(has, t, 0)
+        if self.n_tensors:
+            pk["tensor_rank"] = np.where(has, self.tensor_rank[tc], 0)
+            pk["tensor_itemsize"] = np.where(has, self.tensor_itemsize[tc], 0)
+            pk["tensor_shape"] = np.where(has[:, None], self.tensor_shape[tc], 0)
+            pk["tensor_stride"] = np.where(has[:, None], self.tensor_stride[tc], 0)
+        j = np.arange(APC_TILE_MAX_COLS, dtype=np.int64)[None, :]
+        # producer specs
+        live = j < cols[:, None]
+        sp = np.where(live, rec["src_begin"].astype(np.int64)[:, None] + j, 0)
+        pk["col_codes"] = np.where(live, self.spec_codes[sp], 0)
+        col_tensor = np.where(live, self.spec_tensor[sp], 0)
+        pk["col_tensor"] = col_tensor
+        mixed = (live & ((col_tensor < 0) | (col_tensor != rec["tensor"][:, None]))).any(axis=1)
+        # consumer specs and their strategies
+        live = j < rows[:, None]
+        ts = np.where(live, (rec["tgt_begin"].astype(np.int64) + rb)[:, None] + j, 0)
+        pk["row_codes"] = np.where(live, self.spec_codes[ts], 0)
+        row_tensor = np.where(live, self.spec_tensor[ts], 0)
+        pk["row_tensor"] = row_tensor
+        mixed |= (live & (row_tensor < 0)).any(axis=1)
+        sr = np.where(live, (rec["strat_begin"].astype(np.int64) + rb)[:, None] + j, 0)
+        pk["row_flops"] = np.where(live, self.strat_flops[sr], 0)
+        pk["row_rw_bytes"] = np.where(live, self.strat_rw_bytes[sr], 0)
+        meta = (self.strat_dtype[sr].astype(np.int64) & 0xFF) | ((self.strat_zero_cost[sr] != 0).astype(np.int64) << 8) \
+            | (self.strat_num_args[sr].astype(np.int64) << 16)
+        pk["row_meta"] = np.where(live, meta, 0).astype(np.int32)
+        pk["flags"] = rec["flags"] | np.where(mixed, PACKED_MIXED, 0)
+        # identical edges
+        d = np.arange(APC_PACKED_MAX_DUPS, dtype=np.int64)[None, :]
+        live = d < rec["dup_count"].astype(np.int64)[:, None]
+        if len(self.dup_entry_begin):
+            at = np.where(live, rec["dup_begin"].astype(np.int64)[:, None] + d, 0)
+            pk["dup_entry_begin"] = np.where(live, self.dup_entry_begin[at] + first[:, None], 0)
+            pk["dup_row_begin"] = np.where(live, self.dup_row_begin[at] + rb[:, None], 0)
+        return pk
+
+    def validate_packed(self, packed: np.ndarray) -> None:
+        """The packed records against the tables, through the library's host-side check."""
+        def p(a):
+            return np.ascontiguousarray(a).ctypes.data_as(ctypes.c_void_p)
+
+        keep = [np.ascontiguousarray(a) for a in (
+            self.tensor_rank, self.tensor_itemsize, self.tensor_shape, self.tensor_stride, self.spec_codes, self.spec_tensor,
+            self.strat_flops, self.strat_rw_bytes, self.strat_dtype, self.strat_zero_cost, self.strat_num_args,
+            self.edge_row_begin(), self.tile_records, self.dup_entry_begin, self.dup_row_begin, packed)]
+        (rank, item, shape, stride, codes, owner, flops, rw, dt, zero, nargs, erb, tiles, dups, dup_rows, pk) = keep
+        rc = _native.lib().apc_validate_packed_tiles_host(
+            ctypes.c_int64(self.n_tensors), p(rank), p(item), p(shape), p(stride), ctypes.c_int64(self.n_specs), p(codes), p(owner),
+            ctypes.c_int64(self.n_strategies), p(flops), p(rw), p(dt), p(zero), p(nargs), ctypes.c_int64(self.n_edges), p(erb),
+            ctypes.c_int64(self.n_tiles), p(tiles), ctypes.c_int64(len(dups)), p(dups), p(dup_rows), p(pk))
+        _native.check(rc, "apc_validate_packed_tiles_host")
 
     # ---- checks ------------------------------------------------------------------------
     def validate(self, params) -> None:

@@ -427,8 +427,9 @@ def roofline_of(dev, tables, timing, steps, pass_kind):
     import numpy as np
 
     names = timing["names"]
-    one_launch = "build_tables" in names
-    main = "build_tables" if one_launch else "redistribute_tables"
+    packed = "build_tables_packed" in names
+    one_launch = packed or "build_tables" in names
+    main = "build_tables_packed" if packed else "build_tables" if one_launch else "redistribute_tables"
     in_tiles = dev.row_min is not None and "segmented_min" not in names
     outputs = tuple(k for k in ("comm", "transition", "cost") if getattr(dev, k) is not None)
     spec_table = pass_kind == "all"
@@ -445,7 +446,7 @@ def roofline_of(dev, tables, timing, steps, pass_kind):
     t_kernel = timing["region_ms"] * 1e-3 / steps if single else t_pair
     return {
         "bound": "hbm",
-        "kernel": ("build_tables_kernel" if one_launch else
+        "kernel": ("build_tables_packed_kernel" if packed else "build_tables_kernel" if one_launch else
                    "redistribute_tiles_row_min_kernel" if in_tiles else "redistribute_tiles_kernel"),
         "launch": main + (" (the one launch of the pass)" if single else ""),
         "arrays_written_per_entry": list(outputs),

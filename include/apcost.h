@@ -53,8 +53,9 @@ extern "C" {
 /* Version of this interface: the value apc_version() of a matching library returns.  It changes
  * whenever a struct layout, a limit below or the meaning of an argument changes (2: at most 32
  * identical edges per tile instead of 127; the row-minimum entry points write the minima of the
- * assembled cost whichever arrays are stored).  A binding compares the two before its first call. */
-#define APC_ABI_VERSION 2
+ * assembled cost whichever arrays are stored; 3: packed tiles).  A binding compares the two before its
+ * first call. */
+#define APC_ABI_VERSION 3
 
 #define APC_MAX_RANK 8
 #define APC_MAX_MESH 4
@@ -115,6 +116,8 @@ typedef struct apc_params {
   double inv_mesh[APC_MAX_MESH]; /* 1.0 / mesh_size[i] */
   double inv_hbm_bw;             /* 1.0 / hbm_bw */
   double inv_rw_eff;             /* 1.0 / rw_eff */
+  double inv_compute_eff;        /* 1.0 / compute_eff */
+  double inv_gpu_flops[APC_MAX_DTYPES]; /* 1.0 / gpu_flops[i]; 0 where gpu_flops[i] is 0 */
 } apc_params;
 
 int apc_version(void);
@@ -381,6 +384,80 @@ int apc_redistribute_tables_static(const apc_params *params, int64_t n_tensors, 
                                    const double *pt_values, int64_t n_tiles, const apc_tile *tiles,
                                    const int64_t *dup_entry_begin, int64_t n_entries, double *comm_out,
                                    uint8_t *transition_out, double *cost_out, void *stream);
+
+/* ---- packed tiles: the table pass of a small graph in one round of loads ----------------------
+ * A table of a few million entries is bound by the latency of one workgroup, not by bytes: the
+ * chain "tile record -> spec rows, strategy rows, tensor row, identical edges' offsets -> compute"
+ * costs more than the stores.  A packed tile holds everything one tile reads, copied out of the
+ * tables above by the host into one fixed-size record, so that a workgroup's loads depend on
+ * nothing but its own index.  It describes whole rows of one edge's matrix (cols = the edge's
+ * producer count <= APC_TILE_MAX_COLS, rows <= APC_TILE_MAX_ROWS) and at most APC_PACKED_MAX_DUPS
+ * identical edges.  apc_validate_packed_tiles_host checks every record against the tables it
+ * was copied from.  The values computed from it are those of apc_build_tables_row_min. */
+#define APC_PACKED_MAX_DUPS 16
+#define APC_PACKED_MIXED 0x100 /* flags: some spec of the tile is not a DTensorSpec, or a producer spec names
+                                  another tensor than `tensor`: entries are evaluated one by one */
+typedef struct apc_packed_tile {
+  int32_t rows, cols;      /* consumer / producer strategies of the tile (cols = edge_n_src[edge]) */
+  int32_t flags;           /* edge_flags[edge] | APC_PACKED_MIXED */
+  int32_t dup_count;       /* identical edges that receive the same values */
+  int32_t tensor;          /* spec_tensor of the first producer spec, -1: none */
+  int32_t tensor_rank;     /* rank / itemsize / shape / stride rows of that tensor (zeros when none) */
+  int32_t tensor_itemsize;
+  int32_t edge;
+  int64_t entry_begin;     /* first entry of the tile: edge_entry_begin[edge] + row_begin * cols */
+  int64_t row_begin;       /* its first matrix row: edge_row_begin[edge] + row_begin (rows numbered edge by edge) */
+  int64_t pt_begin;        /* pt_values offset of its first entry (edge_pt_begin[edge] + row_begin * cols), -1: none */
+  int64_t reserved;
+  int64_t tensor_shape[APC_MAX_RANK];
+  int64_t tensor_stride[APC_MAX_RANK];
+  int64_t dup_entry_begin[APC_PACKED_MAX_DUPS]; /* the tile's first entry in every identical edge */
+  int64_t dup_row_begin[APC_PACKED_MAX_DUPS];   /* its first matrix row there */
+  uint32_t col_codes[APC_TILE_MAX_COLS];        /* producer specs: placement codes, tensor rows */
+  int32_t col_tensor[APC_TILE_MAX_COLS];
+  uint32_t row_codes[APC_TILE_MAX_ROWS];        /* consumer specs */
+  int32_t row_tensor[APC_TILE_MAX_ROWS];
+  int64_t row_flops[APC_TILE_MAX_ROWS];         /* the consumer strategies' rows of the strategy table */
+  int64_t row_rw_bytes[APC_TILE_MAX_ROWS];
+  int32_t row_meta[APC_TILE_MAX_ROWS];          /* dtype code (low byte, signed) | zero_cost << 8 | num_args << 16 */
+} apc_packed_tile;
+
+/* Host-side check (HOST pointers) that packed[t] repeats, field by field, what tiles[t] and the
+ * tables say; tiles must hold whole rows (apc_validate_row_minima_host) and at most
+ * APC_PACKED_MAX_DUPS identical edges each.  edge_row_begin[e] = first matrix row of edge e. */
+int apc_validate_packed_tiles_host(int64_t n_tensors, const int32_t *tensor_rank_host, const int32_t *tensor_itemsize_host,
+                                   const int64_t *tensor_shape_host, const int64_t *tensor_stride_host, int64_t n_specs,
+                                   const uint32_t *spec_codes_host, const int32_t *spec_tensor_host, int64_t n_strategies,
+                                   const int64_t *flops_host, const int64_t *rw_bytes_host, const int8_t *dtype_code_host,
+                                   const uint8_t *zero_cost_host, const int32_t *num_args_host, int64_t n_edges,
+                                   const int64_t *edge_row_begin_host, int64_t n_tiles, const apc_tile *tiles_host,
+                                   int64_t n_dups, const int64_t *dup_entry_begin_host, const int64_t *dup_row_begin_host,
+                                   const apc_packed_tile *packed_host);
+
+/* The table pass of a planner over packed tiles, ONE launch: the tensor table, the compute costs,
+ * the assembled cost of every entry and the row minima (what apc_build_tables_row_min writes with
+ * cost_out alone and no spec table; same reference lines, same values).  Every wavefront works
+ * on its own: it reads the tile's record, evaluates whole matrix rows entry by entry in
+ * registers (collective_runtime_estimation.py:37-153 directly, no staging in LDS, no barrier),
+ * takes their minima and stores values and minima to the tile's edge and to every identical
+ * edge.  tensor_* / strategy arrays as in apc_build_tables (a tile whose producer specs name
+ * several tensors reads the tensor table).  cost_out [n_entries], row_min / row_argmin [n_rows]. */
+int apc_build_tables_packed(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
+                            const int32_t *tensor_itemsize, const int64_t *tensor_shape, const int64_t *tensor_stride,
+                            int64_t *tensor_bytes, uint8_t *tensor_contiguous, int64_t n_strategies, const int64_t *flops,
+                            const int64_t *rw_bytes, const int8_t *dtype_code, const uint8_t *zero_cost,
+                            const int32_t *num_args, double *compute_cost, double *compute_cost_per_arg,
+                            int32_t *error_flag, const double *pt_values, int64_t n_tiles, const apc_packed_tile *packed,
+                            int64_t n_entries, double *cost_out, double *row_min, int32_t *row_argmin, void *stream);
+
+/* Measurement aids, no counterpart in the reference.  apc_calibrate_launch enqueues a kernel that
+ * does nothing (n_workgroups workgroups of `threads` threads): launched back to back it shows what
+ * a launch costs on the system before any work.  apc_calibrate_fill enqueues a kernel that only
+ * writes: out[0 .. n) = value, workgroup b taking doubles [b * per_workgroup, (b + 1) *
+ * per_workgroup) (even, >= 2; 256 threads, 16-byte stores; out 16-byte aligned): the ceiling of
+ * the store path for a launch that moves the same bytes as a table build. */
+int apc_calibrate_launch(int64_t n_workgroups, int32_t threads, void *stream);
+int apc_calibrate_fill(double *out, int64_t n, int64_t per_workgroup, double value, void *stream);
 
 #ifdef __cplusplus
 }

@@ -62,6 +62,8 @@ int main() {
   }
   p.inv_hbm_bw = 1.0 / p.hbm_bw;
   p.inv_rw_eff = 1.0 / p.rw_eff;
+  p.inv_compute_eff = 1.0 / p.compute_eff;
+  for (int i = 0; i < APC_MAX_DTYPES; ++i) p.inv_gpu_flops[i] = p.gpu_flops[i] != 0.0 ? 1.0 / p.gpu_flops[i] : 0.0;
 
   // one tensor: [4096, 4096] bf16, contiguous
   const std::vector<int32_t> rank{2}, itemsize{2};

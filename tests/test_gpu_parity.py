@@ -59,16 +59,20 @@ def _run_and_compare(tb: CostTables, mesh, rescale, device):
     # the tiles where every row lies in one tile): all tables in one launch, and two launches
     fits = tb.rows_fit_tiles()
     want_rows = c_oracle.segmented_min(want["cost"], tb.row_ptr()) if fits and tb.n_entries else None
-    for one_launch in (True, False):
+    # ... and, where every tile holds whole rows, the launch over packed tiles (every wavefront on
+    # its own, entries evaluated directly in registers)
+    forms = [(True, False), (False, False)] + ([(True, True)] if tb.packable() else [])
+    for one_launch, packed in forms:
         dp = DeviceCostTables(tb, p, device=device, validate=False)
         step = dp.prepare_step(row_min=fits, fused_inputs=True, one_launch=one_launch, row_min_in_tiles=fits,
-                               outputs=("cost",), spec_table=False)
-        assert tuple(step) == (("build_tables",) if one_launch else ("input_tables", "redistribute_tables"))
+                               outputs=("cost",), spec_table=False, packed=packed)
+        assert tuple(step) == (("build_tables_packed",) if packed else ("build_tables",) if one_launch else
+                               ("input_tables", "redistribute_tables"))
         for launch in step.values():
             launch()
         torch.cuda.synchronize()
         assert dp.comm is None and dp.transition is None
-        assert np.array_equal(dp.cost.cpu().numpy(), want["cost"]), f"cost alone, one_launch={one_launch}"
+        assert np.array_equal(dp.cost.cpu().numpy(), want["cost"]), f"cost alone, one_launch={one_launch}, packed={packed}"
         assert np.array_equal(dp.compute_cost_per_arg.cpu().numpy(), want_pa)
         if want_rows is not None:
             assert np.array_equal(dp.row_min.cpu().numpy(), want_rows[0]) and np.array_equal(dp.row_argmin.cpu().numpy(), want_rows[1])

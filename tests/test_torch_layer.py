@@ -36,7 +36,7 @@ def test_arguments_are_checked_before_any_launch():
     with pytest.raises(RuntimeError, match="must be on the HIP device"):
         ops.segmented_min(f64, i64)
     params = _native.params_tensor(CostModelParams.from_mesh((4, 2)).to_c())
-    assert params.dtype == torch.uint8 and params.numel() == 296  # sizeof(struct apc_params)
+    assert params.dtype == torch.uint8 and params.numel() == 368  # sizeof(struct apc_params)
     i32 = torch.zeros(1, dtype=torch.int32)
     with pytest.raises(RuntimeError, match="struct apc_params"):
         ops.shard_shapes_bytes(params[:-8], i32, i32, i32, i32, i64, i64, 8)

@@ -249,7 +249,7 @@ def test_full_depth_llama3_8b_on_mesh_32x8(gpu_device, fake_pg):
             tb = o.encoded.tables
             assert type(o.backend).__name__ == ("DeviceBackend" if name == "device" else "OracleBackend")
             if name == "device":
-                assert o.backend.launches == ("build_tables",), "the planner's table build is one launch"
+                assert o.backend.launches == ("build_tables_packed",), "the planner's table build is one launch"
                 assert o.backend.dev.comm is None and o.backend.dev.transition is None
             plan = _solve_llama(autop)
             stats = o.solve_stats
