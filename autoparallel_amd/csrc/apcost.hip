@@ -535,8 +535,15 @@ template <int BS>
 __device__ __forceinline__ void compute_costs_block(int64_t block, const apc_params &p, const ComputeCostArgs &a) {
   const int64_t s = block * BS + threadIdx.x;
   if (s >= a.n) return;
-  bool unsupported;
-  const double c = compute_cost_of(p, a.zero_cost[s] != 0, a.rw_bytes[s], a.flops[s], a.dtype[s], unsupported);
+  // (the divisions through the checked reciprocals: the same bits as compute_cost_of, a third of
+  // its instructions; these workgroups share the chip with the ones that write the matrices)
+  const int dt = a.dtype[s];
+  const bool zero = a.zero_cost[s] != 0;
+  const int64_t flops = a.flops[s];
+  const bool known = dt >= 0 && dt < APC_MAX_DTYPES;
+  const double gf = known ? pick<APC_MAX_DTYPES>(p.gpu_flops, dt) : 0.0, inv_gf = known ? pick<APC_MAX_DTYPES>(p.inv_gpu_flops, dt) : 0.0;
+  const double c = compute_cost_through_reciprocals(p, zero, a.rw_bytes[s], flops, gf, inv_gf);
+  const bool unsupported = !zero && flops != 0 && gf == 0.0;
   if (unsupported && a.error_flag) *a.error_flag = 1;
   if (a.compute) a.compute[s] = c;
   if (a.per_arg) a.per_arg[s] = c / (double)a.num_args[s];

@@ -23,6 +23,46 @@ from ..cost_model import DTYPE_CODES
 
 UNSUPPORTED_DTYPE_CODE = 7
 
+
+def einsum_flop(equation, tensors, out=None, **kwargs) -> int:
+    """The flop count the reference registers for ``aten.einsum`` (compute_estimation.py:16-40): two
+    operands; [b, m, k] x [k, n] counts b m n k 2, two rank-3 operands [b, m, k] x [b, m, k2] (the
+    weight-gradient form) count (b m) k k2 2; any other pair of ranks is an error.  The equation
+    string itself is not read."""
+    assert len(tensors) == 2
+    a_shape, b_shape = [x.shape for x in tensors]
+    if len(a_shape) == 3 and len(b_shape) == 3:
+        b, m, k = a_shape
+        b1, n, k2 = b_shape
+        assert b == b1
+        assert m == n
+        return (b * m) * k * k2 * 2
+    if len(a_shape) == 3 and len(b_shape) == 2:
+        b, m, k = a_shape
+        k2, n = b_shape
+        assert k == k2
+        return b * m * n * k * 2
+    raise NotImplementedError(f"Unsupported einsum shapes: {a_shape} {b_shape}")
+
+
+def register_einsum_flop_formula() -> bool:
+    """Registers ``einsum_flop`` in torch's flop registry the way the reference does when it is
+    imported (``register_flop_formula(torch.ops.aten.einsum, get_raw=True)``,
+    compute_estimation.py:16), unless a formula for the operator is already there (the reference
+    itself, in the same process).  Whether ``FlopCounterMode`` consults it is torch's business and
+    the same for both: the installed torch (2.10) looks an operator's overload up before it
+    decomposes it, finds no entry under ``aten.einsum.default`` and counts the matrix products
+    of the decomposition, which for the shapes above are the same numbers."""
+    from torch.utils.flop_counter import flop_registry, register_flop_formula
+
+    if torch.ops.aten.einsum in flop_registry:
+        return False
+    register_flop_formula(torch.ops.aten.einsum, get_raw=True)(einsum_flop)
+    return True
+
+
+register_einsum_flop_formula()
+
 _DTYPE_TO_CODE = {getattr(torch, name): code for name, code in DTYPE_CODES.items()}
 
 

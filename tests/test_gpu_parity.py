@@ -210,16 +210,23 @@ def _golden():
 def test_known_answer_values_on_device(gpu_device):
     """The hand-derived values (tests/golden/known_answers.json) straight from the kernel."""
     R, P, S0, S1 = 0, partial_code(), shard_code(0), shard_code(1)
-    named = {"R": R, "P": P, "S0": S0, "S1": S1}
+    named = {"R": R, "P": P, "S0": S0, "S1": S1, "S2": shard_code(2)}
     g = _golden()
     mesh = tuple(g["environment"]["mesh"])
-    for case in g["redistribute_cost_us"]:
-        src, tgt = tuple(named[x] for x in case["src"]), tuple(named[x] for x in case["tgt"])
-        tb = _two_node_tables(mesh, case["shape"], case["stride"], case["itemsize"], [src], [tgt])
-        d = DeviceCostTables(tb, CostModelParams.from_mesh(mesh), device=gpu_device)
-        comm, trans, _ = d.build_all()
-        assert comm.cpu().numpy()[0] == case["value"], case["note"]
-        assert trans.cpu().numpy()[0] == 1
+    for cases, case_mesh in ((g["redistribute_cost_us"], mesh),
+                             (g["mesh_8x8x8"]["redistribute_cost_us"], tuple(g["mesh_8x8x8"]["environment"]["mesh"]))):
+        for case in cases:
+            src, tgt = tuple(named[x] for x in case["src"]), tuple(named[x] for x in case["tgt"])
+            tb = _two_node_tables(case_mesh, case["shape"], case["stride"], case["itemsize"], [src], [tgt])
+            d = DeviceCostTables(tb, CostModelParams.from_mesh(case_mesh), device=gpu_device)
+            comm, trans, _ = d.build_all()
+            assert comm.cpu().numpy()[0] == case["value"], case["note"]
+            assert trans.cpu().numpy()[0] == 1
+            # the launch over packed tiles (direct evaluation in registers) gives the same value
+            dp = DeviceCostTables(tb, CostModelParams.from_mesh(case_mesh), device=gpu_device)
+            for launch in dp.planner_pass(packed=True).values():
+                launch()
+            assert dp.cost.cpu().numpy()[0] == case["value"] + 1, case["note"]  # + the transition cost; compute cost 0
     # one matrix with the special cases around them
     src = [(S0, S0), (P, P), (S0, S1), (R, R), (S0, R)]
     tgt = [(R, S0), (R, R), (S0, S0), (S0, R), (S0, S1), (P, R)]

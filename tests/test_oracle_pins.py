@@ -112,7 +112,7 @@ def _golden():
         return json.load(f)
 
 
-_NAMED = {"R": R, "P": P, "S0": S0, "S1": S1}
+_NAMED = {"R": R, "P": P, "S0": S0, "S1": S1, "S2": S2}
 
 
 def test_known_answers_2d_mesh():
@@ -127,6 +127,49 @@ def test_known_answers_2d_mesh():
     assert po.redistribute_cost(tuple(_NAMED[x] for x in u["src"]), tuple(_NAMED[x] for x in u["tgt"]), u["shape"],
                                 u["stride"], u["itemsize"], p, u["order"]) == u["value"]
     assert p.bw[0] == g["inter_host_bandwidth_GBps"]
+
+
+def test_known_answers_3d_mesh():
+    """Mesh (8, 8, 8), 8 devices per host: dims 0 and 1 inter-host, dim 2 intra-host.  The running
+    bytes carried across three mesh dims, a reduce-scatter onto a non-dim-0 shard, an all-to-all
+    between two non-dim-0 shards and the non-contiguity charge, from the golden file and written
+    out here term by term (plain arithmetic, none of the oracle's helpers)."""
+    g = _golden()["mesh_8x8x8"]
+    mesh = tuple(g["environment"]["mesh"])
+    p = po.make_params(mesh)
+    assert list(p.bw) == g["environment"]["bandwidth_GBps"] and list(p.lat) == g["environment"]["hop_latency_us"]
+    for case in g["redistribute_cost_us"]:
+        src, tgt = tuple(_NAMED[x] for x in case["src"]), tuple(_NAMED[x] for x in case["tgt"])
+        assert _cost(src, tgt, case["shape"], case["stride"], case["itemsize"], mesh) == case["value"], case["note"]
+    inter, intra = 87.7 * 0.22, 87.7
+
+    def rw(nbytes):
+        return max(nbytes / (3.35 * 1024**4) * 1e6 / 0.70, 7)
+
+    # (S0, P, S1) -> (R, S0, R): gather over dim 0, reduce-scatter on the gathered bytes over dim 1,
+    # gather of a dim-1 shard over dim 2 with its reshuffle
+    gb = 2 * 4096 * 4096 / 64 / 1024 / 1024 / 1024  # Partial does not count as a shard
+    gb *= 8
+    expect = (6.6 + 7 * 2.7) + ((gb * 7 / 8) / inter) * 1e6
+    expect += (6.6 + 7 * 2.7) + ((gb * 7 / 8) / inter) * 1e6
+    gb /= 8
+    gb *= 8
+    expect += (6.6 + 7 * 0.6) + ((gb * 7 / 8) / intra) * 1e6
+    expect += rw(gb * 2 * 1024**3)
+    assert g["redistribute_cost_us"][0]["value"] == expect == _cost((S0, P, S1), (R, S0, R), mesh=mesh)
+    # Partial -> Shard(1): the reshuffle is charged on the bytes before the scatter
+    gb = 4 * 8192 * 4096 / 1024 / 1024 / 1024
+    expect = (6.6 + 7 * 2.7) + ((gb * 7 / 8) / inter) * 1e6
+    expect += rw(gb * 2 * 1024**3)
+    assert g["redistribute_cost_us"][1]["value"] == expect
+    # Shard(1) -> Shard(2): five times the ring term, two reshuffles
+    gb = 2 * 64 * 2048 * 4096 / 8 / 1024 / 1024 / 1024
+    expect = ((6.6 + 7 * 2.7) + ((gb * 7 / 8) / inter) * 1e6) * 5
+    expect += 2 * rw(gb * 2 * 1024**3)
+    assert g["redistribute_cost_us"][2]["value"] == expect
+    # dropping the reshuffle of the dim-1 gather, or charging the reduce-scatter after the division, is seen
+    assert _cost((S0, P, S0), (R, S0, R), mesh=mesh) < g["redistribute_cost_us"][0]["value"]
+    assert _cost((S0, P, S1), (R, S0, R), mesh=mesh) != _cost((S0, R, S1), (R, S0, R), mesh=mesh)
 
 
 def test_hand_expanded_allgather_value():

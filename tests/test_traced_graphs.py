@@ -364,3 +364,49 @@ def test_an_operator_without_a_recipe_takes_the_host_path(fake_pg):
             assert rc.host_nodes and all(n.target.overloadpacket == torch.ops.aten.mm for n in rc.host_nodes)
     finally:
         cost_inputs._CLOSED_FORMS.update(saved)
+
+
+def test_einsum_flop_formula_of_the_reference():
+    """The reference registers its own flop count for ``aten.einsum`` at import
+    (compute_estimation.py:16-40).  The restatement gives the values that formula defines, is
+    registered the same way, and a node with that operator is costed on the host path, through
+    torch's flop counter, as the reference costs it."""
+    from torch.utils.flop_counter import FlopCounterMode, flop_registry
+
+    from autoparallel_amd.graphs import cost_inputs
+
+    def meta(*shape):
+        return torch.empty(shape, device="meta")
+
+    f = cost_inputs.einsum_flop
+    # [b, m, k] x [k, n]: b m n k 2 (hand value: 4 * 8 * 32 * 16 * 2)
+    assert f("bmk,kn->bmn", [meta(4, 8, 16), meta(16, 32)]) == 32768
+    # two rank-3 operands (the weight-gradient form bmk,bmn->kn): (b m) k k2 2
+    assert f("bmk,bmn->kn", [meta(4, 8, 16), meta(4, 8, 32)]) == (4 * 8) * 16 * 32 * 2 == 32768
+    assert f("anything", [meta(2, 3, 5), meta(2, 3, 7)]) == 2 * 3 * 5 * 7 * 2  # the equation is not read
+    with pytest.raises(NotImplementedError, match="Unsupported einsum shapes"):
+        f("mk,kn->mn", [meta(8, 16), meta(16, 32)])
+    with pytest.raises(AssertionError):
+        f("bmk,kn->bmn", [meta(4, 8, 16), meta(15, 32)])  # contraction sizes differ
+    with pytest.raises(AssertionError):
+        f("a,b,c", [meta(2, 2, 2)] * 3)  # two operands only
+    # registered like the reference's (operator packet, raw arguments)
+    registered = flop_registry[torch.ops.aten.einsum]  # (stored unwrapped: it takes the operator's own arguments)
+    assert registered is f or registered.__module__.startswith("autoparallel.")  # (the reference's own, if it is in the process)
+    assert cost_inputs.register_einsum_flop_formula() is False  # a second registration is a no-op, not an error
+    # the count of an einsum node as the host path takes it (the reference's call: the operator on
+    # local-shaped fake tensors under FlopCounterMode): equal to the formula's on the supported shapes
+    a, b = meta(4, 8, 16), meta(16, 32)
+    from torch.utils._pytree import tree_flatten
+
+    flat, spec = tree_flatten(("bmk,kn->bmn", [a, b]))
+    kw_flat, kw_spec = tree_flatten({})
+    flops, rw_bytes, code = cost_inputs._evaluate(torch.ops.aten.einsum.default, flat, [1, 2], [((4, 8, 16), (128, 16, 1)), ((16, 32), (32, 1))],
+                                                  spec, kw_flat, kw_spec, None)
+    assert flops == f("bmk,kn->bmn", [a, b]) and rw_bytes == 4 * (4 * 8 * 16 + 16 * 32 + 4 * 8 * 32) and code == cost_inputs._DTYPE_TO_CODE[torch.float32]
+    with FlopCounterMode(display=False) as counter:
+        torch.ops.aten.einsum.default("bmk,kn->bmn", [a, b])
+    assert counter.get_total_flops() == flops
+    # no device recipe covers the operator: the planner routes the graph to the host path
+    assert torch.ops.aten.einsum not in cost_inputs._CLOSED_FORMS
+    assert torch._C._dispatch_has_kernel_for_dispatch_key(torch.ops.aten.einsum.default.name(), "CompositeImplicitAutograd")
