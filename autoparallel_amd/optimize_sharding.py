@@ -317,11 +317,20 @@ class ShardingOptimizer:
     # declared integral: with a node's and its producers' choices fixed to unit vectors the
     # row / column sum constraints leave exactly one feasible (integral) value for every entry
     # variable.  Same feasible plans and optimum, far fewer branching variables for the solver.
-    # how repeated subgraphs are found when the constructor is asked for them: "neighbourhood" (this
-    # package's refinement of node keys by their surroundings) or "regions" (the reference's region
-    # growing, graph_clustering.py:101-206, which under torch 2.10 fails its own sanity check on
-    # Llama-shaped graphs)
-    clustering = "neighbourhood"
+    # How repeated subgraphs are found when the constructor is asked for them.
+    #   "regions": the reference's region growing over torch's region tracker with the reference's
+    #       links (graph_clustering.py:101-206, optimize_sharding.py:211-231); raises the reference's own
+    #       "Duplicate node ... in region group" where the reference does (every Llama-shaped graph
+    #       under torch 2.10);
+    #   "neighbourhood": this package's refinement of node keys by their surroundings;
+    #   "reference" (default): "regions", and "neighbourhood" only where "regions" ends in that
+    #       error, so that a graph the reference can plan gets the reference's program.  torch's
+    #       region tracker keeps the set of all ancestors of every node (quadratic: 0.9 s on 2 600
+    #       nodes, 16.7 s on the 10 372 nodes of Llama-3-8B, where it then raises), so graphs of
+    #       more than ``regions_max_nodes`` nodes go to "neighbourhood" directly.
+    # ``clustering_used`` records which one produced the links, and why.
+    clustering = "reference"
+    regions_max_nodes = 3000
     # during enumeration torch's own redistribute_cost (whose values the table build replaces) is
     # stubbed by a constant; False leaves it alone (same tables, slower enumeration)
     cheap_enumeration_costs = True
@@ -380,12 +389,13 @@ class ShardingOptimizer:
         logger.info("%s %.3f s", "enumerate_s", self.timings["enumerate_s"])
 
         self.node_representative = {}
+        self.clustering_used = None
         if repeated_subgraphs:
             from .graphs import clustering
 
             t0 = time.perf_counter()
-            find = {"neighbourhood": clustering.cluster_nodes, "regions": clustering.cluster_regions}[self.clustering]
-            self.node_representative = find(self.graph, self.strats)
+            self.node_representative, self.clustering_used = self._find_repeated_subgraphs(clustering)
+            logger.info("repeated subgraphs: %s", self.clustering_used)
             self.timings["cluster_s"] = time.perf_counter() - t0
             logger.info("%s %.3f s", "cluster_s", self.timings["cluster_s"])
         self.ds, self.num_inp_out, self.num_args = self.build_ds()
@@ -403,6 +413,26 @@ class ShardingOptimizer:
         self.add_default_constraints()
 
     # ------------------------------------------------------------------------------------
+    def _find_repeated_subgraphs(self, clustering):
+        """-> (node -> representative, which algorithm produced it and why)."""
+        if self.clustering == "neighbourhood":
+            return clustering.cluster_nodes(self.graph, self.strats), "neighbourhood (asked for)"
+        if self.clustering == "regions":
+            return clustering.cluster_regions(self.graph, self.strats), "regions (asked for)"
+        if self.clustering != "reference":
+            raise ValueError(f"clustering must be 'reference', 'regions' or 'neighbourhood', not {self.clustering!r}")
+        n_nodes = len(self.graph.nodes)
+        if n_nodes > self.regions_max_nodes:
+            return clustering.cluster_nodes(self.graph, self.strats), (
+                f"neighbourhood ({n_nodes} nodes: torch's region tracker is quadratic, regions_max_nodes = "
+                f"{self.regions_max_nodes})")
+        try:
+            return clustering.cluster_regions(self.graph, self.strats), "regions (the reference's links)"
+        except RuntimeError as e:
+            if "Duplicate node" not in str(e):
+                raise
+            return clustering.cluster_nodes(self.graph, self.strats), f"neighbourhood (the reference's algorithm raised: {e})"
+
     def build_sharding_metadata(self):
         self.enumerator = StrategyEnumerator(self.mesh, cheap_costs=self.cheap_enumeration_costs)
         return self.enumerator.enumerate(self.graph)

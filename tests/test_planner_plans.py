@@ -626,3 +626,93 @@ def test_print_costs_for_node(meshes, capsys):
     first = opt.ds[(s_i, 1, 0, 0)]["comm_cost"]
     assert f"{first:.3f}" in out[2]
     assert len(out[0].split("  ")) >= n_cols
+
+
+def _plan_clustered(planner_cls, mesh, clustering=None):
+    model_fn, input_fn = make_model_and_inputs(mesh, "block")
+    with torch.device("meta"):
+        model = model_fn()
+
+    class Planner(planner_cls):
+        pass
+
+    if clustering is not None:
+        class Optimizer(planner_cls.optimizer_cls):
+            pass
+
+        Optimizer.clustering = clustering
+        Planner.optimizer_cls = Optimizer
+    with Planner(model, input_fn, mesh, repeated_subgraphs=True) as autop:
+        autop.add_parameter_memory_constraint(low=0, high=None)
+        placement = autop.optimize_placement()
+        return autop, placement
+
+
+def _reference_links_of_the_block():
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(__file__), "golden", "reference_strategies_and_costs.json")) as f:
+        case = json.load(f)["cases"]["block_32x8"]
+    assert case["cluster_links_error"] is None and len(case["cluster_links"]) == 50
+    return case["cluster_links"]
+
+
+def test_repeated_subgraphs_take_the_references_links_where_its_algorithm_returns(meshes):
+    """``repeated_subgraphs=True`` on the reference's transformer block: the default finds the links
+    the reference's own ``get_identical_regions`` + ``create_cluster_links`` produced on this
+    graph (held by the fixture), i.e. it solves the reference's program; on a Llama-shaped graph,
+    where the reference's function ends in its "Duplicate node" error, the neighbourhood algorithm
+    takes over and says so."""
+    autop, plan = _plan_clustered(OraclePlanner, meshes["2d"])
+    o = autop.sharding_optimizer
+    assert o.clustering == "reference" and o.clustering_used.startswith("regions")
+    assert {n.name: r.name for n, r in o.node_representative.items()} == _reference_links_of_the_block()
+    # the same program as with the reference's algorithm asked for by name; another one than the
+    # neighbourhood algorithm's (which links other node sets on this graph)
+    by_name, plan_by_name = _plan_clustered(OraclePlanner, meshes["2d"], "regions")
+    assert by_name.sharding_optimizer.objective_value() == o.objective_value()
+    assert {n.name: str(s) for n, s in plan.items()} == {n.name: str(s) for n, s in plan_by_name.items()}
+    other, _ = _plan_clustered(OraclePlanner, meshes["2d"], "neighbourhood")
+    assert other.sharding_optimizer.clustering_used.startswith("neighbourhood")
+    assert {n.name: r.name for n, r in other.sharding_optimizer.node_representative.items()} != _reference_links_of_the_block()
+    # linked nodes take one strategy; the clustered optimum is no better than the free one
+    for node, rep in o.node_representative.items():
+        assert str(plan[node]) == str(plan[rep]), (node, rep)
+    free, _ = _plan(OraclePlanner, meshes["2d"], "block", None)
+    assert o.objective_value() >= free.sharding_optimizer.objective_value() * (1 - 1e-12)
+    # (the reference's expected placements of this model are those of the free program: its links tie
+    # the four attention projections to one strategy, which moves the optimum)
+
+
+def test_repeated_subgraphs_fall_back_where_the_references_algorithm_raises(fake_pg):
+    from autoparallel_amd.graphs import workloads
+
+    mesh = workloads.logical_mesh((32, 8))
+    model, input_fn, _, _ = workloads.build_model("llama3_8b", mesh, n_layers=2)
+    with OraclePlanner(model, input_fn, mesh, param_dtype=torch.bfloat16, repeated_subgraphs=True) as autop:
+        o = autop.sharding_optimizer
+        assert o.clustering_used.startswith("neighbourhood (the reference's algorithm raised: Duplicate node")
+        assert len(o.node_representative) > 0
+
+    class Small(OracleOptimizer):
+        regions_max_nodes = 10
+
+    class Planner(OraclePlanner):
+        optimizer_cls = Small
+
+    with Planner(model, input_fn, mesh, param_dtype=torch.bfloat16, repeated_subgraphs=True) as autop:
+        assert "regions_max_nodes" in autop.sharding_optimizer.clustering_used
+
+
+@pytest.mark.gpu
+def test_repeated_subgraphs_with_device_tables_solve_the_references_program(gpu_device, meshes):
+    """The device tables under the reference's links: the plan and objective of the oracle's tables
+    under the same links."""
+    dev, dev_plan = _plan_clustered(AutoParallelPlanner, meshes["2d"])
+    ora, ora_plan = _plan_clustered(OraclePlanner, meshes["2d"])
+    d, o = dev.sharding_optimizer, ora.sharding_optimizer
+    assert type(d.backend).__name__ == "DeviceBackend" and d.clustering_used.startswith("regions")
+    assert {n.name: r.name for n, r in d.node_representative.items()} == _reference_links_of_the_block()
+    assert d.res == o.res and d.objective_value() == o.objective_value()
+    assert {n.name: str(s) for n, s in dev_plan.items()} == {n.name: str(s) for n, s in ora_plan.items()}
