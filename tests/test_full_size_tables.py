@@ -1,6 +1,7 @@
-"""The two large benchmark tables at their full size, every entry against the C oracle: the
-80-layer Llama-3-70B graph on (8, 8, 8) through the planner, and the 200 000-node synthetic DAG
-on (16, 8, 4).  (The Llama-3-8B graph at full depth: test_traced_graphs.py.)"""
+"""The benchmark tables at their full size, every entry against the C oracle: the 80-layer
+Llama-3-70B graph on (8, 8, 8) and the 16-layer DeepSeek-V3 style mixture of experts at its
+stated width on (64, 4) through the planner, and the 200 000-node synthetic DAG on (16, 8, 4).
+(The Llama-3-8B graph at full depth: test_traced_graphs.py.)"""
 
 import numpy as np
 import pytest
@@ -68,6 +69,65 @@ def test_full_depth_llama3_70b_on_mesh_8x8x8(gpu_device, fake_pg):
         entries = np.asarray(o.res_entries, np.int64)
         assert o.objective_value() == float(want["cost"][entries].sum()) > 0
         assert np.isfinite(want["cost"][entries]).all()
+
+
+def test_full_width_dsv3_moe_on_mesh_64x4(gpu_device, fake_pg):
+    """Configuration 4 at its stated size (_testing/models/dsv3.py:1161-1227, 1523): 16 layers, dim
+    7168, multi-head latent attention (q_lora 1536, kv_lora 512, 128 heads, rope dim 64), 256 routed
+    experts of width 2048 with 8 active plus one shared expert, batch 16 x 4096 tokens, mesh (64, 4),
+    the expert regions as ``local_map`` calls, captured through Dynamo.  (The seeded Zipf routing does
+    not enter: planning sees static shapes.)  Flop / byte counts, compute costs, every comm /
+    transition / cost entry and the row minima against the C oracle and the host path; then the
+    pruned solve: its objective is the sum of the oracle's costs of the chosen entries."""
+    from autoparallel_amd.graphs import workloads
+    from autoparallel_amd.graphs.dsv3 import DSV3_16L
+
+    cfg = DSV3_16L
+    assert (cfg.n_layers, cfg.dim, cfg.n_routed_experts, cfg.top_k, cfg.n_shared_experts) == (16, 7168, 256, 8, 1)
+    assert (cfg.q_lora_rank, cfg.kv_lora_rank, cfg.n_heads, cfg.qk_rope_head_dim, cfg.moe_inter_dim) == (1536, 512, 128, 64, 2048)
+    mesh_sizes = (64, 4)
+    mesh = workloads.logical_mesh(mesh_sizes)
+    model, input_fn, _, needs_dynamo = workloads.build_model("dsv3_moe", mesh)
+    assert needs_dynamo and tuple(input_fn().shape) == (16, 4096)
+    with AutoParallelPlanner(model, input_fn, mesh, param_dtype=torch.bfloat16, reduce_dtype=torch.float32,
+                             repeated_subgraphs=True, dynamo=True) as autop:
+        o = autop.sharding_optimizer
+        enc, tb = o.encoded, o.encoded.tables
+        _progress(f"planner built: {len(o.nodes)} nodes, {tb.n_entries} entries, {o.clustering_used}")
+        assert tb.n_entries == 1_073_460
+        assert o.backend.launches == ("build_tables_packed",), "a table this small is one launch over packed tiles"
+        assert sum("local_map_kwargs" in n.meta for n in o.graph.nodes) >= 2 * (cfg.n_layers - cfg.n_dense_layers)
+        device_counts = {k: getattr(tb, k).copy() for k in ("strat_flops", "strat_rw_bytes", "strat_dtype", "strat_zero_cost")}
+        if o.cost_input_stats["strategy_inputs"] == "device":
+            _, lshape, lstride, _, _ = c_oracle.spec_tables(tb.as_dict(), mesh_sizes)
+            fill_flops_and_bytes(enc, o.strats, np.asarray(lshape), np.asarray(lstride))
+            for k, v in device_counts.items():
+                assert np.array_equal(getattr(tb, k), v), k
+            _progress("flop / byte counts equal the host path's")
+        params = po.make_params(mesh_sizes, rescale=2.2)
+        want_compute, want_per_arg = c_oracle.compute_costs(tb.as_dict(), params)[:2]
+        assert np.array_equal(o.compute_cost, want_compute) and np.array_equal(o.compute_cost_per_arg, want_per_arg)
+        want = c_oracle.build_tables(tb.as_dict(), params, per_arg=want_per_arg)
+        for name in ("cost", "comm", "transition"):
+            assert np.array_equal(o.backend.host_array(name), want[name]), name
+            _progress(f"{name} equal")
+        mins, args = o.row_minima()
+        want_min, want_arg = c_oracle.segmented_min(want["cost"], tb.row_ptr())
+        assert np.array_equal(mins, want_min) and np.array_equal(args, want_arg)
+        _progress("row minima equal")
+        from torch.distributed.tensor.placement_types import Replicate, Shard
+
+        autop.add_parameter_memory_constraint(low=None, high=None)
+        # the batch (16) does not divide the mesh's first dim: the sequence is pinned instead
+        autop.add_input_constraints([(Shard(1), Replicate())])
+        autop.add_output_constraints([(Shard(1), Replicate())])
+        autop.optimize_placement()
+        stats = o.solve_stats
+        _progress(f"solved: {stats.get('solved_by')}, {stats.get('columns')} -> {stats.get('columns_after_pruning')} columns")
+        assert stats["incumbent"] is not None and stats["lower_bound"] <= stats["incumbent"] * (1 + 1e-9)
+        entries = np.asarray(o.res_entries, np.int64)
+        assert np.isfinite(want["cost"][entries]).all()
+        assert o.objective_value() == float(want["cost"][entries].sum()) > 0
 
 
 def test_stress_table_at_full_size(gpu_device):
