@@ -62,6 +62,11 @@ def parse_args():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy three times (reference reading for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
+    ap.add_argument("--calibrate-launch", action="store_true",
+                    help="only time an empty kernel launched back to back and plain fills of the bytes the three "
+                         "workloads' launches move (what roofline.launch_floor_us / fill_us come from) and exit")
+    ap.add_argument("--no-cpu-plan", action="store_true",
+                    help="skip the measured plan with the tables built on the host (about 15 s on the default workload)")
     ap.add_argument("--no-traffic", action="store_true",
                     help="skip the HBM-traffic reading (four short child runs of this script under rocprofv3 --pmc)")
     ap.add_argument("--replay-tables", default=None,
@@ -267,6 +272,61 @@ def solve_plan(planner, workload, compare_full=True):
     return out
 
 
+def plan_with_cpu_tables(workload, args, log):
+    """The same plan with the table stage on the host, measured: the planner of this package
+    (capture, enumeration, clustering, encoding, constraints, solver unchanged) with the scalar
+    Python oracle as its table source, the form in which the reference executes this path
+    (examples/example_llama3.py:243-245 times the same stages around ``optimize_placement``).
+    The pruning in front of the solver is off on this leg (its dual ascent runs on the device; the
+    reference has none): the solver receives the full program, as it does in
+    ``solve_s_without_pruning`` of the device leg.  -> stage times in seconds."""
+    import numpy as np
+    import torch
+
+    tests_dir = os.path.join(ROOT, "tests")
+    if tests_dir not in sys.path:
+        sys.path.insert(0, tests_dir)
+    from oracle_backend import OracleBackend  # the checker's table source behind the planner's backend interface
+
+    from autoparallel_amd.api import AutoParallelPlanner
+    from autoparallel_amd.graphs import workloads
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+    from oracle import cost_oracle as po
+
+    stage = {}
+
+    class PythonTables(OracleBackend):
+        def launch_tables(self):
+            t0 = time.perf_counter()
+            out = po.build_tables(self.tables.as_dict(), self.params)
+            self.out = {k: np.asarray(v, np.uint8 if k == "transition" else np.float64) for k, v in out.items()}
+            self.cost = self.out["cost"]
+            self.launches = ("python oracle",)
+            stage["cpu_tables_s"] = time.perf_counter() - t0
+
+    class Optimizer(ShardingOptimizer):
+        backend_cls = PythonTables
+        prune_before_solve = False
+        tile_entries = args.tile_entries
+        dedupe = not args.no_dedupe
+        max_copies = args.max_copies
+
+    class Planner(AutoParallelPlanner):
+        optimizer_cls = Optimizer
+
+    mesh = workloads.logical_mesh(workloads.WORKLOADS[workload][1])
+    model, input_fn, _, needs_dynamo = workloads.build_model(workload, mesh, n_layers=args.layers)
+    t_all = time.perf_counter()
+    with Planner(model, input_fn, mesh, param_dtype=torch.bfloat16, reduce_dtype=torch.float32,
+                 repeated_subgraphs=not args.no_clustering, dynamo=needs_dynamo) as planner:
+        stage.update({k: v for k, v in planner.timings.items() if k in ("capture_s", "optimizer_s")})
+        plan = solve_plan(planner, workload, compare_full=False)
+        stage["constraints_s"], stage["solve_s"], stage["objective"] = plan["constraints_s"], plan["solve_s"], plan["objective"]
+    stage["total_s"] = time.perf_counter() - t_all
+    log.info("plan with the tables built on the host: %.1f s (tables %.1f s)", stage["total_s"], stage["cpu_tables_s"])
+    return stage
+
+
 def cpu_baseline(tables, params, target_seconds):
     """The scalar Python oracle (the reference executes this path as interpreted Python) on
     a prefix of the workload's edges sized for about ``target_seconds`` of CPU work."""
@@ -419,11 +479,59 @@ def verify_pass(dev, tables, params, log):
             "entries": tables.n_entries, "bit_exact": True}
 
 
+def calibrate_launch(nbytes, grid, threads):
+    """What a launch of this shape costs before it does any work, and what a kernel that only
+    writes ``nbytes`` takes (the library's measurement kernels, back to back on the current stream,
+    one HIP event pair around the run): -> (launch_floor_us, fill_us, the fill's doubles per workgroup)."""
+    import ctypes
+
+    import torch
+
+    from autoparallel_amd import _native
+
+    lib = _native.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def timed(fn, k):
+        for _ in range(max(3, k // 10)):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(k):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / k
+
+    k = 200 if nbytes < (256 << 20) else 20
+
+    def empty():
+        _native.check(lib.apc_calibrate_launch(ctypes.c_int64(grid), ctypes.c_int32(threads), stream), "apc_calibrate_launch")
+
+    floor_us = timed(empty, 200)
+    n = nbytes // 8
+    buf = torch.empty(n + 2, dtype=torch.float64, device="cuda:0")
+    best = None
+    for per in (512, 2048, 8192, 16384):
+        def fill():
+            _native.check(lib.apc_calibrate_fill(ctypes.c_void_p(buf.data_ptr()), ctypes.c_int64(n), ctypes.c_int64(per),
+                                                 ctypes.c_double(1.0), stream), "apc_calibrate_fill")
+        us = timed(fill, k)
+        if best is None or us < best[0]:
+            best = (us, per)
+    del buf
+    return floor_us, best[0], best[1]
+
+
 def roofline_of(dev, tables, timing, steps, pass_kind):
     """The launch that writes the cost matrices against the HBM peak, two ways: over the bytes
-    that launch must move (``frac``) and over fixed per-unit prices (``frac_survey_8d``: 9 B per
-    entry, the spec lists and a 64-byte header per edge, 25 B per strategy when the launch also
-    builds the compute costs, 12 B per row minimum it takes)."""
+    that launch must move (``frac``) and over fixed per-unit prices (``frac_survey_8d``: 8 B per
+    entry for each fp64 array the launch writes and 1 B for the transition flag if it does, the
+    spec lists and a 64-byte header per edge, 25 B per strategy when the launch also builds the
+    compute costs, 12 B per row minimum it takes); and against two measured ceilings of this
+    system: an empty launch of the same grid (``launch_floor_us``) and a kernel that only writes
+    the same bytes (``fill_us``; ``frac_of_fill`` = fill_us / the launch's duration)."""
     import numpy as np
 
     names = timing["names"]
@@ -437,13 +545,15 @@ def roofline_of(dev, tables, timing, steps, pass_kind):
     per_edge = int(((tables.edge_n_src.astype(np.int64) + tables.edge_n_tgt.astype(np.int64)) * m + 64).sum())
     per_entry = 8 * ("comm" in outputs) + 1 * ("transition" in outputs) + 8 * ("cost" in outputs)
     launch_bytes = per_entry * tables.n_entries + per_edge + (12 * tables.n_rows if in_tiles else 0)
-    priced = 9 * tables.n_entries + per_edge + (12 * tables.n_rows if in_tiles else 0)
+    priced = per_entry * tables.n_entries + per_edge + (12 * tables.n_rows if in_tiles else 0)
     if one_launch:
         launch_bytes += tables.algorithmic_bytes_input_tables(spec_table=spec_table)
         priced += 25 * tables.n_strategies
     t_pair = timing["kernel_ms"][main] * 1e-3
     single = len(names) == 1
     t_kernel = timing["region_ms"] * 1e-3 / steps if single else t_pair
+    grid, threads = launch_shape(dev, tables, main)
+    floor_us, fill_us, fill_per_wg = calibrate_launch(priced, grid, threads)
     return {
         "bound": "hbm",
         "kernel": ("build_tables_packed_kernel" if packed else "build_tables_kernel" if one_launch else
@@ -451,18 +561,42 @@ def roofline_of(dev, tables, timing, steps, pass_kind):
         "launch": main + (" (the one launch of the pass)" if single else ""),
         "arrays_written_per_entry": list(outputs),
         "row_minima_taken_by_this_launch": bool(in_tiles),
-        "achieved": launch_bytes / t_kernel / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": launch_bytes / t_kernel / 1e9 / HBM_PEAK_GBPS,
-        "frac_survey_8d": priced / t_kernel / 1e9 / HBM_PEAK_GBPS,
+        # algorithmic bytes at fixed per-unit prices: 8 B per entry and fp64 array written (+ 1 B for the
+        # transition flag), the two spec lists and a 64-byte header per edge, 25 B per strategy when the
+        # launch builds the compute costs, 12 B per row minimum it takes
+        "achieved": priced / t_kernel / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": priced / t_kernel / 1e9 / HBM_PEAK_GBPS,
+        # every byte the launch reads or writes (the tensor and strategy table rows in full)
+        "frac_bytes_moved": launch_bytes / t_kernel / 1e9 / HBM_PEAK_GBPS,
         "traffic": None,  # filled in by measure_traffic for the main workload
-        "bytes_per_launch": launch_bytes, "bytes_per_launch_survey_8d": priced,
+        "bytes_per_launch": priced, "bytes_moved_per_launch": launch_bytes,
         "avg_launch_us": t_kernel * 1e6,
+        "launch_floor_us": floor_us, "fill_us": fill_us, "frac_of_fill": fill_us / (t_kernel * 1e6),
+        "calibration": f"apc_calibrate_launch: an empty kernel of the launch's grid ({grid} workgroups of {threads} threads) "
+                       f"back to back; apc_calibrate_fill: a kernel that only writes bytes_per_launch ({fill_per_wg} doubles "
+                       "per workgroup, the fastest of four splits), same timing",
         "avg_launch_us_event_pair_per_launch": t_pair * 1e6,
         "min_launch_us_event_pair_per_launch": timing["kernel_ms_min"][main] * 1e3,
         "timing": ("one HIP event pair on the launch stream around the K back-to-back launches of the timed "
                    "region (the pass is this one kernel), / K" if single else
                    "HIP events around every launch of the kernel inside the timed region"),
     }
+
+
+def launch_shape(dev, tables, main):
+    """(workgroups, threads) of the launch that writes the matrices, as the library sizes it."""
+    import numpy as np
+
+    n_tiles = tables.n_tiles
+    tile_blocks = (n_tiles + 7) // 8 * 8
+    if main == "build_tables_packed":
+        return tile_blocks + (tables.n_tensors + 255) // 256 + (tables.n_strategies + 255) // 256, 256
+    per_tile = tables.n_entries // max(n_tiles, 1)
+    if main == "build_tables":
+        threads = 256 if per_tile >= 1536 else 128 if per_tile >= 512 else 64
+        return tile_blocks + (tables.n_tensors + threads - 1) // threads + (tables.n_strategies + threads - 1) // threads, threads
+    threads = 256 if per_tile >= 4096 else 128 if per_tile >= 512 else 64
+    return tile_blocks, threads
 
 
 def measure(name, args, log, steps, warmup, main_run):
@@ -565,6 +699,14 @@ def main():
     if args.replay_tables:
         replay_tables(args.replay_tables)
         return
+    if args.calibrate_launch:
+        # the three workloads' launch shapes and bytes (bytes_per_launch of their roofline objects)
+        for name, nbytes, grid, threads in (("llama3_8b", 20_766_135, 1352, 256), ("llama3_70b", 596_653_014, 11736, 256),
+                                           ("stress", 3_825_705_690, 426920, 128)):
+            floor_us, fill_us, per = calibrate_launch(nbytes, grid, threads)
+            print(json.dumps({"workload": name, "bytes": nbytes, "grid": grid, "threads": threads, "launch_floor_us": floor_us,
+                              "fill_us": fill_us, "fill_doubles_per_workgroup": per, "fill_TBps": nbytes / fill_us / 1e6}))
+        return
     if args.calibrate_copy:
         src = torch.ones(1 << 27, dtype=torch.float64, device="cuda:0")  # 1 GiB
         dst = torch.empty_like(src)
@@ -607,7 +749,7 @@ def main():
         log.info("traffic reading: %.1f s", time.perf_counter() - t0)
         if read is not None:
             result["roofline"].update(read)
-            result["roofline"]["traffic_over_bytes_per_launch"] = read["traffic"] / result["roofline"]["bytes_per_launch"]
+            result["roofline"]["traffic_over_bytes_moved"] = read["traffic"] / result["roofline"]["bytes_moved_per_launch"]
             copy_factor = read["traffic_reading"]["scale_from_1gib_copy"]
     if planner is not None:
         plan = {"stages_s": {k: round(v, 6) for k, v in host_timings.items()}}
@@ -619,12 +761,25 @@ def main():
             + plan.get("constraints_s", 0.0) + plan.get("solve_s", 0.0)
         plan["total_with_gpu_tables_s"] = other + table_stage
         if "cpu_baseline" in result:
-            # the same plan with the tables built by the CPU port: only the table stage differs
+            # (derived, not a run: the device plan's other stages + the table size / the CPU port's rate)
             cpu_tables = tables.n_entries / result["cpu_baseline"]["value"]
-            plan["cpu_table_stage_s"] = cpu_tables
-            plan["total_with_cpu_tables_s"] = other + cpu_tables
+            plan["derived_cpu_table_stage_s"] = cpu_tables
+            plan["derived_total_with_cpu_tables_s"] = other + cpu_tables
         result["plan_wall_time"] = plan
         planner.__exit__(None, None, None)
+        planner = None
+        if not args.no_cpu_plan and not args.no_solve and not args.no_cpu_baseline:
+            measured = plan_with_cpu_tables(args.workload, args, log)
+            plan["measured_with_cpu_tables"] = {
+                "what": "the same planner run once more with the scalar Python oracle as its table source (1 core), "
+                        "pruning off: capture + optimizer construction (enumerate, cluster, encode, tables) + "
+                        "constraints + solve of the full program",
+                **{k: (round(v, 6) if k != "objective" else v) for k, v in measured.items()}}
+            if "solve_s_without_pruning" in plan:
+                plan["total_with_gpu_tables_without_pruning_s"] = \
+                    plan["total_with_gpu_tables_s"] - plan.get("solve_s", 0.0) + plan["solve_s_without_pruning"]
+            if abs(measured["objective"] - plan.get("objective", measured["objective"])) > 1e-6 * abs(measured["objective"]):
+                raise SystemExit("bench.py: the plan from host-built tables has another objective than the device's")
     del planner, tables
     # ---- the bandwidth-bound tables, beside the headline ---------------------------------------
     extra = {}
@@ -643,7 +798,7 @@ def main():
             read = measure_traffic(tb, o["params"], args.pass_kind, o["roofline"]["kernel"], log, factor=copy_factor)
             if read is not None:
                 o["roofline"].update(read)
-                o["roofline"]["traffic_over_bytes_per_launch"] = read["traffic"] / o["roofline"]["bytes_per_launch"]
+                o["roofline"]["traffic_over_bytes_moved"] = read["traffic"] / o["roofline"]["bytes_moved_per_launch"]
         del tb
         extra[name] = {"workload": o["config"]["workload"], "entries": o["config"]["entries"], "steps": k,
                        "ms_per_step": o["ms_per_step"], "entries_per_s": o["value"], "step": o["config"]["step"],
