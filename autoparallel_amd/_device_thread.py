@@ -48,13 +48,33 @@ def _forget_thread():
 os.register_at_fork(after_in_child=_forget_thread)
 
 
+def _callers_stream():
+    """The caller's current stream, None on a machine without a GPU.  A child forked from a
+    process that had already initialised the GPU cannot use the device at all (torch refuses
+    to initialise it a second time): that is reported as what it is, not as a torch internal."""
+    import torch
+
+    if not torch.cuda.is_available():
+        return None
+    try:
+        return torch.cuda.current_stream()
+    except RuntimeError as e:
+        if "fork" in str(e):
+            raise RuntimeError("apcost: this process was forked from one that had initialised the GPU; a forked child "
+                               "cannot do device work (start workers with the 'spawn' method, or fork before the "
+                               "parent touches the GPU)") from e
+        raise
+
+
 def call(fn, *args, **kwargs):
-    """``fn(*args, **kwargs)`` on the device thread; the result (or the exception) of the call."""
+    """``fn(*args, **kwargs)`` on the device thread; the result (or the exception) of the call.
+    In a forked child the parent's thread is gone and the first call starts a new one; device
+    work there needs a parent that had not initialised the GPU before the fork."""
     if threading.get_ident() == _worker_ident:
         return fn(*args, **kwargs)
     import torch
 
-    stream = torch.cuda.current_stream() if torch.cuda.is_available() else None
+    stream = _callers_stream()
 
     def task():
         if stream is None:

@@ -2197,45 +2197,82 @@ __global__ __launch_bounds__(kBlock) void strategy_bounds_kernel(int64_t n_strat
 // numbered group by group: a group is a set of edges with matrices of the same shape whose
 // entries share variables position by position (one edge when nothing is linked); variable
 // group_var_begin[g] + k sums entry k of every member edge, members in ascending entry order.
-// One thread per variable: neighbouring lanes read neighbouring entries of each member.
+// One workgroup per group (gridDim.y workgroups share a group, each taking every gridDim.y-th
+// run of kBlock variables): which group a variable belongs to is never searched for, what a
+// group needs (its first variable, its size, its member list) is the same for every lane and is
+// fetched once, and neighbouring lanes read neighbouring entries of each member.  The member
+// list goes through LDS, so the loads a thread has in flight are costs and nothing else:
+// kObjectiveMembersAhead members of one variable, or kObjectiveAhead variables of a group with a
+// single member; the additions of a variable stay in member order.
 // ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void cost_objective_kernel(int64_t n_vars, int64_t n_groups,
-                                                                const int64_t *__restrict__ group_var_begin,
+constexpr int kObjectiveAhead = 8;          // variables of a single-member group a thread has in flight
+constexpr int kObjectiveMembersAhead = 8;   // members of a variable a thread has in flight
+
+__global__ __launch_bounds__(kBlock) void cost_objective_kernel(const int64_t *__restrict__ group_var_begin,
                                                                 const int64_t *__restrict__ group_member_begin,
                                                                 const int64_t *__restrict__ member_entry_begin,
                                                                 const double *__restrict__ cost, double inf_replacement,
                                                                 double *__restrict__ objective,
                                                                 uint8_t *__restrict__ forced_zero) {
-  // the group of the workgroup's first variable by bisection, once; every thread then walks on
-  // from there (a workgroup's 256 variables span few groups)
-  __shared__ int64_t s_first_group;
-  const int64_t v0 = (int64_t)blockIdx.x * kBlock;
-  if (threadIdx.x == 0) {
-    int64_t lo = 0, hi = n_groups;  // last group whose first variable is <= v0
-    while (hi - lo > 1) {
-      const int64_t mid = (lo + hi) >> 1;
-      if (group_var_begin[mid] <= v0) lo = mid; else hi = mid;
+  __shared__ int64_t s_first_entry[kBlock];
+  const int tid = threadIdx.x;
+  const int64_t g = blockIdx.x;
+  const int64_t var0 = uniform_load(group_var_begin + g), size = uniform_load(group_var_begin + g + 1) - var0;
+  const int64_t member0 = uniform_load(group_member_begin + g), n_members = uniform_load(group_member_begin + g + 1) - member0;
+  const int64_t begin = (int64_t)blockIdx.y * kBlock, stride = (int64_t)gridDim.y * kBlock;
+  if (begin >= size) return;
+  const double inf = __builtin_inf();
+  auto put = [&](int64_t k, double sum, bool forced) {
+    objective[var0 + k] = sum;
+    forced_zero[var0 + k] = forced ? 1 : 0;
+  };
+  if (n_members == 1) {  // nothing is linked: one entry per variable, kObjectiveAhead variables of a thread in flight
+    const int64_t first = uniform_load(member_entry_begin + member0);
+    for (int64_t base = begin; base < size; base += kObjectiveAhead * stride) {
+      double c[kObjectiveAhead];
+#pragma unroll
+      for (int i = 0; i < kObjectiveAhead; ++i) {
+        const int64_t k = base + i * stride + tid;
+        c[i] = k < size ? cost[first + k] : 0.0;
+      }
+#pragma unroll
+      for (int i = 0; i < kObjectiveAhead; ++i) {
+        const int64_t k = base + i * stride + tid;
+        if (k >= size) continue;
+        const bool bad = !(__builtin_fabs(c[i]) < inf);  // inf or nan: math.isfinite is false
+        put(k, 0.0 + (bad ? inf_replacement : c[i]), bad);
+      }
     }
-    s_first_group = lo;
+    return;
   }
-  __syncthreads();
-  const int64_t v = v0 + threadIdx.x;
-  if (v >= n_vars) return;
-  int64_t lo = s_first_group;
-  while (lo + 1 < n_groups && group_var_begin[lo + 1] <= v) ++lo;
-  const int64_t k = v - group_var_begin[lo];
-  double sum = 0.0;
-  bool forced = false;
-  for (int64_t m = group_member_begin[lo], end = group_member_begin[lo + 1]; m < end; ++m) {
-    double c = cost[member_entry_begin[m] + k];
-    if (!(__builtin_fabs(c) < __builtin_inf())) {  // inf or nan: math.isfinite is false
-      c = inf_replacement;
-      forced = true;
+  for (int64_t base = begin; base < size; base += stride) {  // (the same trips for every thread of the workgroup)
+    const int64_t k = base + tid;
+    const bool active = k < size;
+    double sum = 0.0;
+    bool forced = false;
+    for (int64_t chunk = 0; chunk < n_members; chunk += kBlock) {
+      const int in_chunk = (int)(n_members - chunk < kBlock ? n_members - chunk : kBlock);
+      if (n_members > kBlock || base == begin) {  // (a list of at most kBlock members is staged once)
+        __syncthreads();
+        if (tid < in_chunk) s_first_entry[tid] = member_entry_begin[member0 + chunk + tid];
+        __syncthreads();
+      }
+      for (int at = 0; at < in_chunk; at += kObjectiveMembersAhead) {
+        double c[kObjectiveMembersAhead];
+#pragma unroll
+        for (int i = 0; i < kObjectiveMembersAhead; ++i) c[i] = active && at + i < in_chunk ? cost[s_first_entry[at + i] + k] : 0.0;
+#pragma unroll
+        for (int i = 0; i < kObjectiveMembersAhead; ++i) {
+          if (at + i < in_chunk) {
+            const bool bad = !(__builtin_fabs(c[i]) < inf);
+            forced |= bad;
+            sum += bad ? inf_replacement : c[i];
+          }
+        }
+      }
     }
-    sum += c;
+    if (active) put(k, sum, forced);
   }
-  objective[v] = sum;
-  forced_zero[v] = forced ? 1 : 0;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -2273,13 +2310,11 @@ __device__ __forceinline__ double wave_min(double v) {
   return v;
 }
 
-__global__ __launch_bounds__(kBlock) void diffusion_node_update_kernel(DiffusionArgs a) {
-  __shared__ double s_tot[kDiffusionMaxLabels];
-  const int c = a.nodes[blockIdx.x];
-  const int64_t l0 = a.label_begin[c];
-  const int n_labels = (int)(a.label_begin[c + 1] - l0);
-  const int64_t t0 = a.inc_begin[c], t1 = a.inc_begin[c + 1];
-  if (t1 == t0) return;
+// The update of one class against the matrices where they lie: one pass over every incident
+// matrix for the minima, one for the shares, the matrices taken one after the other.  The path
+// of a class whose matrices do not fit the staging arrays of the kernel below.
+__device__ void diffusion_update_in_memory(const DiffusionArgs &a, double *s_tot, int64_t l0, int n_labels, int64_t t0,
+                                           int64_t t1) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   constexpr int kWaves = kBlock / 64;
   const double inf = __builtin_inf();
@@ -2352,6 +2387,134 @@ __global__ __launch_bounds__(kBlock) void diffusion_node_update_kernel(Diffusion
         }
       }
     }
+  }
+}
+
+// One workgroup per class.  A planning program's classes are small (tens of labels, a handful
+// of incident matrices of a few hundred elements), so an update is a chain of dependent memory
+// round trips and nothing else; the kernel keeps that chain as short as the data allows: the
+// incidence list in one round, every incident matrix into LDS in one round of independent
+// loads (the elements of all matrices numbered through, a thread finds the matrix of an
+// element by bisecting the staged offsets), minima, totals and shares out of LDS, and every
+// element stored once.  Element by element the arithmetic is that of the path above, in the
+// same order: (v - d) where the row has a finite minimum, then + share or +inf.
+constexpr int kDiffusionStagedElements = 8192;  // doubles of LDS for the incident matrices of a class
+constexpr int kDiffusionStagedDegree = 64;      // incident matrices of a class
+constexpr int kDiffusionStagedPairs = 2048;     // (incident matrix, label) pairs of a class
+
+__global__ __launch_bounds__(kBlock) void diffusion_node_update_kernel(DiffusionArgs a) {
+  __shared__ double s_tot[kDiffusionMaxLabels];
+  __shared__ double s_m[kDiffusionStagedElements];
+  __shared__ double s_d[kDiffusionStagedPairs];
+  __shared__ int64_t s_base[kDiffusionStagedDegree];
+  __shared__ int s_off[kDiffusionStagedDegree + 1];
+  __shared__ int s_other[kDiffusionStagedDegree];
+  __shared__ int s_side[kDiffusionStagedDegree];
+  const int c = a.nodes[blockIdx.x];
+  const int64_t l0 = a.label_begin[c];
+  const int n_labels = (int)(a.label_begin[c + 1] - l0);
+  const int64_t t0 = a.inc_begin[c], t1 = a.inc_begin[c + 1];
+  if (t1 == t0) return;
+  if (n_labels > kDiffusionMaxLabels || n_labels < 0) return;  // (the host entry point refuses such a class)
+  const int tid = threadIdx.x;
+  const int64_t degree64 = t1 - t0;
+  if (degree64 > kDiffusionStagedDegree || degree64 * n_labels > kDiffusionStagedPairs) {
+    diffusion_update_in_memory(a, s_tot, l0, n_labels, t0, t1);
+    return;
+  }
+  const int degree = (int)degree64;
+  const double inf = __builtin_inf();
+  // the incidence list: edge, side, where its matrix starts and how many labels the class at
+  // its other end has; the unary vector rides along in the same round
+  double unary = 0.0;
+  if (tid < n_labels) unary = a.unary[l0 + tid];  // (n_labels <= kStagedPairs / degree; labels beyond kBlock below)
+  int size = 0;
+  if (tid < degree) {
+    const int k = a.inc_edge[t0 + tid];
+    const int side = a.inc_side[t0 + tid];
+    const int other_class = side == 0 ? a.edge_j[k] : a.edge_i[k];
+    const int other = (int)(a.label_begin[other_class + 1] - a.label_begin[other_class]);
+    s_base[tid] = a.edge_begin[k];
+    s_other[tid] = other;
+    s_side[tid] = side;
+    size = other * n_labels;
+  }
+  if (tid < 64) {  // degree <= 64: the offsets of the matrices in LDS, a scan within the first wavefront
+    int incl = size;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int o = __shfl_up(incl, off, 64);
+      if (tid >= off) incl += o;
+    }
+    if (tid < degree) s_off[tid + 1] = incl;
+    if (tid == 0) s_off[0] = 0;
+  }
+  __syncthreads();
+  const int total = s_off[degree];
+  if (total > kDiffusionStagedElements || total < 0) {  // uniform: every thread reads the same word
+    diffusion_update_in_memory(a, s_tot, l0, n_labels, t0, t1);
+    return;
+  }
+  auto matrix_of = [&](int g) {  // the incident matrix that holds staged element g: the last t with s_off[t] <= g
+    int lo = 0, hi = degree - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (s_off[mid] <= g) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+  };
+  constexpr int kAhead = 4;  // loads a thread issues before it waits for the first
+  for (int base = 0; base < total; base += kAhead * kBlock) {
+    double v[kAhead];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int g = base + u * kBlock + tid;
+      v[u] = 0.0;
+      if (g < total) {
+        const int t = matrix_of(g);
+        v[u] = a.theta[s_base[t] + (g - s_off[t])];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int g = base + u * kBlock + tid;
+      if (g < total) s_m[g] = v[u];
+    }
+  }
+  __syncthreads();
+  // pull: one thread per (incident matrix, label of the class)
+  const int pairs = degree * n_labels;
+  for (int q = tid; q < pairs; q += kBlock) {
+    const int t = q / n_labels, x = q - t * n_labels;
+    const int other = s_other[t];
+    // rows of the class are contiguous runs of `other` elements; its columns are strided by n_labels
+    const int first = s_off[t] + (s_side[t] == 0 ? x * other : x);
+    const int step = s_side[t] == 0 ? 1 : n_labels;
+    double d = inf;
+    for (int y = 0; y < other; ++y) {
+      const double v = s_m[first + y * step];
+      d = v < d ? v : d;
+    }
+    if (d < inf)
+      for (int y = 0; y < other; ++y) s_m[first + y * step] -= d;
+    s_d[q] = d;
+  }
+  __syncthreads();
+  // totals in incidence order, one division: the share every incident matrix gets back
+  for (int x = tid; x < n_labels; x += kBlock) {
+    double tot = x == tid && tid < n_labels ? unary : a.unary[l0 + x];
+    for (int t = 0; t < degree; ++t) tot += s_d[t * n_labels + x];
+    const bool finite = tot < inf;
+    s_tot[x] = finite ? tot / (double)degree : inf;
+    a.unary[l0 + x] = finite ? 0.0 : inf;
+  }
+  __syncthreads();
+  for (int g = tid; g < total; g += kBlock) {
+    const int t = matrix_of(g);
+    const int e = g - s_off[t];
+    const int x = s_side[t] == 0 ? e / s_other[t] : e % n_labels;
+    const double share = s_tot[x];
+    a.theta[s_base[t] + e] = share < inf ? s_m[g] + share : inf;
   }
 }
 
@@ -2871,10 +3034,14 @@ int apc_cost_objective(int64_t n_vars, int64_t n_groups, const int64_t *group_va
   if (n_groups == 0) return fail(-1, "apc_cost_objective: %lld variables and no group", (long long)n_vars);
   if (!group_var_begin || !group_member_begin || !member_entry_begin || !cost || !objective || !forced_zero)
     return fail(-1, "apc_cost_objective: NULL array");
-  if ((n_vars + kBlock - 1) / kBlock > INT32_MAX) return fail(-1, "n_vars %lld too large", (long long)n_vars);
-  hipLaunchKernelGGL(cost_objective_kernel, dim3(blocks_for(n_vars, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, n_vars,
-                     n_groups, group_var_begin, group_member_begin, member_entry_begin, cost, inf_replacement, objective,
-                     forced_zero);
+  if (n_groups > INT32_MAX) return fail(-1, "apc_cost_objective: %lld groups, at most %d are launched", (long long)n_groups, INT32_MAX);
+  // a program of few groups spreads each over several workgroups (those beyond a group's size
+  // leave at once); with thousands of groups the device is full as it is
+  // (and no more shares than twice what a group of average size fills)
+  const int64_t average_runs = (n_vars / n_groups + kBlock - 1) / kBlock;
+  const int64_t shares = n_groups >= 4096 ? 1 : std::min<int64_t>({64, (4096 + n_groups - 1) / n_groups, 2 * std::max<int64_t>(1, average_runs)});
+  hipLaunchKernelGGL(cost_objective_kernel, dim3((unsigned)n_groups, (unsigned)shares), dim3(kBlock), 0, (hipStream_t)stream,
+                     group_var_begin, group_member_begin, member_entry_begin, cost, inf_replacement, objective, forced_zero);
   return check_launch("apc_cost_objective");
 }
 

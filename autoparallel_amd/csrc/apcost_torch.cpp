@@ -613,7 +613,8 @@ Tensor strategy_bounds(const Tensor &strat_node, const Tensor &node_strat_begin,
 // Sweeps of min-sum diffusion over a labelling problem, in place on theta / unary.
 void diffusion_sweeps_(int64_t n_sweeps, const Tensor &color_begin, const Tensor &color_nodes, const Tensor &label_begin,
                        const Tensor &inc_begin, const Tensor &inc_edge, const Tensor &inc_side, const Tensor &edge_begin,
-                       const Tensor &edge_i, const Tensor &edge_j, int64_t max_labels, const Tensor &theta, const Tensor &unary) {
+                       const Tensor &edge_i, const Tensor &edge_j, int64_t max_labels, int64_t n_labels_total, int64_t n_elements,
+                       const Tensor &theta, const Tensor &unary) {
   TORCH_CHECK(color_begin.device().is_cpu() && color_begin.scalar_type() == at::kLong && color_begin.is_contiguous() && color_begin.numel() >= 1,
               "apcost: color_begin must be a contiguous CPU int64 tensor of n_colors + 1 rows");
   const int32_t *cn = dev<int32_t>(color_nodes, at::kInt, "color_nodes");
@@ -626,6 +627,10 @@ void diffusion_sweeps_(int64_t n_sweeps, const Tensor &color_begin, const Tensor
   TORCH_CHECK(label_begin.numel() >= 1 && inc_begin.numel() == label_begin.numel(), "apcost: label_begin / inc_begin need n_classes + 1 rows each");
   TORCH_CHECK(edge_i.numel() == edge_j.numel() && edge_begin.numel() == edge_i.numel() + 1, "apcost: edge_begin needs n_edges + 1 rows, edge_i / edge_j n_edges");
   TORCH_CHECK(inc_edge.numel() == inc_side.numel(), "apcost: inc_edge and inc_side differ in length");
+  // the ends of the pointer arrays as the host knows them: the kernels index unary by label_begin and theta by edge_begin
+  TORCH_CHECK(unary.numel() == n_labels_total, "apcost: unary has ", unary.numel(), " values, label_begin ends at ", n_labels_total);
+  TORCH_CHECK(theta.numel() == n_elements, "apcost: theta has ", theta.numel(), " values, edge_begin ends at ", n_elements);
+  TORCH_CHECK(color_nodes.numel() == label_begin.numel() - 1, "apcost: color_nodes needs one row per class");
   for (const Tensor *t : {&color_nodes, &label_begin, &inc_begin, &inc_edge, &inc_side, &edge_begin, &edge_i, &edge_j, &unary}) same_device(theta, *t, "an index array");
   const int64_t n_classes = label_begin.numel() - 1;
   on_current_stream(theta.device(), "apc_diffusion_sweeps", [&](void *s) {
@@ -755,7 +760,7 @@ TORCH_LIBRARY(apcost, m) {
         "Tensor edge_row_begin, Tensor row_min) -> Tensor",
         &strategy_bounds);
   m.def("diffusion_sweeps_(int n_sweeps, Tensor color_begin, Tensor color_nodes, Tensor label_begin, Tensor inc_begin, "
-        "Tensor inc_edge, Tensor inc_side, Tensor edge_begin, Tensor edge_i, Tensor edge_j, int max_labels, Tensor(a!) theta, "
+        "Tensor inc_edge, Tensor inc_side, Tensor edge_begin, Tensor edge_i, Tensor edge_j, int max_labels, int n_labels_total, int n_elements, Tensor(a!) theta, "
         "Tensor(b!) unary) -> ()",
         &diffusion_sweeps_);
   m.def("bind_tensor_tables(" APCOST_TENSOR_TABLE ", Tensor tensor_bytes, Tensor tensor_contiguous) -> __torch__.torch.classes.apcost.BoundLaunch",

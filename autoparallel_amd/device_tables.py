@@ -562,7 +562,8 @@ class DeviceCostTables:
         color_begin = torch.from_numpy(np.ascontiguousarray(graph.color_begin, np.int64))
         max_labels = int(np.diff(graph.label_begin).max()) if graph.n_classes else 0
         self.ops.diffusion_sweeps_(int(n_sweeps), color_begin, d["color_nodes"], d["label_begin"], d["inc_begin"],
-                                   d["inc_edge"], d["inc_side"], d["edge_begin"], d["edge_i"], d["edge_j"], max_labels, th, un)
+                                   d["inc_edge"], d["inc_side"], d["edge_begin"], d["edge_i"], d["edge_j"], max_labels,
+                                   int(graph.label_begin[-1]), int(graph.edge_begin[-1]), th, un)
         return th.cpu().numpy(), un.cpu().numpy()
 
     @_guarded

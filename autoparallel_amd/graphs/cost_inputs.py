@@ -14,6 +14,8 @@ as getitem, views: compute_estimation.py:279-291) never reach the shape function
 
 from __future__ import annotations
 
+import math
+
 import numpy as np
 import torch
 from torch.utils._pytree import tree_flatten
@@ -123,7 +125,75 @@ class StrategyRecipes:
         self.host_nodes: list = []
 
 
-def strategy_recipes(encoded, strats) -> StrategyRecipes:
+def _local_shape_stride(tables, row: int, mesh_sizes):
+    """Local shape and stride of spec row ``row`` on the host (compute_estimation.py:211-229:
+    the sharded dim ceil-divided by the mesh dim's size, the stride of the dim before it as
+    well when that dim is not the first) -- the rule the spec-table kernel applies to every
+    row; here for the one row per operator that the recipe check below evaluates."""
+    from ..encoding import KIND_SHARD, code_dim, code_kind, unpack_codes
+
+    t = int(tables.spec_tensor[row])
+    r = int(tables.tensor_rank[t])
+    shape = [int(x) for x in tables.tensor_shape[t][:r]]
+    stride = [int(x) for x in tables.tensor_stride[t][:r]]
+    for n, c in zip(mesh_sizes, unpack_codes(int(tables.spec_codes[row]), len(mesh_sizes))):
+        if code_kind(c) == KIND_SHARD:
+            d = code_dim(c)
+            shape[d] = (shape[d] + n - 1) // n
+            if d - 1 > 0:
+                stride[d - 1] = (stride[d - 1] + n - 1) // n
+    return tuple(shape), tuple(stride)
+
+
+def _recipe_holds(encoded, s_i, node, vals, tensor_pos, node_args, flat_args, treespec, kw_vals, kw_spec, out_rows,
+                  const_bytes, mesh_sizes, n_strategies) -> bool:
+    """Whether a bytes-only recipe gives what the reference's evaluation gives for ``node``
+    (compute_estimation.py:232-243, 334-349 adds the bytes of what the operator RETURNS on the
+    local-shaped arguments; the recipe adds the local bytes of the output specs: equal only
+    while the operator's output shape follows its sharded inputs).  One strategy is evaluated
+    on the host: the first one that shards an argument or an output (a fully replicated
+    strategy cannot tell the two apart), and its flops must be zero."""
+    from ..encoding import KIND_SHARD, code_kind, unpack_codes
+
+    tb = encoded.tables
+    arg_rows = [encoded.input_spec_row[(s_i, k)] for k in range(len(node_args))]
+    M = len(mesh_sizes)
+
+    def sharded(row):
+        return int(tb.spec_tensor[row]) >= 0 and any(code_kind(c) == KIND_SHARD for c in unpack_codes(int(tb.spec_codes[row]), M))
+
+    pick = 0
+    for ss in range(n_strategies):
+        if any(sharded(r + ss) for r in arg_rows + out_rows):
+            pick = ss
+            break
+    if any(int(tb.spec_tensor[r + pick]) < 0 for r in arg_rows):
+        return False  # an argument without a spec: nothing to take a local shape from
+    local = {i: _local_shape_stride(tb, arg_rows[k] + pick, mesh_sizes) for k, i in enumerate(node_args)}
+    shapes = [local.get(i, (tuple(vals[i].shape), tuple(vals[i].stride()))) for i in tensor_pos]
+    mode = getattr(vals[tensor_pos[0]], "fake_mode", None)
+    try:
+        flops, rw_bytes, _ = _evaluate(node.target, vals, tensor_pos, shapes, treespec, kw_vals, kw_spec, mode)
+    except Exception:
+        return False  # the host path reports what the operator cannot run on
+    want = const_bytes
+    for r in arg_rows + out_rows:
+        row = r + pick
+        t = int(tb.spec_tensor[row])
+        if t >= 0:
+            want += math.prod(_local_shape_stride(tb, row, mesh_sizes)[0]) * int(tb.tensor_itemsize[t])
+    return flops == 0 and rw_bytes == want
+
+
+def tb_codes(encoded, rows, n_strategies):
+    """The placement codes of the spec rows of a node (its strategies one after the other per
+    argument / output slot), as bytes: two nodes with the same operator, shapes and codes have
+    the same recipe check."""
+    tb = encoded.tables
+    return [np.ascontiguousarray(tb.spec_codes[r:r + n_strategies]).tobytes() for r in rows]
+
+
+def strategy_recipes(encoded, strats, mesh_sizes=None) -> StrategyRecipes:
     """One recipe per graph node (no per-strategy work on the host).  What the reference does
     per strategy (compute_estimation.py:232-299, 334-349): run the operator on fake tensors of
     the local shard shapes under ``FlopCounterMode`` and add the bytes of every tensor among
@@ -131,12 +201,19 @@ def strategy_recipes(encoded, strats) -> StrategyRecipes:
     specs and output specs (rows of the spec table) plus the bytes of tensor constants; for an
     operator without tensor arguments (a factory) the operator runs on its own arguments, so
     its output is the global tensor whatever the strategy: a constant; flops as the closed
-    form of the operator's entry in torch's flop registry, zero outside the registry."""
+    form of the operator's entry in torch's flop registry, zero outside the registry.
+
+    A bytes-only recipe (an operator outside the flop registry) rests on the operator's output
+    having the local shape of its output spec.  With ``mesh_sizes`` given, that is checked once
+    per distinct (operator, constants, argument shapes and dtypes) by evaluating one sharded
+    strategy on the host the reference's way; a node whose recipe does not hold is listed in
+    ``host_nodes``."""
     from torch.utils.flop_counter import flop_registry
 
     n_nodes = len(encoded.nodes)
     rc = StrategyRecipes(n_nodes)
     rows: list = []
+    checked: dict = {}  # (operator, constants, argument shapes / strides / dtypes) -> the recipe holds
     slots_of: dict = {}
     for (s_i, slot), row in encoded.output_spec_row.items():
         slots_of.setdefault(s_i, []).append(row)
@@ -188,6 +265,19 @@ def strategy_recipes(encoded, strats) -> StrategyRecipes:
         elif packet in flop_registry or torch._C._dispatch_has_kernel_for_dispatch_key(
                 node.target.name(), "CompositeImplicitAutograd"):
             rc.host_nodes.append(node)  # counted by torch, no formula here (or decomposes under the counter)
+        elif mesh_sizes is not None:
+            key = (node.target, tuple(_const_key(v) for i, v in enumerate(vals) if i not in tensor_pos), str(treespec),
+                   tuple(_const_key(v) for v in kw_vals), str(kw_spec),
+                   tuple((tuple(vals[i].shape), tuple(vals[i].stride()), vals[i].dtype, isinstance(flat_args[i], torch.fx.Node))
+                         for i in tensor_pos),
+                   tuple(tb_codes(encoded, arg_rows + slots_of.get(s_i, []), len(strats[node].strategies))))
+            ok = checked.get(key)
+            if ok is None:
+                ok = checked[key] = _recipe_holds(encoded, s_i, node, vals, tensor_pos, node_args, flat_args, treespec, kw_vals,
+                                                  kw_spec, slots_of.get(s_i, []), int(rc.node_const_bytes[s_i]), mesh_sizes,
+                                                  len(strats[node].strategies))
+            if not ok:
+                rc.host_nodes.append(node)
     rc.node_row_begin[n_nodes] = len(rows)
     rc.byte_rows = np.asarray(rows, np.int32)
     return rc

@@ -467,7 +467,7 @@ class ShardingOptimizer:
         # device from per-node recipes; on the host, operator by operator on fake tensors of the
         # local shapes, when the graph holds an operator no recipe covers (or the backend has
         # no device)
-        recipes = strategy_recipes(self.encoded, self.strats) if self.strategy_inputs_on_device else None
+        recipes = strategy_recipes(self.encoded, self.strats, tuple(self.mesh.shape)) if self.strategy_inputs_on_device else None
         on_device = recipes is not None and not recipes.host_nodes and hasattr(self.backend, "strategy_inputs")
         self.cost_input_stats["strategy_inputs"] = "device" if on_device else "host"
         if on_device:

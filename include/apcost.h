@@ -338,7 +338,9 @@ int apc_strategy_bounds(int64_t n_strategies, const int32_t *strat_node, const i
  * group_var_begin[g + 1]) and has members [group_member_begin[g], group_member_begin[g + 1]):
  * edges whose matrices have group_var_begin[g + 1] - group_var_begin[g] entries each and share
  * variables position by position; member_entry_begin[m] is the member's first entry, members
- * of a group in ascending order.  objective[v] / forced_zero[v] are [n_vars]. */
+ * of a group in ascending order.  group_var_begin[0] is 0, group_var_begin[n_groups] is n_vars,
+ * and no group is empty (group_var_begin ascends strictly); the arrays are device memory and
+ * the caller checks them.  objective[v] / forced_zero[v] are [n_vars]. */
 int apc_cost_objective(int64_t n_vars, int64_t n_groups, const int64_t *group_var_begin,
                        const int64_t *group_member_begin, const int64_t *member_entry_begin, const double *cost,
                        double inf_replacement, double *objective, uint8_t *forced_zero, void *stream);
@@ -374,7 +376,9 @@ int apc_diffusion_sweeps(int32_t n_sweeps, int32_t n_colors, const int64_t *colo
  * 2 097 152 strategies; larger tables are rejected with an error.  Two launches on `stream`
  * (staging, then the tiles); no hipMalloc / hipFree, no synchronisation.  Results equal those of
  * apc_input_tables followed by apc_redistribute_tables.  All calls on one GPU share the array:
- * calls that overlap on a GPU (two streams, two threads) race.  A strategy with flops whose
+ * calls that overlap on a GPU (two streams, two threads) race: a call on another stream must be
+ * ordered (an event, a synchronisation) after the previous call's tile launch has finished, not
+ * merely after it was enqueued.  A strategy with flops whose
  * dtype has no throughput on the device row yields NaN costs (there is no error flag). */
 int apc_redistribute_tables_static(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
                                    const int32_t *tensor_itemsize, const int64_t *tensor_shape,

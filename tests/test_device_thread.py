@@ -112,8 +112,15 @@ def test_tables_after_a_warm_up():
 
 
 def test_a_forked_child_starts_its_own_thread():
+    """Covers a parent that has not initialised the GPU (every CPU run, and a GPU process that
+    forks before its first device call): the child gets a worker of its own.  A parent that has
+    initialised the GPU cannot have children that use it; that case is the next test."""
     import os
 
+    import torch
+
+    if torch.cuda.is_initialized():
+        pytest.skip("this process has initialised the GPU: its forked children cannot use the device")
     assert call(lambda: 1) == 1  # the parent's thread exists
     r, w = os.pipe()
     pid = os.fork()
@@ -133,3 +140,23 @@ def test_a_forked_child_starts_its_own_thread():
         os.kill(pid, 9)
     os.waitpid(pid, 0)
     assert got == b"1"
+
+
+def test_a_child_of_a_gpu_parent_is_told_so(monkeypatch):
+    """torch refuses to initialise the GPU in a child forked after the parent did: the caller
+    gets an error that names the situation and the way out."""
+    import torch
+
+    from autoparallel_amd import _device_thread
+
+    def refuse():
+        raise RuntimeError("Cannot re-initialize CUDA in forked subprocess. To use CUDA with multiprocessing, "
+                           "you must use the 'spawn' start method")
+
+    monkeypatch.setattr(torch.cuda, "is_available", lambda: True)
+    monkeypatch.setattr(torch.cuda, "current_stream", refuse)
+    with pytest.raises(RuntimeError, match="forked from one that had initialised the GPU"):
+        _device_thread._callers_stream()
+    monkeypatch.setattr(torch.cuda, "current_stream", lambda: (_ for _ in ()).throw(RuntimeError("something else")))
+    with pytest.raises(RuntimeError, match="something else"):
+        _device_thread._callers_stream()

@@ -111,6 +111,56 @@ def test_planner_pass_and_objective_match_the_oracle(gpu_device, mesh, link, pac
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("n_groups,max_size,max_members", [
+    (350_000, 40, 3),     # four variables per thread; groups of a single variable next to larger ones; a three-round search
+    (3_000, 5000, 2),     # the same kernel over few, large groups
+    (70_000, 30, 9),      # one variable per thread, more members than are in flight at once, a three-round search
+    (1, 700, 33),         # one group
+    (6, 300, 3000),       # more members than a workgroup stages: their offsets straight from memory
+])
+def test_cost_objective_on_synthetic_groups(gpu_device, n_groups, max_size, max_members):
+    """The objective kernel on its own (``torch.ops.apcost.cost_objective``): both of its forms
+    (one / four variables per thread, chosen by the number of variables), groups of one
+    variable, members beyond one round of the member loop, as many groups as take the search
+    for a workgroup's first group three rounds.  Expected values: numpy.bincount, which adds in
+    array order from 0.0 (pinned against the reference's loop in the CPU test above)."""
+    from autoparallel_amd import _native
+
+    rng = np.random.default_rng(n_groups)
+    sizes = rng.integers(1, max_size + 1, n_groups)
+    sizes[rng.random(n_groups) < 0.4] = 1
+    members = rng.integers(1, max_members + 1, n_groups)
+    members[0] = max_members
+    gvb = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+    gmb = np.concatenate([[0], np.cumsum(members)]).astype(np.int64)
+    n_vars = int(gvb[-1])
+    member_size = np.repeat(sizes, members)
+    # the members' entry ranges, in a shuffled order of the groups with gaps between them, ascending inside a group
+    order = rng.permutation(n_groups)
+    group_entries = sizes * members
+    start = np.zeros(n_groups, np.int64)
+    start[order] = np.cumsum(group_entries[order] + 3) - (group_entries[order] + 3)
+    meb = np.repeat(start, members) + (np.arange(gmb[-1]) - np.repeat(gmb[:-1], members)) * member_size
+    n_entries = int((group_entries + 3).sum())
+    cost = rng.uniform(0, 1e4, n_entries)
+    cost[rng.random(n_entries) < 0.01] = np.inf
+    cost[rng.random(n_entries) < 0.001] = np.nan
+    var = np.full(n_entries, -1, np.int64)
+    idx = np.repeat(meb, member_size) + (np.arange(int(member_size.sum())) - np.repeat(np.cumsum(member_size) - member_size, member_size))
+    var[idx] = np.repeat(np.repeat(gvb[:-1], members), member_size) + (idx - np.repeat(meb, member_size))
+    used = var >= 0
+    bad = ~np.isfinite(cost)
+    want = np.bincount(var[used], weights=np.where(bad, 10000.0, cost)[used], minlength=n_vars)
+    want_forced = np.bincount(var[used], weights=bad[used], minlength=n_vars) > 0
+    dev = lambda a: torch.from_numpy(a).to(gpu_device)  # noqa: E731
+    obj, forced = _native.torch_ops().cost_objective(n_vars, dev(gvb), dev(gmb), dev(meb), dev(cost), 10000.0)
+    torch.cuda.synchronize()
+    assert (n_vars >= 1 << 22) == (n_groups == 350_000 or n_groups == 3_000)
+    assert np.array_equal(obj.cpu().numpy(), want)
+    assert np.array_equal(forced.cpu().numpy().astype(bool), want_forced)
+
+
+@pytest.mark.gpu
 def test_planner_pass_on_a_table_whose_rows_do_not_fit_tiles(gpu_device):
     """Producers with more than 64 strategies: the pass writes the cost alone, the row minima are
     taken on request by a segmented minimum over the distinct rows."""

@@ -108,7 +108,7 @@ def test_chain_bound_is_exact():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("seed,n,max_labels", [(0, 8, 5), (1, 40, 70), (2, 25, 130)])
+@pytest.mark.parametrize("seed,n,max_labels", [(0, 8, 5), (1, 40, 70), (2, 25, 130), (3, 150, 24)])
 def test_device_sweeps_equal_the_cpu_restatement(gpu_device, seed, n, max_labels):
     from autoparallel_amd import CostModelParams
     from autoparallel_amd.device_tables import DeviceCostTables
@@ -122,6 +122,47 @@ def test_device_sweeps_equal_the_cpu_restatement(gpu_device, seed, n, max_labels
         want_t, want_u = _sweep(g, theta, unary, chunk)
         theta, unary = dev.diffusion_sweeps(g, theta, unary, chunk)
         assert np.array_equal(theta, want_t) and np.array_equal(unary, want_u), chunk
+
+
+def _star_problem(seed, centre_labels, leaf_labels, p_inf=0.1):
+    """One class joined to every other, the matrices stored either way round."""
+    rng = np.random.default_rng(seed)
+    sizes = [centre_labels] + list(leaf_labels)
+    blocks, costs, var = [], {}, 0
+    for j in range(1, len(sizes)):
+        rows, cols, ci, cj = (sizes[0], sizes[j], 0, j) if j % 2 else (sizes[j], sizes[0], j, 0)
+        m = rng.uniform(0, 100, (rows, cols))
+        m[rng.random(m.shape) < p_inf] = np.inf
+        blocks.append(pruning.Block(var, rows, cols, ci, cj))
+        costs[var] = m
+        var += m.size
+    return pruning.build_label_graph(blocks, sizes, lambda b: costs[b.var_begin], {}, [])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,centre,leaves", [
+    ("more labels than threads of a workgroup", 300, [5, 3, 6]),
+    ("more incident matrices than are staged", 6, [3] * 70),
+    ("as many pairs as are staged", 32, [4] * 64),
+    ("matrices larger than the staging array", 40, [60, 50, 70, 45]),
+    ("a planning program's shape", 16, [16, 12, 9, 16, 15, 15, 8, 12, 16, 16, 22, 24, 16, 16, 16, 16]),
+])
+def test_device_sweeps_on_the_shapes_that_choose_the_kernels_path(gpu_device, name, centre, leaves):
+    """The update kernel stages a class's incident matrices in LDS when their number, the pairs
+    (matrix, label) and the elements fit, and works on them in memory otherwise: the bits of the
+    CPU restatement either way, at the limits and on both sides of them."""
+    from autoparallel_amd import CostModelParams
+    from autoparallel_amd.device_tables import DeviceCostTables
+    from autoparallel_amd.synthetic import stress_dag
+
+    g = _star_problem(7, centre, leaves)
+    dev = DeviceCostTables(stress_dag(seed=1, n_nodes=20, mesh_sizes=(4, 2)), CostModelParams.from_mesh((4, 2)),
+                           device=gpu_device)
+    theta, unary = g.theta, g.unary
+    for chunk in (1, 4):
+        want_t, want_u = _sweep(g, theta, unary, chunk)
+        theta, unary = dev.diffusion_sweeps(g, theta, unary, chunk)
+        assert np.array_equal(theta, want_t) and np.array_equal(unary, want_u), (name, chunk)
 
 
 @pytest.mark.parametrize("seed", range(12))

@@ -338,7 +338,7 @@ def test_strategy_recipes_give_the_flop_counter_path(fake_pg, case):
         o = autop.sharding_optimizer
         assert o.cost_input_stats["strategy_inputs"] == "host"  # the oracle backend has no device
         enc, tb = o.encoded, o.encoded.tables
-        rc = strategy_recipes(enc, o.strats)
+        rc = strategy_recipes(enc, o.strats, mesh)  # (with the check of the bytes-only recipes on, as the planner calls it)
         assert not rc.host_nodes
         _, lshape, _, _, lbytes = c_oracle.spec_tables(tb.as_dict(), mesh)
         strat_node = np.repeat(np.arange(len(enc.nodes)), np.diff(tb.node_strat_begin))
@@ -364,6 +364,41 @@ def test_an_operator_without_a_recipe_takes_the_host_path(fake_pg):
             assert rc.host_nodes and all(n.target.overloadpacket == torch.ops.aten.mm for n in rc.host_nodes)
     finally:
         cost_inputs._CLOSED_FORMS.update(saved)
+
+
+def test_a_bytes_only_recipe_that_does_not_hold_takes_the_host_path(fake_pg, monkeypatch):
+    """A bytes-only recipe rests on the operator returning a tensor of the local shape of its
+    output spec.  At recipe build one sharded strategy per distinct operator call is evaluated
+    the reference's way (compute_estimation.py:232-243, 334-349); an operator whose result
+    differs (here: made to return 8 more bytes, or to count flops) is listed for the host path,
+    and the check runs once per distinct call, not once per node."""
+    from autoparallel_amd.graphs import cost_inputs
+
+    cfg, mesh, batch, seq = CASES["block_1k_batch8_mesh64"]
+    real = cost_inputs._evaluate
+    calls = []
+
+    def evaluate(op, *args):
+        flops, rw_bytes, code = real(op, *args)
+        calls.append(op)
+        if op.overloadpacket == torch.ops.aten.mul:
+            rw_bytes += 8
+        if op.overloadpacket == torch.ops.aten.add:
+            flops += 1
+        return flops, rw_bytes, code
+
+    with _planner(OraclePlanner, cfg, mesh, batch, seq, block=True) as autop:
+        o = autop.sharding_optimizer
+        bytes_only = [n for n in o.encoded.nodes if n.op == "call_function" and not cost_inputs.has_zero_cost(n)
+                      and n.target.overloadpacket not in cost_inputs._CLOSED_FORMS]
+        assert any(n.target.overloadpacket == torch.ops.aten.mul for n in bytes_only)
+        monkeypatch.setattr(cost_inputs, "_evaluate", evaluate)
+        rc = cost_inputs.strategy_recipes(o.encoded, o.strats, mesh)
+        listed = {n.target.overloadpacket for n in rc.host_nodes}
+        assert listed == {torch.ops.aten.mul, torch.ops.aten.add} & {n.target.overloadpacket for n in bytes_only}
+        assert torch.ops.aten.mul in listed
+        assert len(calls) < len(bytes_only) or len(bytes_only) <= len(set(calls))
+        assert not cost_inputs.strategy_recipes(o.encoded, o.strats).host_nodes  # (without mesh sizes nothing is evaluated)
 
 
 def test_einsum_flop_formula_of_the_reference():
