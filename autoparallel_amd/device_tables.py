@@ -455,6 +455,8 @@ class DeviceCostTables:
         if n_groups and (int(group_var_begin[0]) != 0 or int(group_var_begin[-1]) != n_vars
                          or int(group_member_begin[-1]) != len(member_entry_begin)):
             raise ValueError("group pointers do not span the variables / members")
+        if n_groups and not bool((np.diff(np.asarray(group_var_begin, np.int64)) > 0).all()):
+            raise ValueError("every variable group needs at least one variable (the kernel takes one workgroup per group)")
         return self.ops.cost_objective(int(n_vars), gv, gm, me, self.fetch("cost"), float(self.params.inf_replacement_cost))
 
     @_guarded

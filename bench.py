@@ -585,8 +585,6 @@ def roofline_of(dev, tables, timing, steps, pass_kind):
 
 def launch_shape(dev, tables, main):
     """(workgroups, threads) of the launch that writes the matrices, as the library sizes it."""
-    import numpy as np
-
     n_tiles = tables.n_tiles
     tile_blocks = (n_tiles + 7) // 8 * 8
     if main == "build_tables_packed":

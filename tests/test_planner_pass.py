@@ -161,6 +161,22 @@ def test_cost_objective_on_synthetic_groups(gpu_device, n_groups, max_size, max_
 
 
 @pytest.mark.gpu
+def test_cost_objective_refuses_an_empty_group(gpu_device):
+    """The objective kernel takes one workgroup per variable group and never searches for the
+    group of a variable: the host wrapper refuses pointers that do not ascend strictly."""
+    tb = stress_dag(seed=21, n_nodes=60, mesh_sizes=(4, 2))
+    d = DeviceCostTables(tb, CostModelParams.from_mesh((4, 2)), device=gpu_device)
+    for launch in d.planner_pass().values():
+        launch()
+    n_vars, gvb, gmb, meb, _ = _groups(tb, np.random.default_rng(0), False)
+    d.cost_objective(n_vars, gvb, gmb, meb)
+    bad = gvb.copy()
+    bad[3] = bad[2]
+    with pytest.raises(ValueError, match="at least one variable"):
+        d.cost_objective(n_vars, bad, gmb, meb)
+
+
+@pytest.mark.gpu
 def test_planner_pass_on_a_table_whose_rows_do_not_fit_tiles(gpu_device):
     """Producers with more than 64 strategies: the pass writes the cost alone, the row minima are
     taken on request by a segmented minimum over the distinct rows."""
