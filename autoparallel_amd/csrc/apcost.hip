@@ -2398,14 +2398,18 @@ __device__ void diffusion_update_in_memory(const DiffusionArgs &a, double *s_tot
 // element by bisecting the staged offsets), minima, totals and shares out of LDS, and every
 // element stored once.  Element by element the arithmetic is that of the path above, in the
 // same order: (v - d) where the row has a finite minimum, then + share or +inf.
-constexpr int kDiffusionStagedElements = 8192;  // doubles of LDS for the incident matrices of a class
+// (48 KB of LDS in all, so that a compute unit holds three classes: the largest class of the planning programs
+// measured has 3 856 elements and 256 pairs)
+constexpr int kDiffusionStagedElements = 4096;  // doubles of LDS for the incident matrices of a class
 constexpr int kDiffusionStagedDegree = 64;      // incident matrices of a class
-constexpr int kDiffusionStagedPairs = 2048;     // (incident matrix, label) pairs of a class
+constexpr int kDiffusionStagedPairs = 1024;     // (incident matrix, label) pairs of a class
+static_assert(kDiffusionStagedElements >= kDiffusionMaxLabels, "the update in memory keeps its totals where the matrices are staged");
 
 __global__ __launch_bounds__(kBlock) void diffusion_node_update_kernel(DiffusionArgs a) {
-  __shared__ double s_tot[kDiffusionMaxLabels];
   __shared__ double s_m[kDiffusionStagedElements];
   __shared__ double s_d[kDiffusionStagedPairs];
+  __shared__ double s_share[kDiffusionStagedPairs];  // (a staged class has at most kDiffusionStagedPairs labels)
+  double *s_tot = s_m;                               // the update in memory stages no matrix: its totals lie there
   __shared__ int64_t s_base[kDiffusionStagedDegree];
   __shared__ int s_off[kDiffusionStagedDegree + 1];
   __shared__ int s_other[kDiffusionStagedDegree];
@@ -2505,7 +2509,7 @@ __global__ __launch_bounds__(kBlock) void diffusion_node_update_kernel(Diffusion
     double tot = x == tid && tid < n_labels ? unary : a.unary[l0 + x];
     for (int t = 0; t < degree; ++t) tot += s_d[t * n_labels + x];
     const bool finite = tot < inf;
-    s_tot[x] = finite ? tot / (double)degree : inf;
+    s_share[x] = finite ? tot / (double)degree : inf;
     a.unary[l0 + x] = finite ? 0.0 : inf;
   }
   __syncthreads();
@@ -2513,7 +2517,7 @@ __global__ __launch_bounds__(kBlock) void diffusion_node_update_kernel(Diffusion
     const int t = matrix_of(g);
     const int e = g - s_off[t];
     const int x = s_side[t] == 0 ? e / s_other[t] : e % n_labels;
-    const double share = s_tot[x];
+    const double share = s_share[x];
     a.theta[s_base[t] + e] = share < inf ? s_m[g] + share : inf;
   }
 }

@@ -143,7 +143,9 @@ def _star_problem(seed, centre_labels, leaf_labels, p_inf=0.1):
 @pytest.mark.parametrize("name,centre,leaves", [
     ("more labels than threads of a workgroup", 300, [5, 3, 6]),
     ("more incident matrices than are staged", 6, [3] * 70),
-    ("as many pairs as are staged", 32, [4] * 64),
+    ("as many pairs and elements as are staged", 16, [4] * 64),
+    ("one pair of labels more than is staged", 17, [3] * 64),
+    ("a few elements more than are staged", 16, [4] * 63 + [5]),
     ("matrices larger than the staging array", 40, [60, 50, 70, 45]),
     ("a planning program's shape", 16, [16, 12, 9, 16, 15, 15, 8, 12, 16, 16, 22, 24, 16, 16, 16, 16]),
 ])
