@@ -58,6 +58,16 @@ template <typename T>
 __device__ __forceinline__ T uniform_load(const T *p) {
   return *(const APC_CONSTANT T *)p;
 }
+// A plain store that is written through to memory (system scope, no ordering).  What a launch of
+// a few tens of MB leaves in the L2 is written back when the kernel ends, after its last
+// wavefront, and the launch lasts until that is done; written through, the lines leave while the
+// wavefronts still work.  For the tables of a small pass only: a large table streams through the
+// L2 anyway, and its tile kernels lose what the L2 does for them when neighbouring wavefronts fill
+// a line together (write-through there: Llama-3-70B 126 -> 221 us, the stress table 1.19 -> 1.24 ms).
+template <typename T>
+__device__ __forceinline__ void store_through(T *p, T value) {
+  __hip_atomic_store(p, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 typedef int32_t i32x16 __attribute__((ext_vector_type(16)));
 typedef int64_t i64x8 __attribute__((ext_vector_type(8)));
 
@@ -348,15 +358,21 @@ __device__ __forceinline__ void tensor_bytes_and_contiguity(int r, int64_t items
   tensor_bytes_and_contiguity_of(r, itemsize, x, y, nbytes, contiguous);
 }
 
-template <int BS>
+// THROUGH: the rows are written through to memory (the packed pass: see store_through)
+template <int BS, bool THROUGH = false>
 __device__ __forceinline__ void tensor_tables_block(int64_t block, const TensorTableArgs &a) {
   const int64_t t = block * BS + threadIdx.x;
   if (t >= a.n) return;
   int64_t nbytes;
   bool ok;
   tensor_bytes_and_contiguity(a.rank[t], a.itemsize[t], a.shape + t * APC_MAX_RANK, a.stride + t * APC_MAX_RANK, nbytes, ok);
-  a.bytes[t] = nbytes;
-  a.cont[t] = ok ? 1 : 0;
+  if (THROUGH) {
+    store_through(a.bytes + t, nbytes);
+    store_through(a.cont + t, (uint8_t)(ok ? 1 : 0));
+  } else {
+    a.bytes[t] = nbytes;
+    a.cont[t] = ok ? 1 : 0;
+  }
 }
 
 __global__ __launch_bounds__(kBlock) void tensor_tables_kernel(TensorTableArgs a) {
@@ -531,7 +547,7 @@ __device__ __forceinline__ double compute_cost_through_reciprocals(const apc_par
   return t > rw ? t : rw;
 }
 
-template <int BS>
+template <int BS, bool THROUGH = false>
 __device__ __forceinline__ void compute_costs_block(int64_t block, const apc_params &p, const ComputeCostArgs &a) {
   const int64_t s = block * BS + threadIdx.x;
   if (s >= a.n) return;
@@ -545,8 +561,14 @@ __device__ __forceinline__ void compute_costs_block(int64_t block, const apc_par
   const double c = compute_cost_through_reciprocals(p, zero, a.rw_bytes[s], flops, gf, inv_gf);
   const bool unsupported = !zero && flops != 0 && gf == 0.0;
   if (unsupported && a.error_flag) *a.error_flag = 1;
-  if (a.compute) a.compute[s] = c;
-  if (a.per_arg) a.per_arg[s] = c / (double)a.num_args[s];
+  const double per_arg = c / (double)a.num_args[s];
+  if (THROUGH) {
+    if (a.compute) store_through(a.compute + s, c);
+    if (a.per_arg) store_through(a.per_arg + s, per_arg);
+  } else {
+    if (a.compute) a.compute[s] = c;
+    if (a.per_arg) a.per_arg[s] = per_arg;
+  }
 }
 
 __global__ __launch_bounds__(kBlock) void compute_costs_kernel(apc_params p, ComputeCostArgs a) {
@@ -1861,11 +1883,14 @@ __device__ __forceinline__ int64_t from_lane_i64(int64_t v, int lane) {
 // into per-lane 64-bit arithmetic inside a loop over bases).  A store needs no wait before the
 // wavefront ends, and a wait by count for an older load stays correct with younger stores in
 // flight (loads return in order among themselves).
+// (sc0 sc1: the store is written through to memory.  Left in the L2 until the kernel ends, the
+// table's lines are written back after the last wavefront has finished, and a launch of this
+// size waits for that: 10.0 -> 8.6 us on the Llama-3-8B table.)
 // (s_nop 4: a vector-memory instruction may read a scalar register a vector instruction wrote,
 // such as a value fetched from a lane, only five cycles later; the compiler inserts that wait
 // for its own instructions and does not look inside an asm statement.)
 __device__ __forceinline__ void store_at(double *base, uint32_t byte_offset, double value) {
-  __asm__ volatile("s_nop 4\n\tglobal_store_dwordx2 %0, %1, %2" ::"v"(byte_offset), "v"(value), "s"(base) : "memory");
+  __asm__ volatile("s_nop 4\n\tglobal_store_dwordx2 %0, %1, %2 sc0 sc1" ::"v"(byte_offset), "v"(value), "s"(base) : "memory");
 }
 
 struct PackedArgs {
@@ -2036,8 +2061,8 @@ __device__ __forceinline__ void packed_tile(const apc_packed_tile *T, double *co
       const int64_t first_row = from_lane_i64(copies.row0, copy - 1);  // (every lane takes part)
       if (row_live && copy_slot < copies_per_store && copy <= dup_count) {
         const int64_t out = (copy == 0 ? row_begin : first_row) + row0 + q;
-        a.row_min_out[out] = m_q;
-        a.row_arg_out[out] = mc_q;
+        store_through(a.row_min_out + out, m_q);
+        store_through(a.row_arg_out + out, mc_q);
       }
     }
   }
@@ -2057,8 +2082,8 @@ __global__ __launch_bounds__(kBlock) void build_tables_packed_kernel(const apc_p
     return;
   }
   const int64_t tb = b - tile_blocks;
-  if (tb < tensor_blocks) tensor_tables_block<kBlock>(tb, t);
-  else compute_costs_block<kBlock>(tb - tensor_blocks, p, c);
+  if (tb < tensor_blocks) tensor_tables_block<kBlock, true>(tb, t);
+  else compute_costs_block<kBlock, true>(tb - tensor_blocks, p, c);
 }
 
 // ------------------------------------------------------------------------------------------
