@@ -3330,6 +3330,8 @@ __global__ void calibrate_empty_kernel() {}
 
 // Workgroup b writes doubles [b * per_workgroup, (b + 1) * per_workgroup) of out (clipped to n),
 // 16 bytes per lane and store instruction, consecutive lanes consecutive addresses.
+// THROUGH: the stores are written through to memory (store_through), as the packed pass writes.
+template <bool THROUGH>
 __global__ __launch_bounds__(kBlock) void calibrate_fill_kernel(double *__restrict__ out, int64_t n, int64_t per_workgroup,
                                                                 double value) {
   typedef double pair_t __attribute__((ext_vector_type(2)));
@@ -3337,8 +3339,17 @@ __global__ __launch_bounds__(kBlock) void calibrate_fill_kernel(double *__restri
   const int64_t end = begin + per_workgroup < n ? begin + per_workgroup : n;
   const pair_t v = {value, value};
   int64_t i = begin + 2 * (int64_t)threadIdx.x;
-  for (; i + 1 < end; i += 2 * kBlock) *reinterpret_cast<pair_t *>(out + i) = v;
-  if (i < end) out[i] = value;
+  for (; i + 1 < end; i += 2 * kBlock) {
+    if (THROUGH) {
+      __asm__ volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(out + i), "v"(v) : "memory");
+    } else {
+      *reinterpret_cast<pair_t *>(out + i) = v;
+    }
+  }
+  if (i < end) {
+    if (THROUGH) store_through(out + i, value);
+    else out[i] = value;
+  }
 }
 
 }  // namespace
@@ -3352,15 +3363,19 @@ int apc_calibrate_launch(int64_t n_workgroups, int32_t threads, void *stream) {
   return check_launch("apc_calibrate_launch");
 }
 
-int apc_calibrate_fill(double *out, int64_t n, int64_t per_workgroup, double value, void *stream) {
+int apc_calibrate_fill(double *out, int64_t n, int64_t per_workgroup, double value, int32_t write_through, void *stream) {
   if (n < 0 || per_workgroup < 2 || (per_workgroup & 1)) return fail(-1, "apc_calibrate_fill: n >= 0, per_workgroup even and >= 2");
   if (n == 0) return 0;
   if (!out) return fail(-1, "apc_calibrate_fill: NULL array");
   if ((reinterpret_cast<uintptr_t>(out) & 15) != 0) return fail(-1, "apc_calibrate_fill: out must be 16-byte aligned");
   const int64_t blocks = (n + per_workgroup - 1) / per_workgroup;
   if (blocks > INT32_MAX) return fail(-1, "apc_calibrate_fill: too many workgroups");
-  hipLaunchKernelGGL(calibrate_fill_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, (hipStream_t)stream, out, n, per_workgroup,
-                     value);
+  if (write_through)
+    hipLaunchKernelGGL(calibrate_fill_kernel<true>, dim3((unsigned)blocks), dim3(kBlock), 0, (hipStream_t)stream, out, n,
+                       per_workgroup, value);
+  else
+    hipLaunchKernelGGL(calibrate_fill_kernel<false>, dim3((unsigned)blocks), dim3(kBlock), 0, (hipStream_t)stream, out, n,
+                       per_workgroup, value);
   return check_launch("apc_calibrate_fill");
 }
 

@@ -482,7 +482,8 @@ def verify_pass(dev, tables, params, log):
 def calibrate_launch(nbytes, grid, threads):
     """What a launch of this shape costs before it does any work, and what a kernel that only
     writes ``nbytes`` takes (the library's measurement kernels, back to back on the current stream,
-    one HIP event pair around the run): -> (launch_floor_us, fill_us, the fill's doubles per workgroup)."""
+    one HIP event pair around the run): -> (launch_floor_us, fill_us, the fill's doubles per workgroup,
+    whether the fastest fill wrote through to memory)."""
     import ctypes
 
     import torch
@@ -513,15 +514,16 @@ def calibrate_launch(nbytes, grid, threads):
     n = nbytes // 8
     buf = torch.empty(n + 2, dtype=torch.float64, device="cuda:0")
     best = None
-    for per in (512, 2048, 8192, 16384):
-        def fill():
-            _native.check(lib.apc_calibrate_fill(ctypes.c_void_p(buf.data_ptr()), ctypes.c_int64(n), ctypes.c_int64(per),
-                                                 ctypes.c_double(1.0), stream), "apc_calibrate_fill")
-        us = timed(fill, k)
-        if best is None or us < best[0]:
-            best = (us, per)
+    for through in (0, 1):
+        for per in (512, 2048, 8192, 16384):
+            def fill():
+                _native.check(lib.apc_calibrate_fill(ctypes.c_void_p(buf.data_ptr()), ctypes.c_int64(n), ctypes.c_int64(per),
+                                                     ctypes.c_double(1.0), ctypes.c_int32(through), stream), "apc_calibrate_fill")
+            us = timed(fill, k)
+            if best is None or us < best[0]:
+                best = (us, per, through)
     del buf
-    return floor_us, best[0], best[1]
+    return floor_us, best[0], best[1], best[2]
 
 
 def roofline_of(dev, tables, timing, steps, pass_kind):
@@ -553,7 +555,7 @@ def roofline_of(dev, tables, timing, steps, pass_kind):
     single = len(names) == 1
     t_kernel = timing["region_ms"] * 1e-3 / steps if single else t_pair
     grid, threads = launch_shape(dev, tables, main)
-    floor_us, fill_us, fill_per_wg = calibrate_launch(priced, grid, threads)
+    floor_us, fill_us, fill_per_wg, fill_through = calibrate_launch(priced, grid, threads)
     return {
         "bound": "hbm",
         "kernel": ("build_tables_packed_kernel" if packed else "build_tables_kernel" if one_launch else
@@ -574,7 +576,8 @@ def roofline_of(dev, tables, timing, steps, pass_kind):
         "launch_floor_us": floor_us, "fill_us": fill_us, "frac_of_fill": fill_us / (t_kernel * 1e6),
         "calibration": f"apc_calibrate_launch: an empty kernel of the launch's grid ({grid} workgroups of {threads} threads) "
                        f"back to back; apc_calibrate_fill: a kernel that only writes bytes_per_launch ({fill_per_wg} doubles "
-                       "per workgroup, the fastest of four splits), same timing",
+                       f"per workgroup, stores {'written through to memory' if fill_through else 'left to the L2'}: the fastest "
+                       "of four splits x two kinds of store), same timing",
         "avg_launch_us_event_pair_per_launch": t_pair * 1e6,
         "min_launch_us_event_pair_per_launch": timing["kernel_ms_min"][main] * 1e3,
         "timing": ("one HIP event pair on the launch stream around the K back-to-back launches of the timed "
@@ -740,9 +743,10 @@ def main():
         # the three workloads' launch shapes and bytes (bytes_per_launch of their roofline objects)
         for name, nbytes, grid, threads in (("llama3_8b", 20_766_135, 1352, 256), ("llama3_70b", 596_653_014, 11736, 256),
                                            ("stress", 3_825_705_690, 426920, 128)):
-            floor_us, fill_us, per = calibrate_launch(nbytes, grid, threads)
+            floor_us, fill_us, per, through = calibrate_launch(nbytes, grid, threads)
             print(json.dumps({"workload": name, "bytes": nbytes, "grid": grid, "threads": threads, "launch_floor_us": floor_us,
-                              "fill_us": fill_us, "fill_doubles_per_workgroup": per, "fill_TBps": nbytes / fill_us / 1e6}))
+                              "fill_us": fill_us, "fill_doubles_per_workgroup": per, "fill_written_through": bool(through),
+                              "fill_TBps": nbytes / fill_us / 1e6}))
         return
     if args.calibrate_copy:
         src = torch.ones(1 << 27, dtype=torch.float64, device="cuda:0")  # 1 GiB

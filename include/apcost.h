@@ -459,9 +459,12 @@ int apc_build_tables_packed(const apc_params *params, int64_t n_tensors, const i
  * a launch costs on the system before any work.  apc_calibrate_fill enqueues a kernel that only
  * writes: out[0 .. n) = value, workgroup b taking doubles [b * per_workgroup, (b + 1) *
  * per_workgroup) (even, >= 2; 256 threads, 16-byte stores; out 16-byte aligned): the ceiling of
- * the store path for a launch that moves the same bytes as a table build. */
+ * the store path for a launch that moves the same bytes as a table build.  write_through != 0:
+ * the stores are written through to memory instead of being left in the L2 until the kernel ends
+ * (what apc_build_tables_packed does with its own stores; the faster of the two on a launch of a
+ * few tens of MB, the slower on one that streams through the L2). */
 int apc_calibrate_launch(int64_t n_workgroups, int32_t threads, void *stream);
-int apc_calibrate_fill(double *out, int64_t n, int64_t per_workgroup, double value, void *stream);
+int apc_calibrate_fill(double *out, int64_t n, int64_t per_workgroup, double value, int32_t write_through, void *stream);
 
 #ifdef __cplusplus
 }
