@@ -2061,8 +2061,10 @@ __device__ __forceinline__ void packed_tile(const apc_packed_tile *T, double *co
       const int64_t first_row = from_lane_i64(copies.row0, copy - 1);  // (every lane takes part)
       if (row_live && copy_slot < copies_per_store && copy <= dup_count) {
         const int64_t out = (copy == 0 ? row_begin : first_row) + row0 + q;
-        store_through(a.row_min_out + out, m_q);
-        store_through(a.row_arg_out + out, mc_q);
+        // (plain stores: written through, these 8- and 4-byte pieces cost whole sectors of HBM
+        // writes, 21.0 instead of 19.2 MB per launch, for 0.15 us)
+        a.row_min_out[out] = m_q;
+        a.row_arg_out[out] = mc_q;
       }
     }
   }
