@@ -668,3 +668,30 @@ def test_cpp_consumer_of_the_c_abi(gpu_device):
     run = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert run.returncode == 0, run.stdout + run.stderr
     assert "abi consumer ok" in run.stdout
+
+
+@pytest.mark.parametrize("write_through", [0, 1])
+def test_measurement_kernels_do_what_they_say(gpu_device, write_through):
+    """apc_calibrate_fill writes exactly out[0 .. n) (both kinds of store, an odd count, a
+    workgroup that gets a partial run), apc_calibrate_launch runs and touches nothing, and both
+    refuse arguments that make no sense."""
+    import ctypes
+
+    from autoparallel_amd import _native
+
+    lib = _native.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    n = 100_001
+    buf = torch.full((n + 6,), -1.0, dtype=torch.float64, device=gpu_device)
+    rc = lib.apc_calibrate_fill(ctypes.c_void_p(buf.data_ptr()), ctypes.c_int64(n), ctypes.c_int64(2048), ctypes.c_double(3.25),
+                                ctypes.c_int32(write_through), stream)
+    _native.check(rc, "apc_calibrate_fill")
+    _native.check(lib.apc_calibrate_launch(ctypes.c_int64(777), ctypes.c_int32(128), stream), "apc_calibrate_launch")
+    torch.cuda.synchronize()
+    got = buf.cpu().numpy()
+    assert (got[:n] == 3.25).all() and (got[n:] == -1.0).all()
+    assert lib.apc_calibrate_fill(ctypes.c_void_p(buf.data_ptr()), ctypes.c_int64(n), ctypes.c_int64(7), ctypes.c_double(0.0),
+                                  ctypes.c_int32(write_through), stream) != 0
+    assert lib.apc_calibrate_fill(ctypes.c_void_p(buf.data_ptr() + 8), ctypes.c_int64(n), ctypes.c_int64(8), ctypes.c_double(0.0),
+                                  ctypes.c_int32(write_through), stream) != 0
+    assert lib.apc_calibrate_launch(ctypes.c_int64(0), ctypes.c_int32(128), stream) != 0
