@@ -555,6 +555,8 @@ class CostTables:
         # byte counts must convert to fp64 exactly (the kernels divide them as doubles)
         if self.n_tensors:
             r = np.arange(APC_MAX_RANK)[None, :] < self.tensor_rank[:, None]
+            if (np.where(r, self.tensor_shape, 0) < 0).any():
+                raise RuntimeError("tensor sizes must not be negative")
             numel = np.where(r, self.tensor_shape, 1).astype(object).prod(axis=1)
             if (numel * self.tensor_itemsize.astype(object) >= 2**53).any():
                 raise RuntimeError("tensor byte counts must stay below 2**53")

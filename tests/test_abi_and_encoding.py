@@ -304,6 +304,13 @@ def test_validator_rejects_a_tile_with_more_identical_edges_than_the_kernels_sta
             tb.validate(params)
 
 
+def test_validator_rejects_a_negative_tensor_size():
+    tb = _small()
+    tb.tensor_shape[0, 0] = -4
+    with pytest.raises(RuntimeError, match="must not be negative"):
+        tb.validate(CostModelParams.from_mesh((4, 2)))
+
+
 def test_validator_needs_pass_through_values_for_producerless_edges():
     tb = _small()
     e = int(np.nonzero(tb.edge_flags & EDGE_NO_PRODUCER)[0][0])

@@ -87,6 +87,52 @@ def test_operators_match_the_oracle(small_table):
 
 
 @pytest.mark.gpu
+def test_tensor_table_on_shapes_with_empty_and_unit_dims(gpu_device):
+    """Bytes and contiguity (torch spec_to_bytes, check_contiguous_sizes_strides) of hand-made
+    rows: dims of size 0 (after which the expected stride is 0, or the product with sizes below
+    1 counted as 1), dims of size 1 with any stride, rank 0, non-contiguous and permuted strides,
+    random rows; against the oracle and, for contiguity, against torch's own function."""
+    from torch._prims_common import check_contiguous_sizes_strides
+
+    rows = [((), ()), ((5,), (1,)), ((5,), (2,)), ((4, 3), (3, 1)), ((4, 3), (1, 4)), ((4, 1, 3), (3, 77, 1)),
+            ((4, 0, 3), (0, 3, 1)), ((4, 0, 3), (3, 3, 1)), ((4, 0, 3), (0, 0, 1)), ((0,), (1,)), ((0,), (5,)),
+            ((2, 0, 0, 3), (0, 0, 3, 1)), ((2, 0, 0, 3), (3, 3, 3, 1)), ((2, 0, 0, 3), (9, 3, 3, 1)),
+            ((1, 1, 1), (9, 8, 7)), ((2, 3, 4, 5, 6, 7, 8, 9), (181440, 60480, 15120, 3024, 504, 72, 9, 1)),
+            ((2, 3, 4, 5, 6, 7, 8, 9), (181440, 60480, 15120, 3024, 504, 72, 1, 8)), ((3, 1, 0, 1, 2), (0, 5, 2, 9, 1))]
+    rng = np.random.default_rng(5)
+    for _ in range(300):
+        r = int(rng.integers(0, 9))
+        shape = [int(x) for x in rng.choice([0, 1, 1, 2, 3, 5, 8], r)]
+        stride = []
+        z = 1
+        for x in reversed(shape):  # contiguous strides, then some of them disturbed
+            stride.append(z)
+            z *= max(x, 1) if rng.random() < 0.5 else x
+        stride = list(reversed(stride))
+        for i in range(r):
+            if rng.random() < 0.15:
+                stride[i] = int(rng.integers(0, 50))
+        rows.append((tuple(shape), tuple(stride)))
+    n = len(rows)
+    rank = np.asarray([len(s) for s, _ in rows], np.int32)
+    itemsize = np.asarray([(1, 2, 4, 8)[i % 4] for i in range(n)], np.int32)
+    shape = np.zeros((n, 8), np.int64)
+    stride = np.zeros((n, 8), np.int64)
+    for i, (sh, st) in enumerate(rows):
+        shape[i, :len(sh)] = sh
+        stride[i, :len(st)] = st
+    enc = {"tensor_rank": rank, "tensor_itemsize": itemsize, "tensor_shape": shape, "tensor_stride": stride}
+    wb, wc = po.tensor_tables(enc)
+    for (sh, st), c in zip(rows, wc):
+        assert bool(c) == bool(check_contiguous_sizes_strides(sh, st, False)), (sh, st)
+    assert {0, 1} == set(wc) and 0 in wb
+    ops = _native.torch_ops()
+    nbytes, contiguous = ops.tensor_tables(*(_to_device(a, gpu_device) for a in (rank, itemsize, shape, stride)))
+    assert np.array_equal(nbytes.cpu().numpy(), np.asarray(wb, np.int64))
+    assert np.array_equal(contiguous.cpu().numpy(), np.asarray(wc, np.uint8))
+
+
+@pytest.mark.gpu
 def test_lengths_that_disagree_are_rejected(small_table):
     mesh, tb, p, d, want = small_table
     ops = _native.torch_ops()
