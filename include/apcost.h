@@ -445,7 +445,9 @@ int apc_validate_packed_tiles_host(int64_t n_tensors, const int32_t *tensor_rank
  * registers (collective_runtime_estimation.py:37-153 directly, no staging in LDS, no barrier),
  * takes their minima and stores values and minima to the tile's edge and to every identical
  * edge.  tensor_* / strategy arrays as in apc_build_tables (a tile whose producer specs name
- * several tensors reads the tensor table).  cost_out [n_entries], row_min / row_argmin [n_rows]. */
+ * several tensors reads the tensor table).  cost_out [n_entries], row_min / row_argmin [n_rows].
+ * The cost entries and the table rows are written through to memory (a launch of this size would
+ * otherwise wait, after its last wavefront, for the L2 to write them back). */
 int apc_build_tables_packed(const apc_params *params, int64_t n_tensors, const int32_t *tensor_rank,
                             const int32_t *tensor_itemsize, const int64_t *tensor_shape, const int64_t *tensor_stride,
                             int64_t *tensor_bytes, uint8_t *tensor_contiguous, int64_t n_strategies, const int64_t *flops,
