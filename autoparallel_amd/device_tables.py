@@ -41,6 +41,10 @@ def _to_device(a: np.ndarray, device) -> torch.Tensor:
     return torch.from_numpy(a).to(device, non_blocking=False)
 
 
+_TORCH_DTYPE = {np.int32: torch.int32, np.int64: torch.int64, np.uint8: torch.uint8, np.float64: torch.float64,
+                np.int8: torch.int8, np.uint32: torch.int32}
+
+
 class DeviceCostTables:
     @_guarded
     def __init__(self, tables: CostTables, params: CostModelParams, device="cuda:0", validate=True):
@@ -552,21 +556,42 @@ class DeviceCostTables:
     def diffusion_sweeps(self, graph, theta: np.ndarray, unary: np.ndarray, n_sweeps: int):
         """``n_sweeps`` sweeps of min-sum diffusion (``apc_diffusion_sweeps``) over ``graph``
         (``pruning.LabelGraph``) starting from the host arrays ``theta`` / ``unary``; returns the
-        updated pair as new host arrays.  The graph's index arrays are uploaded once."""
+        updated pair as new host arrays (read-only: handed back to the next call unchanged, they
+        are not uploaded again).  The graph's index arrays are uploaded once, as one buffer."""
         cached = getattr(self, "_diffusion_graph", None)
         if cached is None or cached[0] is not graph:
             names = ("color_nodes", "label_begin", "inc_begin", "inc_edge", "inc_side", "edge_begin", "edge_i", "edge_j")
-            cached = (graph, {k: _to_device(np.ascontiguousarray(getattr(graph, k)), self.device) for k in names})
+            # one host buffer, one copy: every array at a 16-byte boundary, viewed with its own dtype on the device
+            arrays = {k: np.ascontiguousarray(getattr(graph, k)) for k in names}
+            offsets, size = {}, 0
+            for k, a in arrays.items():
+                offsets[k] = size
+                size += -(-a.nbytes // 16) * 16
+            packed = np.zeros(max(size, 16), np.uint8)
+            for k, a in arrays.items():
+                packed[offsets[k]:offsets[k] + a.nbytes] = a.view(np.uint8).reshape(-1)
+            on_device = torch.from_numpy(packed).to(self.device)
+            views = {k: on_device[offsets[k]:offsets[k] + a.nbytes].view(_TORCH_DTYPE[a.dtype.type]) for k, a in arrays.items()}
+            cached = (graph, views, on_device)
             self._diffusion_graph = cached
+            self._diffusion_state = None
         d = cached[1]
-        th = torch.from_numpy(np.ascontiguousarray(theta, np.float64)).to(self.device)
-        un = torch.from_numpy(np.ascontiguousarray(unary, np.float64)).to(self.device)
+        state = getattr(self, "_diffusion_state", None)
+        if state is not None and state[0] is theta and state[1] is unary:
+            th, un = state[2], state[3]  # what the last call left on the device, returned as these very arrays
+        else:
+            th = torch.from_numpy(np.ascontiguousarray(theta, np.float64)).to(self.device)
+            un = torch.from_numpy(np.ascontiguousarray(unary, np.float64)).to(self.device)
         color_begin = torch.from_numpy(np.ascontiguousarray(graph.color_begin, np.int64))
         max_labels = int(np.diff(graph.label_begin).max()) if graph.n_classes else 0
         self.ops.diffusion_sweeps_(int(n_sweeps), color_begin, d["color_nodes"], d["label_begin"], d["inc_begin"],
                                    d["inc_edge"], d["inc_side"], d["edge_begin"], d["edge_i"], d["edge_j"], max_labels,
                                    int(graph.label_begin[-1]), int(graph.edge_begin[-1]), th, un)
-        return th.cpu().numpy(), un.cpu().numpy()
+        theta_out, unary_out = th.cpu().numpy(), un.cpu().numpy()
+        theta_out.setflags(write=False)
+        unary_out.setflags(write=False)
+        self._diffusion_state = (theta_out, unary_out, th, un)
+        return theta_out, unary_out
 
     @_guarded
     def strategy_bounds(self, row_min: torch.Tensor) -> torch.Tensor:
